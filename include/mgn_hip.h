@@ -1,0 +1,150 @@
+/*
+ * mgn_hip.h — C ABI of libmgn_hip: MI355X (gfx950) kernels for meganeura's
+ * quantized matmul path, i.e. `matmul` nodes whose B operand is a
+ * `parameter_q4` / `parameter_q8` weight.
+ *
+ * This is the boundary a host runtime binds in place of its own GPU dispatch
+ * for those nodes.  Each entry point names the reference interface it stands
+ * in for (paths relative to the reference checkout, kvark/meganeura v0.2.0).
+ *
+ * Conventions
+ *   - every call returns an mgn_status; nothing throws or aborts across the ABI
+ *     (the reference panics: `unknown parameter`, `rows % 32`; here those are
+ *     MGN_EINVAL / MGN_ENOTFOUND and mgn_last_error() holds the message);
+ *   - handles are opaque and owned by the caller, who frees them with the
+ *     matching *_free / *_destroy before destroying the context;
+ *   - one HIP stream per context; matmul calls are asynchronous on it, like
+ *     Session::step (src/runtime.rs:2843), and mgn_sync is Session::wait
+ *     (src/runtime.rs:2835);
+ *   - a context is thread-compatible, not thread-safe (the reference's Session
+ *     is `&mut self` everywhere);
+ *   - matrices are row-major; a weight is W[K,N] with K = rows = the reduction
+ *     dimension, which must be a multiple of 32 (src/runtime.rs:2037-2040).
+ */
+#ifndef MGN_HIP_H
+#define MGN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum mgn_status {
+  MGN_OK = 0,
+  MGN_EINVAL = 1,    /* bad argument: null handle, rows % 32 != 0, size mismatch */
+  MGN_ENOMEM = 2,    /* host or device allocation failed */
+  MGN_EHIP = 3,      /* a HIP runtime call failed; see mgn_last_error */
+  MGN_ENOTFOUND = 4, /* unknown name (session layer) */
+  MGN_ENODEVICE = 5  /* no usable gfx950 device */
+} mgn_status;
+
+/* compile::WeightFormat::{Q4,Q8} (src/compile.rs:8-29), graph::DType::{Q4_0,Q8_0}
+ * (src/graph.rs:6-27).  Q4 is the asymmetric scale+min format the reference
+ * stores under the name Q4_0. */
+typedef enum mgn_fmt { MGN_FMT_Q4 = 0, MGN_FMT_Q8 = 1 } mgn_fmt;
+
+/* Which kernel family serves a matmul; MGN_ROUTE_AUTO is what a runtime uses.
+ * The others exist so that tests can drive every kernel at every shape. */
+typedef enum mgn_route {
+  MGN_ROUTE_AUTO = 0,
+  MGN_ROUTE_GENERIC = 1, /* scalar f32 fallback, any M */
+  MGN_ROUTE_GEMV = 2,    /* streaming dequant-GEMV, small M */
+  MGN_ROUTE_MFMA = 3     /* nibble/int8 x fp16 on MFMA with per-block rescale */
+} mgn_route;
+
+typedef struct mgn_ctx mgn_ctx;
+typedef struct mgn_buf mgn_buf;
+typedef struct mgn_weight mgn_weight;
+
+/* ---- context: blade_graphics::Context::init + Session::new
+ *      (src/runtime.rs:1513-1524, 2012-2024; device chosen by index as
+ *      MEGANEURA_DEVICE_ID does). */
+mgn_status mgn_ctx_create(int device_id, mgn_ctx** out);
+void mgn_ctx_destroy(mgn_ctx* ctx);
+/* Message of the last failed call on this context ("" if none).  With a null
+ * ctx: the message of the last failed mgn_ctx_create on this thread. */
+const char* mgn_last_error(const mgn_ctx* ctx);
+/* Session::wait (src/runtime.rs:2835-2841). */
+mgn_status mgn_sync(mgn_ctx* ctx);
+/* Test hook: force a kernel family (default MGN_ROUTE_AUTO). */
+mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route);
+
+/* ---- plain device buffers: the reference allocates every plan buffer
+ *      zero-filled (src/runtime.rs:1737-1755) and moves data with memcpy
+ *      through mapped memory (upload_buffer 2552-2558, read_buffer 2623-2629). */
+mgn_status mgn_buf_alloc(mgn_ctx* ctx, size_t bytes, mgn_buf** out); /* zero-filled */
+void mgn_buf_free(mgn_ctx* ctx, mgn_buf* buf);
+size_t mgn_buf_size(const mgn_buf* buf);
+/* Raw device address, for callers that share the buffer with their own kernels. */
+void* mgn_buf_device_ptr(const mgn_buf* buf);
+/* Session::set_input / f32 set_parameter (src/runtime.rs:2496-2504, 2344).
+ * Ordered after earlier work on the context's stream; returns when src may be reused. */
+mgn_status mgn_buf_upload(mgn_ctx* ctx, mgn_buf* buf, size_t offset, const void* src, size_t bytes);
+/* Session::read_output / read_buffer (src/runtime.rs:2612-2629); waits for the stream. */
+mgn_status mgn_buf_download(mgn_ctx* ctx, const mgn_buf* buf, size_t offset, void* dst, size_t bytes);
+
+/* ---- block quantizers on the host, reference byte layout
+ *      TensorType::size_bytes (src/graph.rs:52-68): 20 or 36 bytes per 32-element block. */
+size_t mgn_packed_size(mgn_fmt fmt, size_t rows, size_t cols);
+/* quantize_q4_0 / quantize_q8_0 (src/runtime.rs:2035-2102, 2143-2188), bit-exact.
+ * w: f32 [rows, cols] row-major.  out: mgn_packed_size bytes. */
+mgn_status mgn_quantize_ref(mgn_fmt fmt, const float* w, size_t rows, size_t cols, uint8_t* out);
+/* dequantize_q4_0 / dequantize_q8_0 (src/runtime.rs:2105-2138, 2191-2215), bit-exact. */
+mgn_status mgn_dequantize_ref(mgn_fmt fmt, const uint8_t* in, size_t rows, size_t cols, float* out);
+
+/* ---- quantized weights on the device
+ * Session::set_parameter for a Q4/Q8 parameter (src/runtime.rs:2327-2345):
+ * quantize f32 [rows, cols] and place it in device memory.  The device layout
+ * is private; mgn_weight_export_ref gives back the reference's bytes. */
+mgn_status mgn_weight_create(mgn_ctx* ctx, mgn_fmt fmt, const float* w, size_t rows, size_t cols,
+                             mgn_weight** out);
+/* Same from bytes already in the reference layout (what load_checkpoint copies
+ * back into a Q4/Q8 buffer, src/runtime.rs:4256-4265). */
+mgn_status mgn_weight_create_packed(mgn_ctx* ctx, mgn_fmt fmt, const uint8_t* packed, size_t rows,
+                                    size_t cols, mgn_weight** out);
+/* Same from an f32 [rows, cols] matrix already on the device: the block
+ * quantizer runs as a kernel, bit-exact with mgn_quantize_ref. */
+mgn_status mgn_weight_create_device(mgn_ctx* ctx, mgn_fmt fmt, const mgn_buf* w_f32, size_t rows,
+                                    size_t cols, mgn_weight** out);
+void mgn_weight_free(mgn_ctx* ctx, mgn_weight* w);
+mgn_status mgn_weight_info(const mgn_weight* w, mgn_fmt* fmt, size_t* rows, size_t* cols);
+/* Device-side dequantization to host f32 [rows, cols]; must equal
+ * mgn_dequantize_ref(mgn_quantize_ref(w)) bit for bit. */
+mgn_status mgn_weight_dequantize(mgn_ctx* ctx, const mgn_weight* w, float* out_host);
+/* Device weight back to the reference byte layout (save_checkpoint's dump of a
+ * packed buffer, src/runtime.rs:4218-4226). */
+mgn_status mgn_weight_export_ref(mgn_ctx* ctx, const mgn_weight* w, uint8_t* out_packed);
+
+/* ---- the matmul itself
+ * C[M,N] = A[M,K] x W (+ D[M,N] when d is not null).  A, C, D: f32 row-major
+ * device buffers.  Stands in for the ShaderEntry::{MatMul, MatMulGemv,
+ * FusedMatMulAdd, MatMulGemvAdd} dispatches whose weight_format is Q4/Q8
+ * (src/compile.rs:1381-1421, 1486-1524; bind_dispatch src/runtime.rs:3073-3122).
+ * The kernel family is chosen from (M, K, N) inside, as compile.rs:1390 and
+ * runtime.rs:1634 do for the reference.  Asynchronous on the context's stream.
+ * c must not alias a; c may alias d. */
+mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d,
+                        mgn_buf* c, uint32_t m);
+/* The same with fp16 activations A[M,K] (prefill): fp16 operands on MFMA with
+ * f32 accumulation, the role matmul_coop.wgsl plays for unquantized weights
+ * (src/codegen.rs:1168-1176; quantized weights are excluded from it in the
+ * reference, src/runtime.rs:1634). */
+mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w,
+                             const mgn_buf* d, mgn_buf* c, uint32_t m);
+
+/* ---- GPU timing on the context's stream: Session::set_profiling +
+ *      dump_gpu_timings (src/runtime.rs:1965, 2798-2832) reduced to one
+ *      start/stop pair of HIP events. */
+mgn_status mgn_timer_start(mgn_ctx* ctx);
+mgn_status mgn_timer_stop(mgn_ctx* ctx, float* elapsed_ms); /* waits for the stop event */
+
+/* Library version, and the gfx target the kernels were built for ("gfx950"). */
+const char* mgn_version(void);
+const char* mgn_built_for(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MGN_HIP_H */

@@ -1,0 +1,94 @@
+/*
+ * mgn_session.h — C ABI over the host-side mirror of meganeura's operator
+ * surface for the quantized matmul path: Graph -> build_inference_session ->
+ * Session::{set_parameter, set_input, step, wait, read_output}.
+ *
+ * Only what reaches a quantized `matmul` is mirrored: leaf nodes, matmul, add
+ * (so that MatMul+Add fuses as in the reference), swiglu (so that gate/up
+ * projections fuse into one wide matmul) and rms_norm.  A matmul whose weight
+ * is plain f32 compiles into the plan (routing can be inspected) but is not
+ * executed by this backend: build returns MGN_EINVAL for it.
+ *
+ * Paths cited are relative to the reference checkout.
+ */
+#ifndef MGN_SESSION_H
+#define MGN_SESSION_H
+
+#include "mgn_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mgn_graph mgn_graph;
+typedef struct mgn_session mgn_session;
+
+/* compile::ShaderEntry values that can appear in a plan here
+ * (src/compile.rs ShaderEntry; lowering at 1381-1421, 1486-1524, 1814-1830). */
+typedef enum mgn_shader {
+  MGN_SHADER_MATMUL = 0,
+  MGN_SHADER_MATMUL_GEMV = 1,
+  MGN_SHADER_FUSED_MATMUL_ADD = 2,
+  MGN_SHADER_MATMUL_GEMV_ADD = 3,
+  MGN_SHADER_ADD = 4,
+  MGN_SHADER_SWIGLU = 5,
+  MGN_SHADER_SWIGLU_CONCAT = 6,
+  MGN_SHADER_RMS_NORM = 7
+} mgn_shader;
+
+/* compile::Dispatch (src/compile.rs:435-488), the fields this path uses.
+ * weight_format: 0 = F32, 1 = Q4, 2 = Q8 (compile::WeightFormat). */
+typedef struct mgn_dispatch_info {
+  int32_t shader;          /* mgn_shader */
+  uint32_t workgroups[3];  /* the grid the reference would launch */
+  uint32_t params[4];      /* [m, k, n, 0] for matmuls */
+  int32_t weight_format;
+} mgn_dispatch_info;
+
+/* Graph::new and the builders (src/graph.rs:714-795, 996-999).  Each builder
+ * returns the new node id (>= 0) or a negative mgn_status; the message is in
+ * mgn_graph_last_error.  Shapes are 2-D [rows, cols] (rms_norm weight: [cols]). */
+mgn_graph* mgn_graph_new(void);
+void mgn_graph_free(mgn_graph* g);
+const char* mgn_graph_last_error(const mgn_graph* g);
+int32_t mgn_graph_input(mgn_graph* g, const char* name, size_t rows, size_t cols);
+int32_t mgn_graph_parameter(mgn_graph* g, const char* name, size_t rows, size_t cols);
+int32_t mgn_graph_parameter_q4(mgn_graph* g, const char* name, size_t rows, size_t cols);
+int32_t mgn_graph_parameter_q8(mgn_graph* g, const char* name, size_t rows, size_t cols);
+int32_t mgn_graph_matmul(mgn_graph* g, int32_t a, int32_t b);
+int32_t mgn_graph_add(mgn_graph* g, int32_t a, int32_t b);
+int32_t mgn_graph_swiglu(mgn_graph* g, int32_t gate, int32_t up);
+int32_t mgn_graph_rms_norm(mgn_graph* g, int32_t x, int32_t weight, float eps);
+mgn_status mgn_graph_set_outputs(mgn_graph* g, const int32_t* ids, size_t count);
+
+/* compile only (optimize + compile_with, src/train.rs:272-340 without the GPU
+ * step): works without a device, for routing checks such as
+ * tests/gemv_parity.rs:32-52. */
+mgn_status mgn_graph_compile(const mgn_graph* g, mgn_dispatch_info* out, size_t cap, size_t* count);
+
+/* build_inference_session (src/train.rs:380-389). */
+mgn_status mgn_build_inference_session(const mgn_graph* g, int device_id, mgn_session** out);
+void mgn_session_free(mgn_session* s);
+const char* mgn_session_last_error(const mgn_session* s);
+/* Session::plan().dispatches (src/compile.rs:494-528). */
+size_t mgn_session_num_dispatches(const mgn_session* s);
+mgn_status mgn_session_dispatch_info(const mgn_session* s, size_t index, mgn_dispatch_info* out);
+/* Session::set_parameter (src/runtime.rs:2327-2493): f32 data of rows*cols
+ * elements; quantized on upload for Q4/Q8 parameters; feeds derived
+ * (concatenated) parameters.  Unknown name: MGN_ENOTFOUND (the reference panics). */
+mgn_status mgn_session_set_parameter(mgn_session* s, const char* name, const float* data, size_t len);
+/* Session::set_input (src/runtime.rs:2496-2504). */
+mgn_status mgn_session_set_input(mgn_session* s, const char* name, const float* data, size_t len);
+/* Session::step / wait (src/runtime.rs:2843-2959, 2835-2841). */
+mgn_status mgn_session_step(mgn_session* s);
+mgn_status mgn_session_wait(mgn_session* s);
+/* Session::read_output / read_output_by_index (src/runtime.rs:2612-2638). */
+mgn_status mgn_session_read_output(mgn_session* s, float* out, size_t len);
+mgn_status mgn_session_read_output_by_index(mgn_session* s, size_t index, float* out, size_t len);
+/* The session's context, for timing with mgn_timer_start/stop. */
+mgn_ctx* mgn_session_ctx(mgn_session* s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MGN_SESSION_H */

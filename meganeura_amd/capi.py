@@ -1,0 +1,273 @@
+"""ctypes binding of libmgn_hip.so (include/mgn_hip.h, include/mgn_session.h).
+
+The shared library is the product; this module only declares its entry points.
+There is no fallback: if the library has not been built, loading raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_DIR, "libmgn_hip.so")
+
+OK, EINVAL, ENOMEM, EHIP, ENOTFOUND, ENODEVICE = range(6)
+FMT_Q4, FMT_Q8 = 0, 1
+ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV, ROUTE_MFMA = range(4)
+
+# every symbol include/mgn_hip.h and include/mgn_session.h declare
+HIP_SYMBOLS = [
+    "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync", "mgn_ctx_set_route",
+    "mgn_buf_alloc", "mgn_buf_free", "mgn_buf_size", "mgn_buf_device_ptr", "mgn_buf_upload",
+    "mgn_buf_download", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
+    "mgn_weight_create", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
+    "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_matmul_q",
+    "mgn_matmul_q_f16a", "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
+]
+SESSION_SYMBOLS = [
+    "mgn_graph_new", "mgn_graph_free", "mgn_graph_last_error", "mgn_graph_input", "mgn_graph_parameter",
+    "mgn_graph_parameter_q4", "mgn_graph_parameter_q8", "mgn_graph_matmul", "mgn_graph_add",
+    "mgn_graph_swiglu", "mgn_graph_rms_norm", "mgn_graph_set_outputs", "mgn_graph_compile",
+    "mgn_build_inference_session", "mgn_session_free", "mgn_session_last_error",
+    "mgn_session_num_dispatches", "mgn_session_dispatch_info", "mgn_session_set_parameter",
+    "mgn_session_set_input", "mgn_session_step", "mgn_session_wait", "mgn_session_read_output",
+    "mgn_session_read_output_by_index", "mgn_session_ctx",
+]
+
+
+class DispatchInfo(C.Structure):
+    _fields_ = [
+        ("shader", C.c_int32),
+        ("workgroups", C.c_uint32 * 3),
+        ("params", C.c_uint32 * 4),
+        ("weight_format", C.c_int32),
+    ]
+
+
+class MgnError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"mgn status {status}: {message}")
+        self.status = status
+
+
+_lib = None
+
+
+def load():
+    """Load libmgn_hip.so and declare signatures.  Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "or `make -C meganeura_amd/csrc`; there is no fallback path"
+        )
+    lib = C.CDLL(LIB_PATH)
+    vp, sz, u8p, f32p = C.c_void_p, C.c_size_t, C.POINTER(C.c_uint8), C.POINTER(C.c_float)
+    sig = {
+        "mgn_ctx_create": (C.c_int, [C.c_int, C.POINTER(vp)]),
+        "mgn_ctx_destroy": (None, [vp]),
+        "mgn_last_error": (C.c_char_p, [vp]),
+        "mgn_sync": (C.c_int, [vp]),
+        "mgn_ctx_set_route": (C.c_int, [vp, C.c_int]),
+        "mgn_buf_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
+        "mgn_buf_free": (None, [vp, vp]),
+        "mgn_buf_size": (sz, [vp]),
+        "mgn_buf_device_ptr": (vp, [vp]),
+        "mgn_buf_upload": (C.c_int, [vp, vp, sz, vp, sz]),
+        "mgn_buf_download": (C.c_int, [vp, vp, sz, vp, sz]),
+        "mgn_packed_size": (sz, [C.c_int, sz, sz]),
+        "mgn_quantize_ref": (C.c_int, [C.c_int, vp, sz, sz, vp]),
+        "mgn_dequantize_ref": (C.c_int, [C.c_int, vp, sz, sz, vp]),
+        "mgn_weight_create": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
+        "mgn_weight_create_packed": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
+        "mgn_weight_create_device": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
+        "mgn_weight_free": (None, [vp, vp]),
+        "mgn_weight_info": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(sz), C.POINTER(sz)]),
+        "mgn_weight_dequantize": (C.c_int, [vp, vp, vp]),
+        "mgn_weight_export_ref": (C.c_int, [vp, vp, vp]),
+        "mgn_matmul_q": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
+        "mgn_matmul_q_f16a": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
+        "mgn_timer_start": (C.c_int, [vp]),
+        "mgn_timer_stop": (C.c_int, [vp, C.POINTER(C.c_float)]),
+        "mgn_version": (C.c_char_p, []),
+        "mgn_built_for": (C.c_char_p, []),
+        "mgn_graph_new": (vp, []),
+        "mgn_graph_free": (None, [vp]),
+        "mgn_graph_last_error": (C.c_char_p, [vp]),
+        "mgn_graph_input": (C.c_int32, [vp, C.c_char_p, sz, sz]),
+        "mgn_graph_parameter": (C.c_int32, [vp, C.c_char_p, sz, sz]),
+        "mgn_graph_parameter_q4": (C.c_int32, [vp, C.c_char_p, sz, sz]),
+        "mgn_graph_parameter_q8": (C.c_int32, [vp, C.c_char_p, sz, sz]),
+        "mgn_graph_matmul": (C.c_int32, [vp, C.c_int32, C.c_int32]),
+        "mgn_graph_add": (C.c_int32, [vp, C.c_int32, C.c_int32]),
+        "mgn_graph_swiglu": (C.c_int32, [vp, C.c_int32, C.c_int32]),
+        "mgn_graph_rms_norm": (C.c_int32, [vp, C.c_int32, C.c_int32, C.c_float]),
+        "mgn_graph_set_outputs": (C.c_int, [vp, C.POINTER(C.c_int32), sz]),
+        "mgn_graph_compile": (C.c_int, [vp, C.POINTER(DispatchInfo), sz, C.POINTER(sz)]),
+        "mgn_build_inference_session": (C.c_int, [vp, C.c_int, C.POINTER(vp)]),
+        "mgn_session_free": (None, [vp]),
+        "mgn_session_last_error": (C.c_char_p, [vp]),
+        "mgn_session_num_dispatches": (sz, [vp]),
+        "mgn_session_dispatch_info": (C.c_int, [vp, sz, C.POINTER(DispatchInfo)]),
+        "mgn_session_set_parameter": (C.c_int, [vp, C.c_char_p, vp, sz]),
+        "mgn_session_set_input": (C.c_int, [vp, C.c_char_p, vp, sz]),
+        "mgn_session_step": (C.c_int, [vp]),
+        "mgn_session_wait": (C.c_int, [vp]),
+        "mgn_session_read_output": (C.c_int, [vp, vp, sz]),
+        "mgn_session_read_output_by_index": (C.c_int, [vp, sz, vp, sz]),
+        "mgn_session_ctx": (vp, [vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def _ptr(arr):
+    return arr.ctypes.data_as(C.c_void_p)
+
+
+# ---- host quantizers (no GPU needed) -------------------------------------------
+
+def packed_size(fmt, rows, cols):
+    return int(load().mgn_packed_size(fmt, rows, cols))
+
+
+def quantize_ref(fmt, w):
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    rows, cols = w.shape
+    out = np.zeros(packed_size(fmt, rows, cols), dtype=np.uint8)
+    st = load().mgn_quantize_ref(fmt, _ptr(w), rows, cols, _ptr(out))
+    if st != OK:
+        raise MgnError(st, "quantize_ref: rows (K dim) must be a multiple of 32")
+    return out
+
+
+def dequantize_ref(fmt, packed, rows, cols):
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    out = np.empty((rows, cols), dtype=np.float32)
+    st = load().mgn_dequantize_ref(fmt, _ptr(packed), rows, cols, _ptr(out))
+    if st != OK:
+        raise MgnError(st, "dequantize_ref: bad arguments")
+    return out
+
+
+# ---- thin object wrappers over the handles -----------------------------------------
+
+class Context:
+    def __init__(self, device_id=0):
+        self.lib = load()
+        h = C.c_void_p()
+        st = self.lib.mgn_ctx_create(device_id, C.byref(h))
+        if st != OK:
+            raise MgnError(st, self.lib.mgn_last_error(None).decode())
+        self.h = h
+
+    def check(self, st):
+        if st != OK:
+            raise MgnError(st, self.lib.mgn_last_error(self.h).decode())
+
+    def close(self):
+        if self.h:
+            self.lib.mgn_ctx_destroy(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def set_route(self, route):
+        self.check(self.lib.mgn_ctx_set_route(self.h, route))
+
+    def sync(self):
+        self.check(self.lib.mgn_sync(self.h))
+
+    def timer_start(self):
+        self.check(self.lib.mgn_timer_start(self.h))
+
+    def timer_stop(self):
+        ms = C.c_float()
+        self.check(self.lib.mgn_timer_stop(self.h, C.byref(ms)))
+        return ms.value
+
+    def buffer(self, nbytes):
+        return Buffer(self, nbytes)
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr)
+        b = Buffer(self, arr.nbytes)
+        b.upload(arr)
+        return b
+
+    def weight(self, fmt, w):
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        h = C.c_void_p()
+        self.check(self.lib.mgn_weight_create(self.h, fmt, _ptr(w), w.shape[0], w.shape[1], C.byref(h)))
+        return Weight(self, h, fmt, w.shape[0], w.shape[1])
+
+    def weight_from_packed(self, fmt, packed, rows, cols):
+        packed = np.ascontiguousarray(packed, dtype=np.uint8)
+        assert packed.size == packed_size(fmt, rows, cols)
+        h = C.c_void_p()
+        self.check(self.lib.mgn_weight_create_packed(self.h, fmt, _ptr(packed), rows, cols, C.byref(h)))
+        return Weight(self, h, fmt, rows, cols)
+
+    def weight_from_device(self, fmt, buf, rows, cols):
+        h = C.c_void_p()
+        self.check(self.lib.mgn_weight_create_device(self.h, fmt, buf.h, rows, cols, C.byref(h)))
+        return Weight(self, h, fmt, rows, cols)
+
+    def matmul_q(self, a, w, c, m, d=None):
+        self.check(self.lib.mgn_matmul_q(self.h, a.h, w.h, d.h if d is not None else None, c.h, m))
+
+    def matmul_q_f16a(self, a, w, c, m, d=None):
+        self.check(self.lib.mgn_matmul_q_f16a(self.h, a.h, w.h, d.h if d is not None else None, c.h, m))
+
+
+class Buffer:
+    def __init__(self, ctx, nbytes):
+        self.ctx = ctx
+        h = C.c_void_p()
+        ctx.check(ctx.lib.mgn_buf_alloc(ctx.h, nbytes, C.byref(h)))
+        self.h = h
+        self.nbytes = nbytes
+
+    def upload(self, arr, offset=0):
+        arr = np.ascontiguousarray(arr)
+        self.ctx.check(self.ctx.lib.mgn_buf_upload(self.ctx.h, self.h, offset, _ptr(arr), arr.nbytes))
+
+    def download(self, dtype, count, offset=0):
+        out = np.empty(count, dtype=dtype)
+        self.ctx.check(self.ctx.lib.mgn_buf_download(self.ctx.h, self.h, offset, _ptr(out), out.nbytes))
+        return out
+
+    def free(self):
+        if self.h:
+            self.ctx.lib.mgn_buf_free(self.ctx.h, self.h)
+            self.h = None
+
+
+class Weight:
+    def __init__(self, ctx, h, fmt, rows, cols):
+        self.ctx, self.h, self.fmt, self.rows, self.cols = ctx, h, fmt, rows, cols
+
+    def dequantize(self):
+        out = np.empty((self.rows, self.cols), dtype=np.float32)
+        self.ctx.check(self.ctx.lib.mgn_weight_dequantize(self.ctx.h, self.h, _ptr(out)))
+        return out
+
+    def export_ref(self):
+        out = np.empty(packed_size(self.fmt, self.rows, self.cols), dtype=np.uint8)
+        self.ctx.check(self.ctx.lib.mgn_weight_export_ref(self.ctx.h, self.h, _ptr(out)))
+        return out
+
+    def free(self):
+        if self.h:
+            self.ctx.lib.mgn_weight_free(self.ctx.h, self.h)
+            self.h = None

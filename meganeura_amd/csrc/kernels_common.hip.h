@@ -1,0 +1,68 @@
+// Device helpers shared by the kernel translation units (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "mgn_internal.h"
+
+namespace mgn {
+
+// IEEE half bits -> float.  v_cvt_f32_f16 keeps half subnormals (the f16
+// denormal mode of a HIP kernel is "preserve"), matching half::f16::to_f32
+// (src/runtime.rs:2122-2123), not the shader's flush-to-zero decoder
+// (src/codegen.rs:739-746).
+__device__ __forceinline__ float half_bits_to_float(uint32_t bits) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Streaming (read-once) loads: the weight is far larger than what is reused.
+__device__ __forceinline__ uint4 stream_load_u128(const void* p) {
+  const u32x4 v = __builtin_nontemporal_load((const u32x4*)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint32_t stream_load_u32(const void* p) {
+  return __builtin_nontemporal_load((const uint32_t*)p);
+}
+__device__ __forceinline__ uint16_t stream_load_u16(const void* p) {
+  return __builtin_nontemporal_load((const uint16_t*)p);
+}
+
+// Byte N of a word as float: the compiler selects v_cvt_f32_ubyteN for these.
+__device__ __forceinline__ float ubyte0(uint32_t v) { return (float)(v & 0xFFu); }
+__device__ __forceinline__ float ubyte1(uint32_t v) { return (float)((v >> 8) & 0xFFu); }
+__device__ __forceinline__ float ubyte2(uint32_t v) { return (float)((v >> 16) & 0xFFu); }
+__device__ __forceinline__ float ubyte3(uint32_t v) { return (float)(v >> 24); }
+
+// One DPP move: lane i receives src from the lane the control word selects.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+  return __builtin_bit_cast(float, r);
+}
+
+constexpr int kDppQuadXor1 = 0xB1;     // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;     // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+
+// Sum over aligned groups of WIDTH consecutive lanes (WIDTH a power of two up to
+// 64); every lane of a group ends with the group's sum.
+template <int WIDTH>
+__device__ __forceinline__ float group_sum(float v) {
+  if constexpr (WIDTH >= 2) v += dpp_move<kDppQuadXor1>(v);
+  if constexpr (WIDTH >= 4) v += dpp_move<kDppQuadXor2>(v);
+  if constexpr (WIDTH >= 8) v += dpp_move<kDppRowHalfMirror>(v);
+  if constexpr (WIDTH >= 16) v += dpp_move<kDppRowMirror>(v);
+  if constexpr (WIDTH >= 32) v += __shfl_xor(v, 16, 64);
+  if constexpr (WIDTH >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+#define MGN_HIP_LAUNCH_CHECK()                      \
+  do {                                              \
+    hipError_t e__ = hipGetLastError();             \
+    if (e__ != hipSuccess) return (int)e__;         \
+  } while (0)
+
+}  // namespace mgn

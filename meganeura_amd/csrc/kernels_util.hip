@@ -1,0 +1,235 @@
+// Layout and conversion kernels: device-side dequantize, the bit-exact block
+// quantizer, and conversion between the reference's Q8 byte layout and the
+// device layout.  None of these is on the per-token path.
+#include "kernels_common.hip.h"
+#include "session.h"
+
+namespace mgn {
+namespace {
+
+// One thread per (block row kb, column n), n fastest, so the f32 side is
+// coalesced across the wave while each thread owns one whole block.
+// dequantize_q4_0 / dequantize_q8_0 (src/runtime.rs:2105-2138, 2191-2215):
+// nibble * d + m has an exact product, so the fused form rounds identically.
+__global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, float* __restrict__ out) {
+  const uint32_t n = blockIdx.x * 256 + threadIdx.x;
+  const uint32_t kb = blockIdx.y;
+  if (n >= w.n) return;
+  const uint32_t bpc = w.k / 32;
+  const size_t b = (size_t)n * bpc + kb;
+  float* dst = out + (size_t)kb * 32 * w.n + n;
+  if (w.fmt == MGN_FMT_Q4) {
+    const uint32_t dm = ((const uint32_t*)w.meta)[b];
+    const float d = half_bits_to_float(dm & 0xFFFFu), m = half_bits_to_float(dm >> 16);
+    const uint4 q = ((const uint4*)w.quants)[b];
+    const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+      for (int j = 0; j < 8; j++)
+        dst[(size_t)(t * 8 + j) * w.n] = __fmaf_rn((float)((words[t] >> (4 * j)) & 0xFu), d, m);
+  } else {
+    const float s = half_bits_to_float(((const uint16_t*)w.meta)[b]);
+    const uint4* qp = (const uint4*)w.quants + b * 2;
+    const uint4 q0 = qp[0], q1 = qp[1];
+    const uint32_t words[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        dst[(size_t)(t * 4 + j) * w.n] = (float)(int8_t)(words[t] >> (8 * j)) * s;
+  }
+}
+
+// Reference Q8 block (36 bytes: f16 scale, 2 pad bytes, 32 int8;
+// src/runtime.rs:2150-2186) <-> device arrays (u16 scale, 32-byte quants).
+__global__ __launch_bounds__(256) void export_q8_kernel(const uint16_t* __restrict__ scales,
+                                                        const uint32_t* __restrict__ quants, size_t nb,
+                                                        uint32_t* __restrict__ out) {
+  const size_t b = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (b >= nb) return;
+  out[b * 9] = scales[b];
+#pragma unroll
+  for (int i = 0; i < 8; i++) out[b * 9 + 1 + i] = quants[b * 8 + i];
+}
+
+__global__ __launch_bounds__(256) void import_q8_kernel(const uint32_t* __restrict__ ref, size_t nb,
+                                                        uint16_t* __restrict__ scales,
+                                                        uint32_t* __restrict__ quants) {
+  const size_t b = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (b >= nb) return;
+  scales[b] = (uint16_t)ref[b * 9];
+#pragma unroll
+  for (int i = 0; i < 8; i++) quants[b * 8 + i] = ref[b * 9 + 1 + i];
+}
+
+__device__ __forceinline__ float clamp_keep_nan(float v, float lo, float hi) {
+  return v < lo ? lo : (v > hi ? hi : v);
+}
+
+// quantize_q4_0 / quantize_q8_0 (src/runtime.rs:2035-2102, 2143-2188) as a
+// kernel, one thread per block.  Every f32 operation rounds separately (no
+// contraction), division and roundf are the correctly rounded device forms,
+// and the f16 stores use round-to-nearest-even conversion, so the bytes equal
+// the host quantizer's.
+#pragma clang fp contract(off)
+__global__ __launch_bounds__(256) void quantize_kernel(int fmt, const float* __restrict__ w, uint32_t k,
+                                                       uint32_t n_cols, void* __restrict__ meta,
+                                                       void* __restrict__ quants) {
+  const uint32_t n = blockIdx.x * 256 + threadIdx.x;
+  const uint32_t kb = blockIdx.y;
+  if (n >= n_cols) return;
+  const uint32_t bpc = k / 32;
+  const size_t b = (size_t)n * bpc + kb;
+  const float* src = w + (size_t)kb * 32 * n_cols + n;
+  float v[32];
+#pragma unroll
+  for (int i = 0; i < 32; i++) v[i] = src[(size_t)i * n_cols];
+  if (fmt == MGN_FMT_Q4) {
+    float bmin = INFINITY, bmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      if (v[i] < bmin) bmin = v[i];
+      if (v[i] > bmax) bmax = v[i];
+    }
+    const float d = bmax > bmin ? (bmax - bmin) / 15.0f : 1.0f;
+    const float m = bmin;
+    const float d_inv = d > 0.0f ? 1.0f / d : 0.0f;
+    const uint32_t dbits = __builtin_bit_cast(uint16_t, (_Float16)d);
+    const uint32_t mbits = __builtin_bit_cast(uint16_t, (_Float16)m);
+    ((uint32_t*)meta)[b] = dbits | (mbits << 16);
+    uint32_t words[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      float t = clamp_keep_nan(roundf((v[i] - m) * d_inv), 0.0f, 15.0f);
+      uint32_t nib = (t != t) ? 0u : (uint32_t)t;
+      words[i / 8] |= nib << (4 * (i % 8));
+    }
+    ((uint4*)quants)[b] = make_uint4(words[0], words[1], words[2], words[3]);
+  } else {
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      float a = fabsf(v[i]);
+      if (a > amax) amax = a;
+    }
+    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+    const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+    ((uint16_t*)meta)[b] = __builtin_bit_cast(uint16_t, (_Float16)scale);
+    uint32_t words[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      float t = clamp_keep_nan(roundf(v[i] * inv), -128.0f, 127.0f);
+      int q = (t != t) ? 0 : (int)t;
+      words[i / 4] |= (uint32_t)(q & 0xFF) << (8 * (i % 4));
+    }
+    uint4* qp = (uint4*)quants + b * 2;
+    qp[0] = make_uint4(words[0], words[1], words[2], words[3]);
+    qp[1] = make_uint4(words[4], words[5], words[6], words[7]);
+  }
+}
+
+// ---- pointwise companions of the matmul in a decode layer ----
+
+__global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                  float* __restrict__ out, size_t len) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < len) out[i] = a[i] + b[i];
+}
+
+// src/shaders/swiglu_concat.wgsl:20-32: silu(gate) * up with sig = 1 / (1 + exp(-gate))
+__device__ __forceinline__ float swiglu_value(float gate, float up) {
+  const float sig = 1.0f / (1.0f + expf(-gate));
+  return gate * sig * up;
+}
+
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                     float* __restrict__ out, size_t len) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < len) out[i] = swiglu_value(gate[i], up[i]);
+}
+
+__global__ __launch_bounds__(256) void swiglu_concat_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                            size_t len, uint32_t half_n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= len) return;
+  const size_t row = i / half_n, col = i % half_n;
+  const float* p = in + row * 2 * half_n;
+  out[i] = swiglu_value(p[col], p[half_n + col]);
+}
+
+// src/shaders/rms_norm.wgsl:1-57: one workgroup of 256 per row, strided sum of
+// squares, tree reduction, x * rsqrt(mean_sq + eps) * weight.
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const float* __restrict__ wt,
+                                                       float* __restrict__ out, uint32_t cols, float eps) {
+  __shared__ float wg[256];
+  const uint32_t tid = threadIdx.x;
+  const float* src = x + (size_t)blockIdx.x * cols;
+  float ss = 0.0f;
+  for (uint32_t j = tid; j < cols; j += 256) ss = __fmaf_rn(src[j], src[j], ss);
+  wg[tid] = ss;
+  __syncthreads();
+  for (uint32_t stride = 128; stride > 0; stride >>= 1) {
+    if (tid < stride) wg[tid] += wg[tid + stride];
+    __syncthreads();
+  }
+  const float r = 1.0f / sqrtf(wg[0] / (float)cols + eps);
+  float* dst = out + (size_t)blockIdx.x * cols;
+  for (uint32_t j = tid; j < cols; j += 256) dst[j] = src[j] * r * wt[j];
+}
+
+}  // namespace
+
+int launch_add(ihipStream_t* s, const float* a, const float* b, float* out, size_t len) {
+  hipLaunchKernelGGL(add_kernel, dim3((unsigned)((len + 255) / 256)), dim3(256), 0, s, a, b, out, len);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+int launch_swiglu(ihipStream_t* s, const float* gate, const float* up, float* out, size_t len) {
+  hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((len + 255) / 256)), dim3(256), 0, s, gate, up, out, len);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+int launch_swiglu_concat(ihipStream_t* s, const float* in, float* out, size_t len, uint32_t half_n) {
+  hipLaunchKernelGGL(swiglu_concat_kernel, dim3((unsigned)((len + 255) / 256)), dim3(256), 0, s, in, out, len, half_n);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+int launch_rms_norm(ihipStream_t* s, const float* x, const float* weight, float* out, uint32_t rows, uint32_t cols,
+                    float eps) {
+  hipLaunchKernelGGL(rms_norm_kernel, dim3(rows), dim3(256), 0, s, x, weight, out, cols, eps);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_dequantize(ihipStream_t* s, const WeightView& w, float* out_dev) {
+  dim3 grid((w.n + 255) / 256, w.k / 32);
+  hipLaunchKernelGGL(dequantize_kernel, grid, dim3(256), 0, s, w, out_dev);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_export_q8(ihipStream_t* s, const WeightView& w, uint8_t* out_dev) {
+  const size_t nb = (size_t)(w.k / 32) * w.n;
+  hipLaunchKernelGGL(export_q8_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s,
+                     (const uint16_t*)w.meta, (const uint32_t*)w.quants, nb, (uint32_t*)out_dev);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* meta, void* quants) {
+  hipLaunchKernelGGL(import_q8_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s,
+                     (const uint32_t*)ref_dev, nb, (uint16_t*)meta, (uint32_t*)quants);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, uint32_t n, void* meta,
+                    void* quants) {
+  dim3 grid((n + 255) / 256, k / 32);
+  hipLaunchKernelGGL(quantize_kernel, grid, dim3(256), 0, s, fmt, w_dev, k, n, meta, quants);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace mgn

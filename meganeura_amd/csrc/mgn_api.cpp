@@ -1,0 +1,387 @@
+// C ABI of libmgn_hip: contexts, buffers, quantized weights, matmul dispatch.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "mgn_internal.h"
+
+namespace {
+
+thread_local std::string g_create_error;
+
+mgn_status fail(mgn_ctx* ctx, mgn_status st, const std::string& msg) {
+  if (ctx) ctx->err = msg; else g_create_error = msg;
+  return st;
+}
+
+mgn_status hip_fail(mgn_ctx* ctx, const char* what, hipError_t e) {
+  return fail(ctx, MGN_EHIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define MGN_HIP(ctx, call)                                   \
+  do {                                                       \
+    hipError_t e_ = (call);                                  \
+    if (e_ != hipSuccess) return hip_fail(ctx, #call, e_);   \
+  } while (0)
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+size_t meta_elem(mgn_fmt fmt) { return fmt == MGN_FMT_Q4 ? 4 : 2; }
+size_t quant_elem(mgn_fmt fmt) { return fmt == MGN_FMT_Q4 ? 16 : 32; }
+
+bool valid_fmt(mgn_fmt fmt) { return fmt == MGN_FMT_Q4 || fmt == MGN_FMT_Q8; }
+
+mgn::WeightView view_of(const mgn_weight* w) {
+  return mgn::WeightView{w->meta, w->quants, (uint32_t)w->rows, (uint32_t)w->cols, (int)w->fmt};
+}
+
+// Device storage for a [rows, cols] weight, contents undefined.
+mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn_weight** out) {
+  if (!ctx || !out) return fail(ctx, MGN_EINVAL, "null argument");
+  *out = nullptr;
+  if (!valid_fmt(fmt)) return fail(ctx, MGN_EINVAL, "unknown weight format");
+  if (rows == 0 || cols == 0) return fail(ctx, MGN_EINVAL, "empty weight");
+  if (rows % 32 != 0) return fail(ctx, MGN_EINVAL, "quantized weights require rows (K dim) to be a multiple of 32");
+  if (rows > 0xFFFFFFE0ull || cols > 0xFFFFFFFFull) return fail(ctx, MGN_EINVAL, "weight dimension exceeds 32 bits");
+  auto* w = new (std::nothrow) mgn_weight();
+  if (!w) return fail(ctx, MGN_ENOMEM, "out of host memory");
+  w->fmt = fmt;
+  w->rows = rows;
+  w->cols = cols;
+  w->nb = (rows / 32) * cols;
+  w->meta_bytes = w->nb * meta_elem(fmt);
+  w->quant_bytes = w->nb * quant_elem(fmt);
+  const size_t q_off = align_up(w->meta_bytes, 256);
+  // 256 spare bytes: kernels may over-read one vector past the last block
+  hipError_t e = hipMalloc(&w->base, q_off + w->quant_bytes + 256);
+  if (e != hipSuccess) {
+    delete w;
+    return e == hipErrorOutOfMemory ? fail(ctx, MGN_ENOMEM, "out of device memory") : hip_fail(ctx, "hipMalloc", e);
+  }
+  w->meta = w->base;
+  w->quants = (char*)w->base + q_off;
+  *out = w;
+  return MGN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mgn_version(void) { return "0.1.0"; }
+const char* mgn_built_for(void) { return "gfx950"; }
+
+mgn_status mgn_ctx_create(int device_id, mgn_ctx** out) {
+  if (!out) return fail(nullptr, MGN_EINVAL, "null out pointer");
+  *out = nullptr;
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count == 0) return fail(nullptr, MGN_ENODEVICE, "no HIP device visible");
+  if (device_id < 0 || device_id >= count) return fail(nullptr, MGN_EINVAL, "device_id out of range");
+  hipDeviceProp_t prop;
+  MGN_HIP(nullptr, hipGetDeviceProperties(&prop, device_id));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(nullptr, MGN_ENODEVICE, std::string("kernels are built for gfx950, device is ") + prop.gcnArchName);
+  MGN_HIP(nullptr, hipSetDevice(device_id));
+  auto* ctx = new (std::nothrow) mgn_ctx();
+  if (!ctx) return fail(nullptr, MGN_ENOMEM, "out of host memory");
+  ctx->device = device_id;
+  ctx->num_cus = prop.multiProcessorCount;
+  if ((e = hipStreamCreate(&ctx->stream)) != hipSuccess || (e = hipEventCreate(&ctx->ev_start)) != hipSuccess ||
+      (e = hipEventCreate(&ctx->ev_stop)) != hipSuccess) {
+    mgn_ctx_destroy(ctx);
+    return hip_fail(nullptr, "stream/event creation", e);
+  }
+  *out = ctx;
+  return MGN_OK;
+}
+
+void mgn_ctx_destroy(mgn_ctx* ctx) {
+  if (!ctx) return;
+  if (ctx->stream) {
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipStreamDestroy(ctx->stream);
+  }
+  if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+  if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+  delete ctx;
+}
+
+const char* mgn_last_error(const mgn_ctx* ctx) { return ctx ? ctx->err.c_str() : g_create_error.c_str(); }
+
+mgn_status mgn_sync(mgn_ctx* ctx) {
+  if (!ctx) return MGN_EINVAL;
+  MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return MGN_OK;
+}
+
+mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route) {
+  if (!ctx) return MGN_EINVAL;
+  if (route < MGN_ROUTE_AUTO || route > MGN_ROUTE_MFMA) return fail(ctx, MGN_EINVAL, "unknown route");
+  ctx->route = route;
+  return MGN_OK;
+}
+
+// ---- buffers ----
+
+mgn_status mgn_buf_alloc(mgn_ctx* ctx, size_t bytes, mgn_buf** out) {
+  if (!ctx || !out) return fail(ctx, MGN_EINVAL, "null argument");
+  *out = nullptr;
+  auto* b = new (std::nothrow) mgn_buf();
+  if (!b) return fail(ctx, MGN_ENOMEM, "out of host memory");
+  b->bytes = bytes;
+  const size_t alloc = align_up(bytes < 4 ? 4 : bytes, 256);  // the reference's minimum is 4 bytes
+  hipError_t e = hipMalloc(&b->ptr, alloc);
+  if (e != hipSuccess) {
+    delete b;
+    return e == hipErrorOutOfMemory ? fail(ctx, MGN_ENOMEM, "out of device memory") : hip_fail(ctx, "hipMalloc", e);
+  }
+  e = hipMemsetAsync(b->ptr, 0, alloc, ctx->stream);
+  if (e != hipSuccess) {
+    (void)hipFree(b->ptr);
+    delete b;
+    return hip_fail(ctx, "hipMemsetAsync", e);
+  }
+  *out = b;
+  return MGN_OK;
+}
+
+void mgn_buf_free(mgn_ctx* ctx, mgn_buf* buf) {
+  if (!buf) return;
+  if (ctx) (void)hipStreamSynchronize(ctx->stream);
+  if (buf->ptr) (void)hipFree(buf->ptr);
+  delete buf;
+}
+
+size_t mgn_buf_size(const mgn_buf* buf) { return buf ? buf->bytes : 0; }
+void* mgn_buf_device_ptr(const mgn_buf* buf) { return buf ? buf->ptr : nullptr; }
+
+mgn_status mgn_buf_upload(mgn_ctx* ctx, mgn_buf* buf, size_t offset, const void* src, size_t bytes) {
+  if (!ctx || !buf || (!src && bytes)) return fail(ctx, MGN_EINVAL, "null argument");
+  if (offset > buf->bytes || bytes > buf->bytes - offset) return fail(ctx, MGN_EINVAL, "upload exceeds buffer size");
+  if (bytes == 0) return MGN_OK;
+  MGN_HIP(ctx, hipMemcpyAsync((char*)buf->ptr + offset, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return MGN_OK;
+}
+
+mgn_status mgn_buf_download(mgn_ctx* ctx, const mgn_buf* buf, size_t offset, void* dst, size_t bytes) {
+  if (!ctx || !buf || (!dst && bytes)) return fail(ctx, MGN_EINVAL, "null argument");
+  if (offset > buf->bytes || bytes > buf->bytes - offset) return fail(ctx, MGN_EINVAL, "download exceeds buffer size");
+  if (bytes == 0) return mgn_sync(ctx);
+  MGN_HIP(ctx, hipMemcpyAsync(dst, (const char*)buf->ptr + offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return MGN_OK;
+}
+
+// ---- host quantizers ----
+
+size_t mgn_packed_size(mgn_fmt fmt, size_t rows, size_t cols) {
+  if (!valid_fmt(fmt)) return 0;
+  return (rows / 32) * cols * (fmt == MGN_FMT_Q4 ? 20 : 36);
+}
+
+mgn_status mgn_quantize_ref(mgn_fmt fmt, const float* w, size_t rows, size_t cols, uint8_t* out) {
+  if (!valid_fmt(fmt) || rows % 32 != 0) return MGN_EINVAL;
+  if (rows == 0 || cols == 0) return MGN_OK;
+  if (!w || !out) return MGN_EINVAL;
+  if (fmt == MGN_FMT_Q4) mgn::quantize_q4_host(w, rows, cols, out);
+  else mgn::quantize_q8_host(w, rows, cols, out);
+  return MGN_OK;
+}
+
+mgn_status mgn_dequantize_ref(mgn_fmt fmt, const uint8_t* in, size_t rows, size_t cols, float* out) {
+  if (!valid_fmt(fmt) || rows % 32 != 0) return MGN_EINVAL;
+  if (rows == 0 || cols == 0) return MGN_OK;
+  if (!in || !out) return MGN_EINVAL;
+  if (fmt == MGN_FMT_Q4) mgn::dequantize_q4_host(in, rows, cols, out);
+  else mgn::dequantize_q8_host(in, rows, cols, out);
+  return MGN_OK;
+}
+
+// ---- weights ----
+
+mgn_status mgn_weight_create_packed(mgn_ctx* ctx, mgn_fmt fmt, const uint8_t* packed, size_t rows, size_t cols,
+                                    mgn_weight** out) {
+  if (!packed) return fail(ctx, MGN_EINVAL, "null argument");
+  mgn_weight* w = nullptr;
+  mgn_status st = weight_alloc(ctx, fmt, rows, cols, &w);
+  if (st != MGN_OK) return st;
+  hipError_t e = hipSuccess;
+  void* tmp = nullptr;
+  if (fmt == MGN_FMT_Q4) {
+    // the reference layout is already "all scale|min words, then all nibbles"
+    e = hipMemcpyAsync(w->meta, packed, w->meta_bytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess)
+      e = hipMemcpyAsync(w->quants, packed + w->meta_bytes, w->quant_bytes, hipMemcpyHostToDevice, ctx->stream);
+  } else {
+    const size_t bytes = w->nb * 36;
+    e = hipMalloc(&tmp, bytes);
+    if (e == hipSuccess) e = hipMemcpyAsync(tmp, packed, bytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = (hipError_t)mgn::launch_import_q8(ctx->stream, (const uint8_t*)tmp, w->nb, w->meta, w->quants);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (tmp) (void)hipFree(tmp);
+  if (e != hipSuccess) {
+    mgn_weight_free(ctx, w);
+    return hip_fail(ctx, "weight upload", e);
+  }
+  *out = w;
+  return MGN_OK;
+}
+
+mgn_status mgn_weight_create(mgn_ctx* ctx, mgn_fmt fmt, const float* wdata, size_t rows, size_t cols,
+                             mgn_weight** out) {
+  if (!ctx || !out || !wdata) return fail(ctx, MGN_EINVAL, "null argument");
+  *out = nullptr;
+  if (!valid_fmt(fmt)) return fail(ctx, MGN_EINVAL, "unknown weight format");
+  if (rows % 32 != 0) return fail(ctx, MGN_EINVAL, "quantized weights require rows (K dim) to be a multiple of 32");
+  if (rows == 0 || cols == 0) return fail(ctx, MGN_EINVAL, "empty weight");
+  std::vector<uint8_t> packed;
+  try {
+    packed.resize(mgn_packed_size(fmt, rows, cols));
+  } catch (const std::bad_alloc&) {
+    return fail(ctx, MGN_ENOMEM, "out of host memory");
+  }
+  mgn_quantize_ref(fmt, wdata, rows, cols, packed.data());
+  return mgn_weight_create_packed(ctx, fmt, packed.data(), rows, cols, out);
+}
+
+mgn_status mgn_weight_create_device(mgn_ctx* ctx, mgn_fmt fmt, const mgn_buf* w_f32, size_t rows, size_t cols,
+                                    mgn_weight** out) {
+  if (!w_f32) return fail(ctx, MGN_EINVAL, "null argument");
+  mgn_weight* w = nullptr;
+  mgn_status st = weight_alloc(ctx, fmt, rows, cols, &w);
+  if (st != MGN_OK) return st;
+  if (w_f32->bytes / sizeof(float) < rows * cols) {
+    mgn_weight_free(ctx, w);
+    return fail(ctx, MGN_EINVAL, "source buffer smaller than rows*cols floats");
+  }
+  hipError_t e = (hipError_t)mgn::launch_quantize(ctx->stream, (int)fmt, (const float*)w_f32->ptr, (uint32_t)rows,
+                                                  (uint32_t)cols, w->meta, w->quants);
+  if (e != hipSuccess) {
+    mgn_weight_free(ctx, w);
+    return hip_fail(ctx, "quantize kernel", e);
+  }
+  *out = w;
+  return MGN_OK;
+}
+
+void mgn_weight_free(mgn_ctx* ctx, mgn_weight* w) {
+  if (!w) return;
+  if (ctx) (void)hipStreamSynchronize(ctx->stream);
+  if (w->base) (void)hipFree(w->base);
+  delete w;
+}
+
+mgn_status mgn_weight_info(const mgn_weight* w, mgn_fmt* fmt, size_t* rows, size_t* cols) {
+  if (!w) return MGN_EINVAL;
+  if (fmt) *fmt = w->fmt;
+  if (rows) *rows = w->rows;
+  if (cols) *cols = w->cols;
+  return MGN_OK;
+}
+
+mgn_status mgn_weight_dequantize(mgn_ctx* ctx, const mgn_weight* w, float* out_host) {
+  if (!ctx || !w || !out_host) return fail(ctx, MGN_EINVAL, "null argument");
+  const size_t bytes = w->rows * w->cols * sizeof(float);
+  float* tmp = nullptr;
+  hipError_t e = hipMalloc((void**)&tmp, bytes);
+  if (e != hipSuccess) return e == hipErrorOutOfMemory ? fail(ctx, MGN_ENOMEM, "out of device memory") : hip_fail(ctx, "hipMalloc", e);
+  e = (hipError_t)mgn::launch_dequantize(ctx->stream, view_of(w), tmp);
+  if (e == hipSuccess) e = hipMemcpyAsync(out_host, tmp, bytes, hipMemcpyDeviceToHost, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  (void)hipFree(tmp);
+  if (e != hipSuccess) return hip_fail(ctx, "dequantize", e);
+  return MGN_OK;
+}
+
+mgn_status mgn_weight_export_ref(mgn_ctx* ctx, const mgn_weight* w, uint8_t* out_packed) {
+  if (!ctx || !w || !out_packed) return fail(ctx, MGN_EINVAL, "null argument");
+  hipError_t e = hipSuccess;
+  void* tmp = nullptr;
+  if (w->fmt == MGN_FMT_Q4) {
+    e = hipMemcpyAsync(out_packed, w->meta, w->meta_bytes, hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess)
+      e = hipMemcpyAsync(out_packed + w->meta_bytes, w->quants, w->quant_bytes, hipMemcpyDeviceToHost, ctx->stream);
+  } else {
+    const size_t bytes = w->nb * 36;
+    e = hipMalloc(&tmp, bytes);
+    if (e == hipSuccess) e = (hipError_t)mgn::launch_export_q8(ctx->stream, view_of(w), (uint8_t*)tmp);
+    if (e == hipSuccess) e = hipMemcpyAsync(out_packed, tmp, bytes, hipMemcpyDeviceToHost, ctx->stream);
+  }
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (tmp) (void)hipFree(tmp);
+  if (e != hipSuccess) return hip_fail(ctx, "weight export", e);
+  return MGN_OK;
+}
+
+// ---- matmul ----
+
+static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, const mgn_weight* w, const mgn_buf* d,
+                              mgn_buf* c, uint32_t m) {
+  if (!ctx || !a || !w || !c) return fail(ctx, MGN_EINVAL, "null argument");
+  if (m == 0) return MGN_OK;
+  const size_t k = w->rows, n = w->cols;
+  const size_t a_elem = a_is_f16 ? 2 : 4;
+  if (a->bytes / a_elem < (size_t)m * k) return fail(ctx, MGN_EINVAL, "A is smaller than m*K elements");
+  if (c->bytes / 4 < (size_t)m * n) return fail(ctx, MGN_EINVAL, "C is smaller than m*N floats");
+  if (d && d->bytes / 4 < (size_t)m * n) return fail(ctx, MGN_EINVAL, "D is smaller than m*N floats");
+  if (c->ptr == a->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
+  mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus};
+  mgn_route route = ctx->route;
+  if (route == MGN_ROUTE_AUTO) {
+    if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV;
+    else if (mgn::mfma_supported(x)) route = MGN_ROUTE_MFMA;
+    else route = MGN_ROUTE_GENERIC;
+  }
+  int rc;
+  switch (route) {
+    case MGN_ROUTE_GEMV:
+      if (!mgn::gemv_supported(x)) return fail(ctx, MGN_EINVAL, "GEMV route does not support this shape");
+      rc = mgn::launch_matmul_gemv(ctx->stream, x);
+      break;
+    case MGN_ROUTE_MFMA:
+      if (!mgn::mfma_supported(x)) return fail(ctx, MGN_EINVAL, "MFMA route does not support this shape");
+      rc = mgn::launch_matmul_mfma(ctx->stream, x);
+      break;
+    default:
+      rc = mgn::launch_matmul_generic(ctx->stream, x);
+      break;
+  }
+  if (rc != 0) return hip_fail(ctx, "kernel launch", (hipError_t)rc);
+  return MGN_OK;
+}
+
+mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
+                        uint32_t m) {
+  return matmul_impl(ctx, a, false, w, d, c, m);
+}
+
+mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
+                             uint32_t m) {
+  return matmul_impl(ctx, a_f16, true, w, d, c, m);
+}
+
+// ---- timing ----
+
+mgn_status mgn_timer_start(mgn_ctx* ctx) {
+  if (!ctx) return MGN_EINVAL;
+  MGN_HIP(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+  return MGN_OK;
+}
+
+mgn_status mgn_timer_stop(mgn_ctx* ctx, float* elapsed_ms) {
+  if (!ctx || !elapsed_ms) return fail(ctx, MGN_EINVAL, "null argument");
+  MGN_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
+  MGN_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
+  MGN_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
+  return MGN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,83 @@
+// Internal declarations shared by the translation units of libmgn_hip.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <string>
+
+#include "../../include/mgn_hip.h"
+
+struct ihipStream_t;
+struct ihipEvent_t;
+
+namespace mgn {
+
+// ---- host quantizers (quant_host.cpp) ----
+uint16_t f32_to_f16_bits(float f);
+float f16_bits_to_f32(uint16_t h);
+void quantize_q4_host(const float* w, size_t rows, size_t cols, uint8_t* out);
+void quantize_q8_host(const float* w, size_t rows, size_t cols, uint8_t* out);
+void dequantize_q4_host(const uint8_t* in, size_t rows, size_t cols, float* out);
+void dequantize_q8_host(const uint8_t* in, size_t rows, size_t cols, float* out);
+
+// ---- device view of a quantized weight ----
+// Blocks are numbered b = n * (K/32) + kb, as in the reference, so one output
+// column's blocks are contiguous.  Scales and quants live in separate arrays:
+//   Q4: meta[b] = u32 (d_f16 | m_f16 << 16), quants[b] = 16 bytes of nibbles
+//       -> byte for byte the reference layout, split at nb*4;
+//   Q8: meta[b] = u16 scale_f16,             quants[b] = 32 int8
+//       -> the reference's 36-byte blocks with the pad dropped and scales
+//          gathered, so quants are 32-byte aligned for 128-bit loads.
+struct WeightView {
+  const void* meta;
+  const void* quants;
+  uint32_t k, n;  // rows, cols
+  int fmt;        // mgn_fmt
+};
+
+struct LaunchArgs {
+  WeightView w;
+  const void* a;   // [m, k] f32 or f16
+  const float* d;  // [m, n] or null
+  float* c;        // [m, n]
+  uint32_t m;
+  bool a_is_f16;
+  int num_cus;
+};
+
+// kernels.hip
+int launch_dequantize(ihipStream_t* s, const WeightView& w, float* out_dev);  // out [k, n] f32
+int launch_export_q8(ihipStream_t* s, const WeightView& w, uint8_t* out_dev);  // 36-byte blocks
+int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* meta, void* quants);
+int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, uint32_t n, void* meta,
+                    void* quants);
+int launch_matmul_generic(ihipStream_t* s, const LaunchArgs& a);
+bool gemv_supported(const LaunchArgs& a);
+int launch_matmul_gemv(ihipStream_t* s, const LaunchArgs& a);
+bool mfma_supported(const LaunchArgs& a);
+int launch_matmul_mfma(ihipStream_t* s, const LaunchArgs& a);
+
+}  // namespace mgn
+
+struct mgn_ctx {
+  int device = 0;
+  int num_cus = 0;
+  ihipStream_t* stream = nullptr;
+  ihipEvent_t* ev_start = nullptr;
+  ihipEvent_t* ev_stop = nullptr;
+  mgn_route route = MGN_ROUTE_AUTO;
+  std::string err;
+};
+
+struct mgn_buf {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+
+struct mgn_weight {
+  mgn_fmt fmt;
+  size_t rows = 0, cols = 0, nb = 0;
+  void* base = nullptr;    // one allocation
+  void* meta = nullptr;    // into base
+  void* quants = nullptr;  // into base, 256-byte aligned
+  size_t meta_bytes = 0, quant_bytes = 0;
+};

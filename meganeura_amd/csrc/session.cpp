@@ -1,0 +1,631 @@
+// Graph building, the two matmul fusions, plan compilation and the Session
+// verbs for the quantized matmul path.  See session.h for what is mirrored.
+#include "session.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+
+namespace mgn {
+
+// ---------------------------------------------------------------- Graph ----
+
+NodeId Graph::add_raw_node(Op op, std::vector<NodeId> inputs, TensorType ty, std::string name, float eps) {
+  const NodeId id = (NodeId)nodes_.size();
+  nodes_.push_back(Node{id, op, std::move(name), std::move(inputs), std::move(ty), eps});
+  return id;
+}
+
+const Node& Graph::node(NodeId id) const {
+  if (id >= nodes_.size()) throw GraphError("node id out of range");
+  return nodes_[id];
+}
+
+bool Graph::is_output(NodeId id) const { return std::find(outputs_.begin(), outputs_.end(), id) != outputs_.end(); }
+
+static NodeId leaf(Graph& g, Op op, const std::string& name, std::vector<size_t> shape, DType dt) {
+  if (shape.empty()) throw GraphError("leaf node needs a shape");
+  for (size_t s : shape)
+    if (s == 0) throw GraphError("zero-sized dimension");
+  return g.add_raw_node(op, {}, TensorType{std::move(shape), dt}, name);
+}
+
+NodeId Graph::input(const std::string& name, std::vector<size_t> shape) {
+  return leaf(*this, Op::Input, name, std::move(shape), DType::F32);
+}
+NodeId Graph::parameter(const std::string& name, std::vector<size_t> shape) {
+  return leaf(*this, Op::Parameter, name, std::move(shape), DType::F32);
+}
+// src/graph.rs:752-773: only the dtype tag differs; the shape stays logical [K, N].
+NodeId Graph::parameter_q4(const std::string& name, std::vector<size_t> shape) {
+  return leaf(*this, Op::Parameter, name, std::move(shape), DType::Q4_0);
+}
+NodeId Graph::parameter_q8(const std::string& name, std::vector<size_t> shape) {
+  return leaf(*this, Op::Parameter, name, std::move(shape), DType::Q8_0);
+}
+
+// src/graph.rs:787-795
+NodeId Graph::matmul(NodeId a, NodeId b) {
+  const auto& as = node(a).ty.shape;
+  const auto& bs = node(b).ty.shape;
+  if (as.size() != 2 || bs.size() != 2) throw GraphError("matmul requires 2D tensors");
+  if (as[1] != bs[0]) throw GraphError("matmul inner dimensions must match");
+  return add_raw_node(Op::MatMul, {a, b}, TensorType{{as[0], bs[1]}, DType::F32});
+}
+
+// src/graph.rs:821-827
+NodeId Graph::add(NodeId a, NodeId b) {
+  if (node(a).ty.shape != node(b).ty.shape) throw GraphError("add requires matching shapes");
+  return add_raw_node(Op::Add, {a, b}, TensorType{node(a).ty.shape, DType::F32});
+}
+
+// src/graph.rs:996-999
+NodeId Graph::swiglu(NodeId gate, NodeId up) {
+  if (node(gate).ty.shape != node(up).ty.shape) throw GraphError("swiglu requires matching shapes");
+  return add_raw_node(Op::SwiGLU, {gate, up}, TensorType{node(gate).ty.shape, DType::F32});
+}
+
+// src/graph.rs:1029-1040
+NodeId Graph::rms_norm(NodeId x, NodeId weight, float eps) {
+  const auto& xs = node(x).ty.shape;
+  const auto& ws = node(weight).ty.shape;
+  if (xs.size() != 2) throw GraphError("rms_norm requires 2D input");
+  if (ws.size() != 1) throw GraphError("rms_norm weight must be 1D");
+  if (xs[1] != ws[0]) throw GraphError("rms_norm weight size must match last dim");
+  return add_raw_node(Op::RmsNorm, {x, weight}, TensorType{xs, DType::F32}, {}, eps);
+}
+
+void Graph::set_outputs(std::vector<NodeId> ids) {
+  for (NodeId id : ids) (void)node(id);
+  outputs_ = std::move(ids);
+}
+
+// ------------------------------------------------------------- optimize ----
+
+static size_t use_count(const Graph& g, NodeId id) {
+  size_t n = 0;
+  for (const Node& nd : g.nodes())
+    if (nd.op != Op::Nop && std::find(nd.inputs.begin(), nd.inputs.end(), id) != nd.inputs.end()) n++;
+  return n;
+}
+
+// src/optimize.rs:724-767: Add(MatMul(a,b), d) -> FusedMatMulAdd(a,b,d) when the
+// matmul feeds only this Add and is not itself a graph output.
+static bool apply_matmul_add_fusions(Graph& g) {
+  bool changed = false;
+  const size_t count = g.nodes().size();
+  for (size_t id = 0; id < count; id++) {
+    const Node& nd = g.nodes()[id];
+    if (nd.op != Op::Add) continue;
+    const NodeId lhs = nd.inputs[0], rhs = nd.inputs[1];
+    NodeId mm, addend;
+    if (g.node(lhs).op == Op::MatMul) {
+      mm = lhs;
+      addend = rhs;
+    } else if (g.node(rhs).op == Op::MatMul) {
+      mm = rhs;
+      addend = lhs;
+    } else {
+      continue;
+    }
+    if (use_count(g, mm) != 1 || g.is_output(mm)) continue;
+    const NodeId a = g.node(mm).inputs[0], b = g.node(mm).inputs[1];
+    g.nodes_mut()[id].op = Op::FusedMatMulAdd;
+    g.nodes_mut()[id].inputs = {a, b, addend};
+    g.nodes_mut()[mm].op = Op::Nop;
+    changed = true;
+  }
+  return changed;
+}
+
+// src/optimize.rs:776-879: SwiGLU(MatMul(h,Wg), MatMul(h,Wu)) -> SwiGLUConcat(MatMul(h, [Wg|Wu])).
+// The concatenated parameter is named "<gate>+<up>", keeps the sources' dtype
+// (848-854) and is recorded as a derived parameter so that set_parameter on
+// either source refills it (842-847).
+static bool apply_swiglu_concat_fusions(Graph& g) {
+  bool changed = false;
+  const size_t count = g.nodes().size();
+  for (size_t id = 0; id < count; id++) {
+    if (g.nodes()[id].op != Op::SwiGLU) continue;
+    const NodeId gate_id = g.nodes()[id].inputs[0], up_id = g.nodes()[id].inputs[1];
+    const Node gate = g.node(gate_id), up = g.node(up_id);
+    if (gate.op != Op::MatMul || up.op != Op::MatMul) continue;
+    if (gate.inputs[0] != up.inputs[0]) continue;
+    if (use_count(g, gate_id) != 1 || use_count(g, up_id) != 1) continue;
+    if (g.is_output(gate_id) || g.is_output(up_id)) continue;
+    const NodeId h = gate.inputs[0], w_gate = gate.inputs[1], w_up = up.inputs[1];
+    const Node wg = g.node(w_gate), wu = g.node(w_up);
+    if (wg.ty.shape.size() != 2 || wu.ty.shape.size() != 2) continue;
+    if (wg.ty.shape != wu.ty.shape) continue;
+    if (wg.op != Op::Parameter || wu.op != Op::Parameter) continue;
+    // The reference keeps the gate's dtype even if the up projection's differs;
+    // a mixed pair would then be quantized in a format its owner did not ask
+    // for, so here a mixed pair is simply left unfused.
+    if (wg.ty.dtype != wu.ty.dtype) continue;
+    const size_t in_f = wg.ty.shape[0], out_f = wg.ty.shape[1];
+    const std::string name = wg.name + "+" + wu.name;
+    g.derived_params.push_back(DerivedParam{name, {{wg.name, out_f}, {wu.name, out_f}}, in_f});
+    const NodeId concat_w =
+        g.add_raw_node(Op::Parameter, {}, TensorType{{in_f, 2 * out_f}, wg.ty.dtype}, name);
+    const size_t m = g.node(h).ty.shape[0];
+    const NodeId wide = g.add_raw_node(Op::MatMul, {h, concat_w}, TensorType{{m, 2 * out_f}, DType::F32});
+    Node& sw = g.nodes_mut()[id];
+    sw.op = Op::SwiGLUConcat;
+    sw.inputs = {wide};
+    sw.ty = TensorType{{m, out_f}, DType::F32};
+    g.nodes_mut()[gate_id].op = Op::Nop;
+    g.nodes_mut()[up_id].op = Op::Nop;
+    changed = true;
+  }
+  return changed;
+}
+
+Graph optimize(const Graph& src) {
+  Graph g = src;
+  for (int iter = 0; iter < 8; iter++) {
+    bool changed = apply_matmul_add_fusions(g);
+    changed |= apply_swiglu_concat_fusions(g);
+    if (!changed) break;
+  }
+  return g;
+}
+
+// -------------------------------------------------------------- compile ----
+
+static std::vector<NodeId> toposort(const Graph& g) {
+  // fusion appends nodes (the wide matmul) after their consumer, so order by dependencies
+  const size_t n = g.nodes().size();
+  std::vector<int> state(n, 0);
+  std::vector<NodeId> order;
+  order.reserve(n);
+  std::vector<std::pair<NodeId, size_t>> stack;
+  for (NodeId root = 0; root < n; root++) {
+    if (state[root]) continue;
+    stack.push_back({root, 0});
+    state[root] = 1;
+    while (!stack.empty()) {
+      auto& [id, next] = stack.back();
+      const Node& nd = g.nodes()[id];
+      if (next < nd.inputs.size()) {
+        const NodeId in = nd.inputs[next++];
+        if (state[in] == 0) {
+          state[in] = 1;
+          stack.push_back({in, 0});
+        } else if (state[in] == 1) {
+          throw GraphError("cycle in graph");
+        }
+      } else {
+        state[id] = 2;
+        order.push_back(id);
+        stack.pop_back();
+      }
+    }
+  }
+  return order;
+}
+
+ExecutionPlan compile(const Graph& g) {
+  ExecutionPlan plan;
+  std::map<NodeId, int> node_buf;
+  // pass 1 (src/compile.rs:1201-1262): a buffer per live node; quantized parameters are
+  // registered with (format, rows = shape[0], cols = shape[1]) (1229-1241)
+  for (const Node& nd : g.nodes()) {
+    if (nd.op == Op::Nop) continue;
+    const int buf = (int)plan.buffers.size();
+    plan.buffers.push_back(std::max<size_t>(nd.ty.size_bytes(), 4));
+    node_buf[nd.id] = buf;
+    if (nd.op == Op::Parameter) {
+      plan.param_buffers.push_back({nd.name, buf});
+      const WeightFormat wf = weight_format_from(nd.ty.dtype);
+      if (wf != WeightFormat::F32) {
+        const auto& sh = nd.ty.shape;
+        plan.weight_buffers[buf] = WeightBufferInfo{wf, sh[0], sh.size() >= 2 ? sh[1] : 1};
+      }
+    } else if (nd.op == Op::Input) {
+      plan.input_buffers.push_back({nd.name, buf});
+    }
+  }
+  for (const DerivedParam& dp : g.derived_params) {
+    for (const auto& pb : plan.param_buffers)
+      if (pb.first == dp.name) plan.derived_params.push_back({pb.second, dp.sources, dp.rows});
+  }
+  auto buf_of = [&](NodeId id) {
+    auto it = node_buf.find(id);
+    if (it == node_buf.end()) throw GraphError("node consumed after being fused away");
+    return it->second;
+  };
+  // pass 2: one dispatch per compute node
+  for (NodeId id : toposort(g)) {
+    const Node& nd = g.nodes()[id];
+    Dispatch d{};
+    d.output_buffer = nd.op == Op::Nop ? -1 : buf_of(id);
+    switch (nd.op) {
+      case Op::Input:
+      case Op::Parameter:
+      case Op::Nop:
+        continue;
+      case Op::MatMul:
+      case Op::FusedMatMulAdd: {
+        // src/compile.rs:1381-1421, 1486-1524: M == 1 and N % 4 == 0 take the GEMV entry
+        // with grid [N/4,1,1]; everything else the 64x64 tiled entry
+        const auto& as = g.node(nd.inputs[0]).ty.shape;
+        const Node& bn = g.node(nd.inputs[1]);
+        const uint32_t m = (uint32_t)as[0], k = (uint32_t)as[1], n = (uint32_t)bn.ty.shape[1];
+        const bool fused = nd.op == Op::FusedMatMulAdd;
+        if (m == 1 && n % 4 == 0) {
+          d.shader = fused ? MGN_SHADER_MATMUL_GEMV_ADD : MGN_SHADER_MATMUL_GEMV;
+          d.workgroups[0] = n / 4, d.workgroups[1] = 1, d.workgroups[2] = 1;
+        } else {
+          d.shader = fused ? MGN_SHADER_FUSED_MATMUL_ADD : MGN_SHADER_MATMUL;
+          d.workgroups[0] = (n + 63) / 64, d.workgroups[1] = (m + 63) / 64, d.workgroups[2] = 1;
+        }
+        d.input_buffers = {buf_of(nd.inputs[0]), buf_of(nd.inputs[1])};
+        if (fused) d.input_buffers.push_back(buf_of(nd.inputs[2]));
+        d.params[0] = m, d.params[1] = k, d.params[2] = n, d.params[3] = 0;
+        d.weight_format = weight_format_from(bn.ty.dtype);
+        break;
+      }
+      case Op::Add:
+      case Op::SwiGLU: {
+        const uint32_t len = (uint32_t)nd.ty.num_elements();
+        d.shader = nd.op == Op::Add ? MGN_SHADER_ADD : MGN_SHADER_SWIGLU;
+        d.workgroups[0] = (len + 255) / 256, d.workgroups[1] = 1, d.workgroups[2] = 1;
+        d.input_buffers = {buf_of(nd.inputs[0]), buf_of(nd.inputs[1])};
+        d.params[0] = len;
+        break;
+      }
+      case Op::SwiGLUConcat: {
+        // src/compile.rs:1814-1830
+        const uint32_t len = (uint32_t)nd.ty.num_elements();
+        d.shader = MGN_SHADER_SWIGLU_CONCAT;
+        d.workgroups[0] = (len + 255) / 256, d.workgroups[1] = 1, d.workgroups[2] = 1;
+        d.input_buffers = {buf_of(nd.inputs[0])};
+        d.params[0] = len, d.params[1] = (uint32_t)nd.ty.shape[1];
+        break;
+      }
+      case Op::RmsNorm: {
+        // src/compile.rs:1851-1872 (the hand-written entry: one workgroup per row)
+        const auto& xs = g.node(nd.inputs[0]).ty.shape;
+        d.shader = MGN_SHADER_RMS_NORM;
+        d.workgroups[0] = (uint32_t)xs[0], d.workgroups[1] = 1, d.workgroups[2] = 1;
+        d.input_buffers = {buf_of(nd.inputs[0]), buf_of(nd.inputs[1])};
+        d.params[0] = (uint32_t)xs[0], d.params[1] = (uint32_t)xs[1];
+        std::memcpy(&d.params[2], &nd.eps, 4);
+        d.eps = nd.eps;
+        break;
+      }
+    }
+    plan.dispatches.push_back(std::move(d));
+  }
+  for (NodeId out : g.outputs()) plan.output_buffers.push_back(buf_of(out));
+  return plan;
+}
+
+// -------------------------------------------------------------- Session ----
+
+void Session::check(mgn_status st, const char* what) {
+  if (st != MGN_OK) throw std::runtime_error(std::string(what) + ": " + mgn_last_error(ctx_));
+}
+
+static bool is_matmul(mgn_shader s) { return s <= MGN_SHADER_MATMUL_GEMV_ADD; }
+
+Session::Session(ExecutionPlan plan, int device_id) : plan_(std::move(plan)) {
+  // This backend serves matmuls whose weight is quantized; a plain f32 weight
+  // stays with the host runtime's own dispatch.
+  for (const Dispatch& d : plan_.dispatches)
+    if (is_matmul(d.shader) && d.weight_format == WeightFormat::F32)
+      throw std::runtime_error("matmul with an f32 weight is not on the quantized path of this backend");
+  mgn_status st = mgn_ctx_create(device_id, &ctx_);
+  if (st != MGN_OK) throw std::runtime_error(std::string("mgn_ctx_create: ") + mgn_last_error(nullptr));
+  buffers_.assign(plan_.buffers.size(), nullptr);
+  weights_.assign(plan_.buffers.size(), nullptr);
+  try {
+    // every plan buffer exists and is zero-filled up front (src/runtime.rs:1737-1755);
+    // a quantized parameter gets its device storage when it is first set
+    for (size_t i = 0; i < plan_.buffers.size(); i++)
+      if (!plan_.weight_buffers.count((int)i)) check(mgn_buf_alloc(ctx_, plan_.buffers[i], &buffers_[i]), "mgn_buf_alloc");
+  } catch (...) {
+    release();
+    throw;
+  }
+}
+
+Session::~Session() { release(); }
+
+void Session::release() {
+  if (!ctx_) return;
+  (void)mgn_sync(ctx_);  // Drop waits for the GPU first (src/runtime.rs:4339-4345)
+  for (mgn_buf* b : buffers_) mgn_buf_free(ctx_, b);
+  for (mgn_weight* w : weights_) mgn_weight_free(ctx_, w);
+  buffers_.clear();
+  weights_.clear();
+  mgn_ctx_destroy(ctx_);
+  ctx_ = nullptr;
+}
+
+void Session::upload_weight(int buf, const WeightBufferInfo& info, const float* data) {
+  mgn_weight* fresh = nullptr;
+  const mgn_fmt fmt = info.fmt == WeightFormat::Q4 ? MGN_FMT_Q4 : MGN_FMT_Q8;
+  check(mgn_weight_create(ctx_, fmt, data, info.rows, info.cols, &fresh), "mgn_weight_create");
+  mgn_weight_free(ctx_, weights_[buf]);  // waits for in-flight work that may still read it
+  weights_[buf] = fresh;
+}
+
+// src/runtime.rs:2327-2493
+void Session::set_parameter(const std::string& name, const float* data, size_t len) {
+  for (const auto& pb : plan_.param_buffers) {
+    if (pb.first != name) continue;
+    const int buf = pb.second;
+    auto wb = plan_.weight_buffers.find(buf);
+    if (wb != plan_.weight_buffers.end()) {
+      if (len != wb->second.rows * wb->second.cols) throw std::invalid_argument("parameter '" + name + "': length is not rows*cols");
+      upload_weight(buf, wb->second, data);
+    } else {
+      if (len * 4 > plan_.buffers[buf]) throw std::invalid_argument("parameter '" + name + "': data exceeds buffer");
+      check(mgn_buf_upload(ctx_, buffers_[buf], 0, data, len * 4), "mgn_buf_upload");
+    }
+    // derived (horizontally concatenated) parameters fed by this source (2349-2432)
+    for (const auto& dp : plan_.derived_params) {
+      bool feeds = false;
+      size_t total_cols = 0;
+      for (const auto& s : dp.sources) {
+        feeds |= s.first == name;
+        total_cols += s.second;
+      }
+      if (!feeds) continue;
+      auto dwb = plan_.weight_buffers.find(dp.buffer);
+      const size_t rows = dp.rows;
+      // f32 staging copy of the whole concatenated matrix, kept across calls (2373-2391)
+      std::vector<float>& staging = weight_staging_[dp.buffer];
+      if (staging.empty()) staging.assign(rows * total_cols, 0.0f);
+      size_t col_off = 0;
+      for (const auto& s : dp.sources) {
+        if (s.first == name) {
+          if (len != rows * s.second) throw std::invalid_argument("parameter '" + name + "': length does not match derived source");
+          for (size_t r = 0; r < rows; r++)
+            std::memcpy(&staging[r * total_cols + col_off], data + r * s.second, s.second * sizeof(float));
+        }
+        col_off += s.second;
+      }
+      if (dwb != plan_.weight_buffers.end())
+        upload_weight(dp.buffer, dwb->second, staging.data());  // re-quantize the whole matrix (2392-2406)
+      else
+        check(mgn_buf_upload(ctx_, buffers_[dp.buffer], 0, staging.data(), staging.size() * 4), "mgn_buf_upload");
+    }
+    return;
+  }
+  throw std::out_of_range("unknown parameter: " + name);
+}
+
+// src/runtime.rs:2496-2504
+void Session::set_input(const std::string& name, const float* data, size_t len) {
+  for (const auto& ib : plan_.input_buffers) {
+    if (ib.first != name) continue;
+    if (len * 4 > plan_.buffers[ib.second]) throw std::invalid_argument("input '" + name + "': data exceeds buffer");
+    check(mgn_buf_upload(ctx_, buffers_[ib.second], 0, data, len * 4), "mgn_buf_upload");
+    return;
+  }
+  throw std::out_of_range("unknown input: " + name);
+}
+
+// src/runtime.rs:2843-2959: replay the dispatch list on the stream; returns after
+// submission.  Stream order stands in for the barriers between dependency groups.
+void Session::step() {
+  for (const Dispatch& d : plan_.dispatches) {
+    float* out = (float*)buffers_[d.output_buffer]->ptr;
+    auto fin = [&](size_t i) { return (const float*)buffers_[d.input_buffers[i]]->ptr; };
+    int rc = 0;
+    switch (d.shader) {
+      case MGN_SHADER_MATMUL:
+      case MGN_SHADER_MATMUL_GEMV:
+      case MGN_SHADER_FUSED_MATMUL_ADD:
+      case MGN_SHADER_MATMUL_GEMV_ADD: {
+        mgn_weight* w = weights_[d.input_buffers[1]];
+        if (!w) throw std::runtime_error("quantized parameter was never set");
+        const mgn_buf* addend = d.input_buffers.size() > 2 ? buffers_[d.input_buffers[2]] : nullptr;
+        check(mgn_matmul_q(ctx_, buffers_[d.input_buffers[0]], w, addend, buffers_[d.output_buffer], d.params[0]),
+              "mgn_matmul_q");
+        break;
+      }
+      case MGN_SHADER_ADD:
+        rc = launch_add(ctx_->stream, fin(0), fin(1), out, d.params[0]);
+        break;
+      case MGN_SHADER_SWIGLU:
+        rc = launch_swiglu(ctx_->stream, fin(0), fin(1), out, d.params[0]);
+        break;
+      case MGN_SHADER_SWIGLU_CONCAT:
+        rc = launch_swiglu_concat(ctx_->stream, fin(0), out, d.params[0], d.params[1]);
+        break;
+      case MGN_SHADER_RMS_NORM:
+        rc = launch_rms_norm(ctx_->stream, fin(0), fin(1), out, d.params[0], d.params[1], d.eps);
+        break;
+    }
+    if (rc != 0) throw std::runtime_error(std::string("kernel launch: ") + hipGetErrorString((hipError_t)rc));
+  }
+}
+
+void Session::wait() { check(mgn_sync(ctx_), "mgn_sync"); }
+
+void Session::read_output_by_index(size_t index, float* out, size_t len) {
+  if (index >= plan_.output_buffers.size()) throw std::out_of_range("output index out of range");
+  const int buf = plan_.output_buffers[index];
+  if (!buffers_[buf]) throw std::runtime_error("output is a quantized parameter");
+  if (len * 4 > plan_.buffers[buf]) throw std::invalid_argument("read_output: length exceeds buffer");
+  check(mgn_buf_download(ctx_, buffers_[buf], 0, out, len * 4), "mgn_buf_download");
+}
+
+std::unique_ptr<Session> build_inference_session(const Graph& g, int device_id) {
+  return std::make_unique<Session>(compile(optimize(g)), device_id);
+}
+
+}  // namespace mgn
+
+// ------------------------------------------------------------ C wrappers ----
+
+struct mgn_graph {
+  mgn::Graph g;
+  std::string err;
+};
+
+struct mgn_session {
+  std::unique_ptr<mgn::Session> s;
+  std::string err;
+};
+
+namespace {
+
+thread_local std::string g_build_error;
+
+template <class F>
+int32_t graph_node(mgn_graph* g, F&& f) {
+  if (!g) return -(int32_t)MGN_EINVAL;
+  try {
+    return (int32_t)f();
+  } catch (const std::exception& e) {
+    g->err = e.what();
+    return -(int32_t)MGN_EINVAL;
+  }
+}
+
+std::vector<size_t> shape2(size_t rows, size_t cols) { return cols == 0 ? std::vector<size_t>{rows} : std::vector<size_t>{rows, cols}; }
+
+void fill_info(const mgn::Dispatch& d, mgn_dispatch_info* out) {
+  out->shader = d.shader;
+  for (int i = 0; i < 3; i++) out->workgroups[i] = d.workgroups[i];
+  for (int i = 0; i < 4; i++) out->params[i] = d.params[i];
+  out->weight_format = (int32_t)d.weight_format;
+}
+
+template <class F>
+mgn_status session_call(mgn_session* s, F&& f) {
+  if (!s || !s->s) return MGN_EINVAL;
+  try {
+    f();
+    return MGN_OK;
+  } catch (const std::out_of_range& e) {
+    s->err = e.what();
+    return MGN_ENOTFOUND;
+  } catch (const std::invalid_argument& e) {
+    s->err = e.what();
+    return MGN_EINVAL;
+  } catch (const std::bad_alloc&) {
+    s->err = "out of host memory";
+    return MGN_ENOMEM;
+  } catch (const std::exception& e) {
+    s->err = e.what();
+    return MGN_EHIP;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+mgn_graph* mgn_graph_new(void) { return new (std::nothrow) mgn_graph(); }
+void mgn_graph_free(mgn_graph* g) { delete g; }
+const char* mgn_graph_last_error(const mgn_graph* g) { return g ? g->err.c_str() : g_build_error.c_str(); }
+
+// a 1-D shape is passed as cols == 0
+int32_t mgn_graph_input(mgn_graph* g, const char* name, size_t rows, size_t cols) {
+  return graph_node(g, [&] { return g->g.input(name ? name : "", shape2(rows, cols)); });
+}
+int32_t mgn_graph_parameter(mgn_graph* g, const char* name, size_t rows, size_t cols) {
+  return graph_node(g, [&] { return g->g.parameter(name ? name : "", shape2(rows, cols)); });
+}
+int32_t mgn_graph_parameter_q4(mgn_graph* g, const char* name, size_t rows, size_t cols) {
+  return graph_node(g, [&] { return g->g.parameter_q4(name ? name : "", shape2(rows, cols)); });
+}
+int32_t mgn_graph_parameter_q8(mgn_graph* g, const char* name, size_t rows, size_t cols) {
+  return graph_node(g, [&] { return g->g.parameter_q8(name ? name : "", shape2(rows, cols)); });
+}
+int32_t mgn_graph_matmul(mgn_graph* g, int32_t a, int32_t b) {
+  return graph_node(g, [&] { return g->g.matmul((mgn::NodeId)a, (mgn::NodeId)b); });
+}
+int32_t mgn_graph_add(mgn_graph* g, int32_t a, int32_t b) {
+  return graph_node(g, [&] { return g->g.add((mgn::NodeId)a, (mgn::NodeId)b); });
+}
+int32_t mgn_graph_swiglu(mgn_graph* g, int32_t gate, int32_t up) {
+  return graph_node(g, [&] { return g->g.swiglu((mgn::NodeId)gate, (mgn::NodeId)up); });
+}
+int32_t mgn_graph_rms_norm(mgn_graph* g, int32_t x, int32_t weight, float eps) {
+  return graph_node(g, [&] { return g->g.rms_norm((mgn::NodeId)x, (mgn::NodeId)weight, eps); });
+}
+
+mgn_status mgn_graph_set_outputs(mgn_graph* g, const int32_t* ids, size_t count) {
+  if (!g || (!ids && count)) return MGN_EINVAL;
+  try {
+    std::vector<mgn::NodeId> v(ids, ids + count);
+    g->g.set_outputs(std::move(v));
+    return MGN_OK;
+  } catch (const std::exception& e) {
+    g->err = e.what();
+    return MGN_EINVAL;
+  }
+}
+
+mgn_status mgn_graph_compile(const mgn_graph* g, mgn_dispatch_info* out, size_t cap, size_t* count) {
+  if (!g || !count) return MGN_EINVAL;
+  try {
+    const mgn::ExecutionPlan plan = mgn::compile(mgn::optimize(g->g));
+    *count = plan.dispatches.size();
+    for (size_t i = 0; i < plan.dispatches.size() && i < cap && out; i++) fill_info(plan.dispatches[i], &out[i]);
+    return MGN_OK;
+  } catch (const std::exception& e) {
+    g_build_error = e.what();
+    return MGN_EINVAL;
+  }
+}
+
+mgn_status mgn_build_inference_session(const mgn_graph* g, int device_id, mgn_session** out) {
+  if (!g || !out) return MGN_EINVAL;
+  *out = nullptr;
+  auto* s = new (std::nothrow) mgn_session();
+  if (!s) return MGN_ENOMEM;
+  try {
+    s->s = mgn::build_inference_session(g->g, device_id);
+  } catch (const mgn::GraphError& e) {
+    g_build_error = e.what();
+    delete s;
+    return MGN_EINVAL;
+  } catch (const std::exception& e) {
+    g_build_error = e.what();
+    delete s;
+    return std::strstr(e.what(), "mgn_ctx_create") ? MGN_ENODEVICE : MGN_EINVAL;
+  }
+  *out = s;
+  return MGN_OK;
+}
+
+void mgn_session_free(mgn_session* s) { delete s; }
+const char* mgn_session_last_error(const mgn_session* s) { return s ? s->err.c_str() : g_build_error.c_str(); }
+
+size_t mgn_session_num_dispatches(const mgn_session* s) { return s && s->s ? s->s->plan().dispatches.size() : 0; }
+
+mgn_status mgn_session_dispatch_info(const mgn_session* s, size_t index, mgn_dispatch_info* out) {
+  if (!s || !s->s || !out || index >= s->s->plan().dispatches.size()) return MGN_EINVAL;
+  fill_info(s->s->plan().dispatches[index], out);
+  return MGN_OK;
+}
+
+mgn_status mgn_session_set_parameter(mgn_session* s, const char* name, const float* data, size_t len) {
+  if (!name || !data) return MGN_EINVAL;
+  return session_call(s, [&] { s->s->set_parameter(name, data, len); });
+}
+mgn_status mgn_session_set_input(mgn_session* s, const char* name, const float* data, size_t len) {
+  if (!name || !data) return MGN_EINVAL;
+  return session_call(s, [&] { s->s->set_input(name, data, len); });
+}
+mgn_status mgn_session_step(mgn_session* s) { return session_call(s, [&] { s->s->step(); }); }
+mgn_status mgn_session_wait(mgn_session* s) { return session_call(s, [&] { s->s->wait(); }); }
+mgn_status mgn_session_read_output(mgn_session* s, float* out, size_t len) {
+  if (!out) return MGN_EINVAL;
+  return session_call(s, [&] { s->s->read_output(out, len); });
+}
+mgn_status mgn_session_read_output_by_index(mgn_session* s, size_t index, float* out, size_t len) {
+  if (!out) return MGN_EINVAL;
+  return session_call(s, [&] { s->s->read_output_by_index(index, out, len); });
+}
+mgn_ctx* mgn_session_ctx(mgn_session* s) { return s && s->s ? s->s->ctx() : nullptr; }
+
+}  // extern "C"

@@ -1,0 +1,167 @@
+// Host-side mirror of meganeura's Graph / compile / Session for the quantized
+// matmul path.  Paths cited are relative to the reference checkout.
+#pragma once
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "mgn_internal.h"
+#include "../../include/mgn_session.h"
+
+namespace mgn {
+
+using NodeId = uint32_t;
+
+// graph::DType (src/graph.rs:5-16); F16/U32 do not occur on this path.
+enum class DType { F32, Q4_0, Q8_0 };
+
+// compile::WeightFormat (src/compile.rs:8-29)
+enum class WeightFormat { F32 = 0, Q4 = 1, Q8 = 2 };
+inline WeightFormat weight_format_from(DType d) {
+  return d == DType::Q4_0 ? WeightFormat::Q4 : d == DType::Q8_0 ? WeightFormat::Q8 : WeightFormat::F32;
+}
+
+// TensorType (src/graph.rs:29-68)
+struct TensorType {
+  std::vector<size_t> shape;
+  DType dtype = DType::F32;
+  size_t num_elements() const {
+    size_t n = 1;
+    for (size_t s : shape) n *= s;
+    return n;
+  }
+  // block-level sizing for quantized types (src/graph.rs:52-68)
+  size_t size_bytes() const {
+    const size_t blocks = (num_elements() + 31) / 32;
+    if (dtype == DType::Q4_0) return blocks * 20;
+    if (dtype == DType::Q8_0) return blocks * 36;
+    return num_elements() * 4;
+  }
+};
+
+enum class Op { Input, Parameter, MatMul, Add, SwiGLU, RmsNorm, FusedMatMulAdd, SwiGLUConcat, Nop };
+
+struct Node {
+  NodeId id;
+  Op op;
+  std::string name;  // Input / Parameter
+  std::vector<NodeId> inputs;
+  TensorType ty;
+  float eps = 0.0f;  // RmsNorm
+};
+
+// graph::DerivedParam with ParamTransform::HorizontalConcat (src/graph.rs:521-545)
+struct DerivedParam {
+  std::string name;
+  std::vector<std::pair<std::string, size_t>> sources;  // (name, cols)
+  size_t rows;
+};
+
+struct GraphError : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
+class Graph {
+ public:
+  NodeId input(const std::string& name, std::vector<size_t> shape);
+  NodeId parameter(const std::string& name, std::vector<size_t> shape);
+  NodeId parameter_q4(const std::string& name, std::vector<size_t> shape);
+  NodeId parameter_q8(const std::string& name, std::vector<size_t> shape);
+  NodeId matmul(NodeId a, NodeId b);
+  NodeId add(NodeId a, NodeId b);
+  NodeId swiglu(NodeId gate, NodeId up);
+  NodeId rms_norm(NodeId x, NodeId weight, float eps);
+  void set_outputs(std::vector<NodeId> ids);
+
+  const Node& node(NodeId id) const;
+  const std::vector<Node>& nodes() const { return nodes_; }
+  std::vector<Node>& nodes_mut() { return nodes_; }
+  const std::vector<NodeId>& outputs() const { return outputs_; }
+  bool is_output(NodeId id) const;
+  NodeId add_raw_node(Op op, std::vector<NodeId> inputs, TensorType ty, std::string name = {}, float eps = 0.0f);
+  std::vector<DerivedParam> derived_params;
+
+ private:
+  std::vector<Node> nodes_;
+  std::vector<NodeId> outputs_;
+};
+
+// optimize::apply_matmul_add_fusions + apply_swiglu_concat_fusions
+// (src/optimize.rs:724-767, 776-879), run to a fixpoint as the reference's loop
+// does (src/optimize.rs:645-665).
+Graph optimize(const Graph& g);
+
+struct Dispatch {
+  mgn_shader shader;
+  uint32_t workgroups[3];
+  std::vector<int> input_buffers;
+  int output_buffer;
+  uint32_t params[4];
+  WeightFormat weight_format = WeightFormat::F32;
+  float eps = 0.0f;
+};
+
+// compile::ExecutionPlan (src/compile.rs:494-528), the fields this path uses.
+struct WeightBufferInfo {
+  WeightFormat fmt;
+  size_t rows, cols;
+};
+struct ExecutionPlan {
+  std::vector<size_t> buffers;  // byte sizes
+  std::vector<Dispatch> dispatches;
+  std::vector<std::pair<std::string, int>> param_buffers;
+  std::vector<std::pair<std::string, int>> input_buffers;
+  std::vector<int> output_buffers;
+  std::map<int, WeightBufferInfo> weight_buffers;
+  struct Derived {
+    int buffer;
+    std::vector<std::pair<std::string, size_t>> sources;
+    size_t rows;
+  };
+  std::vector<Derived> derived_params;
+};
+
+// compile::compile_with for the ops above (src/compile.rs:1199-1272, 1381-1421, 1486-1524).
+ExecutionPlan compile(const Graph& g);
+
+class Session {
+ public:
+  Session(ExecutionPlan plan, int device_id);
+  ~Session();
+  Session(const Session&) = delete;
+  Session& operator=(const Session&) = delete;
+
+  const ExecutionPlan& plan() const { return plan_; }
+  void set_parameter(const std::string& name, const float* data, size_t len);
+  void set_input(const std::string& name, const float* data, size_t len);
+  void step();
+  void wait();
+  void read_output(float* out, size_t len) { read_output_by_index(0, out, len); }
+  void read_output_by_index(size_t index, float* out, size_t len);
+  mgn_ctx* ctx() { return ctx_; }
+
+ private:
+  void upload_weight(int buf, const WeightBufferInfo& info, const float* data);
+  void check(mgn_status st, const char* what);
+  void release();
+  ExecutionPlan plan_;
+  mgn_ctx* ctx_ = nullptr;
+  std::vector<mgn_buf*> buffers_;        // f32 buffers (null for quantized params)
+  std::vector<mgn_weight*> weights_;     // quantized params (null otherwise)
+  std::map<int, std::vector<float>> weight_staging_;  // src/runtime.rs:2373-2376
+};
+
+// build_inference_session (src/train.rs:380-389): optimize -> compile -> Session.
+std::unique_ptr<Session> build_inference_session(const Graph& g, int device_id = 0);
+
+// pointwise kernels of the session layer (kernels_util.hip)
+int launch_add(ihipStream_t* s, const float* a, const float* b, float* out, size_t len);
+int launch_swiglu(ihipStream_t* s, const float* gate, const float* up, float* out, size_t len);
+int launch_swiglu_concat(ihipStream_t* s, const float* in, float* out, size_t len, uint32_t half_n);
+int launch_rms_norm(ihipStream_t* s, const float* x, const float* weight, float* out, uint32_t rows, uint32_t cols,
+                    float eps);
+
+}  // namespace mgn

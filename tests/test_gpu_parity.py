@@ -1,0 +1,178 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI.
+
+Bars: dequantized weights and packed bytes bit-exact; matmul outputs within
+1e-3 relative OR 1e-4 absolute of the f32 sequential-k result on the oracle's
+dequantized weights (helper semantics of tests/gemv_parity.rs:61-72)."""
+import numpy as np
+import pytest
+
+from helpers import Q4, Q8, bits, ref_test_inputs_q4_matmul
+from meganeura_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+REL, ABS = 1e-3, 1e-4
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+def run_matmul(ctx, fmt, x, w_or_weight, route=capi.ROUTE_AUTO, d=None, f16=False):
+    m, k = x.shape
+    weight = w_or_weight if isinstance(w_or_weight, capi.Weight) else ctx.weight(fmt, w_or_weight)
+    n = weight.cols
+    a = ctx.upload(x.astype(np.float16) if f16 else x)
+    c = ctx.buffer(m * n * 4)
+    dbuf = ctx.upload(d) if d is not None else None
+    ctx.set_route(route)
+    try:
+        (ctx.matmul_q_f16a if f16 else ctx.matmul_q)(a, weight, c, m, dbuf)
+        out = c.download(np.float32, m * n).reshape(m, n)
+    finally:
+        ctx.set_route(capi.ROUTE_AUTO)
+        a.free(); c.free()
+        if dbuf is not None:
+            dbuf.free()
+        if weight is not w_or_weight:
+            weight.free()
+    return out
+
+
+# ---- weights: bit-exact ------------------------------------------------------------------
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("shape", [(32, 1), (64, 7), (576, 192), (1536, 576), (1024, 300)])
+def test_device_weight_is_bit_exact(ctx, orc, fmt, shape):
+    k, n = shape
+    w = synth.normal(7 + k + n, k * n, 0.02).reshape(k, n)
+    want_packed = orc.quantize(fmt, w)
+    want = orc.dequantize(fmt, want_packed, k, n)
+    wt = ctx.weight(fmt, w)
+    assert (bits(wt.dequantize()) == bits(want)).all()
+    assert (wt.export_ref() == want_packed).all()
+    wt.free()
+    # the same weight from pre-packed bytes and from the device-side quantizer
+    wt = ctx.weight_from_packed(fmt, want_packed, k, n)
+    assert (bits(wt.dequantize()) == bits(want)).all()
+    wt.free()
+    src = ctx.upload(w)
+    wt = ctx.weight_from_device(fmt, src, k, n)
+    assert (wt.export_ref() == want_packed).all()
+    wt.free(); src.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+def test_device_weight_extreme_scales(ctx, orc, fmt):
+    # half-subnormal scales must decode as the half crate does (kept, not flushed),
+    # and the device quantizer must agree on ties, zero and constant blocks
+    rng = np.random.default_rng(12)
+    k, n = 64, 48
+    w = rng.standard_normal((k, n)).astype(np.float32)
+    w[:, 0] *= 1e-6
+    w[:, 1] *= 3e-8
+    w[:, 2] *= 1e3
+    w[:, 3] = 0.0
+    w[:, 4] = 0.375
+    w[:32, 5] = np.linspace(0, 15, 32, dtype=np.float32)
+    w[:32, 6] = np.arange(32, dtype=np.float32) * 0.5
+    w[0, 7] = 127.0
+    w[1:5, 7] = [0.5, 2.5, -0.5, -2.5]
+    want_packed = orc.quantize(fmt, w)
+    want = orc.dequantize(fmt, want_packed, k, n)
+    wt = ctx.weight(fmt, w)
+    assert (bits(wt.dequantize()) == bits(want)).all()
+    wt.free()
+    src = ctx.upload(w)
+    wt = ctx.weight_from_device(fmt, src, k, n)
+    assert (wt.export_ref() == want_packed).all()
+    assert (bits(wt.dequantize()) == bits(want)).all()
+    wt.free(); src.free()
+
+
+def test_weight_errors(ctx):
+    with pytest.raises(capi.MgnError, match="multiple of 32"):
+        ctx.weight(Q4, np.zeros((48, 8), np.float32))
+    wt = ctx.weight(Q4, np.zeros((64, 8), np.float32))
+    a = ctx.buffer(4 * 10)
+    c = ctx.buffer(4 * 8)
+    with pytest.raises(capi.MgnError, match="smaller"):
+        ctx.matmul_q(a, wt, c, 1)
+    a.free(); c.free(); wt.free()
+
+
+# ---- matmul: every route at small and ragged shapes ----------------------------------------
+
+ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv": capi.ROUTE_GEMV, "auto": capi.ROUTE_AUTO}
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("route", ["generic", "gemv", "auto"])
+@pytest.mark.parametrize("m,k,n", [
+    (1, 32, 1), (1, 64, 3), (1, 576, 192), (1, 576, 577), (1, 1536, 576), (1, 1024, 100),
+    (2, 576, 65), (3, 2048, 130), (4, 4096, 257), (1, 14336, 64), (1, 3072, 1024),
+])
+def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
+    x = synth.normal(1000 + m + k + n, m * k).reshape(m, k)
+    w = synth.normal(2000 + m + k + n, k * n, 0.02).reshape(k, n)
+    d = synth.normal(3000 + n, m * n).reshape(m, n)
+    deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
+    try:
+        got = run_matmul(ctx, fmt, x, w, ROUTES[route])
+        got_d = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d)
+    except capi.MgnError as e:
+        if route == "gemv" and "does not support" in str(e):
+            pytest.skip("shape outside the GEMV kernel's range")
+        raise
+    orc.assert_close(got, orc.matmul_f32(x, deq), REL, ABS)
+    orc.assert_close(got_d, orc.matmul_f32(x, deq, d), REL, ABS)
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m,k,n", [(5, 64, 70), (6, 1024, 2048), (16, 576, 130), (17, 256, 64), (64, 128, 96), (130, 96, 67)])
+def test_larger_m(ctx, orc, fmt, m, k, n):
+    x = synth.normal(11 + m + k + n, m * k).reshape(m, k)
+    w = synth.normal(12 + m + k + n, k * n, 0.02).reshape(k, n)
+    d = synth.normal(13 + n, m * n).reshape(m, n)
+    deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
+    for route in ("generic", "auto"):
+        got = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d)
+        orc.assert_close(got, orc.matmul_f32(x, deq, d), REL, ABS)
+        # fp16 activations: the oracle multiplies the rounded values
+        x16 = x.astype(np.float16).astype(np.float32)
+        got = run_matmul(ctx, fmt, x, w, ROUTES[route], f16=True)
+        orc.assert_close(got, orc.matmul_f32(x16, deq), REL, ABS)
+
+
+def test_reference_q4_matmul_correctness_inputs(ctx, orc):
+    # tests/gpu_smoke.rs:2681-2771 (m=6, k=1024, n=2048; the reference's own bar is abs 0.1)
+    a, b = ref_test_inputs_q4_matmul()
+    packed = orc.quantize(Q4, b)
+    want = orc.matmul_packed(Q4, a, packed, 2048)
+    for route in ("generic", "auto"):
+        got = run_matmul(ctx, Q4, a, b, ROUTES[route])
+        assert np.abs(got - want).max() < 0.1
+        orc.assert_close(got, want, REL, ABS)
+    # and row by row through the M=1 route
+    for r in (0, 5):
+        got = run_matmul(ctx, Q4, a[r:r + 1], b)
+        orc.assert_close(got, want[r:r + 1], REL, ABS)
+
+
+def test_linearity_and_zero_input(ctx):
+    # size-independent properties: W(0) = 0; W(x + y) = W(x) + W(y) to rounding; W(2x) = 2 W(x) exactly
+    k, n = 4096, 1024
+    w = synth.weights(5, k, n)
+    wt = ctx.weight(Q4, w)
+    x = synth.activations(5, 1, k)
+    y = synth.activations(5, 1, k, which=1)
+    fx = run_matmul(ctx, Q4, x, wt)
+    assert (run_matmul(ctx, Q4, np.zeros_like(x), wt) == 0).all()
+    assert (run_matmul(ctx, Q4, 2 * x, wt) == 2 * fx).all()
+    fy = run_matmul(ctx, Q4, y, wt)
+    fxy = run_matmul(ctx, Q4, x + y, wt)
+    assert np.abs(fxy - (fx + fy)).max() < 2e-4
+    wt.free()

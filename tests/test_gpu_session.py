@@ -1,0 +1,164 @@
+"""The Graph / Session surface end to end on the GPU, written after the
+reference's own tests (tests/gpu_smoke.rs, tests/gemv_parity.rs)."""
+import numpy as np
+import pytest
+
+from helpers import Q4, Q8, gemv_parity_inputs, golden_ratio_weights, ref_test_inputs_q4_matmul
+from meganeura_amd import capi, synth
+from meganeura_amd.graph import Graph, ShaderEntry, build_inference_session
+
+pytestmark = pytest.mark.gpu
+
+
+def test_q4_matmul_correctness(orc):
+    # tests/gpu_smoke.rs:2681-2771
+    m, k, n = 6, 1024, 2048
+    g = Graph()
+    a = g.input("a", [m, k])
+    b = g.parameter_q4("b", [k, n])
+    g.set_outputs([g.matmul(a, b)])
+    sess = build_inference_session(g)
+    a_data, b_data = ref_test_inputs_q4_matmul()
+    sess.set_input("a", a_data)
+    sess.set_parameter("b", b_data)
+    sess.step()
+    sess.wait()
+    out = sess.read_output(m * n)
+    b_deq = orc.dequantize(Q4, orc.quantize(Q4, b_data), k, n)
+    cpu = orc.matmul_f32(a_data, b_deq).reshape(-1)
+    assert not np.isnan(out).any()
+    assert np.abs(cpu - out).max() < 0.1
+    orc.assert_close(out, cpu, 1e-3, 1e-4)
+    sess.close()
+
+
+@pytest.mark.parametrize("quant", ["q4", "q8"])
+@pytest.mark.parametrize("k,n,seed", [(64, 64, 1), (576, 576, 2), (576, 1536, 3), (1536, 576, 4), (576, 49152, 5), (64, 66, 6)])
+def test_gemv_shapes(orc, quant, k, n, seed):
+    # tests/gemv_parity.rs:74-130 shapes, with the weight quantized
+    fmt = Q4 if quant == "q4" else Q8
+    a, b = gemv_parity_inputs(k, n, seed)
+    g = Graph()
+    an = g.input("a", [1, k])
+    bn = (g.parameter_q4 if quant == "q4" else g.parameter_q8)("b", [k, n])
+    g.set_outputs([g.matmul(an, bn)])
+    sess = build_inference_session(g)
+    gemv = [d for d in sess.plan() if d.shader == ShaderEntry.MatMulGemv]
+    assert len(gemv) == (1 if n % 4 == 0 else 0)
+    sess.set_input("a", a)
+    sess.set_parameter("b", b)
+    sess.step()
+    sess.wait()
+    gpu = sess.read_output(n)
+    cpu = orc.matmul_f32(a, orc.dequantize(fmt, orc.quantize(fmt, b), k, n)).reshape(-1)
+    orc.assert_close(gpu, cpu, 1e-3, 1e-4)
+    sess.close()
+
+
+@pytest.mark.parametrize("k,n,seed", [(1536, 576, 100), (576, 576, 101), (2048, 720, 102)])
+def test_gemv_add_shapes(orc, k, n, seed):
+    # tests/gemv_parity.rs:133-196: MatMul + Add fuses and takes the GemvAdd entry at M = 1
+    a, b = gemv_parity_inputs(k, n, seed)
+    d = np.sin(np.arange(n, dtype=np.float32) * np.float32(0.01)).reshape(1, n)
+    g = Graph()
+    an = g.input("a", [1, k])
+    bn = g.parameter_q4("b", [k, n])
+    dn = g.parameter("d", [1, n])
+    g.set_outputs([g.add(g.matmul(an, bn), dn)])
+    sess = build_inference_session(g)
+    assert [x.shader for x in sess.plan()] == [ShaderEntry.MatMulGemvAdd]
+    sess.set_input("a", a)
+    sess.set_parameter("b", b)
+    sess.set_parameter("d", d)
+    sess.step()
+    sess.wait()
+    gpu = sess.read_output(n)
+    cpu = orc.matmul_f32(a, orc.dequantize(Q4, orc.quantize(Q4, b), k, n), d).reshape(-1)
+    orc.assert_close(gpu, cpu, 1e-3, 1e-4)
+    sess.close()
+
+
+def _silu_mul(gate, up):
+    gate = gate.astype(np.float32)
+    sig = np.float32(1) / (np.float32(1) + np.exp(-gate, dtype=np.float32))
+    return gate * sig * up
+
+
+@pytest.mark.parametrize("seq,hidden,ffn", [(1, 576, 1536), (6, 1024, 3072)])
+def test_q4_mlp_block_with_fused_gate_up(orc, seq, hidden, ffn):
+    # the MLP half of tests/gpu_smoke.rs:2824-2835 (q4_layer_nan_hunt), with values checked:
+    # x + down(swiglu(gate(h), up(h))), gate/up fused into one wide matmul on a derived weight
+    g = Graph()
+    x = g.input("x", [seq, hidden])
+    ln = g.parameter("ln2", [hidden])
+    h = g.rms_norm(x, ln, 1e-6)
+    gate = g.matmul(h, g.parameter_q4("wg", [hidden, ffn]))
+    up = g.matmul(h, g.parameter_q4("wu", [hidden, ffn]))
+    act = g.swiglu(gate, up)
+    out = g.add(x, g.matmul(act, g.parameter_q4("wd", [ffn, hidden])))
+    g.set_outputs([out])
+    sess = build_inference_session(g)
+    shaders = [d.shader for d in sess.plan()]
+    mm = ShaderEntry.MatMulGemv if seq == 1 else ShaderEntry.MatMul
+    mma = ShaderEntry.MatMulGemvAdd if seq == 1 else ShaderEntry.FusedMatMulAdd
+    assert shaders == [ShaderEntry.RmsNorm, mm, ShaderEntry.SwiGLUConcat, mma]
+
+    xv = synth.normal(77, seq * hidden).reshape(seq, hidden)
+    wg = golden_ratio_weights(hidden * ffn).reshape(hidden, ffn) * np.float32(0.1)
+    wu = synth.normal(78, hidden * ffn, 0.02).reshape(hidden, ffn)
+    wd = synth.normal(79, ffn * hidden, 0.02).reshape(ffn, hidden)
+    sess.set_input("x", xv)
+    sess.set_parameter("ln2", np.ones(hidden, np.float32))
+    sess.set_parameter("wg", wg)
+    sess.set_parameter("wu", wu)
+    sess.set_parameter("wd", wd)
+    with pytest.raises(KeyError, match="unknown parameter"):
+        sess.set_parameter("nope", wd)
+    sess.step()
+    sess.wait()
+    got = sess.read_output(seq * hidden).reshape(seq, hidden)
+
+    deq = lambda w: orc.dequantize(Q4, orc.quantize(Q4, w), *w.shape)
+    hn = xv * (np.float32(1) / np.sqrt((xv.astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-6)).astype(np.float32)
+    gate_o = orc.matmul_f64(hn, deq(wg))
+    up_o = orc.matmul_f64(hn, deq(wu))
+    want = orc.matmul_f64(_silu_mul(gate_o, up_o), deq(wd), xv)
+    assert np.isfinite(got).all()
+    # three chained ops: compare with a bar scaled to the block's output, not the single-matmul bar
+    orc.assert_close(got, want, 2e-3, 2e-4)
+
+    # setting one source again re-quantizes the derived weight (src/runtime.rs:2347-2406)
+    sess.set_parameter("wu", np.zeros_like(wu))
+    sess.step()
+    sess.wait()
+    got0 = sess.read_output(seq * hidden).reshape(seq, hidden)
+    orc.assert_close(got0, xv, 1e-6, 1e-6)
+    sess.close()
+
+
+def test_q8_session_and_stepping_twice(orc):
+    m, k, n = 1, 576, 1536
+    g = Graph()
+    a = g.input("a", [m, k])
+    b = g.parameter_q8("b", [k, n])
+    g.set_outputs([g.matmul(a, b)])
+    sess = build_inference_session(g)
+    w = synth.weights(1, k, n)
+    deq = orc.dequantize(Q8, orc.quantize(Q8, w), k, n)
+    sess.set_parameter("b", w)
+    for which in (0, 1):
+        x = synth.activations(1, m, k, which=which)
+        sess.set_input("a", x)
+        sess.step()
+        sess.wait()
+        orc.assert_close(sess.read_output(n), orc.matmul_f32(x, deq), 1e-3, 1e-4)
+    sess.close()
+
+
+def test_f32_weight_matmul_is_refused():
+    g = Graph()
+    a = g.input("a", [1, 64])
+    b = g.parameter("b", [64, 64])
+    g.set_outputs([g.matmul(a, b)])
+    with pytest.raises(capi.MgnError, match="quantized path"):
+        build_inference_session(g)

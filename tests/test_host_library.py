@@ -1,0 +1,174 @@
+"""CPU-side checks of the shipped library: the C ABI loads and exports every
+declared symbol, the host quantizers equal the oracle byte for byte, and the
+graph compiler routes matmuls as the reference does.  No GPU call is made."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from helpers import Q4, Q8, bits, gemv_parity_inputs
+from meganeura_amd import capi, synth
+from meganeura_amd.graph import Graph, ShaderEntry, WeightFormat
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    declared = set()
+    for header in ("mgn_hip.h", "mgn_session.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        declared |= set(re.findall(r"\b(mgn_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(capi.HIP_SYMBOLS) | set(capi.SESSION_SYMBOLS)
+    for name in sorted(declared):
+        assert hasattr(lib, name), name
+    assert capi.load().mgn_built_for() == b"gfx950"
+
+
+def test_no_product_file_touches_the_oracle():
+    for base, _, files in os.walk(os.path.join(ROOT, "meganeura_amd")):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(base, f), errors="ignore").read()
+                assert "liboracle" not in text and "import oracle" not in text and "from oracle" not in text, f
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("shape", [(32, 1), (64, 7), (576, 192), (1536, 100), (4096, 33)])
+def test_host_quantizer_equals_oracle(orc, fmt, shape):
+    k, n = shape
+    w = synth.normal(100 + k + n + fmt, k * n, 0.02).reshape(k, n)
+    w[0, 0] = 0.0
+    if n > 2:
+        w[:32, 1] = 0.25          # constant block
+        w[:32, 2] = 0.0           # zero block
+    packed = capi.quantize_ref(fmt, w)
+    want = orc.quantize(fmt, w)
+    assert packed.size == capi.packed_size(fmt, k, n) == want.size
+    assert (packed == want).all()
+    got = capi.dequantize_ref(fmt, packed, k, n)
+    assert (bits(got) == bits(orc.dequantize(fmt, want, k, n))).all()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+def test_host_quantizer_extreme_values(orc, fmt):
+    rng = np.random.default_rng(4)
+    k, n = 64, 40
+    w = rng.standard_normal((k, n)).astype(np.float32)
+    w[:, 0] *= 1e-7       # f16-subnormal scales
+    w[:, 1] *= 1e-10      # scales that round to zero in f16
+    w[:, 2] *= 1e4
+    w[:, 3] *= 1e6        # scales overflow f16 -> inf
+    w[5, 4] = np.nan
+    w[6, 5] = np.inf
+    w[7, 6] = -np.inf
+    w[:, 7] = np.float32(1e-45)
+    w[:32, 8] = np.linspace(0, 15, 32, dtype=np.float32)   # exact ties at .5 steps
+    w[:32, 9] = np.arange(32, dtype=np.float32) * 0.5
+    with np.errstate(all="ignore"):
+        packed = capi.quantize_ref(fmt, w)
+        want = orc.quantize(fmt, w)
+        assert (packed == want).all()
+        a = capi.dequantize_ref(fmt, packed, k, n)
+        b = orc.dequantize(fmt, want, k, n)
+    nan = np.isnan(b)
+    assert (np.isnan(a) == nan).all() and (bits(a)[~nan] == bits(b)[~nan]).all()
+
+
+def test_host_quantizer_rejects_ragged_rows():
+    # src/runtime.rs:2037-2040: "Q4 requires rows (K dim) to be a multiple of 32"
+    with pytest.raises(capi.MgnError):
+        capi.quantize_ref(Q4, np.zeros((48, 4), np.float32))
+    with pytest.raises(capi.MgnError):
+        capi.quantize_ref(Q8, np.zeros((31, 4), np.float32))
+    assert capi.packed_size(Q4, 576, 1536) == 552960   # src/graph.rs:52-68
+    assert capi.packed_size(Q8, 576, 1536) == 995328
+    assert capi.packed_size(Q4, 4096, 14336) == 36700160
+
+
+def test_context_creation_fails_cleanly_without_gpu():
+    lib = capi.load()
+    h = ctypes.c_void_p()
+    st = lib.mgn_ctx_create(10_000, ctypes.byref(h))
+    assert st != capi.OK and not h.value
+    assert lib.mgn_last_error(None)
+
+
+# ---- routing: tests/gemv_parity.rs:32-52, 157-174 -------------------------------------
+
+def _plan(m, k, n, quant="q4", add=False):
+    g = Graph()
+    a = g.input("a", [m, k])
+    b = {"q4": g.parameter_q4, "q8": g.parameter_q8, "f32": g.parameter}[quant]("b", [k, n])
+    out = g.matmul(a, b)
+    if add:
+        out = g.add(out, g.parameter("d", [m, n]))
+    g.set_outputs([out])
+    return g.compile()
+
+
+@pytest.mark.parametrize("quant", ["q4", "q8", "f32"])
+def test_m1_routes_to_gemv_iff_n_multiple_of_4(quant):
+    fmt = {"q4": WeightFormat.Q4, "q8": WeightFormat.Q8, "f32": WeightFormat.F32}[quant]
+    for n in (576, 1536, 49152, 192):
+        (d,) = _plan(1, 576, n, quant)
+        assert d.shader == ShaderEntry.MatMulGemv and d.workgroups == [n // 4, 1, 1]
+        assert d.params == [1, 576, n, 0] and d.weight_format == fmt
+    (d,) = _plan(1, 64, 66, quant)
+    assert d.shader == ShaderEntry.MatMul and d.workgroups == [2, 1, 1]
+    (d,) = _plan(6, 1024, 2048, quant)
+    assert d.shader == ShaderEntry.MatMul and d.workgroups == [32, 1, 1] and d.params == [6, 1024, 2048, 0]
+    (d,) = _plan(512, 1024, 3072, quant)
+    assert d.workgroups == [48, 8, 1]
+
+
+def test_matmul_add_fuses_and_routes():
+    (d,) = _plan(1, 1536, 576, "q4", add=True)
+    assert d.shader == ShaderEntry.MatMulGemvAdd and d.workgroups == [144, 1, 1]
+    (d,) = _plan(4, 1536, 576, "q8", add=True)
+    assert d.shader == ShaderEntry.FusedMatMulAdd and d.weight_format == WeightFormat.Q8
+
+
+def test_matmul_that_is_an_output_is_not_fused():
+    g = Graph()
+    a = g.input("a", [1, 64])
+    b = g.parameter_q4("b", [64, 64])
+    mm = g.matmul(a, b)
+    out = g.add(mm, g.parameter("d", [1, 64]))
+    g.set_outputs([out, mm])
+    shaders = [d.shader for d in g.compile()]
+    assert shaders == [ShaderEntry.MatMulGemv, ShaderEntry.Add]
+
+
+def test_swiglu_of_two_matmuls_becomes_one_wide_matmul():
+    # src/optimize.rs:776-879; the concatenated weight keeps the Q4 dtype (848-854)
+    g = Graph()
+    h = g.input("h", [1, 576])
+    gate = g.matmul(h, g.parameter_q4("w_gate", [576, 1536]))
+    up = g.matmul(h, g.parameter_q4("w_up", [576, 1536]))
+    act = g.swiglu(gate, up)
+    down = g.matmul(act, g.parameter_q4("w_down", [1536, 576]))
+    out = g.add(g.input("resid", [1, 576]), down)
+    g.set_outputs([out])
+    plan = g.compile()
+    assert [d.shader for d in plan] == [ShaderEntry.MatMulGemv, ShaderEntry.SwiGLUConcat, ShaderEntry.MatMulGemvAdd]
+    assert plan[0].params == [1, 576, 3072, 0] and plan[0].weight_format == WeightFormat.Q4
+    assert plan[1].params[:2] == [1536, 1536]
+    assert plan[2].params == [1, 1536, 576, 0]
+
+
+def test_graph_builder_errors():
+    g = Graph()
+    a = g.input("a", [2, 64])
+    b = g.parameter_q4("b", [32, 8])
+    with pytest.raises(ValueError, match="inner dimensions"):
+        g.matmul(a, b)
+    with pytest.raises(ValueError, match="matching shapes"):
+        g.add(a, b)
+    v = g.parameter("v", [64])
+    with pytest.raises(ValueError, match="2D"):
+        g.matmul(a, v)
+    assert g.rms_norm(a, v, 1e-6) >= 0
