@@ -1,0 +1,247 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized matmul path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--sweep]
+
+A step is one launch of the hot kernel over one batch of synthetic input: by
+default the Q4 batch-1 GEMV at the Llama-3-8B FFN shape W[4096,14336] (the
+configuration the headline metric is quoted on).  Steps rotate through enough
+distinct copies of the weight (>= 512 MiB) that no step finds its weight in a
+cache: the figure is an HBM figure.  Inputs are resident in HBM before the
+timed region; the region is bracketed by HIP events recorded on the stream the
+kernels run on, with a device synchronisation on both sides.
+
+Prints ONE JSON line on stdout.  `--sweep` additionally measures every
+BASELINE configuration (cache-cold and cache-warm) and writes the table to
+stderr and, if the directory exists, to gpurun_out/bench_sweep.json.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, vendor figure
+MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA, vendor figure
+
+Q4, Q8 = 0, 1
+
+# name: (fmt, m, k, n, residual, fp16 activations, BASELINE config index)
+WORKLOADS = {
+    "c5_q4_m1_4096x14336": (Q4, 1, 4096, 14336, False, False, 5),
+    "c5_q4_m1_14336x4096": (Q4, 1, 14336, 4096, False, False, 5),
+    "c5_q8_m1_4096x14336": (Q8, 1, 4096, 14336, False, False, 5),
+    "c5_q8_m1_14336x4096": (Q8, 1, 14336, 4096, False, False, 5),
+    "c5_q4_m4_4096x14336": (Q4, 4, 4096, 14336, False, False, 5),
+    "c5_q4_m16_4096x14336": (Q4, 16, 4096, 14336, False, False, 5),
+    "c5_q8_m4_4096x14336": (Q8, 4, 4096, 14336, False, False, 5),
+    "c5_q8_m16_4096x14336": (Q8, 16, 4096, 14336, False, False, 5),
+    "c5_q4_m4_14336x4096": (Q4, 4, 14336, 4096, False, False, 5),
+    "c5_q4_m16_14336x4096": (Q4, 16, 14336, 4096, False, False, 5),
+    "c3_q4_lm_head_576x49152": (Q4, 1, 576, 49152, False, False, 3),
+    "c1_q8_up_576x1536": (Q8, 1, 576, 1536, False, False, 1),
+    "c2_q4_q_576x576": (Q4, 1, 576, 576, False, False, 2),
+    "c2_q4_kv_576x192": (Q4, 1, 576, 192, False, False, 2),
+    "c2_q4_o_576x576_add": (Q4, 1, 576, 576, True, False, 2),
+    "c2_q4_gate_up_576x3072": (Q4, 1, 576, 3072, False, False, 2),
+    "c2_q4_down_1536x576_add": (Q4, 1, 1536, 576, True, False, 2),
+    "c4_q4_prefill_up_512x1024x3072": (Q4, 512, 1024, 3072, False, True, 4),
+    "c4_q4_prefill_down_512x3072x1024": (Q4, 512, 3072, 1024, False, True, 4),
+}
+HEADLINE = "c5_q4_m1_4096x14336"
+
+
+def algorithmic_bytes(fmt, m, k, n, resid, f16):
+    """Bytes one call must move: packed weight once (20 B per Q4 block; 34 B per Q8
+    block, the reference's 2 pad bytes are not credited), activations, output
+    (and the residual when there is one)."""
+    blocks = (k // 32) * n
+    wbytes = blocks * (20 if fmt == Q4 else 34)
+    return wbytes + (2 if f16 else 4) * m * k + 4 * m * n * (2 if resid else 1)
+
+
+class Workload:
+    def __init__(self, ctx, name, min_rotate_bytes):
+        from meganeura_amd import capi, synth
+
+        self.name = name
+        fmt, m, k, n, resid, f16, cfg = WORKLOADS[name]
+        self.fmt, self.m, self.k, self.n, self.resid, self.f16 = fmt, m, k, n, resid, f16
+        self.ctx = ctx
+        self.w_host = synth.weights(cfg, k, n)
+        self.x_host = synth.activations(cfg, m, k)
+        self.packed = capi.quantize_ref(fmt, self.w_host)
+        dev_bytes = (k // 32) * n * (20 if fmt == Q4 else 34)
+        copies = max(2, -(-min_rotate_bytes // dev_bytes)) if min_rotate_bytes else 1
+        self.weights = [ctx.weight_from_packed(fmt, self.packed, k, n) for _ in range(copies)]
+        xs = self.x_host.astype(np.float16) if f16 else self.x_host
+        self.a = ctx.upload(xs)
+        self.c = ctx.buffer(m * n * 4)
+        self.d_host = synth.activations(cfg, m, n, which=3) if resid else None
+        self.d = ctx.upload(self.d_host) if resid else None
+        self.bytes = algorithmic_bytes(fmt, m, k, n, resid, f16)
+        self.flops = 2.0 * m * n * k
+        self.fn = ctx.matmul_q_f16a if f16 else ctx.matmul_q
+        self.i = 0
+
+    def step(self):
+        w = self.weights[self.i % len(self.weights)]
+        self.i += 1
+        self.fn(self.a, w, self.c, self.m, self.d)
+
+    def run(self, steps, warmup):
+        for _ in range(warmup):
+            self.step()
+        self.ctx.sync()
+        self.ctx.timer_start()
+        for _ in range(steps):
+            self.step()
+        ms = self.ctx.timer_stop()  # waits for the stop event
+        self.ctx.sync()
+        return ms / steps
+
+    def output(self):
+        return self.c.download(np.float32, self.m * self.n).reshape(self.m, self.n)
+
+    def free(self):
+        for w in self.weights:
+            w.free()
+        self.a.free()
+        self.c.free()
+        if self.d is not None:
+            self.d.free()
+
+
+def cpu_baseline(wl, budget_s=20.0):
+    """The reference's tiled dequant-on-load algorithm restated for the CPU
+    (oracle/mgn_oracle.c: orc_matmul_q_tiled), one OpenMP task per workgroup, on
+    this box's host cores.  Checker infrastructure used as the timing baseline
+    only; it is never part of the product path."""
+    import oracle
+
+    x = wl.x_host.astype(np.float16).astype(np.float32) if wl.f16 else wl.x_host
+    packed_ref = oracle.quantize(wl.fmt, wl.w_host)
+    t0 = time.perf_counter()
+    out = oracle.matmul_packed(wl.fmt, x, packed_ref, wl.n, wl.d_host, tiled=True)
+    first = time.perf_counter() - t0
+    reps = int(max(1, min(10, budget_s / max(first, 1e-3) - 1)))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        oracle.matmul_packed(wl.fmt, x, packed_ref, wl.n, wl.d_host, tiled=True)
+    per = (time.perf_counter() - t0) / reps
+    return out, {
+        "value": wl.bytes / per / 1e9,
+        "unit": "GB/s",
+        "cores": oracle.num_threads(),
+        "kind": "port",
+        "ms_per_call": per * 1e3,
+        "sample": f"{reps + 1} full calls of {wl.name} (64x64x32-tiled per-element dequant, "
+                  "the reference shader's algorithm, OpenMP over workgroups)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--sweep", action="store_true", help="also measure every configuration (stderr)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no multi-GPU part (column-parallel "
+                 "sharding needs no exchange); run with --gpus 1")
+
+    from meganeura_amd import capi
+    import oracle
+
+    ctx = capi.Context(0)
+    wl = Workload(ctx, args.workload, 512 << 20)
+    ms = wl.run(args.steps, args.warmup)
+    got = wl.output()
+
+    is_gemm = wl.m > 16
+    gbs = wl.bytes / (ms * 1e-3) / 1e9
+    tflops = wl.flops / (ms * 1e-3) / 1e12
+
+    # the timed kernel's result is checked against the oracle before it is reported
+    x = wl.x_host.astype(np.float16).astype(np.float32) if wl.f16 else wl.x_host
+    want = oracle.matmul_packed(wl.fmt, x, oracle.quantize(wl.fmt, wl.w_host), wl.n, wl.d_host)
+    oracle.assert_close(got, want, 1e-3, 1e-4)
+
+    cpu = None
+    if not args.no_cpu:
+        cpu_out, cpu = cpu_baseline(wl)
+        oracle.assert_close(cpu_out, want, 1e-3, 1e-4)
+
+    # cache-warm figure for the same shape (one weight, reused every step)
+    warm = Workload(ctx, args.workload, 0)
+    warm_ms = warm.run(args.steps, args.warmup)
+    warm.free()
+
+    if is_gemm:
+        roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": tflops / MFMA_F16_PEAK_TFLOPS, "traffic": None}
+    else:
+        roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": gbs / HBM_PEAK_GBS, "traffic": None}
+    line = {
+        "metric": "Q4/Q8 GEMV HBM GB/s (% of peak) + us/call; prefill dequant-GEMM TFLOP/s",
+        "value": tflops if is_gemm else gbs,
+        "unit": "TFLOP/s" if is_gemm else "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "us_per_call": ms * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload,
+            "format": "q4" if wl.fmt == Q4 else "q8",
+            "m": wl.m, "k": wl.k, "n": wl.n,
+            "algorithmic_bytes": wl.bytes,
+            "cache": f"cold: rotating {len(wl.weights)} weight copies",
+        },
+        "roofline": roof,
+        "cpu_baseline": cpu,
+        "cache_warm": {"us_per_call": warm_ms * 1e3, "GB/s": wl.bytes / (warm_ms * 1e-3) / 1e9},
+        "pct_of_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
+    }
+    wl.free()
+
+    if args.sweep:
+        rows = []
+        for name in WORKLOADS:
+            row = {"workload": name}
+            for label, rot in (("cold", 512 << 20), ("warm", 0)):
+                w = Workload(ctx, name, rot)
+                t = w.run(max(50, args.steps // 2), args.warmup)
+                row[label + "_us"] = t * 1e3
+                row[label + "_GBs"] = w.bytes / (t * 1e-3) / 1e9
+                row[label + "_TFLOPs"] = w.flops / (t * 1e-3) / 1e12
+                row["bytes"] = w.bytes
+                w.free()
+            row["cold_pct_hbm"] = 100.0 * row["cold_GBs"] / HBM_PEAK_GBS
+            rows.append(row)
+            print(json.dumps(row), file=sys.stderr, flush=True)
+        out_dir = os.path.join(ROOT, "gpurun_out")
+        if os.path.isdir(out_dir):
+            with open(os.path.join(out_dir, "bench_sweep.json"), "w") as f:
+                json.dump(rows, f, indent=1)
+
+    ctx.close()
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

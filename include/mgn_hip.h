@@ -49,9 +49,10 @@ typedef enum mgn_fmt { MGN_FMT_Q4 = 0, MGN_FMT_Q8 = 1 } mgn_fmt;
  * The others exist so that tests can drive every kernel at every shape. */
 typedef enum mgn_route {
   MGN_ROUTE_AUTO = 0,
-  MGN_ROUTE_GENERIC = 1, /* scalar f32 fallback, any M */
-  MGN_ROUTE_GEMV = 2,    /* streaming dequant-GEMV, small M */
-  MGN_ROUTE_MFMA = 3     /* nibble/int8 x fp16 on MFMA with per-block rescale */
+  MGN_ROUTE_GENERIC = 1,   /* scalar f32 fallback, any M */
+  MGN_ROUTE_GEMV_VALU = 2, /* streaming dequant-GEMV on the vector ALU, M <= 4 */
+  MGN_ROUTE_GEMV_MFMA = 3, /* streaming dequant-GEMV, raw quants x split-fp16 activations on MFMA, M <= 2 */
+  MGN_ROUTE_GEMM_MFMA = 4  /* tiled dequant-GEMM on MFMA, larger M */
 } mgn_route;
 
 typedef struct mgn_ctx mgn_ctx;

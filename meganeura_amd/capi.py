@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_DIR, "libmgn_hip.so")
 
 OK, EINVAL, ENOMEM, EHIP, ENOTFOUND, ENODEVICE = range(6)
 FMT_Q4, FMT_Q8 = 0, 1
-ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV, ROUTE_MFMA = range(4)
+ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA = range(5)
 
 # every symbol include/mgn_hip.h and include/mgn_session.h declare
 HIP_SYMBOLS = [

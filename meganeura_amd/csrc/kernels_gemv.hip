@@ -32,14 +32,34 @@ struct XRegs {
   float sx[MR];     // plain sum of the 32 activations
 };
 
+// Activations reach the lanes through LDS: the workgroup copies the M rows of A
+// with coalesced 128-bit loads into rows of 36 floats per 32-element block (the
+// 4-float pad makes the per-lane 128-bit reads below conflict-free: lane l
+// starts at dword 36*l, and 36*l mod 64 hits each multiple of 4 once per 16
+// lanes), then every lane lifts its own block into registers.
+constexpr int kXStride = 36;
+
+template <int MR>
+__device__ __forceinline__ void stage_x(float* __restrict__ xs, const float* __restrict__ a, uint32_t m,
+                                        uint32_t k) {
+  const uint32_t bpc = k / 32;
+  for (uint32_t r = 0; r < (uint32_t)MR && r < m; r++) {
+    const float4* src = (const float4*)(a + (size_t)r * k);
+    float* dst = xs + (size_t)r * bpc * kXStride;
+    for (uint32_t i = threadIdx.x; i < k / 4; i += blockDim.x)
+      *(float4*)(dst + (i >> 3) * kXStride + (i & 7) * 4) = src[i];
+  }
+}
+
 template <int FMT, int MR>
-__device__ __forceinline__ void load_x(XRegs<MR>& xr, const float* __restrict__ a, uint32_t m, uint32_t k,
+__device__ __forceinline__ void load_x(XRegs<MR>& xr, const float* __restrict__ xs, uint32_t m, uint32_t k,
                                        uint32_t kb, bool ok) {
+  const uint32_t bpc = k / 32;
 #pragma unroll
   for (int r = 0; r < MR; r++) {
     float s = 0.0f;
     if (ok && (uint32_t)r < m) {
-      const float4* p = (const float4*)(a + (size_t)r * k + (size_t)kb * 32);
+      const float4* p = (const float4*)(xs + ((size_t)r * bpc + kb) * kXStride);
 #pragma unroll
       for (int j = 0; j < 8; j++) {
         const float4 v = p[j];
@@ -144,7 +164,10 @@ constexpr int max_waves() { return MR >= 4 ? 4 : 8; }
 template <int FMT, int KBW, int MR, int U>
 __global__ __launch_bounds__(64 * max_waves<MR>()) void gemv_kernel(WeightView w, const float* __restrict__ a, const float* __restrict__ d,
                             float* __restrict__ c, uint32_t m, uint32_t steps, uint32_t kgc) {
-  extern __shared__ float red[];  // [kgc][MR][cols_per_wg], used when kgc > 1
+  extern __shared__ float lds[];
+  const uint32_t x_floats = MR * (w.k / 32) * kXStride;
+  float* xs = lds;               // [MR][bpc][36] staged activations
+  float* red = lds + x_floats;   // [kgc][MR][cols_per_wg], used when kgc > 1
   constexpr int NW = 64 / KBW;
   const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const uint32_t kg = wave % kgc, wn = wave / kgc, wnc = (blockDim.x >> 6) / kgc;
@@ -165,9 +188,11 @@ __global__ __launch_bounds__(64 * max_waves<MR>()) void gemv_kernel(WeightView w
       blk[u].load(w, ok ? (size_t)n * bpc + kb : 0);  // block 0 always exists
     }
   };
-  issue(0);  // weights first: the activation loads below hit in cache
+  issue(0);  // weights first: they are in flight while the activations are staged
+  stage_x<MR>(xs, a, m, w.k);
+  __syncthreads();
   XRegs<MR> xr;
-  load_x<FMT, MR>(xr, a, m, w.k, kb, kb_ok);
+  load_x<FMT, MR>(xr, xs, m, w.k, kb, kb_ok);
 
   for (uint32_t step = 0; step < steps; step += U) {
     RawBlock<FMT> cur[U];
@@ -254,10 +279,21 @@ int launch_gemv_t(ihipStream_t* s, const LaunchArgs& x) {
   const GemvPlan p = plan_gemv(x.w.k, x.w.n, x.num_cus, max_waves<MR>());
   const dim3 grid(p.grid), block(64 * p.kgc * p.wnc);
   const uint32_t nw = 64 / p.kbw;
-  const size_t lds = p.kgc > 1 ? (size_t)p.kgc * MR * p.steps * nw * p.wnc * sizeof(float) : 0;
-#define MGN_GEMV(KBW)                                                                                 \
-  hipLaunchKernelGGL((gemv_kernel<FMT, KBW, MR, kUnroll>), grid, block, lds, s, x.w, (const float*)x.a, \
-                     x.d, x.c, x.m, p.steps, p.kgc)
+  const size_t lds = ((size_t)MR * (x.w.k / 32) * kXStride +
+                      (p.kgc > 1 ? (size_t)p.kgc * MR * p.steps * nw * p.wnc : 0)) * sizeof(float);
+  // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+#define MGN_GEMV(KBW)                                                                                   \
+  do {                                                                                                  \
+    auto kern = gemv_kernel<FMT, KBW, MR, kUnroll>;                                                     \
+    static bool big_lds_enabled = false;                                                                \
+    if (lds > 64 * 1024 && !big_lds_enabled) {                                                          \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                         160 * 1024);                                                   \
+      if (e != hipSuccess) return (int)e;                                                               \
+      big_lds_enabled = true;                                                                           \
+    }                                                                                                   \
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x.w, (const float*)x.a, x.d, x.c, x.m, p.steps, p.kgc); \
+  } while (0)
   switch (p.kbw) {
     case 64: MGN_GEMV(64); break;
     case 32: MGN_GEMV(32); break;
@@ -275,7 +311,9 @@ bool gemv_supported(const LaunchArgs& x) {
   if (x.a_is_f16 || x.m == 0 || x.m > 4) return false;
   const uint32_t mw = x.m > 2 ? max_waves<4>() : max_waves<1>();
   const GemvPlan p = plan_gemv(x.w.k, x.w.n, x.num_cus, mw);
-  return p.kgc <= mw;  // all K groups of a column must fit in one workgroup
+  const size_t x_bytes = (size_t)(x.m > 2 ? 4 : x.m) * (x.w.k / 32) * kXStride * sizeof(float);
+  // all K groups of a column must fit in one workgroup, the staged activations in LDS
+  return p.kgc <= mw && x_bytes <= 128 * 1024;
 }
 
 int launch_matmul_gemv(ihipStream_t* s, const LaunchArgs& x) {

@@ -1,7 +1,7 @@
-// Placeholder until the MFMA kernels land: no shape is claimed.
+// Placeholder until the tiled MFMA GEMM lands: no shape is claimed.
 #include "kernels_common.hip.h"
 
 namespace mgn {
-bool mfma_supported(const LaunchArgs&) { return false; }
-int launch_matmul_mfma(ihipStream_t*, const LaunchArgs&) { return (int)hipErrorNotSupported; }
+bool gemm_mfma_supported(const LaunchArgs&) { return false; }
+int launch_matmul_gemm_mfma(ihipStream_t*, const LaunchArgs&) { return (int)hipErrorNotSupported; }
 }  // namespace mgn

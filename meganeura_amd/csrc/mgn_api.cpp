@@ -47,7 +47,8 @@ mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn
   if (!valid_fmt(fmt)) return fail(ctx, MGN_EINVAL, "unknown weight format");
   if (rows == 0 || cols == 0) return fail(ctx, MGN_EINVAL, "empty weight");
   if (rows % 32 != 0) return fail(ctx, MGN_EINVAL, "quantized weights require rows (K dim) to be a multiple of 32");
-  if (rows > 0xFFFFFFE0ull || cols > 0xFFFFFFFFull) return fail(ctx, MGN_EINVAL, "weight dimension exceeds 32 bits");
+  if (rows > 0xFFFFFFE0ull || cols > 0xFFFFFFFFull || (rows / 32) * cols >= 0x7FFFFFFFull)
+    return fail(ctx, MGN_EINVAL, "weight too large: block count must stay below 2^31");
   auto* w = new (std::nothrow) mgn_weight();
   if (!w) return fail(ctx, MGN_ENOMEM, "out of host memory");
   w->fmt = fmt;
@@ -56,8 +57,9 @@ mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn
   w->nb = (rows / 32) * cols;
   w->meta_bytes = w->nb * meta_elem(fmt);
   w->quant_bytes = w->nb * quant_elem(fmt);
-  const size_t q_off = align_up(w->meta_bytes, 256);
-  // 256 spare bytes: kernels may over-read one vector past the last block
+  // One extra all-zero block (index nb) follows the real ones in both arrays: lanes
+  // that have no block of their own load it and contribute exactly zero.
+  const size_t q_off = align_up(w->meta_bytes + 16, 256);
   hipError_t e = hipMalloc(&w->base, q_off + w->quant_bytes + 256);
   if (e != hipSuccess) {
     delete w;
@@ -65,6 +67,13 @@ mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn
   }
   w->meta = w->base;
   w->quants = (char*)w->base + q_off;
+  e = hipMemsetAsync((char*)w->meta + w->meta_bytes, 0, 16, ctx->stream);
+  if (e == hipSuccess) e = hipMemsetAsync((char*)w->quants + w->quant_bytes, 0, 256, ctx->stream);
+  if (e != hipSuccess) {
+    (void)hipFree(w->base);
+    delete w;
+    return hip_fail(ctx, "hipMemsetAsync", e);
+  }
   *out = w;
   return MGN_OK;
 }
@@ -122,7 +131,7 @@ mgn_status mgn_sync(mgn_ctx* ctx) {
 
 mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route) {
   if (!ctx) return MGN_EINVAL;
-  if (route < MGN_ROUTE_AUTO || route > MGN_ROUTE_MFMA) return fail(ctx, MGN_EINVAL, "unknown route");
+  if (route < MGN_ROUTE_AUTO || route > MGN_ROUTE_GEMM_MFMA) return fail(ctx, MGN_EINVAL, "unknown route");
   ctx->route = route;
   return MGN_OK;
 }
@@ -336,19 +345,24 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus};
   mgn_route route = ctx->route;
   if (route == MGN_ROUTE_AUTO) {
-    if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV;
-    else if (mgn::mfma_supported(x)) route = MGN_ROUTE_MFMA;
+    if (mgn::gemv_mfma_supported(x)) route = MGN_ROUTE_GEMV_MFMA;
+    else if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV_VALU;
+    else if (mgn::gemm_mfma_supported(x)) route = MGN_ROUTE_GEMM_MFMA;
     else route = MGN_ROUTE_GENERIC;
   }
   int rc;
   switch (route) {
-    case MGN_ROUTE_GEMV:
-      if (!mgn::gemv_supported(x)) return fail(ctx, MGN_EINVAL, "GEMV route does not support this shape");
+    case MGN_ROUTE_GEMV_VALU:
+      if (!mgn::gemv_supported(x)) return fail(ctx, MGN_EINVAL, "GEMV_VALU route does not support this shape");
       rc = mgn::launch_matmul_gemv(ctx->stream, x);
       break;
-    case MGN_ROUTE_MFMA:
-      if (!mgn::mfma_supported(x)) return fail(ctx, MGN_EINVAL, "MFMA route does not support this shape");
-      rc = mgn::launch_matmul_mfma(ctx->stream, x);
+    case MGN_ROUTE_GEMV_MFMA:
+      if (!mgn::gemv_mfma_supported(x)) return fail(ctx, MGN_EINVAL, "GEMV_MFMA route does not support this shape");
+      rc = mgn::launch_matmul_gemv_mfma(ctx->stream, x);
+      break;
+    case MGN_ROUTE_GEMM_MFMA:
+      if (!mgn::gemm_mfma_supported(x)) return fail(ctx, MGN_EINVAL, "GEMM_MFMA route does not support this shape");
+      rc = mgn::launch_matmul_gemm_mfma(ctx->stream, x);
       break;
     default:
       rc = mgn::launch_matmul_generic(ctx->stream, x);

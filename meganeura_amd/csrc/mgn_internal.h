@@ -27,6 +27,7 @@ void dequantize_q8_host(const uint8_t* in, size_t rows, size_t cols, float* out)
 //   Q8: meta[b] = u16 scale_f16,             quants[b] = 32 int8
 //       -> the reference's 36-byte blocks with the pad dropped and scales
 //          gathered, so quants are 32-byte aligned for 128-bit loads.
+// Both arrays carry one extra all-zero block at index nb = (K/32)*N.
 struct WeightView {
   const void* meta;
   const void* quants;
@@ -53,8 +54,10 @@ int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, ui
 int launch_matmul_generic(ihipStream_t* s, const LaunchArgs& a);
 bool gemv_supported(const LaunchArgs& a);
 int launch_matmul_gemv(ihipStream_t* s, const LaunchArgs& a);
-bool mfma_supported(const LaunchArgs& a);
-int launch_matmul_mfma(ihipStream_t* s, const LaunchArgs& a);
+bool gemv_mfma_supported(const LaunchArgs& a);
+int launch_matmul_gemv_mfma(ihipStream_t* s, const LaunchArgs& a);
+bool gemm_mfma_supported(const LaunchArgs& a);
+int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& a);
 
 }  // namespace mgn
 

@@ -106,11 +106,12 @@ def test_weight_errors(ctx):
 
 # ---- matmul: every route at small and ragged shapes ----------------------------------------
 
-ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv": capi.ROUTE_GEMV, "auto": capi.ROUTE_AUTO}
+ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv_valu": capi.ROUTE_GEMV_VALU, "gemv_mfma": capi.ROUTE_GEMV_MFMA,
+          "gemm_mfma": capi.ROUTE_GEMM_MFMA, "auto": capi.ROUTE_AUTO}
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-@pytest.mark.parametrize("route", ["generic", "gemv", "auto"])
+@pytest.mark.parametrize("route", ["generic", "gemv_valu", "gemv_mfma", "auto"])
 @pytest.mark.parametrize("m,k,n", [
     (1, 32, 1), (1, 64, 3), (1, 576, 192), (1, 576, 577), (1, 1536, 576), (1, 1024, 100),
     (2, 576, 65), (3, 2048, 130), (4, 4096, 257), (1, 14336, 64), (1, 3072, 1024),
@@ -124,8 +125,8 @@ def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
         got = run_matmul(ctx, fmt, x, w, ROUTES[route])
         got_d = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d)
     except capi.MgnError as e:
-        if route == "gemv" and "does not support" in str(e):
-            pytest.skip("shape outside the GEMV kernel's range")
+        if route.startswith("gemv") and "does not support" in str(e):
+            pytest.skip("shape outside this GEMV kernel's range")
         raise
     orc.assert_close(got, orc.matmul_f32(x, deq), REL, ABS)
     orc.assert_close(got_d, orc.matmul_f32(x, deq, d), REL, ABS)
