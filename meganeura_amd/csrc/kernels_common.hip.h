@@ -59,6 +59,15 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for
+// every outstanding global load of the wave (its fences cover global memory),
+// which would stall a kernel that keeps weight loads in flight across the barrier.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 #define MGN_HIP_LAUNCH_CHECK()                      \
   do {                                              \
     hipError_t e__ = hipGetLastError();             \

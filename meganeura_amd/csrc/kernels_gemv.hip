@@ -190,7 +190,7 @@ __global__ __launch_bounds__(64 * max_waves<MR>()) void gemv_kernel(WeightView w
   };
   issue(0);  // weights first: they are in flight while the activations are staged
   stage_x<MR>(xs, a, m, w.k);
-  __syncthreads();
+  lds_barrier();
   XRegs<MR> xr;
   load_x<FMT, MR>(xr, xs, m, w.k, kb, kb_ok);
 
@@ -221,7 +221,7 @@ __global__ __launch_bounds__(64 * max_waves<MR>()) void gemv_kernel(WeightView w
     }
   }
   if (kgc > 1) {
-    __syncthreads();
+    lds_barrier();
     for (uint32_t idx = threadIdx.x; idx < MR * cols_per_wg; idx += blockDim.x) {
       const uint32_t r = idx / cols_per_wg, col = idx % cols_per_wg;
       const uint32_t n = blockIdx.x * cols_per_wg + col;

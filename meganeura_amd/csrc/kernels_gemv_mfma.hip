@@ -5,51 +5,52 @@
 // every nibble to f32 and multiplying it on the vector ALU costs three times
 // that and makes the kernel ALU-bound.  Here the vector ALU only masks nibbles
 // into place (5 instructions per 8 weights); the multiply-adds run on
-// v_mfma_f32_4x4x4_16B_f16, whose 16 independent 4x4 blocks fit the problem:
-//   lane (b, i), b = lane/4, i = lane%4, supplies "row i" of block b's A:
-//     four weights of quant block (column 4q+i, K block kb0+b);
-//   lane (b, j) supplies "column j" of block b's B: four activations of K block
-//     kb0+b, j = 2*row for the high half of an fp16 split, 2*row+1 for the low;
-//   lane (b, j) receives D[i][j], i = 0..3: the four columns' partial sums.
+// v_mfma_f32_4x4x4_16B_f16, whose 16 independent 4x4 blocks fit the problem.
+// With b = lane/4 the MFMA block and i, j = lane%4:
+//   lane (b, j) supplies column j of block b's B operand: four weights of ITS OWN
+//     quant block (output column 4q+j, K block kb0+b);
+//   lane (b, i) supplies row i of block b's A operand: four activations of K block
+//     kb0+b; row 0/1 = high/low half of an fp16 split of activation row 0, row
+//     2/3 the same for activation row 1;
+//   lane (b, j) receives D[i][j], i = 0..3: the dot products of its own weights
+//     with the four activation rows, so scaling by the block's d stays in-lane.
 // Eight such MFMAs cover one 32-element quant block per lane.
 //
-// Exactness.  A nibble n masked to bits 0-3 (or 4-7) of an fp16 is the
-// subnormal n * 2^-24 (n * 2^-20): exact, and the matrix cores do not flush
-// fp16 subnormals.  Activations are split x = hi + lo into two fp16 after
+// Exactness.  A nibble n masked to bits 4-7 of an fp16 is the subnormal
+// n * 2^-20, and the matrix cores do not flush fp16 subnormals.  (Bits 0-3,
+// n * 2^-24, would save the shifts but is measurably worse: the MFMA datapath
+// aligns products by the operands' nominal exponents and drops low bits of
+// mantissas with many leading zeros.  Q8 bytes, q + 128 in bits 0-7, have few
+// leading zeros and are fine.)  Activations are split x = hi + lo into two fp16 after
 // scaling the row by a power of two (|x| < 2^12), so products are exact in f32
 // and only the f32 accumulation rounds: the result carries ~21 bits of x, not
 // 11.  Per block the identity used is
-//   sum_k (n_k d + m) x_k = d * (sum_k n_k x_k - 8 sum_k x_k) + (m + 8 d) * sum_k x_k :
+//   sum_k (n_k d + m) x_k = d * (sum_k n_k x_k - 8 S) + (m + 8 d) * S,  S = sum_k x_k :
 // the nibbles are centred (n - 8) so that neither term is large against the
-// result, and the "- 8 sum x" enters as the MFMA chain's initial accumulator,
-// i.e. before anything is scaled or summed across blocks; accumulating
+// result, and "- 8 S" enters as the MFMA chain's initial accumulator, i.e.
+// before anything is scaled or summed across blocks; accumulating
 // d * sum(n x) and m * sum(x) separately down a column would cancel
 // catastrophically.  Q8 bytes are biased to unsigned (q + 128) and the bias
-// leaves the same way (- 128 sum x as the initial accumulator).
+// leaves the same way (- 128 S as the initial accumulator).
 //
-// A wave owns four adjacent columns and walks K sixteen blocks at a time, so
-// its four accumulators stay in registers down the whole column; cross-lane
-// sums happen once per column quad.  The activations' B operands are prepared
-// once per workgroup in LDS, laid out so that consecutive lanes read
-// consecutive 16-byte chunks.
+// A wave owns four adjacent columns and walks K sixteen blocks at a time, so a
+// lane's accumulator stays in a register down the whole column; the 16 lanes
+// of a column are summed once per column quad.  The activations' A operands
+// are prepared once per workgroup in LDS, laid out so that consecutive lanes
+// read consecutive 16-byte chunks.
 #include "kernels_common.hip.h"
 
 namespace mgn {
 namespace {
 
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr float kTwoPow24 = 16777216.0f;
+// fp16 bit patterns used as operands stand for value * 2^-kOperandShift
+template <int FMT>
+constexpr float operand_scale() { return FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f; }  // 2^20, 2^24
 constexpr int kMaxTasks = 2;  // activation chunks a thread prepares, per row
-
-__device__ __forceinline__ uint32_t pack_half2(float lo, float hi) {
-  const uint32_t a = __builtin_bit_cast(uint16_t, (_Float16)lo);
-  const uint32_t b = __builtin_bit_cast(uint16_t, (_Float16)hi);
-  return a | (b << 16);
-}
-
-__device__ __forceinline__ float half_residual(float v) { return v - (float)(_Float16)v; }
 
 __device__ __forceinline__ half4 as_half4(uint32_t lo, uint32_t hi) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -57,8 +58,15 @@ __device__ __forceinline__ half4 as_half4(uint32_t lo, uint32_t hi) {
   return __builtin_bit_cast(half4, v);
 }
 
-constexpr int kQuadBcast[4] = {0x00, 0x55, 0xAA, 0xFF};  // quad_perm:[i,i,i,i]
-constexpr int kRowRor4 = 0x124, kRowRor8 = 0x128;        // rotate right within a row of 16
+// two floats -> packed fp16 pair, truncating: the low halves computed from the
+// residual make up for the truncation
+__device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
+}
+__device__ __forceinline__ float half_lo(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[0]; }
+__device__ __forceinline__ float half_hi(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[1]; }
+
+constexpr int kRowRor4 = 0x124, kRowRor8 = 0x128;  // rotate right within a row of 16 lanes
 
 // sum over the 16 lanes sharing lane%4 (every such lane ends with the total)
 __device__ __forceinline__ float sum_over_blocks(float v) {
@@ -92,47 +100,35 @@ struct Raw<MGN_FMT_Q8> {
 };
 
 // LDS image of the activations, per workgroup:
-//   chunk planes  xb[c][kb * NJ + j]  (uint4), c = 0..3: the B operands of the two MFMAs
-//                 that consume elements 8c..8c+7 of K block kb, B column j;
-//   sx24[r][kb]   2^-24 * sum of the (scaled) activations of K block kb, row r.
-// Q4 pairs nibble k with k+4 in one fp16x2 mask, and odd nibbles sit 4 bits higher
-// (2^-20 instead of 2^-24), so the chunk is (x0,x4,x2,x6 | x1,x5,x3,x7 / 16).
+//   chunk planes  xa[c][kb * NJ + j]  (uint4), c = 0..3: the A-operand rows of the two
+//                 MFMAs that consume elements 8c..8c+7 of K block kb; j = 2*row (high
+//                 halves) or 2*row + 1 (low halves);
+//   cinit[kb][row] = -bias / operand_scale * S(kb, row), the chain's initial accumulator.
+// Q4 pairs nibble k with k+4 in one fp16x2 mask, so the chunk is (x0,x4,x2,x6 | x1,x5,x3,x7).
 // Q8 bytes come out in natural order: (x0,x1,x2,x3 | x4,x5,x6,x7).
-// *s_hi / *s_lo get sum_k of the value nibble/byte k is multiplied with in the hi / lo
-// column (for Q4's odd elements that is 16 * fp16(x/16)), in f32.
 template <int FMT>
-__device__ __forceinline__ void make_chunks(const float (&x)[8], uint4& hi, uint4& lo, float* s_hi, float* s_lo) {
+__device__ __forceinline__ void make_chunks(const float (&x)[8], uint4& hi, uint4& lo) {
   float p[8];
   if constexpr (FMT == MGN_FMT_Q4) {
-    const float o = 0.0625f;
     p[0] = x[0], p[1] = x[4], p[2] = x[2], p[3] = x[6];
-    p[4] = x[1] * o, p[5] = x[5] * o, p[6] = x[3] * o, p[7] = x[7] * o;
+    p[4] = x[1], p[5] = x[5], p[6] = x[3], p[7] = x[7];
   } else {
 #pragma unroll
     for (int i = 0; i < 8; i++) p[i] = x[i];
   }
-  hi = make_uint4(pack_half2(p[0], p[1]), pack_half2(p[2], p[3]), pack_half2(p[4], p[5]), pack_half2(p[6], p[7]));
-  float r[8];
+  hi = make_uint4(pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7]));
+  const uint32_t h[4] = {hi.x, hi.y, hi.z, hi.w};
+  uint32_t l[4];
 #pragma unroll
-  for (int i = 0; i < 8; i++) r[i] = half_residual(p[i]);
-  lo = make_uint4(pack_half2(r[0], r[1]), pack_half2(r[2], r[3]), pack_half2(r[4], r[5]), pack_half2(r[6], r[7]));
-  float h[8], l[8];
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    h[i] = (float)(_Float16)p[i];
-    l[i] = (float)(_Float16)r[i];
-  }
-  const float sc = FMT == MGN_FMT_Q4 ? 16.0f : 1.0f;  // second half of a Q4 chunk is x/16
-  *s_hi = ((h[0] + h[1]) + (h[2] + h[3])) + sc * ((h[4] + h[5]) + (h[6] + h[7]));
-  *s_lo = ((l[0] + l[1]) + (l[2] + l[3])) + sc * ((l[4] + l[5]) + (l[6] + l[7]));
+  for (int i = 0; i < 4; i++) l[i] = pack_rtz(p[2 * i] - half_lo(h[i]), p[2 * i + 1] - half_hi(h[i]));
+  lo = make_uint4(l[0], l[1], l[2], l[3]);
 }
 
 // Power of two that brings the row's largest magnitude below 2^12 (1 if the row
-// is all zero or not finite).  Returns the scale; *inv gets its reciprocal.
-__device__ __forceinline__ float row_scale(float amax, float* inv) {
-  const uint32_t bits = __builtin_bit_cast(uint32_t, amax);
-  const int e = (int)(bits >> 23) - 127;  // floor(log2(amax)) for normal values
-  if (bits == 0 || e >= 128 || e <= -100) {
+// is all zero or not finite).  amax_bits: the IEEE bits of max |x|.
+__device__ __forceinline__ float row_scale(uint32_t amax_bits, float* inv) {
+  const int e = (int)(amax_bits >> 23) - 127;  // floor(log2(amax)) for normal values
+  if (amax_bits == 0 || e >= 128 || e <= -100) {
     *inv = 1.0f;
     return 1.0f;
   }
@@ -141,117 +137,105 @@ __device__ __forceinline__ float row_scale(float amax, float* inv) {
   return __builtin_bit_cast(float, (uint32_t)(127 + sh) << 23);
 }
 
-// blockDim.x = 64 * ksc * wnc.  Wave w: K split ks = w % ksc, quad lane wn = w / ksc.
-// The workgroup owns quads [blockIdx.x * qpw, +qpw); wave (ks, wn) takes quads wn, wn+wnc, ...
-// and K blocks [ks * spk * 16, (ks+1) * spk * 16).
-template <int FMT, int MROWS, int U>
+// blockDim.x = 64 * ksc * wnc.  Wave w: K split ks = w % ksc, quad slot wn = w / ksc.
+// The workgroup owns quads [blockIdx.x * wnc, +wnc); wave (ks, wn) takes quad wn and the
+// K steps [ks * STEPS, (ks+1) * STEPS) of 16 blocks each.  Every wave issues all of its
+// STEPS block loads up front and then runs straight-line code: with no branch around a
+// load the compiler's wait counts are exact, so step s starts as soon as its own block
+// has arrived while the later ones are still in flight.
+template <int FMT, int MROWS, int STEPS>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const float* __restrict__ a,
                                                          const float* __restrict__ dres, float* __restrict__ c,
-                                                         uint32_t m, uint32_t qpw, uint32_t ksc, uint32_t spk) {
+                                                         uint32_t m, uint32_t ksc) {
   constexpr int NJ = 2 * MROWS;
   extern __shared__ uint4 lds4[];
   const uint32_t bpc = w.k / 32;
   const uint32_t bpc_pad = (bpc + 15) & ~15u;
   const uint32_t plane = bpc_pad * NJ;
-  uint4* xb = lds4;                                  // [4][plane]
-  float* sx24 = (float*)(lds4 + 4 * plane);          // [MROWS][bpc_pad]
-  float* cinit = sx24 + MROWS * bpc_pad;             // [bpc_pad][NJ]: -bias * 2^-24 * sum of column j's operands
-  float* red = cinit + plane;                        // [qpw][ksc][MROWS][4]
-  float* scratch = red + qpw * ksc * MROWS * 4;      // [16 waves][MROWS] row maxima, then [MROWS] scales
+  const uint32_t nwaves = blockDim.x >> 6, wnc = nwaves / ksc;
+  uint4* xa = lds4;                                   // [4][plane]
+  float* cinit = (float*)(lds4 + 4 * plane);          // [bpc_pad][MROWS]
+  float* red = cinit + bpc_pad * MROWS;               // [wnc][ksc][MROWS][4]
+  uint32_t* amax_bits = (uint32_t*)(red + wnc * ksc * MROWS * 4);  // [MROWS]
 
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   // everything derived from the wave index is wave-uniform: keep it in scalar registers
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t nwaves = blockDim.x >> 6;
-  const uint32_t ks = wave % ksc, wn = wave / ksc, wnc = nwaves / ksc;
-  const uint32_t b = lane >> 2, i = lane & 3;        // MFMA block, row (A) / column (B) within it
-  const uint32_t quad0 = blockIdx.x * qpw;
+  const uint32_t ks = wave % ksc, wn = wave / ksc;
+  const uint32_t b = lane >> 2, i = lane & 3;
+  const uint32_t quad0 = blockIdx.x * wnc;
   const uint32_t nquads = (w.n + 3) / 4;
-
-  // This wave's work, linearised: quads first, first + wnc, ... below q_end, each walked
-  // in my_steps steps of 16 K blocks.  A producer cursor (pq, pst) runs U steps ahead of
-  // the consumer cursor (cq, cst) and keeps a ring of U raw blocks in flight per lane.
+  const uint32_t quad = quad0 + wn;
   const uint32_t steps_total = bpc_pad / 16;
-  const uint32_t step_begin = ks * spk;
-  const uint32_t my_steps = step_begin >= steps_total ? 0u : min(spk, steps_total - step_begin);
-  const uint32_t first = quad0 + wn;
-  const uint32_t q_end = my_steps == 0 ? 0u : min(quad0 + qpw, nquads);
-  const uint32_t kb_first = step_begin * 16 + b;      // this lane's K block at step 0
-  const uint32_t zero_block = bpc * w.n;              // an all-zero block behind the last real one
-  Raw<FMT> ring[U];
-  uint32_t pq = first, pst = 0;
-  uint32_t pblk = 0;  // block index the producer loads next (valid while pn_ok)
-  bool pn_ok = false;
-  auto produce = [&](int u) {
-    if (pq < q_end) {  // wave-uniform
-      if (pst == 0) {
-        const uint32_t n = pq * 4 + i;
-        pn_ok = n < w.n;
-        pblk = n * bpc + kb_first;
-      }
-      const bool ok = pn_ok && kb_first + pst * 16 < bpc;
-      ring[u].load(w, ok ? pblk : zero_block);
-      pblk += 16;
-      if (++pst == my_steps) {
-        pst = 0;
-        pq += wnc;
-      }
-    }
-  };
+  const uint32_t step_begin = ks * STEPS;
+  // a wave past the last K step (or past the last quad) keeps running on the zero block:
+  // it contributes nothing and clamps its LDS reads to step 0
+  const bool wave_live = step_begin < steps_total && quad < nquads;
+  const uint32_t kb_first = (wave_live ? step_begin : 0u) * 16 + b;  // this lane's K block at step 0
+  const uint32_t zero_block = bpc * w.n;  // an all-zero block behind the last real one
+
   // Memory returns a wave's loads in issue order, so the (small, cache-resident)
-  // activation loads go first and the weight ring right behind them: the activation
+  // activation loads go first and the weight loads right behind them: the activation
   // prep below then waits for its own data only, while the weights stream in.
-  // One task = 8 consecutive activations of one row = one B chunk; the 4 tasks of a K
+  // One task = 8 consecutive activations of one row = one A chunk; the 4 tasks of a K
   // block sit in one lane quad.  A thread holds at most kMaxTasks tasks in registers.
   float4 xraw[kMaxTasks][MROWS][2];
 #pragma unroll
   for (int tt = 0; tt < kMaxTasks; tt++) {
     const uint32_t t = tid + tt * blockDim.x, kb = t >> 2, ch = t & 3;
+    const bool live = kb < bpc;
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
-      if (kb < bpc && (uint32_t)r < m) {
-        const float4* src = (const float4*)(a + (size_t)r * w.k + (size_t)kb * 32 + ch * 8);
-        xraw[tt][r][0] = src[0];
-        xraw[tt][r][1] = src[1];
-      } else {
-        xraw[tt][r][0] = xraw[tt][r][1] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      }
+      // always load (from element 0 when there is nothing to load) and zero afterwards
+      const bool ok = live && (uint32_t)r < m;
+      const float4* src = (const float4*)(a + (ok ? (size_t)r * w.k + (size_t)kb * 32 + ch * 8 : (size_t)0));
+      xraw[tt][r][0] = src[0];
+      xraw[tt][r][1] = src[1];
     }
   }
+  Raw<FMT> blk[STEPS];
+  {
+    const uint32_t n = quad * 4 + i;
+    const uint32_t base = n * bpc + kb_first;
+    const bool n_ok = wave_live && n < w.n;
 #pragma unroll
-  for (int u = 0; u < U; u++) produce(u);
-  for (uint32_t t = tid; t < qpw * ksc * MROWS * 4; t += blockDim.x) red[t] = 0.0f;
+    for (int s = 0; s < STEPS; s++) {
+      const bool ok = n_ok && step_begin + s < steps_total && kb_first + s * 16 < bpc;
+      blk[s].load(w, ok ? base + s * 16 : zero_block);
+    }
+  }
+  for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += blockDim.x) red[t] = 0.0f;
+  if (tid < (uint32_t)MROWS) amax_bits[tid] = 0;
+  lds_barrier();
 
   // ---- activations -> LDS (once per workgroup) ----
   float inv_scale[MROWS];
   {
-    float scale[MROWS];
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
       float am = 0.0f;
 #pragma unroll
-      for (int tt = 0; tt < kMaxTasks; tt++)
+      for (int tt = 0; tt < kMaxTasks; tt++) {
+        const bool ok = ((tid + tt * blockDim.x) >> 2) < bpc && (uint32_t)r < m;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
+          if (!ok) xraw[tt][r][h] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
           const float4 v = xraw[tt][r][h];
           am = fmaxf(am, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
         }
-      // NaN never wins fmaxf; infinities do and switch scaling off in row_scale
+      }
+      // NaN never wins fmaxf; infinities do and switch scaling off in row_scale.
+      // |x| orders like its bit pattern, so an integer max over the workgroup will do.
       am = fmaxf(am, dpp_move<kDppQuadXor1>(am));
       am = fmaxf(am, dpp_move<kDppQuadXor2>(am));
       am = fmaxf(am, dpp_move<kDppRowHalfMirror>(am));
       am = fmaxf(am, dpp_move<kDppRowMirror>(am));
-      am = fmaxf(am, __shfl_xor(am, 16, 64));
-      am = fmaxf(am, __shfl_xor(am, 32, 64));
-      if (lane == 0) scratch[(tid >> 6) * MROWS + r] = am;
+      if ((lane & 15) == 0) atomicMax(&amax_bits[r], __builtin_bit_cast(uint32_t, am));
     }
-    __syncthreads();
+    lds_barrier();
+    float scale[MROWS];
 #pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      float v = 0.0f;
-      for (uint32_t wv = 0; wv < nwaves; wv++) v = fmaxf(v, scratch[wv * MROWS + r]);
-      scale[r] = row_scale(v, &inv_scale[r]);
-    }
+    for (int r = 0; r < MROWS; r++) scale[r] = row_scale(amax_bits[r], &inv_scale[r]);
 #pragma unroll
     for (int tt = 0; tt < kMaxTasks; tt++) {
       const uint32_t t = tid + tt * blockDim.x, kb = t >> 2, ch = t & 3;
@@ -262,133 +246,87 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
           const float x[8] = {v0.x * scale[r], v0.y * scale[r], v0.z * scale[r], v0.w * scale[r],
                               v1.x * scale[r], v1.y * scale[r], v1.z * scale[r], v1.w * scale[r]};
           uint4 hi, lo;
-          float s_hi, s_lo;
-          make_chunks<FMT>(x, hi, lo, &s_hi, &s_lo);
-          xb[ch * plane + kb * NJ + 2 * r] = hi;
-          xb[ch * plane + kb * NJ + 2 * r + 1] = lo;
-          s_hi += dpp_move<kDppQuadXor1>(s_hi);
-          s_hi += dpp_move<kDppQuadXor2>(s_hi);
-          s_lo += dpp_move<kDppQuadXor1>(s_lo);
-          s_lo += dpp_move<kDppQuadXor2>(s_lo);
-          if (ch == 0) {
-            constexpr float bias = FMT == MGN_FMT_Q4 ? 8.0f : 128.0f;
-            // the m-term uses the same split values the MFMAs see, so the result is the
-            // exact dot product with hi + lo up to f32 rounding
-            sx24[r * bpc_pad + kb] = (s_hi + s_lo) * (1.0f / kTwoPow24);
-            cinit[kb * NJ + 2 * r] = s_hi * (-bias / kTwoPow24);
-            cinit[kb * NJ + 2 * r + 1] = s_lo * (-bias / kTwoPow24);
-          }
+          make_chunks<FMT>(x, hi, lo);
+          xa[ch * plane + kb * NJ + 2 * r] = hi;
+          xa[ch * plane + kb * NJ + 2 * r + 1] = lo;
+          float s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+          s += dpp_move<kDppQuadXor1>(s);
+          s += dpp_move<kDppQuadXor2>(s);
+          constexpr float bias = FMT == MGN_FMT_Q4 ? 8.0f : 128.0f;
+          if (ch == 0) cinit[kb * MROWS + r] = s * (-bias / operand_scale<FMT>());
         }
       }
     }
   }
-  __syncthreads();
+  lds_barrier();
 
-  // ---- main loop ----
-  // Lanes i >= NJ have no B column of their own; they re-read column i % NJ (a broadcast in
-  // LDS) and their sums are never looked at.  Byte offsets into the chunk planes / sx24:
-  const uint32_t x_lane = ((kb_first * NJ) + (i % NJ)) * 16;
-  const uint32_t sx_lane = kb_first * 4;
-  const uint32_t ci_lane = (kb_first * NJ + (i % NJ)) * 4;
-  const char* xb_bytes = (const char*)xb;
-  const char* sx_bytes = (const char*)sx24;
-  const char* ci_bytes = (const char*)cinit;
-  floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};  // lane (b, j): sum over K of d * D[i][j], i = 0..3
-  float macc[MROWS];                       // lane (b, i): sum over K of m * sum(x) for column 4q+i
+  // ---- the K walk: STEPS blocks per lane, straight-line ----
+  // Lanes i >= NJ have no activation row of their own; they re-read row i % NJ (a broadcast
+  // in LDS) and the D entries they produce are never looked at.
+  const char* xa_lane = (const char*)xa + ((kb_first * NJ) + (i % NJ)) * 16;
+  const char* ci_lane = (const char*)cinit + kb_first * MROWS * 4;
+  float acc[MROWS];  // lane (b, j): sum over this lane's K blocks for column 4*quad+j, per row
 #pragma unroll
-  for (int r = 0; r < MROWS; r++) macc[r] = 0.0f;
-  uint32_t cq = first, cst = 0;
-  while (cq < q_end) {
+  for (int r = 0; r < MROWS; r++) acc[r] = 0.0f;
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-      if (cq < q_end) {  // wave-uniform
-        const Raw<FMT> cur = ring[u];
-        produce(u);
-        // B operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks
-        const uint32_t x_off = x_lane + cst * (16 * NJ * 16);
-        uint4 bx[4];
+  for (int s = 0; s < STEPS; s++) {
+    // steps past the end of K multiply the zero block; keep their LDS reads in range
+    const uint32_t so = (step_begin + s < steps_total) ? (uint32_t)s : 0u;
+    const Raw<FMT>& cur = blk[s];
+    // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks
+    uint4 ax[4];
 #pragma unroll
-        for (int ch = 0; ch < 4; ch++) bx[ch] = *(const uint4*)(xb_bytes + x_off + ch * plane * 16);
-        float sxv[MROWS];
+    for (int ch = 0; ch < 4; ch++) ax[ch] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + ch * plane * 16);
+    float ci[MROWS];
 #pragma unroll
-        for (int r = 0; r < MROWS; r++) sxv[r] = *(const float*)(sx_bytes + sx_lane + cst * 64 + r * bpc_pad * 4);
-        const float ci = *(const float*)(ci_bytes + ci_lane + cst * (16 * NJ * 4));
-        floatx4 dsum = {ci, ci, ci, ci};  // the centring term rides in as the chain's start value
-        float dscale, mterm;
-        if constexpr (FMT == MGN_FMT_Q4) {
-          const uint32_t words[4] = {cur.q.x, cur.q.y, cur.q.z, cur.q.w};
+    for (int r = 0; r < MROWS; r++) ci[r] = *(const float*)(ci_lane + so * (16 * MROWS * 4) + r * 4);
+    // the centring term rides in as the chain's start value (rows 2r and 2r+1 add up later)
+    floatx4 dsum = {ci[0], 0.0f, MROWS > 1 ? ci[MROWS - 1] : 0.0f, 0.0f};
+    if constexpr (FMT == MGN_FMT_Q4) {
+      const uint32_t words[4] = {cur.q.x, cur.q.y, cur.q.z, cur.q.w};
 #pragma unroll
-          for (int ch = 0; ch < 4; ch++) {
-            const uint32_t wd = words[ch], w8 = wd >> 8;
-            const uint32_t e0 = wd & 0x000F000Fu, o0 = wd & 0x00F000F0u;  // (n0,n4) 2^-24, (n1,n5) 2^-20
-            const uint32_t e1 = w8 & 0x000F000Fu, o1 = w8 & 0x00F000F0u;  // (n2,n6),       (n3,n7)
-            dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(e0, e1), as_half4(bx[ch].x, bx[ch].y), dsum, 0, 0, 0);
-            dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(o0, o1), as_half4(bx[ch].z, bx[ch].w), dsum, 0, 0, 0);
-          }
-          dscale = half_bits_to_float(cur.meta & 0xFFFFu);
-          mterm = __fmaf_rn(8.0f, dscale, half_bits_to_float(cur.meta >> 16));  // m + 8 d
-        } else {
-          const uint32_t words[8] = {cur.q0.x, cur.q0.y, cur.q0.z, cur.q0.w, cur.q1.x, cur.q1.y, cur.q1.z, cur.q1.w};
+      for (int ch = 0; ch < 4; ch++) {
+        // every nibble pair goes to bits 4-7 / 20-23: n * 2^-20 in each fp16 half
+        const uint32_t wd = words[ch];
+        const uint32_t e0 = (wd << 4) & 0x00F000F0u, o0 = wd & 0x00F000F0u;         // (n0,n4), (n1,n5)
+        const uint32_t e1 = (wd >> 4) & 0x00F000F0u, o1 = (wd >> 8) & 0x00F000F0u;  // (n2,n6), (n3,n7)
+        dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[ch].x, ax[ch].y), as_half4(e0, e1), dsum, 0, 0, 0);
+        dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[ch].z, ax[ch].w), as_half4(o0, o1), dsum, 0, 0, 0);
+      }
+    } else {
+      const uint32_t words[8] = {cur.q0.x, cur.q0.y, cur.q0.z, cur.q0.w, cur.q1.x, cur.q1.y, cur.q1.z, cur.q1.w};
 #pragma unroll
-          for (int ch = 0; ch < 4; ch++) {
+      for (int ch = 0; ch < 4; ch++) {
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-              const uint32_t u8 = words[2 * ch + h] ^ 0x80808080u;  // q + 128 in every byte
-              const uint32_t lo2 = __builtin_amdgcn_perm(0u, u8, 0x0c010c00u);  // (b0, b1) as fp16 mantissas
-              const uint32_t hi2 = __builtin_amdgcn_perm(0u, u8, 0x0c030c02u);  // (b2, b3)
-              const half4 bop = h == 0 ? as_half4(bx[ch].x, bx[ch].y) : as_half4(bx[ch].z, bx[ch].w);
-              dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(lo2, hi2), bop, dsum, 0, 0, 0);
-            }
-          }
-          dscale = half_bits_to_float(cur.meta & 0xFFFFu);
-          mterm = 0.0f;  // symmetric format: nothing besides the centred sum
-        }
-        // acc[i] += d(column i of this block) * D[i]: d sits in lane (b, i), a quad broadcast away
-        acc[0] = __fmaf_rn(dpp_move<kQuadBcast[0]>(dscale), dsum[0], acc[0]);
-        acc[1] = __fmaf_rn(dpp_move<kQuadBcast[1]>(dscale), dsum[1], acc[1]);
-        acc[2] = __fmaf_rn(dpp_move<kQuadBcast[2]>(dscale), dsum[2], acc[2]);
-        acc[3] = __fmaf_rn(dpp_move<kQuadBcast[3]>(dscale), dsum[3], acc[3]);
-#pragma unroll
-        for (int r = 0; r < MROWS; r++)
-          if constexpr (FMT == MGN_FMT_Q4) macc[r] = __fmaf_rn(mterm, sxv[r], macc[r]);
-
-        if (cst + 1 == my_steps) {
-          // ---- end of a column quad: the one cross-lane reduction ----
-          // acc[col] in lane (b, j): add the hi/lo pair (j ^ 1), then all 16 blocks b
-          float tot[4];
-#pragma unroll
-          for (int col = 0; col < 4; col++) {
-            float v = acc[col];
-            v += dpp_move<kDppQuadXor1>(v);
-            tot[col] = sum_over_blocks(v);  // lanes j = 2r, 2r+1: row r's sum for column `col`
-            acc[col] = 0.0f;
-          }
-#pragma unroll
-          for (int r = 0; r < MROWS; r++) {
-            const float mt = sum_over_blocks(macc[r]);  // lane (., i): column i's m-term, row r
-            macc[r] = 0.0f;
-            const float m0 = dpp_move<kQuadBcast[0]>(mt), m1 = dpp_move<kQuadBcast[1]>(mt);
-            const float m2 = dpp_move<kQuadBcast[2]>(mt), m3 = dpp_move<kQuadBcast[3]>(mt);
-            if (lane == (uint32_t)(2 * r)) {
-              const float os = kTwoPow24 * inv_scale[r];
-              float* dst = red + (((cq - quad0) * ksc + ks) * MROWS + r) * 4;
-              dst[0] = (tot[0] + m0) * os;
-              dst[1] = (tot[1] + m1) * os;
-              dst[2] = (tot[2] + m2) * os;
-              dst[3] = (tot[3] + m3) * os;
-            }
-          }
-        }
-        if (++cst == my_steps) {
-          cst = 0;
-          cq += wnc;
+        for (int h = 0; h < 2; h++) {
+          const uint32_t u8 = words[2 * ch + h] ^ 0x80808080u;  // q + 128 in every byte
+          const uint32_t lo2 = __builtin_amdgcn_perm(0u, u8, 0x0c010c00u);  // (b0, b1) as fp16 mantissas
+          const uint32_t hi2 = __builtin_amdgcn_perm(0u, u8, 0x0c030c02u);  // (b2, b3)
+          const half4 aop = h == 0 ? as_half4(ax[ch].x, ax[ch].y) : as_half4(ax[ch].z, ax[ch].w);
+          dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(aop, as_half4(lo2, hi2), dsum, 0, 0, 0);
         }
       }
     }
+    const float dscale = half_bits_to_float(cur.meta & 0xFFFFu);
+#pragma unroll
+    for (int r = 0; r < MROWS; r++) {
+      acc[r] = __fmaf_rn(dscale, dsum[2 * r] + dsum[2 * r + 1], acc[r]);
+      if constexpr (FMT == MGN_FMT_Q4) {
+        // (m + 8 d) * S with S = -ci * operand_scale / 8: fold the -1/8 into the block constant
+        const float mneg = __fmaf_rn(-0.125f, half_bits_to_float(cur.meta >> 16), -dscale);
+        acc[r] = __fmaf_rn(mneg, ci[r], acc[r]);
+      }
+    }
   }
-  __syncthreads();
+  // ---- sum the 16 lanes of each column ----
+#pragma unroll
+  for (int r = 0; r < MROWS; r++) {
+    const float tot = sum_over_blocks(acc[r]);
+    if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot * (operand_scale<FMT>() * inv_scale[r]);
+  }
+  lds_barrier();
   // ---- combine the K splits, add the residual, store ----
-  for (uint32_t t = tid; t < qpw * MROWS * 4; t += blockDim.x) {
+  for (uint32_t t = tid; t < wnc * MROWS * 4; t += blockDim.x) {
     const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
     const uint32_t n = (quad0 + ql) * 4 + col;
     if (r < m && n < w.n) {
@@ -401,48 +339,44 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
 }
 
 struct MfmaGemvPlan {
-  uint32_t ksc, wnc, qpw, spk, grid;
+  uint32_t ksc, wnc, steps, grid;
   size_t lds;
 };
 
-// raw blocks in flight per lane: 8 x 20 B for Q4, 6 x 34 B for Q8
-template <int FMT>
-constexpr int ring_depth() { return FMT == MGN_FMT_Q4 ? 8 : 6; }
+constexpr uint32_t kMaxSteps = 8;  // blocks a lane holds in flight: 8 x 20 B (Q4) or 8 x 34 B (Q8)
 
 bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, MfmaGemvPlan* out) {
   const uint32_t bpc = k / 32, bpc_pad = (bpc + 15) & ~15u;
   const uint32_t steps_total = bpc_pad / 16;
   const uint32_t nquads = (n + 3) / 4;
   MfmaGemvPlan p{};
+  // K splits: at least enough that a wave's share fits in its registers; more when there
+  // are too few column quads to give every CU a handful of waves
+  uint32_t ksc = (steps_total + kMaxSteps - 1) / kMaxSteps;
+  if (ksc > 16) return false;
+  const uint32_t want_waves = (uint32_t)num_cus * 8;
+  while (ksc < 16 && nquads * ksc < want_waves && (steps_total + ksc) / (ksc + 1) >= 2) ksc++;
+  p.steps = (steps_total + ksc - 1) / ksc;
+  p.ksc = (steps_total + p.steps - 1) / p.steps;  // drop splits that would get no step
   // quads per workgroup: spread the quads evenly over the CUs (one workgroup per CU when
   // there is enough work), so the activations are prepared as few times as possible
-  p.qpw = std::max<uint32_t>(1, (nquads + num_cus - 1) / num_cus);
-  // K splits: keep at least ~12 waves per workgroup busy when a workgroup has few quads,
-  // but leave every wave a few steps of its own
-  uint32_t ksc = 1;
-  while (p.qpw * ksc < 12 && ksc * 2 <= 16 && steps_total / (ksc * 2) >= 2) ksc *= 2;
-  p.ksc = ksc;
-  p.spk = (steps_total + ksc - 1) / ksc;
-  p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(p.qpw, 16 / ksc));
-  // enough threads to prepare the activations (waves beyond the quads only help there)
+  const uint32_t max_wnc = 16 / p.ksc;
+  p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (nquads + num_cus - 1) / num_cus));
+  // enough threads to prepare the activations (waves without a quad only help there)
   const uint32_t prep_waves = (bpc_pad * 4 + kMaxTasks * 64 - 1) / (kMaxTasks * 64);
-  p.wnc = std::min<uint32_t>(16 / ksc, std::max<uint32_t>(p.wnc, (prep_waves + ksc - 1) / ksc));
-  p.grid = (nquads + p.qpw - 1) / p.qpw;
+  p.wnc = std::max<uint32_t>(p.wnc, (prep_waves + p.ksc - 1) / p.ksc);
+  if (p.wnc > max_wnc) return false;
+  p.grid = (nquads + p.wnc - 1) / p.wnc;
   const size_t nj = 2 * mrows;
-  p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)mrows * bpc_pad * 4 + (size_t)bpc_pad * nj * 4 +
-          (size_t)p.qpw * ksc * mrows * 16 + (size_t)16 * mrows * 4 + 64;
+  p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 4 + (size_t)p.wnc * p.ksc * mrows * 16 + 64;
   if (p.lds > 150 * 1024) return false;
-  // every thread prepares at most kMaxTasks activation chunks per row
-  if ((size_t)bpc_pad * 4 > (size_t)kMaxTasks * 64 * p.ksc * p.wnc) return false;
   *out = p;
   return true;
 }
 
-template <int FMT, int MROWS>
-int launch_t(ihipStream_t* s, const LaunchArgs& x) {
-  MfmaGemvPlan p;
-  if (!plan_mfma_gemv(x.w.k, x.w.n, MROWS, x.num_cus, &p)) return (int)hipErrorInvalidValue;
-  auto kern = gemv_mfma_kernel<FMT, MROWS, ring_depth<FMT>()>;
+template <int FMT, int MROWS, int STEPS>
+int launch_steps(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
+  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS>;
   static bool big_lds_enabled = false;
   if (p.lds > 64 * 1024 && !big_lds_enabled) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -450,9 +384,26 @@ int launch_t(ihipStream_t* s, const LaunchArgs& x) {
     big_lds_enabled = true;
   }
   hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, x.w, (const float*)x.a, x.d, x.c, x.m,
-                     p.qpw, p.ksc, p.spk);
+                     p.ksc);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
+}
+
+template <int FMT, int MROWS>
+int launch_t(ihipStream_t* s, const LaunchArgs& x) {
+  MfmaGemvPlan p;
+  if (!plan_mfma_gemv(x.w.k, x.w.n, MROWS, x.num_cus, &p)) return (int)hipErrorInvalidValue;
+  switch (p.steps) {
+    case 1: return launch_steps<FMT, MROWS, 1>(s, x, p);
+    case 2: return launch_steps<FMT, MROWS, 2>(s, x, p);
+    case 3: return launch_steps<FMT, MROWS, 3>(s, x, p);
+    case 4: return launch_steps<FMT, MROWS, 4>(s, x, p);
+    case 5: return launch_steps<FMT, MROWS, 5>(s, x, p);
+    case 6: return launch_steps<FMT, MROWS, 6>(s, x, p);
+    case 7: return launch_steps<FMT, MROWS, 7>(s, x, p);
+    case 8: return launch_steps<FMT, MROWS, 8>(s, x, p);
+    default: return (int)hipErrorInvalidValue;
+  }
 }
 
 }  // namespace
