@@ -40,6 +40,21 @@
 // read consecutive 16-byte chunks.
 #include "kernels_common.hip.h"
 
+#ifdef MGN_TRACE
+// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.
+__device__ unsigned long long* mgn_trace_ptr = nullptr;
+extern "C" int mgn_debug_set_trace(void* p) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(mgn_trace_ptr), &p, sizeof(p));
+}
+#define MGN_STAMP(slot)                                                                          \
+  do {                                                                                           \
+    if (mgn_trace_ptr && (threadIdx.x & 63) == 0)                                                \
+      mgn_trace_ptr[((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 16 + (slot)] = __builtin_readcyclecounter(); \
+  } while (0)
+#else
+#define MGN_STAMP(slot) do {} while (0)
+#endif
+
 namespace mgn {
 namespace {
 
@@ -51,6 +66,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 template <int FMT>
 constexpr float operand_scale() { return FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f; }  // 2^20, 2^24
 constexpr int kMaxTasks = 2;  // activation chunks a thread prepares, per row
+constexpr int kDepth = 3;     // weight blocks in flight per lane ahead of the one in use
 
 __device__ __forceinline__ half4 as_half4(uint32_t lo, uint32_t hi) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -158,6 +174,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   float* red = cinit + bpc_pad * MROWS;               // [wnc][ksc][MROWS][4]
   uint32_t* amax_bits = (uint32_t*)(red + wnc * ksc * MROWS * 4);  // [MROWS]
 
+  MGN_STAMP(0);
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   // everything derived from the wave index is wave-uniform: keep it in scalar registers
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -193,20 +210,23 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
       xraw[tt][r][1] = src[1];
     }
   }
+  // Weight blocks: kDepth loads run ahead of the step that consumes them.  That is enough
+  // to keep the memory system busy; issuing every load up front would only park the wave
+  // in the load queue (which drains at HBM speed) before it could prepare any activations.
   Raw<FMT> blk[STEPS];
-  {
-    const uint32_t n = quad * 4 + i;
-    const uint32_t base = n * bpc + kb_first;
-    const bool n_ok = wave_live && n < w.n;
+  const uint32_t wbase = (quad * 4 + i) * bpc + kb_first;
+  const bool n_ok = wave_live && quad * 4 + i < w.n;
+  auto fetch = [&](int s) {
+    const bool ok = n_ok && step_begin + s < steps_total && kb_first + s * 16 < bpc;
+    blk[s].load(w, ok ? wbase + s * 16 : zero_block);
+  };
 #pragma unroll
-    for (int s = 0; s < STEPS; s++) {
-      const bool ok = n_ok && step_begin + s < steps_total && kb_first + s * 16 < bpc;
-      blk[s].load(w, ok ? base + s * 16 : zero_block);
-    }
-  }
+  for (int s = 0; s < STEPS && s < kDepth; s++) fetch(s);
   for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += blockDim.x) red[t] = 0.0f;
   if (tid < (uint32_t)MROWS) amax_bits[tid] = 0;
+  MGN_STAMP(1);
   lds_barrier();
+  MGN_STAMP(2);
 
   // ---- activations -> LDS (once per workgroup) ----
   float inv_scale[MROWS];
@@ -232,7 +252,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
       am = fmaxf(am, dpp_move<kDppRowMirror>(am));
       if ((lane & 15) == 0) atomicMax(&amax_bits[r], __builtin_bit_cast(uint32_t, am));
     }
+    MGN_STAMP(3);
     lds_barrier();
+    MGN_STAMP(4);
     float scale[MROWS];
 #pragma unroll
     for (int r = 0; r < MROWS; r++) scale[r] = row_scale(amax_bits[r], &inv_scale[r]);
@@ -258,7 +280,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
       }
     }
   }
+  MGN_STAMP(5);
   lds_barrier();
+  MGN_STAMP(6);
 
   // ---- the K walk: STEPS blocks per lane, straight-line ----
   // Lanes i >= NJ have no activation row of their own; they re-read row i % NJ (a broadcast
@@ -272,6 +296,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   for (int s = 0; s < STEPS; s++) {
     // steps past the end of K multiply the zero block; keep their LDS reads in range
     const uint32_t so = (step_begin + s < steps_total) ? (uint32_t)s : 0u;
+    if (s + kDepth < STEPS) fetch(s + kDepth);
     const Raw<FMT>& cur = blk[s];
     // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks
     uint4 ax[4];
@@ -317,14 +342,19 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
         acc[r] = __fmaf_rn(mneg, ci[r], acc[r]);
       }
     }
+    if (s == 0) MGN_STAMP(7);
+    if (s == 3) MGN_STAMP(8);
   }
+  MGN_STAMP(9);
   // ---- sum the 16 lanes of each column ----
 #pragma unroll
   for (int r = 0; r < MROWS; r++) {
     const float tot = sum_over_blocks(acc[r]);
     if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot * (operand_scale<FMT>() * inv_scale[r]);
   }
+  MGN_STAMP(10);
   lds_barrier();
+  MGN_STAMP(11);
   // ---- combine the K splits, add the residual, store ----
   for (uint32_t t = tid; t < wnc * MROWS * 4; t += blockDim.x) {
     const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
@@ -336,6 +366,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
       c[o] = dres ? v + dres[o] : v;
     }
   }
+  MGN_STAMP(12);
 }
 
 struct MfmaGemvPlan {
