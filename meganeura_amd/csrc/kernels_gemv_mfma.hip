@@ -22,7 +22,9 @@
 // aligns products by the operands' nominal exponents and drops low bits of
 // mantissas with many leading zeros.  Q8 bytes, q + 128 in bits 0-7, have few
 // leading zeros and are fine.)  Activations are split x = hi + lo into two fp16 after
-// scaling the row by a power of two (|x| < 2^12), so products are exact in f32
+// scaling each 32-element K block by its own power of two (|x| < 2^12; the
+// scale needs only the block's four preparing lanes, no workgroup-wide
+// reduction), so products are exact in f32
 // and only the f32 accumulation rounds: the result carries ~21 bits of x, not
 // 11.  Per block the identity used is
 //   sum_k (n_k d + m) x_k = d * (sum_k n_k x_k - 8 S) + (m + 8 d) * S,  S = sum_k x_k :
@@ -119,7 +121,8 @@ struct Raw<MGN_FMT_Q8> {
 //   chunk planes  xa[c][kb * NJ + j]  (uint4), c = 0..3: the A-operand rows of the two
 //                 MFMAs that consume elements 8c..8c+7 of K block kb; j = 2*row (high
 //                 halves) or 2*row + 1 (low halves);
-//   cinit[kb][row] = -bias / operand_scale * S(kb, row), the chain's initial accumulator.
+//   cinit[kb][row] = { -bias / operand_scale * S(kb, row), the chain's initial accumulator;
+//                      operand_scale / block scale, which undoes both scalings afterwards }.
 // Q4 pairs nibble k with k+4 in one fp16x2 mask, so the chunk is (x0,x4,x2,x6 | x1,x5,x3,x7).
 // Q8 bytes come out in natural order: (x0,x1,x2,x3 | x4,x5,x6,x7).
 template <int FMT>
@@ -140,11 +143,12 @@ __device__ __forceinline__ void make_chunks(const float (&x)[8], uint4& hi, uint
   lo = make_uint4(l[0], l[1], l[2], l[3]);
 }
 
-// Power of two that brings the row's largest magnitude below 2^12 (1 if the row
-// is all zero or not finite).  amax_bits: the IEEE bits of max |x|.
-__device__ __forceinline__ float row_scale(uint32_t amax_bits, float* inv) {
+// Power of two that brings a block's largest magnitude below 2^12 (1 if the block
+// is all zero, tiny or not finite).  *inv gets the reciprocal.
+__device__ __forceinline__ float block_scale(float amax, float* inv) {
+  const uint32_t amax_bits = __builtin_bit_cast(uint32_t, amax);
   const int e = (int)(amax_bits >> 23) - 127;  // floor(log2(amax)) for normal values
-  if (amax_bits == 0 || e >= 128 || e <= -100) {
+  if (amax_bits == 0 || e >= 100 || e <= -100) {
     *inv = 1.0f;
     return 1.0f;
   }
@@ -170,9 +174,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   const uint32_t plane = bpc_pad * NJ;
   const uint32_t nwaves = blockDim.x >> 6, wnc = nwaves / ksc;
   uint4* xa = lds4;                                   // [4][plane]
-  float* cinit = (float*)(lds4 + 4 * plane);          // [bpc_pad][MROWS]
-  float* red = cinit + bpc_pad * MROWS;               // [wnc][ksc][MROWS][4]
-  uint32_t* amax_bits = (uint32_t*)(red + wnc * ksc * MROWS * 4);  // [MROWS]
+  float2* cinit = (float2*)(lds4 + 4 * plane);        // [bpc_pad][MROWS]
+  float* red = (float*)(cinit + bpc_pad * MROWS);     // [wnc][ksc][MROWS][4]
 
   MGN_STAMP(0);
   const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -223,60 +226,36 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
 #pragma unroll
   for (int s = 0; s < STEPS && s < kDepth; s++) fetch(s);
   for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += blockDim.x) red[t] = 0.0f;
-  if (tid < (uint32_t)MROWS) amax_bits[tid] = 0;
   MGN_STAMP(1);
-  lds_barrier();
-  MGN_STAMP(2);
 
   // ---- activations -> LDS (once per workgroup) ----
-  float inv_scale[MROWS];
-  {
 #pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      float am = 0.0f;
+  for (int tt = 0; tt < kMaxTasks; tt++) {
+    const uint32_t t = tid + tt * blockDim.x, kb = t >> 2, ch = t & 3;
+    if (t < bpc_pad * 4) {  // whole waves take this branch together (bpc_pad * 4 is a multiple of 64)
 #pragma unroll
-      for (int tt = 0; tt < kMaxTasks; tt++) {
-        const bool ok = ((tid + tt * blockDim.x) >> 2) < bpc && (uint32_t)r < m;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          if (!ok) xraw[tt][r][h] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-          const float4 v = xraw[tt][r][h];
-          am = fmaxf(am, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
-        }
-      }
-      // NaN never wins fmaxf; infinities do and switch scaling off in row_scale.
-      // |x| orders like its bit pattern, so an integer max over the workgroup will do.
-      am = fmaxf(am, dpp_move<kDppQuadXor1>(am));
-      am = fmaxf(am, dpp_move<kDppQuadXor2>(am));
-      am = fmaxf(am, dpp_move<kDppRowHalfMirror>(am));
-      am = fmaxf(am, dpp_move<kDppRowMirror>(am));
-      if ((lane & 15) == 0) atomicMax(&amax_bits[r], __builtin_bit_cast(uint32_t, am));
-    }
-    MGN_STAMP(3);
-    lds_barrier();
-    MGN_STAMP(4);
-    float scale[MROWS];
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) scale[r] = row_scale(amax_bits[r], &inv_scale[r]);
-#pragma unroll
-    for (int tt = 0; tt < kMaxTasks; tt++) {
-      const uint32_t t = tid + tt * blockDim.x, kb = t >> 2, ch = t & 3;
-      if (t < bpc_pad * 4) {  // whole waves take this branch together (bpc_pad * 4 is a multiple of 64)
-#pragma unroll
-        for (int r = 0; r < MROWS; r++) {
-          const float4 v0 = xraw[tt][r][0], v1 = xraw[tt][r][1];
-          const float x[8] = {v0.x * scale[r], v0.y * scale[r], v0.z * scale[r], v0.w * scale[r],
-                              v1.x * scale[r], v1.y * scale[r], v1.z * scale[r], v1.w * scale[r]};
-          uint4 hi, lo;
-          make_chunks<FMT>(x, hi, lo);
-          xa[ch * plane + kb * NJ + 2 * r] = hi;
-          xa[ch * plane + kb * NJ + 2 * r + 1] = lo;
-          float s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
-          s += dpp_move<kDppQuadXor1>(s);
-          s += dpp_move<kDppQuadXor2>(s);
-          constexpr float bias = FMT == MGN_FMT_Q4 ? 8.0f : 128.0f;
-          if (ch == 0) cinit[kb * MROWS + r] = s * (-bias / operand_scale<FMT>());
-        }
+      for (int r = 0; r < MROWS; r++) {
+        float4 v0 = xraw[tt][r][0], v1 = xraw[tt][r][1];
+        if (!(kb < bpc && (uint32_t)r < m)) v0 = v1 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        // block maximum over the quad's 32 values; NaN never wins fmaxf, an infinity
+        // does and switches scaling off
+        float am = fmaxf(fmaxf(fmaxf(fabsf(v0.x), fabsf(v0.y)), fmaxf(fabsf(v0.z), fabsf(v0.w))),
+                         fmaxf(fmaxf(fabsf(v1.x), fabsf(v1.y)), fmaxf(fabsf(v1.z), fabsf(v1.w))));
+        am = fmaxf(am, dpp_move<kDppQuadXor1>(am));
+        am = fmaxf(am, dpp_move<kDppQuadXor2>(am));
+        float inv;
+        const float scale = block_scale(am, &inv);
+        const float x[8] = {v0.x * scale, v0.y * scale, v0.z * scale, v0.w * scale,
+                            v1.x * scale, v1.y * scale, v1.z * scale, v1.w * scale};
+        uint4 hi, lo;
+        make_chunks<FMT>(x, hi, lo);
+        xa[ch * plane + kb * NJ + 2 * r] = hi;
+        xa[ch * plane + kb * NJ + 2 * r + 1] = lo;
+        float s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+        s += dpp_move<kDppQuadXor1>(s);
+        s += dpp_move<kDppQuadXor2>(s);
+        constexpr float bias = FMT == MGN_FMT_Q4 ? 8.0f : 128.0f;
+        if (ch == 0) cinit[kb * MROWS + r] = make_float2(s * (-bias / operand_scale<FMT>()), inv * operand_scale<FMT>());
       }
     }
   }
@@ -288,7 +267,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   // Lanes i >= NJ have no activation row of their own; they re-read row i % NJ (a broadcast
   // in LDS) and the D entries they produce are never looked at.
   const char* xa_lane = (const char*)xa + ((kb_first * NJ) + (i % NJ)) * 16;
-  const char* ci_lane = (const char*)cinit + kb_first * MROWS * 4;
+  const char* ci_lane = (const char*)cinit + kb_first * MROWS * 8;
   float acc[MROWS];  // lane (b, j): sum over this lane's K blocks for column 4*quad+j, per row
 #pragma unroll
   for (int r = 0; r < MROWS; r++) acc[r] = 0.0f;
@@ -302,11 +281,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
     uint4 ax[4];
 #pragma unroll
     for (int ch = 0; ch < 4; ch++) ax[ch] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + ch * plane * 16);
-    float ci[MROWS];
+    float2 ci[MROWS];  // {chain start value, factor that undoes the operand and block scales}
 #pragma unroll
-    for (int r = 0; r < MROWS; r++) ci[r] = *(const float*)(ci_lane + so * (16 * MROWS * 4) + r * 4);
+    for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_lane + so * (16 * MROWS * 8) + r * 8);
     // the centring term rides in as the chain's start value (rows 2r and 2r+1 add up later)
-    floatx4 dsum = {ci[0], 0.0f, MROWS > 1 ? ci[MROWS - 1] : 0.0f, 0.0f};
+    floatx4 dsum = {ci[0].x, 0.0f, MROWS > 1 ? ci[MROWS - 1].x : 0.0f, 0.0f};
     if constexpr (FMT == MGN_FMT_Q4) {
       const uint32_t words[4] = {cur.q.x, cur.q.y, cur.q.z, cur.q.w};
 #pragma unroll
@@ -335,12 +314,13 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
     const float dscale = half_bits_to_float(cur.meta & 0xFFFFu);
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
-      acc[r] = __fmaf_rn(dscale, dsum[2 * r] + dsum[2 * r + 1], acc[r]);
+      float v = dscale * (dsum[2 * r] + dsum[2 * r + 1]);
       if constexpr (FMT == MGN_FMT_Q4) {
         // (m + 8 d) * S with S = -ci * operand_scale / 8: fold the -1/8 into the block constant
         const float mneg = __fmaf_rn(-0.125f, half_bits_to_float(cur.meta >> 16), -dscale);
-        acc[r] = __fmaf_rn(mneg, ci[r], acc[r]);
+        v = __fmaf_rn(mneg, ci[r].x, v);
       }
+      acc[r] = __fmaf_rn(v, ci[r].y, acc[r]);
     }
     if (s == 0) MGN_STAMP(7);
     if (s == 3) MGN_STAMP(8);
@@ -350,7 +330,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
 #pragma unroll
   for (int r = 0; r < MROWS; r++) {
     const float tot = sum_over_blocks(acc[r]);
-    if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot * (operand_scale<FMT>() * inv_scale[r]);
+    if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot;
   }
   MGN_STAMP(10);
   lds_barrier();
@@ -399,7 +379,7 @@ bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, MfmaGem
   if (p.wnc > max_wnc) return false;
   p.grid = (nquads + p.wnc - 1) / p.wnc;
   const size_t nj = 2 * mrows;
-  p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 4 + (size_t)p.wnc * p.ksc * mrows * 16 + 64;
+  p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 8 + (size_t)p.wnc * p.ksc * mrows * 16 + 64;
   if (p.lds > 150 * 1024) return false;
   *out = p;
   return true;
