@@ -40,6 +40,8 @@
 // of a column are summed once per column quad.  The activations' A operands
 // are prepared once per workgroup in LDS, laid out so that consecutive lanes
 // read consecutive 16-byte chunks.
+#include <cstdlib>
+
 #include "kernels_common.hip.h"
 
 #ifdef MGN_TRACE
@@ -68,7 +70,10 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 template <int FMT>
 constexpr float operand_scale() { return FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f; }  // 2^20, 2^24
 constexpr int kMaxTasks = 2;  // activation chunks a thread prepares, per row
-constexpr int kDepth = 3;     // weight blocks in flight per lane ahead of the one in use
+#ifndef MGN_GEMV_DEPTH
+#define MGN_GEMV_DEPTH 3
+#endif
+constexpr int kDepth = MGN_GEMV_DEPTH;  // weight blocks in flight per lane ahead of the one in use
 
 __device__ __forceinline__ half4 as_half4(uint32_t lo, uint32_t hi) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -327,6 +332,20 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   }
   MGN_STAMP(9);
   // ---- sum the 16 lanes of each column ----
+  if (ksc == 1) {
+    // no K split: lanes 0..3 hold the four finished columns of this wave's quad
+#pragma unroll
+    for (int r = 0; r < MROWS; r++) {
+      const float tot = sum_over_blocks(acc[r]);
+      const uint32_t n = quad * 4 + lane;
+      if (lane < 4 && wave_live && (uint32_t)r < m && n < w.n) {
+        const size_t o = (size_t)r * w.n + n;
+        c[o] = dres ? tot + dres[o] : tot;
+      }
+    }
+    MGN_STAMP(12);
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < MROWS; r++) {
     const float tot = sum_over_blocks(acc[r]);
@@ -373,6 +392,7 @@ bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, MfmaGem
   // there is enough work), so the activations are prepared as few times as possible
   const uint32_t max_wnc = 16 / p.ksc;
   p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (nquads + num_cus - 1) / num_cus));
+  if (const char* e = getenv("MGN_DEV_WNC")) p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (uint32_t)atoi(e)));
   // enough threads to prepare the activations (waves without a quad only help there)
   const uint32_t prep_waves = (bpc_pad * 4 + kMaxTasks * 64 - 1) / (kMaxTasks * 64);
   p.wnc = std::max<uint32_t>(p.wnc, (prep_waves + p.ksc - 1) / p.ksc);
