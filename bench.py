@@ -55,6 +55,10 @@ WORKLOADS = {
 }
 HEADLINE = "c5_q4_m1_4096x14336"
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
+# same counters read for a 256 MiB device copy (profiles/gemv_mfma_q4_m1_4096x14336.md).
+MEASURED_TRAFFIC_BYTES = {"c5_q4_m1_4096x14336": 37.02e6}
+
 
 def algorithmic_bytes(fmt, m, k, n, resid, f16):
     """Bytes one call must move: packed weight once (20 B per Q4 block; 34 B per Q8
@@ -153,6 +157,9 @@ def main():
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
     ap.add_argument("--sweep", action="store_true", help="also measure every configuration (stderr)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--profile", action="store_true",
+                    help="for rocprofv3 runs: only the timed cache-cold workload plus one 256 MiB device copy "
+                         "(a known size to calibrate FETCH_SIZE / WRITE_SIZE against); no CPU leg, no warm leg")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (column-parallel "
@@ -175,22 +182,33 @@ def main():
     want = oracle.matmul_packed(wl.fmt, x, oracle.quantize(wl.fmt, wl.w_host), wl.n, wl.d_host)
     oracle.assert_close(got, want, 1e-3, 1e-4)
 
+    if args.profile:
+        args.no_cpu = True
+        cal = 256 << 20
+        src, dst = ctx.buffer(cal), ctx.buffer(cal)
+        ctx.copy(dst, src, cal)
+        ctx.sync()
+        src.free()
+        dst.free()
+
     cpu = None
     if not args.no_cpu:
         cpu_out, cpu = cpu_baseline(wl)
         oracle.assert_close(cpu_out, want, 1e-3, 1e-4)
 
     # cache-warm figure for the same shape (one weight, reused every step)
-    warm = Workload(ctx, args.workload, 0)
-    warm_ms = warm.run(args.steps, args.warmup)
-    warm.free()
+    warm_ms = None
+    if not args.profile:
+        warm = Workload(ctx, args.workload, 0)
+        warm_ms = warm.run(args.steps, args.warmup)
+        warm.free()
 
     if is_gemm:
         roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": tflops / MFMA_F16_PEAK_TFLOPS, "traffic": None}
     else:
         roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": gbs / HBM_PEAK_GBS, "traffic": None}
+                "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
     line = {
         "metric": "Q4/Q8 GEMV HBM GB/s (% of peak) + us/call; prefill dequant-GEMM TFLOP/s",
         "value": tflops if is_gemm else gbs,
@@ -214,7 +232,8 @@ def main():
         },
         "roofline": roof,
         "cpu_baseline": cpu,
-        "cache_warm": {"us_per_call": warm_ms * 1e3, "GB/s": wl.bytes / (warm_ms * 1e-3) / 1e9},
+        "cache_warm": None if warm_ms is None else
+        {"us_per_call": warm_ms * 1e3, "GB/s": wl.bytes / (warm_ms * 1e-3) / 1e9},
         "pct_of_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
     }
     wl.free()

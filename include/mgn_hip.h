@@ -86,6 +86,11 @@ mgn_status mgn_buf_upload(mgn_ctx* ctx, mgn_buf* buf, size_t offset, const void*
 /* Session::read_output / read_buffer (src/runtime.rs:2612-2629); waits for the stream. */
 mgn_status mgn_buf_download(mgn_ctx* ctx, const mgn_buf* buf, size_t offset, void* dst, size_t bytes);
 
+/* Device-to-device copy on the context's stream (asynchronous).  The reference has no
+ * such call (its buffers are host-mapped); it is here for callers that stage data on
+ * the device, and it gives profilers a copy of known size to calibrate byte counters. */
+mgn_status mgn_buf_copy(mgn_ctx* ctx, mgn_buf* dst, const mgn_buf* src, size_t bytes);
+
 /* ---- block quantizers on the host, reference byte layout
  *      TensorType::size_bytes (src/graph.rs:52-68): 20 or 36 bytes per 32-element block. */
 size_t mgn_packed_size(mgn_fmt fmt, size_t rows, size_t cols);

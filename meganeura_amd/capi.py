@@ -19,7 +19,7 @@ ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA = r
 HIP_SYMBOLS = [
     "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync", "mgn_ctx_set_route",
     "mgn_buf_alloc", "mgn_buf_free", "mgn_buf_size", "mgn_buf_device_ptr", "mgn_buf_upload",
-    "mgn_buf_download", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
+    "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_matmul_q",
     "mgn_matmul_q_f16a", "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
@@ -77,6 +77,7 @@ def load():
         "mgn_buf_device_ptr": (vp, [vp]),
         "mgn_buf_upload": (C.c_int, [vp, vp, sz, vp, sz]),
         "mgn_buf_download": (C.c_int, [vp, vp, sz, vp, sz]),
+        "mgn_buf_copy": (C.c_int, [vp, vp, vp, sz]),
         "mgn_packed_size": (sz, [C.c_int, sz, sz]),
         "mgn_quantize_ref": (C.c_int, [C.c_int, vp, sz, sz, vp]),
         "mgn_dequantize_ref": (C.c_int, [C.c_int, vp, sz, sz, vp]),
@@ -198,6 +199,9 @@ class Context:
 
     def buffer(self, nbytes):
         return Buffer(self, nbytes)
+
+    def copy(self, dst, src, nbytes):
+        self.check(self.lib.mgn_buf_copy(self.h, dst.h, src.h, nbytes))
 
     def upload(self, arr):
         arr = np.ascontiguousarray(arr)

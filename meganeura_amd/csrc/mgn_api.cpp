@@ -188,6 +188,14 @@ mgn_status mgn_buf_download(mgn_ctx* ctx, const mgn_buf* buf, size_t offset, voi
   return MGN_OK;
 }
 
+mgn_status mgn_buf_copy(mgn_ctx* ctx, mgn_buf* dst, const mgn_buf* src, size_t bytes) {
+  if (!ctx || !dst || !src) return fail(ctx, MGN_EINVAL, "null argument");
+  if (bytes > dst->bytes || bytes > src->bytes) return fail(ctx, MGN_EINVAL, "copy exceeds buffer size");
+  if (bytes == 0) return MGN_OK;
+  MGN_HIP(ctx, hipMemcpyAsync(dst->ptr, src->ptr, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+  return MGN_OK;
+}
+
 // ---- host quantizers ----
 
 size_t mgn_packed_size(mgn_fmt fmt, size_t rows, size_t cols) {
