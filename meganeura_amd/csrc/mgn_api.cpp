@@ -354,8 +354,8 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   mgn_route route = ctx->route;
   if (route == MGN_ROUTE_AUTO) {
     if (mgn::gemv_mfma_supported(x)) route = MGN_ROUTE_GEMV_MFMA;
-    else if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV_VALU;
     else if (mgn::gemm_mfma_supported(x)) route = MGN_ROUTE_GEMM_MFMA;
+    else if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV_VALU;
     else route = MGN_ROUTE_GENERIC;
   }
   int rc;

@@ -111,7 +111,7 @@ ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv_valu": capi.ROUTE_GEMV_VALU, "gem
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-@pytest.mark.parametrize("route", ["generic", "gemv_valu", "gemv_mfma", "auto"])
+@pytest.mark.parametrize("route", ["generic", "gemv_valu", "gemv_mfma", "gemm_mfma", "auto"])
 @pytest.mark.parametrize("m,k,n", [
     (1, 32, 1), (1, 64, 3), (1, 576, 192), (1, 576, 577), (1, 1536, 576), (1, 1024, 100),
     (2, 576, 65), (3, 2048, 130), (4, 4096, 257), (1, 14336, 64), (1, 3072, 1024),
@@ -125,7 +125,7 @@ def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
         got = run_matmul(ctx, fmt, x, w, ROUTES[route])
         got_d = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d)
     except capi.MgnError as e:
-        if route.startswith("gemv") and "does not support" in str(e):
+        if route != "generic" and "does not support" in str(e):
             pytest.skip("shape outside this GEMV kernel's range")
         raise
     orc.assert_close(got, orc.matmul_f32(x, deq), REL, ABS)
@@ -139,7 +139,7 @@ def test_larger_m(ctx, orc, fmt, m, k, n):
     w = synth.normal(12 + m + k + n, k * n, 0.02).reshape(k, n)
     d = synth.normal(13 + n, m * n).reshape(m, n)
     deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
-    for route in ("generic", "auto"):
+    for route in ("generic", "gemm_mfma", "auto"):
         got = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d)
         orc.assert_close(got, orc.matmul_f32(x, deq, d), REL, ABS)
         # fp16 activations: the oracle multiplies the rounded values
