@@ -31,8 +31,28 @@
 // Work split: grid.y = row tiles; a workgroup owns `wnc` column tiles and splits
 // every 32-block K chunk `ksc` ways among its waves; partial tiles meet in LDS.
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 
 #include "kernels_common.hip.h"
+
+#ifdef MGN_TRACE
+// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.
+__device__ unsigned long long* mgn_gemm_trace_ptr = nullptr;
+extern "C" int mgn_debug_set_trace_gemm(void* p) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(mgn_gemm_trace_ptr), &p, sizeof(p));
+}
+#define MGN_GSTAMP_INIT() unsigned long long* const trace_base = mgn_gemm_trace_ptr
+#define MGN_GSTAMP(slot)                                                                                \
+  do {                                                                                                  \
+    if (trace_base && (threadIdx.x & 63) == 0)                                                          \
+      trace_base[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 16 + (slot)] = \
+          __builtin_readcyclecounter();                                                                 \
+  } while (0)
+#else
+#define MGN_GSTAMP_INIT() do {} while (0)
+#define MGN_GSTAMP(slot) do {} while (0)
+#endif
 
 namespace mgn {
 namespace {
@@ -42,8 +62,6 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kChunkBlocks = 32;  // K blocks staged in LDS at a time (1024 k)
-constexpr int kAhead = 3;         // weight blocks in flight per lane ahead of the one in use
 
 __device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
   const u32x4_t v = {a, b, c, d};
@@ -64,28 +82,6 @@ __device__ __forceinline__ void swap32(uint32_t& a, uint32_t& b) {
   b = r[1];
 }
 
-template <int FMT>
-struct RawBlk;
-template <>
-struct RawBlk<MGN_FMT_Q4> {
-  uint4 q;
-  uint32_t meta;
-  __device__ __forceinline__ void load(const WeightView& w, size_t b) {
-    q = stream_load_u128((const uint4*)w.quants + b);
-    meta = stream_load_u32((const uint32_t*)w.meta + b);
-  }
-};
-template <>
-struct RawBlk<MGN_FMT_Q8> {
-  uint4 q0, q1;
-  uint32_t meta;
-  __device__ __forceinline__ void load(const WeightView& w, size_t b) {
-    q0 = stream_load_u128((const uint4*)w.quants + b * 2);
-    q1 = stream_load_u128((const uint4*)w.quants + b * 2 + 1);
-    meta = stream_load_u16((const uint16_t*)w.meta + b);
-  }
-};
-
 // one dword of nibbles -> B operand (8 fp16): (n0,n4),(n1,n5),(n2,n6),(n3,n7), each n * 2^-20
 __device__ __forceinline__ half8 nibbles_to_operand(uint32_t wd) {
   return as_half8((wd << 4) & 0x00F000F0u, wd & 0x00F000F0u, (wd >> 4) & 0x00F000F0u, (wd >> 8) & 0x00F000F0u);
@@ -97,147 +93,165 @@ __device__ __forceinline__ half8 bytes_to_operand(uint32_t w0, uint32_t w1) {
                   __builtin_amdgcn_perm(0u, u1, 0x0c010c00u), __builtin_amdgcn_perm(0u, u1, 0x0c030c02u));
 }
 
-// LDS per workgroup:
-//   aimg[(lb * 2 + h) * 64 + lane]  (uint4): A operand of the MFMA that covers k = 16h..16h+15
-//                                   of local block lb, for A lane `lane` = row + 32 * g
-//   simg[(lb / 2) * 64 + lane]      (uint4): A operand of the step's additive MFMA; lanes < 32 hold
-//                                   (mean_hi, mean_lo) of blocks 2p and 2p+1 in the first two dwords,
-//                                   everything else stays zero
+// LDS per workgroup, two buffers b = chunk parity (CB = 8 * ksc K blocks per chunk):
+//   aimg[b][(lb * 2 + h) * 64 + lane]  (uint4): A operand of the MFMA that covers k = 16h..16h+15
+//                                      of local block lb, for A lane `lane` = row + 32 * g
+//   simg[b][(lb / 2) * 64 + lane]      (uint4): A operand of a step's additive MFMA; lanes < 32 hold
+//                                      (mean_hi, mean_lo) of blocks 2p and 2p+1 in the first two
+//                                      dwords, everything else stays zero
 // The element order inside an A operand follows the B side: Q4 pairs k with k+4, Q8 is natural.
+constexpr int kSteps = 4;  // steps per wave per chunk; a step is two K blocks
+// bytes per column of a parked weight slice: 8 blocks + 16 bytes of padding
+constexpr int slice_stride(int fmt) { return fmt == MGN_FMT_Q4 ? 8 * 16 + 16 : 8 * 32 + 16; }
+typedef uint32_t u32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x2_unaligned __attribute__((ext_vector_type(2), aligned(2)));
+
+struct GemmArgs {
+  WeightView w;
+  const void* a;
+  const float* dres;
+  float* c;
+  float* scratch;      // [parts][row tiles * ROWS][n] partial results when parts > 1
+  uint32_t* counters;  // one arrival counter per (row tile, column group), zero between launches
+  uint32_t m, ksc, wnc, nch, parts, colgroups;
+};
+
 template <int FMT>
-__device__ __forceinline__ void order_for_operand(const float (&x)[8], float (&p)[8]) {
+__device__ __forceinline__ uint4 f16_operand(uint4 v) {
   if constexpr (FMT == MGN_FMT_Q4) {
-    p[0] = x[0], p[1] = x[4], p[2] = x[1], p[3] = x[5], p[4] = x[2], p[5] = x[6], p[6] = x[3], p[7] = x[7];
+    return make_uint4(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                      __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
   } else {
-#pragma unroll
-    for (int i = 0; i < 8; i++) p[i] = x[i];
+    return v;
   }
 }
 
-// grid = (column-tile groups, row tiles).  blockDim.x = 64 * ksc * wnc.
-// SPC = steps per chunk per wave = kChunkBlocks / (2 * ksc); a step is two K blocks.
-template <int FMT, bool F32A, int SPC>
-__global__ __launch_bounds__(1024) void gemm_mfma_kernel(WeightView w, const void* __restrict__ a_any,
-                                                         const float* __restrict__ dres, float* __restrict__ c,
-                                                         uint32_t m, uint32_t ksc) {
-  constexpr int ROWS = F32A ? 16 : 32;           // real rows per tile
-  constexpr int NI = F32A ? 8 : 16;              // result registers per lane
-  constexpr int TPT = F32A ? 4 : 8;              // staging tasks per thread per chunk (>= 512 threads)
-  constexpr int NTASK = ROWS * kChunkBlocks * 4;  // one task = 8 consecutive k of one row
+// grid = (column groups * parts, row tiles); blockDim.x = 64 * ksc * wnc, ksc in {1, 2}.
+// A workgroup owns wnc column tiles of one row tile and K blocks
+// [part * nch * CB, (part + 1) * nch * CB); within a chunk wave (ks, wn) takes the
+// 8 blocks starting at 8 * ks.  While a chunk is being multiplied, the next chunk's
+// activations are in flight to registers and the weight ring is refilled one chunk ahead.
+// TPT = staging tasks per thread per chunk (one task = 8 consecutive k of one row).
+template <int FMT, bool F32A, int TPT>
+__global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kernel(GemmArgs g) {
+  constexpr int ROWS = F32A ? 16 : 32;  // real rows per tile
+  constexpr int NI = F32A ? 8 : 16;     // result registers per lane
   constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;
   extern __shared__ uint4 lds4[];
-  uint4* aimg = lds4;
-  uint4* simg = lds4 + kChunkBlocks * 2 * 64;
-  float* red = (float*)lds4;  // reused after the K loop: [wave][NI][64]
+  const WeightView& w = g.w;
+  const uint32_t ksc = g.ksc, wnc = g.wnc;
+  const uint32_t cb = 8 * ksc;                  // blocks per chunk
+  const uint32_t a_stride = cb * 2 * 64;        // uint4 per aimg buffer
+  const uint32_t s_stride = (cb / 2) * 64;      // uint4 per simg buffer
+  uint4* const aimg = lds4;
+  uint4* const simg = lds4 + 2 * a_stride;
+  float* const red = (float*)lds4;  // reused after the K loop: [wn][NI][64]
 
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t nwaves = blockDim.x >> 6, wnc = nwaves / ksc;
   const uint32_t ks = wave % ksc, wn = wave / ksc;
-  const uint32_t cl = lane & 31, g = lane >> 5;
+  const uint32_t cl = lane & 31, gh = lane >> 5;
   const uint32_t bpc = w.k / 32;
   const uint32_t n_tiles = (w.n + 31) / 32;
-  const uint32_t col_tile = blockIdx.x * wnc + wn;
+  const uint32_t cg = blockIdx.x / g.parts, part = blockIdx.x % g.parts;
+  const uint32_t col_tile = cg * wnc + wn;
   const uint32_t n = col_tile * 32 + cl;
   const bool n_ok = col_tile < n_tiles && n < w.n;
   const uint32_t row0 = blockIdx.y * ROWS;
   const uint32_t zero_block = bpc * w.n;
-  const uint32_t nchunks = (bpc + kChunkBlocks - 1) / kChunkBlocks;
-  const uint32_t split_first = ks * (2 * SPC);  // this wave's first local block in every chunk
+  const uint32_t chunk0 = part * g.nch;  // first chunk of this workgroup
 
-  // the additive operands' unused slots must read as zero for the whole kernel
-  for (uint32_t t = tid; t < (kChunkBlocks / 2) * 64; t += blockDim.x) simg[t] = make_uint4(0, 0, 0, 0);
-  lds_barrier();
+  MGN_GSTAMP_INIT();
+  MGN_GSTAMP(0);
 
-  floatx16 acc;
+  // ---- per-thread staging tasks: task t = (lb * ROWS + r) * 4 + sub, sub = 2h + g ----
+  uint32_t t_lb[TPT], t_slot[TPT], t_r[TPT];
+  size_t t_off[TPT];
+  bool t_rowok[TPT], t_live[TPT];
 #pragma unroll
-  for (int i = 0; i < 16; i++) acc[i] = 0.0f;
-
-  for (uint32_t chunk = 0; chunk < nchunks; chunk++) {
-    const uint32_t kb_chunk = chunk * kChunkBlocks;
-    // ---- 1. activation loads for this thread's staging tasks (oldest in the queue) ----
-    // task t = (lb * ROWS + r) * 4 + sub, sub = 2h + g: the four tasks of a (row, block) are a lane quad
-    uint4 raw[TPT][F32A ? 2 : 1];
+  for (int tt = 0; tt < TPT; tt++) {
+    const uint32_t t = tid + tt * blockDim.x;
+    const uint32_t sub = t & 3, r = (t >> 2) % ROWS, lb = (t >> 2) / ROWS;
+    t_lb[tt] = lb;
+    t_r[tt] = r;
+    t_live[tt] = lb < cb;
+    t_rowok[tt] = t_live[tt] && row0 + r < g.m;
+    t_off[tt] = t_rowok[tt] ? (size_t)(row0 + r) * w.k + (size_t)lb * 32 + sub * 8 : (size_t)0;
+    t_slot[tt] = (lb * 2 + (sub >> 1)) * 64 + 32 * (sub & 1) + r;
+  }
+  uint4 raw[TPT][F32A ? 2 : 1];
+  auto load_a = [&](uint32_t chunk) {  // unconditional loads; dead tasks re-read element 0
+    const uint32_t kb_chunk = chunk * cb;
 #pragma unroll
     for (int tt = 0; tt < TPT; tt++) {
-      const uint32_t t = tid + tt * blockDim.x;
-      const uint32_t sub = t & 3, r = (t >> 2) % ROWS, lb = (t >> 2) / ROWS;
-      const uint32_t row = row0 + r, kb = kb_chunk + lb;
-      const bool ok = t < NTASK && row < m && kb < bpc;
-      const size_t off = ok ? (size_t)row * w.k + (size_t)kb * 32 + sub * 8 : (size_t)0;
+      const bool ok = t_rowok[tt] && kb_chunk + t_lb[tt] < bpc;
+      const size_t off = ok ? t_off[tt] + (size_t)kb_chunk * 32 : (size_t)0;
       if constexpr (F32A) {
-        const uint4* src = (const uint4*)((const float*)a_any + off);
+        const uint4* src = (const uint4*)((const float*)g.a + off);
         raw[tt][0] = src[0];
         raw[tt][1] = src[1];
       } else {
-        raw[tt][0] = *(const uint4*)((const _Float16*)a_any + off);
+        raw[tt][0] = *(const uint4*)((const _Float16*)g.a + off);
       }
     }
-    // ---- 2. first weight blocks of the chunk go out right behind them ----
-    RawBlk<FMT> blk[SPC];
-    const uint32_t kb_wave = kb_chunk + split_first + g;  // this lane's block in step 0
-    const uint32_t wbase = n * bpc + kb_wave;
-    auto fetch = [&](int s) {
-      const bool ok = n_ok && kb_wave + 2 * s < bpc;
-      blk[s].load(w, ok ? wbase + 2 * s : zero_block);
-    };
-#pragma unroll
-    for (int s = 0; s < SPC && s < kAhead; s++) fetch(s);
-
-    // ---- 3. stage the chunk's A operands ----
+  };
+  auto stage = [&](uint32_t chunk, uint32_t buf) {
+    const uint32_t kb_chunk = chunk * cb;
+    uint4* const ab = aimg + buf * a_stride;
+    uint32_t* const sb = (uint32_t*)(simg + buf * s_stride);
 #pragma unroll
     for (int tt = 0; tt < TPT; tt++) {
-      const uint32_t t = tid + tt * blockDim.x;
-      if (t < NTASK) {  // whole waves together: NTASK and blockDim.x are multiples of 64
-        const uint32_t sub = t & 3, r = (t >> 2) % ROWS, lb = (t >> 2) / ROWS;
-        const uint32_t h = sub >> 1, gg = sub & 1;
-        const bool ok = row0 + r < m && kb_chunk + lb < bpc;
+      const bool ok = t_rowok[tt] && kb_chunk + t_lb[tt] < bpc;
+      const uint32_t lb = t_lb[tt], r = t_r[tt];
+      float s_hi, s_lo = 0.0f;
+      uint4 op_hi, op_lo;
+      if constexpr (F32A) {
+        const uint4 v0 = raw[tt][0], v1 = raw[tt][1];
+        const uint32_t bits[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
         float x[8], p[8];
-        if constexpr (F32A) {
-          const uint4 v0 = raw[tt][0], v1 = raw[tt][1];
-          const uint32_t bits[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
-          for (int e = 0; e < 8; e++) x[e] = ok ? __builtin_bit_cast(float, bits[e]) : 0.0f;
+        for (int e = 0; e < 8; e++) x[e] = ok ? __builtin_bit_cast(float, bits[e]) : 0.0f;
+        if constexpr (FMT == MGN_FMT_Q4) {
+          p[0] = x[0], p[1] = x[4], p[2] = x[1], p[3] = x[5], p[4] = x[2], p[5] = x[6], p[6] = x[3], p[7] = x[7];
         } else {
-          const uint4 v = raw[tt][0];
-          const uint32_t pr[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
-            x[2 * e] = ok ? half_lo(pr[e]) : 0.0f;
-            x[2 * e + 1] = ok ? half_hi(pr[e]) : 0.0f;
-          }
+          for (int e = 0; e < 8; e++) p[e] = x[e];
         }
-        order_for_operand<FMT>(x, p);
-        const uint32_t slot = (lb * 2 + h) * 64 + 32 * gg;
-        float s_hi, s_lo = 0.0f;
-        if constexpr (F32A) {
-          const uint32_t hp[4] = {pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7])};
-          float res[8], hs = 0.0f;
+        const uint32_t hp[4] = {pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7])};
+        float res[8], hs = 0.0f;
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const float f0 = half_lo(hp[e]), f1 = half_hi(hp[e]);
-            res[2 * e] = p[2 * e] - f0;
-            res[2 * e + 1] = p[2 * e + 1] - f1;
-            hs += f0 + f1;
-            s_lo += res[2 * e] + res[2 * e + 1];
-          }
-          s_hi = hs;
-          aimg[slot + r] = make_uint4(hp[0], hp[1], hp[2], hp[3]);
-          aimg[slot + 16 + r] =
-              make_uint4(pack_rtz(res[0], res[1]), pack_rtz(res[2], res[3]), pack_rtz(res[4], res[5]), pack_rtz(res[6], res[7]));
-        } else {
-          s_hi = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
-          aimg[slot + r] = make_uint4(pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7]));
+        for (int e = 0; e < 4; e++) {
+          const float f0 = half_lo(hp[e]), f1 = half_hi(hp[e]);
+          res[2 * e] = p[2 * e] - f0;
+          res[2 * e + 1] = p[2 * e + 1] - f1;
+          hs += f0 + f1;
+          s_lo += res[2 * e] + res[2 * e + 1];
         }
-        // block mean (sum over the quad's 32 values / 32), split into two fp16
-        s_hi += dpp_move<kDppQuadXor1>(s_hi);
-        s_hi += dpp_move<kDppQuadXor2>(s_hi);
-        if constexpr (F32A) {
-          s_lo += dpp_move<kDppQuadXor1>(s_lo);
-          s_lo += dpp_move<kDppQuadXor2>(s_lo);
-        }
-        if (sub == 0) {
-          uint32_t* sdst = (uint32_t*)(simg + (lb >> 1) * 64) + (lb & 1);
+        s_hi = hs;
+        op_hi = make_uint4(hp[0], hp[1], hp[2], hp[3]);
+        op_lo = make_uint4(pack_rtz(res[0], res[1]), pack_rtz(res[2], res[3]), pack_rtz(res[4], res[5]), pack_rtz(res[6], res[7]));
+      } else {
+        uint4 v = raw[tt][0];
+        if (!ok) v = make_uint4(0, 0, 0, 0);
+        const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+        s_hi = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v.x), ones, 0.0f, false);
+        s_hi = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v.y), ones, s_hi, false);
+        s_hi = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v.z), ones, s_hi, false);
+        s_hi = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v.w), ones, s_hi, false);
+        op_hi = f16_operand<FMT>(v);
+      }
+      // block mean (sum over the lane quad's 32 values / 32), split into two fp16
+      s_hi += dpp_move<kDppQuadXor1>(s_hi);
+      s_hi += dpp_move<kDppQuadXor2>(s_hi);
+      if constexpr (F32A) {
+        s_lo += dpp_move<kDppQuadXor1>(s_lo);
+        s_lo += dpp_move<kDppQuadXor2>(s_lo);
+      }
+      if (t_live[tt]) {
+        ab[t_slot[tt]] = op_hi;
+        if constexpr (F32A) ab[t_slot[tt] + 16] = op_lo;
+        if ((tid & 3) == 0) {
+          uint32_t* sdst = sb + (lb >> 1) * 256 + (lb & 1);
           const float mean = s_hi * 0.03125f;
           const uint32_t mh = pack_rtz(mean, 0.0f);
           sdst[r * 4] = (mh & 0xFFFFu) | (pack_rtz(mean - half_lo(mh), 0.0f) << 16);
@@ -249,19 +263,96 @@ __global__ __launch_bounds__(1024) void gemm_mfma_kernel(WeightView w, const voi
         }
       }
     }
-    lds_barrier();
+  };
 
-    // ---- 4. this wave's steps of the chunk ----
+  const uint32_t lb_wave = ks * (2 * kSteps);  // this wave's first local block in every chunk
+  // ---- weight slices: a wave's 8 blocks x 32 columns of a chunk ----
+  // Loaded as whole runs of a column's blocks (128 bytes of nibbles or 256 bytes of
+  // int8: 8 or 16 lanes per column, NL loads), parked in a wave-private LDS area with
+  // a padded column stride, and read back one block per lane (column lane%32, block
+  // 2s + lane/32) for step s.  Loading in the operand's own lane order instead would
+  // take 32 bytes from each cache line at a time and fetch every line several times.
+  // The scale words of the slice are one load per lane (4 blocks), broadcast across
+  // the wave halves.
+  constexpr int QB = FMT == MGN_FMT_Q4 ? 16 : 32;  // quant bytes per block
+  constexpr int NL = QB / 4;                       // 16-byte loads per lane per slice
+  constexpr int LPC = QB / 2;                      // lanes per column in one load
+  constexpr int CPL = 64 / LPC;                    // columns per load
+  constexpr int kStride = slice_stride(FMT);
+  uint4 wq[NL];
+  uint4 wm;  // Q4: scale|min words of 4 blocks; Q8: x, y = four fp16 scales
+  uint8_t* const wbuf = (uint8_t*)(lds4 + 2 * a_stride + 2 * s_stride) + wave * (32 * kStride);
+  auto fetch_slice = [&](uint32_t chunk, bool chunk_ok) {
+    const uint32_t kb0 = chunk * cb + lb_wave;
+    const bool tile_ok = chunk_ok && col_tile < n_tiles;
 #pragma unroll
-    for (int s = 0; s < SPC; s++) {
-      if (s + kAhead < SPC) fetch(s + kAhead);
-      const RawBlk<FMT>& cur = blk[s];
-      const uint32_t lb0 = split_first + 2 * s;  // local index of the step's first block
-      uint32_t meta0 = cur.meta, meta1 = cur.meta;
-      swap32(meta0, meta1);  // meta0: block lb0 for every lane, meta1: block lb0 + 1
-      half8 bop[2][2];       // [block][h]
+    for (int j = 0; j < NL; j++) {
+      const uint32_t nn = col_tile * 32 + CPL * j + lane / LPC, piece = lane % LPC;
+      const uint32_t kb = kb0 + piece / (QB / 16);
+      const bool ok = tile_ok && nn < w.n && kb < bpc;
+      const size_t idx = ok ? ((size_t)nn * bpc + kb0) * (QB / 16) + piece : (size_t)zero_block * (QB / 16);
+      wq[j] = stream_load_u128((const uint4*)w.quants + idx);
+    }
+    // blocks past the end of the column carry zero quants; their scale words must be zero too
+    const uint32_t kbm = kb0 + 4 * gh;
+    const bool okm = tile_ok && n_ok && kbm < bpc;
+    const bool ok1 = okm && kbm + 1 < bpc, ok2 = okm && kbm + 2 < bpc, ok3 = okm && kbm + 3 < bpc;
+    if constexpr (FMT == MGN_FMT_Q4) {
+      const u32x4_unaligned v =
+          __builtin_nontemporal_load((const u32x4_unaligned*)((const uint32_t*)w.meta + (okm ? n * bpc + kbm : zero_block)));
+      wm = make_uint4(okm ? v.x : 0u, ok1 ? v.y : 0u, ok2 ? v.z : 0u, ok3 ? v.w : 0u);
+    } else {
+      const u32x2_unaligned v =
+          __builtin_nontemporal_load((const u32x2_unaligned*)((const uint16_t*)w.meta + (okm ? n * bpc + kbm : zero_block)));
+      wm = make_uint4(okm ? v.x & 0xFFFFu : 0u, ok1 ? v.x >> 16 : 0u, ok2 ? v.y & 0xFFFFu : 0u, ok3 ? v.y >> 16 : 0u);
+    }
+  };
+  uint32_t mb[8];  // scale words of the slice's 8 blocks, the same in every lane
+  auto park_slice = [&]() {
+#pragma unroll
+    for (int j = 0; j < NL; j++) *(uint4*)(wbuf + (CPL * j + lane / LPC) * kStride + (lane % LPC) * 16) = wq[j];
+    const uint32_t mm[4] = {wm.x, wm.y, wm.z, wm.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      uint32_t lo = mm[e], hi = mm[e];
+      swap32(lo, hi);  // lo: lower half's word (block e) in every lane, hi: upper half's (block 4 + e)
+      mb[e] = lo;
+      mb[4 + e] = hi;
+    }
+  };
+
+  load_a(chunk0);
+  fetch_slice(chunk0, true);
+  MGN_GSTAMP(1);
+  // the additive operands' unused slots must read as zero for the whole kernel
+  for (uint32_t t = tid; t < 2 * s_stride; t += blockDim.x) simg[t] = make_uint4(0, 0, 0, 0);
+  lds_barrier();
+  stage(chunk0, 0);
+  MGN_GSTAMP(2);
+  lds_barrier();
+  MGN_GSTAMP(3);
+
+  floatx16 acc;
+#pragma unroll
+  for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+
+  for (uint32_t c = 0; c < g.nch; c++) {
+    const uint32_t chunk = chunk0 + c, buf = c & 1;
+    const bool more = c + 1 < g.nch;
+    load_a(more ? chunk + 1 : chunk);  // next chunk's activations travel while this one is multiplied
+    const uint4* const ab = aimg + buf * a_stride;
+    const uint4* const sb = simg + buf * s_stride;
+    park_slice();
+    fetch_slice(chunk + 1, more);
+#pragma unroll
+    for (int s = 0; s < kSteps; s++) {
+      const uint32_t lb0 = lb_wave + 2 * s;  // local index of the step's first block
+      const uint32_t meta0 = mb[2 * s], meta1 = mb[2 * s + 1];  // block lb0, block lb0 + 1
+      half8 bop[2][2];                                            // [block][h]
+      const uint4* const wsrc = (const uint4*)(wbuf + cl * kStride + (2 * s + gh) * QB);
       if constexpr (FMT == MGN_FMT_Q4) {
-        uint32_t r0 = cur.q.x, r1 = cur.q.y, r2 = cur.q.z, r3 = cur.q.w;
+        const uint4 q = wsrc[0];
+        uint32_t r0 = q.x, r1 = q.y, r2 = q.z, r3 = q.w;
         swap32(r0, r1);  // r0: block 0, k 0-7 | 8-15;   r1: block 1, same
         swap32(r2, r3);  // r2: block 0, k 16-23 | 24-31; r3: block 1, same
         bop[0][0] = nibbles_to_operand(r0);
@@ -269,8 +360,9 @@ __global__ __launch_bounds__(1024) void gemm_mfma_kernel(WeightView w, const voi
         bop[0][1] = nibbles_to_operand(r2);
         bop[1][1] = nibbles_to_operand(r3);
       } else {
-        uint32_t r0 = cur.q0.x, r1 = cur.q0.y, r2 = cur.q0.z, r3 = cur.q0.w;
-        uint32_t r4 = cur.q1.x, r5 = cur.q1.y, r6 = cur.q1.z, r7 = cur.q1.w;
+        const uint4 q0 = wsrc[0], q1 = wsrc[1];
+        uint32_t r0 = q0.x, r1 = q0.y, r2 = q0.z, r3 = q0.w;
+        uint32_t r4 = q1.x, r5 = q1.y, r6 = q1.z, r7 = q1.w;
         swap32(r0, r2);
         swap32(r1, r3);  // (r0, r1): block 0, k 0-7 | 8-15;   (r2, r3): block 1, same
         swap32(r4, r6);
@@ -285,7 +377,7 @@ __global__ __launch_bounds__(1024) void gemm_mfma_kernel(WeightView w, const voi
         floatx16 dsum;
 #pragma unroll
         for (int i = 0; i < 16; i++) dsum[i] = 0.0f;
-        const uint4* ap = aimg + ((lb0 + t) * 2) * 64 + lane;
+        const uint4* ap = ab + ((lb0 + t) * 2) * 64 + lane;
         dsum = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ap[0]), bop[t][0], dsum, 0, 0, 0);
         dsum = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ap[64]), bop[t][1], dsum, 0, 0, 0);
         const float dq = half_bits_to_float((t == 0 ? meta0 : meta1) & 0xFFFFu) * kOpScale;
@@ -308,75 +400,199 @@ __global__ __launch_bounds__(1024) void gemm_mfma_kernel(WeightView w, const voi
         add0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add0) * kb);
         add1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add1) * kb);
       }
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(simg[(lb0 >> 1) * 64 + lane]),
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(sb[(lb0 >> 1) * 64 + lane]),
                                                     as_half8(add0, add1, add0, add1), acc, 0, 0, 0);
     }
-    lds_barrier();  // the next chunk's staging overwrites aimg
+    if (c == 0) MGN_GSTAMP(4);
+    if (more) stage(chunk + 1, buf ^ 1);  // the other buffer was last read before the previous barrier
+    lds_barrier();
+    if (c == 0) MGN_GSTAMP(5);
   }
+  MGN_GSTAMP(6);
 
-  // ---- combine the K splits through LDS, add the residual, store ----
+  // ---- combine the two K halves of the workgroup ----
   // D layout: lane -> column lane%32; register i -> tile row 8*(i/4) + 4*(lane/32) + i%4.
   // With f32 activations rows r and r+16 (registers i and i+8) are the hi and lo parts.
   float outv[NI];
 #pragma unroll
   for (int i = 0; i < NI; i++) outv[i] = F32A ? acc[i] + acc[i + 8] : acc[i];
+  if (ksc == 2) {
+    if (ks == 1) {
 #pragma unroll
-  for (int i = 0; i < NI; i++) red[(wave * NI + i) * 64 + lane] = outv[i];
-  lds_barrier();
-  for (uint32_t idx = tid; idx < wnc * NI * 64; idx += blockDim.x) {
-    const uint32_t ln = idx & 63, i = (idx >> 6) % NI, tile = idx / (64 * NI);
-    const uint32_t row = row0 + 8 * (i >> 2) + 4 * (ln >> 5) + (i & 3);
-    const uint32_t col = (blockIdx.x * wnc + tile) * 32 + (ln & 31);
-    if (row < m && col < w.n) {
-      float v = 0.0f;
-      for (uint32_t s = 0; s < ksc; s++) v += red[((tile * ksc + s) * NI + i) * 64 + ln];
-      const size_t o = (size_t)row * w.n + col;
-      c[o] = dres ? v + dres[o] : v;
+      for (int i = 0; i < NI; i++) red[(wn * NI + i) * 64 + lane] = outv[i];
+    }
+    lds_barrier();
+    if (ks == 0) {
+#pragma unroll
+      for (int i = 0; i < NI; i++) outv[i] += red[(wn * NI + i) * 64 + lane];
     }
   }
+  const bool writer = ks == 0 && n_ok;
+
+  if (g.parts > 1) {
+    // ---- K parts of other workgroups: the last one to arrive adds them up in part order ----
+    // Each XCD has its own L2, so partial tiles travel as device-scope relaxed atomics
+    // (write-through stores, L2-coherent loads); a device-scope fence would write back
+    // and invalidate the whole L2 instead.  The barrier's wait for outstanding stores
+    // orders them before the arrival counter.
+    const size_t plane = (size_t)gridDim.y * ROWS * w.n;  // floats per part
+    float* const mine = g.scratch + (size_t)part * plane + (size_t)row0 * w.n + n;
+    if (writer) {
+#pragma unroll
+      for (int i = 0; i < NI; i++)
+        __hip_atomic_store(mine + (size_t)(8 * (i >> 2) + 4 * gh + (i & 3)) * w.n, outv[i], __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    MGN_GSTAMP(8);
+    __syncthreads();
+    MGN_GSTAMP(9);
+    uint32_t* const flag = (uint32_t*)lds4;
+    if (tid == 0) {
+      uint32_t* ctr = g.counters + blockIdx.y * g.colgroups + cg;
+      const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = seen == g.parts - 1;
+      if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+      *flag = last ? 1u : 0u;
+    }
+    __syncthreads();
+    MGN_GSTAMP(10);
+    if (*flag == 0u) return;
+    if (writer) {
+      // every part comes from memory, this workgroup's own included: NI loads of a part in
+      // flight together, parts added in order
+      const float* const base = g.scratch + (size_t)row0 * w.n + n;
+      float sum[NI];
+#pragma unroll
+      for (int i = 0; i < NI; i++) sum[i] = 0.0f;
+      constexpr int PB = F32A ? 4 : 2;  // parts in flight together
+      for (uint32_t p0 = 0; p0 < g.parts; p0 += PB) {
+        float tmp[PB][NI];
+#pragma unroll
+        for (int j = 0; j < PB; j++) {
+          const uint32_t p = p0 + j < g.parts ? p0 + j : g.parts - 1;
+#pragma unroll
+          for (int i = 0; i < NI; i++)
+            tmp[j][i] = __hip_atomic_load(base + p * plane + (size_t)(8 * (i >> 2) + 4 * gh + (i & 3)) * w.n,
+                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int j = 0; j < PB; j++) {
+          if (p0 + j < g.parts) {
+#pragma unroll
+            for (int i = 0; i < NI; i++) sum[i] += tmp[j][i];
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NI; i++) outv[i] = sum[i];
+    }
+  }
+  if (writer) {
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+      const uint32_t row = row0 + 8 * (i >> 2) + 4 * gh + (i & 3);
+      if (row < g.m) {
+        const size_t o = (size_t)row * w.n + n;
+        g.c[o] = g.dres ? outv[i] + g.dres[o] : outv[i];
+      }
+    }
+  }
+  MGN_GSTAMP(7);
+}
+
+size_t gemm_lds_bytes(int fmt, uint32_t ksc, uint32_t wnc) {
+  const uint32_t cb = 8 * ksc;
+  return std::max<size_t>((size_t)2 * (cb * 2 * 64 + (cb / 2) * 64) * 16 + (size_t)ksc * wnc * 32 * slice_stride(fmt),
+                          (size_t)wnc * 16 * 64 * 4);
 }
 
 struct GemmPlan {
-  uint32_t ksc, wnc, spc, grid_x, grid_y;
-  size_t lds;
+  uint32_t ksc, wnc, tpt, nch, parts, colgroups, grid_y;
+  size_t lds, scratch_bytes;
 };
 
-bool plan_gemm(uint32_t m, uint32_t n, bool f32a, int num_cus, GemmPlan* out) {
+// Picks the workgroup shape and the K split.  The kernel is bound by what a compute
+// unit has to pull in (weights for its columns, activations for its K range), so the
+// model is: rounds of workgroups over the CUs x bytes per workgroup.
+bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
+  const bool f32a = !x.a_is_f16;
   const uint32_t rows = f32a ? 16 : 32;
-  GemmPlan p{};
-  p.grid_y = (m + rows - 1) / rows;
-  if (p.grid_y > 65535) return false;
-  const uint32_t n_tiles = (n + 31) / 32;
-  // K splits: enough waves for ~8 per CU, in powers of two up to 16
-  const uint64_t tiles = (uint64_t)p.grid_y * n_tiles;
-  uint32_t ksc = 1;
-  while (ksc < 16 && tiles * ksc < (uint64_t)num_cus * 8) ksc *= 2;
-  p.ksc = ksc;
-  p.spc = kChunkBlocks / (2 * ksc);
-  // column tiles per workgroup: as many as fit (the activations are staged once per workgroup),
-  // fewer only if that would leave a fifth of the CUs without a workgroup
-  uint32_t wnc = std::min<uint32_t>(16 / ksc, n_tiles);
-  auto groups = [&](uint32_t v) { return (uint64_t)p.grid_y * ((n_tiles + v - 1) / v); };
-  while (wnc > 1 && groups(wnc) * 5 < (uint64_t)num_cus * 4) wnc--;
-  // staging assumes at least 512 threads; waves without a column tile only help staging
-  wnc = std::max<uint32_t>(wnc, (8 + ksc - 1) / ksc);
-  p.wnc = wnc;
-  p.grid_x = (n_tiles + wnc - 1) / wnc;
-  p.lds = (size_t)(kChunkBlocks * 2 * 64 + (kChunkBlocks / 2) * 64) * 16;
-  *out = p;
+  const uint32_t bpc = x.w.k / 32, n_tiles = (x.w.n + 31) / 32;
+  const uint32_t grid_y = (x.m + rows - 1) / rows;
+  if (x.m == 0 || bpc == 0 || grid_y > 65535) return false;
+  const double wblock = x.w.fmt == MGN_FMT_Q4 ? 20.0 * 32 : 34.0 * 32;  // bytes per K block of a column tile
+  const double ablock = rows * 32.0 * (f32a ? 4 : 2);
+  const uint32_t max_tasks = f32a ? 8 : 16;  // staging tasks per chunk per ksc, in units of 64 threads
+  double best = 0;
+  GemmPlan bp{};
+  for (uint32_t ksc = 1; ksc <= 2; ksc++) {
+    const uint32_t cb = 8 * ksc, chunks = (bpc + cb - 1) / cb;
+    // Q8 slices are twice the size: at most 8 waves fit the LDS (and get 256 registers each)
+    for (uint32_t wnc = (x.w.fmt == MGN_FMT_Q8 ? 8 : 16) / ksc; wnc >= 1; wnc--) {
+      const uint32_t tpt = (max_tasks + wnc - 1) / wnc;
+      if (tpt > 4) break;
+      if (gemm_lds_bytes(x.w.fmt, ksc, wnc) > 160 * 1024) continue;
+      if (wnc > n_tiles && wnc * ksc > 8 && wnc > 4) continue;  // idle waves only help staging up to a point
+      const uint32_t colgroups = (n_tiles + wnc - 1) / wnc;
+      for (uint32_t nch = chunks; nch >= 1; nch--) {
+        const uint32_t parts = (chunks + nch - 1) / nch;
+        if ((chunks + parts - 1) / parts != nch) continue;  // same split, already seen
+        const uint64_t wgs = (uint64_t)grid_y * colgroups * parts;
+        const size_t scratch = parts > 1 ? (size_t)parts * grid_y * rows * x.w.n * 4 : 0;
+        if (scratch > x.scratch_bytes || (parts > 1 && (uint64_t)grid_y * colgroups > x.n_counters)) break;
+        if (wgs * 64 * ksc * wnc > (uint64_t)x.num_cus * 4096 && parts > 1) break;  // far more than enough already
+        const double rounds = (double)((wgs + x.num_cus - 1) / x.num_cus);
+        const double per_wg = nch * cb * (std::min(wnc, n_tiles) * wblock + ablock) + 32768.0 +
+                              (parts > 1 ? 2.0 * wnc * 32 * rows * 4 + 16384.0 : 0.0);
+        // few waves hide little latency; a task count that does not divide over the threads
+        // leaves part of the workgroup idle while the rest stages twice
+        const double cost = rounds * per_wg * (ksc * wnc < 8 ? 1.5 : 1.0) * (max_tasks % wnc ? 1.15 : 1.0) * (tpt > 2 ? 1.25 : 1.0);
+        if (best == 0 || cost < best) {
+          best = cost;
+          bp.ksc = ksc, bp.wnc = wnc, bp.tpt = tpt <= 1 ? 1 : tpt <= 2 ? 2 : 4;
+          bp.nch = nch, bp.parts = parts, bp.colgroups = colgroups, bp.grid_y = grid_y;
+          bp.scratch_bytes = scratch;
+        }
+      }
+    }
+  }
+#ifdef MGN_TRACE  // development build only: force a plan, print the chosen one
+  if (const char* dev = getenv("MGN_DEV_GEMM")) {
+    unsigned a = 0, b = 0, c = 0;
+    if (sscanf(dev, "%u,%u,%u", &a, &b, &c) == 3) {
+      const uint32_t cb = 8 * a, chunks = (bpc + cb - 1) / cb;
+      bp.ksc = a, bp.wnc = b, bp.parts = c;
+      bp.nch = (chunks + c - 1) / c;
+      bp.parts = (chunks + bp.nch - 1) / bp.nch;
+      bp.colgroups = (n_tiles + b - 1) / b;
+      const uint32_t tpt = (max_tasks + b - 1) / b;
+      bp.tpt = tpt <= 1 ? 1 : tpt <= 2 ? 2 : 4;
+      bp.grid_y = grid_y;
+      best = 1;
+    }
+  }
+  if (getenv("MGN_DEV_PLAN"))
+    fprintf(stderr, "gemm plan m=%u k=%u n=%u: ksc=%u wnc=%u parts=%u nch=%u tpt=%u wgs=%u\n", x.m, x.w.k, x.w.n, bp.ksc, bp.wnc,
+            bp.parts, bp.nch, bp.tpt, bp.colgroups * bp.parts * bp.grid_y);
+#endif
+  if (best == 0 || (uint64_t)bp.colgroups * bp.parts > 0x7fffffffu) return false;
+  const uint32_t cb = 8 * bp.ksc;
+  bp.lds = gemm_lds_bytes(x.w.fmt, bp.ksc, bp.wnc);
+  *out = bp;
   return true;
 }
 
-template <int FMT, bool F32A, int SPC>
-int launch_spc(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
-  auto kern = gemm_mfma_kernel<FMT, F32A, SPC>;
+template <int FMT, bool F32A, int TPT>
+int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
+  auto kern = gemm_mfma_kernel<FMT, F32A, TPT>;
   static bool big_lds_enabled = false;
   if (!big_lds_enabled) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) return (int)e;
     big_lds_enabled = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.grid_x, p.grid_y), dim3(64 * p.ksc * p.wnc), p.lds, s, x.w, x.a, x.d, x.c, x.m, p.ksc);
+  GemmArgs g{x.w, x.a, x.d, x.c, (float*)x.scratch, x.counters, x.m, p.ksc, p.wnc, p.nch, p.parts, p.colgroups};
+  hipLaunchKernelGGL(kern, dim3(p.colgroups * p.parts, p.grid_y), dim3(64 * p.ksc * p.wnc), p.lds, s, g);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }
@@ -384,23 +600,19 @@ int launch_spc(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
 template <int FMT, bool F32A>
 int launch_fa(ihipStream_t* s, const LaunchArgs& x) {
   GemmPlan p;
-  if (!plan_gemm(x.m, x.w.n, F32A, x.num_cus, &p)) return (int)hipErrorInvalidValue;
-  switch (p.spc) {
-    case 16: return launch_spc<FMT, F32A, 16>(s, x, p);
-    case 8: return launch_spc<FMT, F32A, 8>(s, x, p);
-    case 4: return launch_spc<FMT, F32A, 4>(s, x, p);
-    case 2: return launch_spc<FMT, F32A, 2>(s, x, p);
-    case 1: return launch_spc<FMT, F32A, 1>(s, x, p);
-    default: return (int)hipErrorInvalidValue;
+  if (!plan_gemm(x, &p)) return (int)hipErrorInvalidValue;
+  switch (p.tpt) {
+    case 1: return launch_tpt<FMT, F32A, 1>(s, x, p);
+    case 2: return launch_tpt<FMT, F32A, 2>(s, x, p);
+    default: return launch_tpt<FMT, F32A, 4>(s, x, p);
   }
 }
 
 }  // namespace
 
 bool gemm_mfma_supported(const LaunchArgs& x) {
-  if (x.m == 0) return false;
   GemmPlan p;
-  return plan_gemm(x.m, x.w.n, !x.a_is_f16, x.num_cus, &p);
+  return plan_gemm(x, &p);
 }
 
 int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& x) {

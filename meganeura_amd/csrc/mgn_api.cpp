@@ -106,6 +106,17 @@ mgn_status mgn_ctx_create(int device_id, mgn_ctx** out) {
     mgn_ctx_destroy(ctx);
     return hip_fail(nullptr, "stream/event creation", e);
   }
+  // workspace of the split-K matmul kernels: partial tiles, then 4096 arrival counters
+  constexpr size_t kScratchBytes = (size_t)16 << 20;
+  constexpr uint32_t kCounters = 4096;
+  if ((e = hipMalloc(&ctx->scratch, kScratchBytes + kCounters * sizeof(uint32_t))) != hipSuccess ||
+      (e = hipMemsetAsync((char*)ctx->scratch + kScratchBytes, 0, kCounters * sizeof(uint32_t), ctx->stream)) != hipSuccess) {
+    mgn_ctx_destroy(ctx);
+    return hip_fail(nullptr, "workspace allocation", e);
+  }
+  ctx->scratch_bytes = kScratchBytes;
+  ctx->counters = (uint32_t*)((char*)ctx->scratch + kScratchBytes);
+  ctx->n_counters = kCounters;
   *out = ctx;
   return MGN_OK;
 }
@@ -116,6 +127,7 @@ void mgn_ctx_destroy(mgn_ctx* ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipStreamDestroy(ctx->stream);
   }
+  if (ctx->scratch) (void)hipFree(ctx->scratch);
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
   if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
   delete ctx;
@@ -350,7 +362,8 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   if (c->bytes / 4 < (size_t)m * n) return fail(ctx, MGN_EINVAL, "C is smaller than m*N floats");
   if (d && d->bytes / 4 < (size_t)m * n) return fail(ctx, MGN_EINVAL, "D is smaller than m*N floats");
   if (c->ptr == a->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
-  mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus};
+  mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus,
+                    ctx->scratch,  ctx->scratch_bytes, ctx->counters, ctx->n_counters};
   mgn_route route = ctx->route;
   if (route == MGN_ROUTE_AUTO) {
     if (mgn::gemv_mfma_supported(x)) route = MGN_ROUTE_GEMV_MFMA;

@@ -43,6 +43,11 @@ struct LaunchArgs {
   uint32_t m;
   bool a_is_f16;
   int num_cus;
+  // context-owned workspace for kernels that split K across workgroups
+  void* scratch = nullptr;
+  size_t scratch_bytes = 0;
+  uint32_t* counters = nullptr;  // all zero between launches
+  uint32_t n_counters = 0;
 };
 
 // kernels.hip
@@ -68,6 +73,10 @@ struct mgn_ctx {
   ihipEvent_t* ev_start = nullptr;
   ihipEvent_t* ev_stop = nullptr;
   mgn_route route = MGN_ROUTE_AUTO;
+  void* scratch = nullptr;  // split-K partial results + arrival counters, one allocation
+  size_t scratch_bytes = 0;
+  uint32_t* counters = nullptr;
+  uint32_t n_counters = 0;
   std::string err;
 };
 
