@@ -8,28 +8,33 @@
 // the MFMA operand and the block scale is applied to the accumulators:
 //
 //   v_mfma_f32_32x32x16_f16, wave tile = 32 activation rows x 32 weight columns.
-//   B operand: lane (c, g), c = lane%32, g = lane/32, holds 8 weights of column c:
-//     a lane loads one whole quant block (column c, K block kb0+g: one 128-bit load)
-//     and v_permlane32_swap hands the partner lane the half it needs, so after two
-//     swaps the wave holds, for both K blocks, the k-slices the instruction wants.
-//     Nibbles are masked to fp16 bits 4-7 (n * 2^-20, exact; see the GEMV kernel for
-//     why not bits 0-3), Q8 bytes (q + 128) to bits 0-7.
+//   B operand: lane (c, g), c = lane%32, g = lane/32, holds 8 weights of column c.
+//     The quants come from memory as whole runs of a column's blocks, are parked in a
+//     wave-private LDS slice, and each lane reads back one whole block (column c, K
+//     block 2s+g); v_permlane32_swap hands the partner lane the half it needs, so
+//     after two swaps the wave holds, for both K blocks of a step, the k-slices the
+//     instruction wants.  Nibbles are masked to fp16 bits 4-7 (n * 2^-20, exact; see
+//     the GEMV kernel for why not bits 0-3), Q8 bytes (q + 128) to bits 0-7.
 //   A operand: the activations, re-laid once per workgroup and K chunk into LDS in
 //     exactly the per-lane order the instruction reads (consecutive lanes read
-//     consecutive 16 bytes).  f32 activations are split hi + lo into two fp16 rows
+//     consecutive 16 bytes), double-buffered so the next chunk is staged while this
+//     one is multiplied.  f32 activations are split hi + lo into two fp16 rows
 //     (rows r and r+16 of the tile; the two partial results sit in the same lane
 //     and are added at the end), so a tile carries 16 real rows; fp16 activations
-//     fill all 32 rows.
+//     fill all 32 rows.  f32 activations are not rescaled: |x| must stay below 65504.
 //   Per quant block: two MFMAs (K = 32) into a fresh accumulator D, then
 //     acc += d * D on the vector ALU (16 FMAs per lane).  The format's additive part
 //     (m * sum(x) for Q4, -128 * scale * sum(x) for Q8's byte bias) is one more MFMA
-//     per step that accumulates straight into acc: its A operand is the block's
-//     mean activation (hi, lo), its B operand 32*m taken from the scale|min word.
-//     Adding both parts of a block into the same accumulator within a step keeps
-//     the running sum small even when the two parts are individually large.
+//     per step into a second accumulator: its A operand is the block's mean
+//     activation (hi, lo), its B operand 32*m (or -4096*scale) taken from the scale
+//     word, so |m| < 2048 and scale < 16 are required.  Both accumulators are f32;
+//     their sum is taken once at the end.
 //
-// Work split: grid.y = row tiles; a workgroup owns `wnc` column tiles and splits
-// every 32-block K chunk `ksc` ways among its waves; partial tiles meet in LDS.
+// Work split: grid.y = row tiles; a workgroup owns `wnc` column tiles; K is cut into
+// chunks of 8*ksc blocks which the workgroup walks in order (ksc waves share a chunk),
+// and, when there are too few tiles to fill the chip, into `parts` ranges handled by
+// different workgroups whose partial tiles the last one to finish adds up in part
+// order (deterministic).
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -37,17 +42,19 @@
 #include "kernels_common.hip.h"
 
 #ifdef MGN_TRACE
-// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.
-__device__ unsigned long long* mgn_gemm_trace_ptr = nullptr;
+// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.  The
+// buffer travels as a kernel argument, so a stamp is one clock read and one store.
+static unsigned long long* g_gemm_trace_host = nullptr;
 extern "C" int mgn_debug_set_trace_gemm(void* p) {
-  return (int)hipMemcpyToSymbol(HIP_SYMBOL(mgn_gemm_trace_ptr), &p, sizeof(p));
+  g_gemm_trace_host = (unsigned long long*)p;
+  return 0;
 }
-#define MGN_GSTAMP_INIT() unsigned long long* const trace_base = mgn_gemm_trace_ptr
-#define MGN_GSTAMP(slot)                                                                                \
-  do {                                                                                                  \
-    if (trace_base && (threadIdx.x & 63) == 0)                                                          \
-      trace_base[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 16 + (slot)] = \
-          __builtin_readcyclecounter();                                                                 \
+#define MGN_GSTAMP_INIT()                                                                                  \
+  unsigned long long* const trace_base =                                                                   \
+      g.trace ? g.trace + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 16 : nullptr
+#define MGN_GSTAMP(slot)                                                                  \
+  do {                                                                                    \
+    if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = __builtin_readcyclecounter(); \
   } while (0)
 #else
 #define MGN_GSTAMP_INIT() do {} while (0)
@@ -114,6 +121,9 @@ struct GemmArgs {
   float* scratch;      // [parts][row tiles * ROWS][n] partial results when parts > 1
   uint32_t* counters;  // one arrival counter per (row tile, column group), zero between launches
   uint32_t m, ksc, wnc, nch, parts, colgroups;
+#ifdef MGN_TRACE
+  unsigned long long* trace;
+#endif
 };
 
 template <int FMT>
@@ -133,7 +143,7 @@ __device__ __forceinline__ uint4 f16_operand(uint4 v) {
 // activations are in flight to registers and the weight ring is refilled one chunk ahead.
 // TPT = staging tasks per thread per chunk (one task = 8 consecutive k of one row).
 template <int FMT, bool F32A, int TPT>
-__global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kernel(GemmArgs g) {
+__global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
   constexpr int ROWS = F32A ? 16 : 32;  // real rows per tile
   constexpr int NI = F32A ? 8 : 16;     // result registers per lane
   constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;
@@ -332,9 +342,9 @@ __global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kern
   lds_barrier();
   MGN_GSTAMP(3);
 
-  floatx16 acc;
+  floatx16 acc, acc2;  // scaled quant sums (vector ALU), additive parts (MFMA)
 #pragma unroll
-  for (int i = 0; i < 16; i++) acc[i] = 0.0f;
+  for (int i = 0; i < 16; i++) acc[i] = acc2[i] = 0.0f;
 
   for (uint32_t c = 0; c < g.nch; c++) {
     const uint32_t chunk = chunk0 + c, buf = c & 1;
@@ -344,8 +354,11 @@ __global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kern
     const uint4* const sb = simg + buf * s_stride;
     park_slice();
     fetch_slice(chunk + 1, more);
-#pragma unroll
-    for (int s = 0; s < kSteps; s++) {
+    // Software pipeline over the steps: the MFMAs of step s + 1 are issued before the vector
+    // ALU scales the results of step s, so the matrix cores work through one step while the
+    // ALU finishes the previous one.  The scheduling fences keep the compiler from undoing it.
+    floatx16 dsum[2][2];  // [step parity][block]
+    auto issue_step = [&](int s) {
       const uint32_t lb0 = lb_wave + 2 * s;  // local index of the step's first block
       const uint32_t meta0 = mb[2 * s], meta1 = mb[2 * s + 1];  // block lb0, block lb0 + 1
       half8 bop[2][2];                                            // [block][h]
@@ -372,19 +385,8 @@ __global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kern
         bop[0][1] = bytes_to_operand(r4, r5);
         bop[1][1] = bytes_to_operand(r6, r7);
       }
-#pragma unroll
-      for (int t = 0; t < 2; t++) {
-        floatx16 dsum;
-#pragma unroll
-        for (int i = 0; i < 16; i++) dsum[i] = 0.0f;
-        const uint4* ap = ab + ((lb0 + t) * 2) * 64 + lane;
-        dsum = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ap[0]), bop[t][0], dsum, 0, 0, 0);
-        dsum = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(ap[64]), bop[t][1], dsum, 0, 0, 0);
-        const float dq = half_bits_to_float((t == 0 ? meta0 : meta1) & 0xFFFFu) * kOpScale;
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc[i] = __fmaf_rn(dq, dsum[i], acc[i]);
-      }
-      // additive part of both blocks: mean(x) * (32 * m), straight into acc
+      // additive part of both blocks: mean(x) * (32 * m), into its own accumulator so that this
+      // MFMA chain and the vector ALU's chain never wait for each other
       uint32_t add0, add1;
       if constexpr (FMT == MGN_FMT_Q4) {
         add0 = __builtin_amdgcn_perm(meta0, meta0, 0x07060706u);  // (m, m) of block 0
@@ -400,8 +402,40 @@ __global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kern
         add0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add0) * kb);
         add1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add1) * kb);
       }
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(sb[(lb0 >> 1) * 64 + lane]),
-                                                    as_half8(add0, add1, add0, add1), acc, 0, 0, 0);
+      uint4 aop[2][2];
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const uint4* ap = ab + ((lb0 + t) * 2) * 64 + lane;
+        aop[t][0] = ap[0];
+        aop[t][1] = ap[64];
+      }
+      const uint4 sop = sb[(lb0 >> 1) * 64 + lane];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        floatx16 z;
+#pragma unroll
+        for (int i = 0; i < 16; i++) z[i] = 0.0f;
+        z = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(aop[t][0]), bop[t][0], z, 0, 0, 0);
+        dsum[s & 1][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(aop[t][1]), bop[t][1], z, 0, 0, 0);
+      }
+      acc2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(sop), as_half8(add0, add1, add0, add1), acc2, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto scale_step = [&](int s) {
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        const float dq = half_bits_to_float(mb[2 * s + t] & 0xFFFFu) * kOpScale;
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[i] = __fmaf_rn(dq, dsum[s & 1][t][i], acc[i]);
+      }
+    };
+    issue_step(0);
+#pragma unroll
+    for (int s = 0; s < kSteps; s++) {
+      if (s + 1 < kSteps) issue_step(s + 1);
+      scale_step(s);
+      asm volatile("" : "+v"(acc));  // the scaling stays here, between the two MFMA groups
     }
     if (c == 0) MGN_GSTAMP(4);
     if (more) stage(chunk + 1, buf ^ 1);  // the other buffer was last read before the previous barrier
@@ -415,7 +449,7 @@ __global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kern
   // With f32 activations rows r and r+16 (registers i and i+8) are the hi and lo parts.
   float outv[NI];
 #pragma unroll
-  for (int i = 0; i < NI; i++) outv[i] = F32A ? acc[i] + acc[i + 8] : acc[i];
+  for (int i = 0; i < NI; i++) outv[i] = F32A ? (acc[i] + acc2[i]) + (acc[i + 8] + acc2[i + 8]) : acc[i] + acc2[i];
   if (ksc == 2) {
     if (ks == 1) {
 #pragma unroll
@@ -432,9 +466,9 @@ __global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kern
   if (g.parts > 1) {
     // ---- K parts of other workgroups: the last one to arrive adds them up in part order ----
     // Each XCD has its own L2, so partial tiles travel as device-scope relaxed atomics
-    // (write-through stores, L2-coherent loads); a device-scope fence would write back
-    // and invalidate the whole L2 instead.  The barrier's wait for outstanding stores
-    // orders them before the arrival counter.
+    // (write-through stores, L2-coherent loads), with a single release fence per
+    // workgroup; a fence in every wave plus an acquire on the reading side would write
+    // back and invalidate the whole L2 hundreds of times.
     const size_t plane = (size_t)gridDim.y * ROWS * w.n;  // floats per part
     float* const mine = g.scratch + (size_t)part * plane + (size_t)row0 * w.n + n;
     if (writer) {
@@ -449,6 +483,9 @@ __global__ __launch_bounds__(FMT == MGN_FMT_Q8 ? 512 : 1024) void gemm_mfma_kern
     uint32_t* const flag = (uint32_t*)lds4;
     if (tid == 0) {
       uint32_t* ctr = g.counters + blockIdx.y * g.colgroups + cg;
+      // one device-scope release per workgroup: the barrier above ordered every wave's
+      // stores before it, and it makes them visible to the other XCDs before the count
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
       const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const bool last = seen == g.parts - 1;
       if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
@@ -527,8 +564,8 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
   GemmPlan bp{};
   for (uint32_t ksc = 1; ksc <= 2; ksc++) {
     const uint32_t cb = 8 * ksc, chunks = (bpc + cb - 1) / cb;
-    // Q8 slices are twice the size: at most 8 waves fit the LDS (and get 256 registers each)
-    for (uint32_t wnc = (x.w.fmt == MGN_FMT_Q8 ? 8 : 16) / ksc; wnc >= 1; wnc--) {
+    // at most 8 waves: each gets 256 registers, and Q8 slices of more would not fit the LDS
+    for (uint32_t wnc = 8 / ksc; wnc >= 1; wnc--) {
       const uint32_t tpt = (max_tasks + wnc - 1) / wnc;
       if (tpt > 4) break;
       if (gemm_lds_bytes(x.w.fmt, ksc, wnc) > 160 * 1024) continue;
@@ -592,6 +629,9 @@ int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
     big_lds_enabled = true;
   }
   GemmArgs g{x.w, x.a, x.d, x.c, (float*)x.scratch, x.counters, x.m, p.ksc, p.wnc, p.nch, p.parts, p.colgroups};
+#ifdef MGN_TRACE
+  g.trace = g_gemm_trace_host;
+#endif
   hipLaunchKernelGGL(kern, dim3(p.colgroups * p.parts, p.grid_y), dim3(64 * p.ksc * p.wnc), p.lds, s, g);
   MGN_HIP_LAUNCH_CHECK();
   return 0;

@@ -177,3 +177,36 @@ def test_linearity_and_zero_input(ctx):
     fxy = run_matmul(ctx, Q4, x + y, wt)
     assert np.abs(fxy - (fx + fy)).max() < 2e-4
     wt.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+def test_split_k_is_repeatable(ctx, orc, fmt):
+    """Few tiles and a long K: the tiled kernel splits K across workgroups and the last
+    one to arrive adds the partial tiles in part order.  Alternating two inputs makes a
+    partial tile left over from the previous call wrong for this one, so a stale read
+    shows; the result must also be the same bits every time."""
+    m, k, n = 16, 4096, 2048
+    w = synth.normal(91 + fmt, k * n, 0.02).reshape(k, n)
+    wt = ctx.weight(fmt, w)
+    packed = orc.quantize(fmt, w)
+    xs = [synth.normal(92 + i, m * k, 1.0).reshape(m, k) for i in range(2)]
+    bufs = [ctx.upload(x) for x in xs]
+    c = ctx.buffer(m * n * 4)
+    ctx.set_route(capi.ROUTE_GEMM_MFMA)
+    try:
+        first = []
+        for i in range(2):
+            ctx.matmul_q(bufs[i], wt, c, m, None)
+            first.append(c.download(np.float32, m * n).reshape(m, n))
+            orc.assert_close(first[i], orc.matmul_packed(fmt, xs[i], packed, n), REL, ABS)
+        for it in range(40):
+            i = it & 1
+            ctx.matmul_q(bufs[i], wt, c, m, None)
+            got = c.download(np.float32, m * n).reshape(m, n)
+            assert (bits(got) == bits(first[i])).all(), f"call {it} differs from the first call with the same input"
+    finally:
+        ctx.set_route(capi.ROUTE_AUTO)
+        for b in bufs:
+            b.free()
+        c.free()
+        wt.free()
