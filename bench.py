@@ -56,8 +56,12 @@ WORKLOADS = {
 HEADLINE = "c5_q4_m1_4096x14336"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
-# same counters read for a 256 MiB device copy (profiles/gemv_mfma_q4_m1_4096x14336.md).
-MEASURED_TRAFFIC_BYTES = {"c5_q4_m1_4096x14336": 37.02e6}
+# same counters read for a 256 MiB device copy (one summary per workload under profiles/).
+MEASURED_TRAFFIC_BYTES = {
+    "c5_q4_m1_4096x14336": 37.02e6,
+    "c5_q4_m16_4096x14336": 48.4e6,
+    "c4_q4_prefill_up_512x1024x3072": 18.8e6,
+}
 
 
 def algorithmic_bytes(fmt, m, k, n, resid, f16):
@@ -205,7 +209,7 @@ def main():
 
     if is_gemm:
         roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": tflops / MFMA_F16_PEAK_TFLOPS, "traffic": None}
+                "frac": tflops / MFMA_F16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
     else:
         roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
