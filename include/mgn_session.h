@@ -82,6 +82,13 @@ mgn_status mgn_session_set_input(mgn_session* s, const char* name, const float* 
 /* Session::step / wait (src/runtime.rs:2843-2959, 2835-2841). */
 mgn_status mgn_session_step(mgn_session* s);
 mgn_status mgn_session_wait(mgn_session* s);
+/* The reference records a step's dispatches into one command buffer and submits it once
+ * (src/runtime.rs:2843-2959).  Here a step is captured into one HIP graph the second time it
+ * runs after the weights were set and replayed from then on; `enable = 0` keeps every step as
+ * individual launches.  On by default.  mgn_session_graph_active reports whether the next
+ * step will be a graph replay (1) or individual launches (0). */
+mgn_status mgn_session_set_graph_replay(mgn_session* s, int enable);
+int mgn_session_graph_active(const mgn_session* s);
 /* Session::read_output / read_output_by_index (src/runtime.rs:2612-2638). */
 mgn_status mgn_session_read_output(mgn_session* s, float* out, size_t len);
 mgn_status mgn_session_read_output_by_index(mgn_session* s, size_t index, float* out, size_t len);

@@ -31,7 +31,8 @@ SESSION_SYMBOLS = [
     "mgn_build_inference_session", "mgn_session_free", "mgn_session_last_error",
     "mgn_session_num_dispatches", "mgn_session_dispatch_info", "mgn_session_set_parameter",
     "mgn_session_set_input", "mgn_session_step", "mgn_session_wait", "mgn_session_read_output",
-    "mgn_session_read_output_by_index", "mgn_session_ctx",
+    "mgn_session_read_output_by_index", "mgn_session_ctx", "mgn_session_set_graph_replay",
+    "mgn_session_graph_active",
 ]
 
 
@@ -119,6 +120,8 @@ def load():
         "mgn_session_read_output": (C.c_int, [vp, vp, sz]),
         "mgn_session_read_output_by_index": (C.c_int, [vp, sz, vp, sz]),
         "mgn_session_ctx": (vp, [vp]),
+        "mgn_session_set_graph_replay": (C.c_int, [vp, C.c_int]),
+        "mgn_session_graph_active": (C.c_int, [vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -167,15 +170,25 @@ class Context:
         if st != OK:
             raise MgnError(st, self.lib.mgn_last_error(None).decode())
         self.h = h
+        self.owned = True
+
+    @classmethod
+    def borrowed(cls, handle):
+        """View of a context owned by someone else (a session's): never destroyed here."""
+        self = cls.__new__(cls)
+        self.lib = load()
+        self.h = C.c_void_p(handle)
+        self.owned = False
+        return self
 
     def check(self, st):
         if st != OK:
             raise MgnError(st, self.lib.mgn_last_error(self.h).decode())
 
     def close(self):
-        if self.h:
+        if self.h and self.owned:
             self.lib.mgn_ctx_destroy(self.h)
-            self.h = None
+        self.h = None
 
     def __enter__(self):
         return self

@@ -45,17 +45,30 @@
 #include "kernels_common.hip.h"
 
 #ifdef MGN_TRACE
-// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.
-__device__ unsigned long long* mgn_trace_ptr = nullptr;
+// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.  The
+// buffer travels as a kernel argument, so a stamp is one clock read and one store.
+static unsigned long long* g_gemv_trace_host = nullptr;
 extern "C" int mgn_debug_set_trace(void* p) {
-  return (int)hipMemcpyToSymbol(HIP_SYMBOL(mgn_trace_ptr), &p, sizeof(p));
+  g_gemv_trace_host = (unsigned long long*)p;
+  return 0;
 }
+#define MGN_TRACE_PARAM , unsigned long long* trace_arg
+#define MGN_TRACE_ARG , g_gemv_trace_host
+#define MGN_STAMP_INIT() \
+  unsigned long long* const trace_base = trace_arg ? trace_arg + ((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 16 : nullptr
 #define MGN_STAMP(slot)                                                                          \
   do {                                                                                           \
-    if (mgn_trace_ptr && (threadIdx.x & 63) == 0)                                                \
-      mgn_trace_ptr[((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 16 + (slot)] = __builtin_readcyclecounter(); \
+    if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = __builtin_readcyclecounter();   \
+  } while (0)
+#define MGN_STAMP_WALL(slot)                                                        \
+  do {                                                                             \
+    if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = wall_clock64();  \
   } while (0)
 #else
+#define MGN_STAMP_WALL(slot) do {} while (0)
+#define MGN_TRACE_PARAM
+#define MGN_TRACE_ARG
+#define MGN_STAMP_INIT() do {} while (0)
 #define MGN_STAMP(slot) do {} while (0)
 #endif
 
@@ -171,7 +184,7 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 template <int FMT, int MROWS, int STEPS>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const float* __restrict__ a,
                                                          const float* __restrict__ dres, float* __restrict__ c,
-                                                         uint32_t m, uint32_t ksc) {
+                                                         uint32_t m, uint32_t ksc MGN_TRACE_PARAM) {
   constexpr int NJ = 2 * MROWS;
   extern __shared__ uint4 lds4[];
   const uint32_t bpc = w.k / 32;
@@ -182,7 +195,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   float2* cinit = (float2*)(lds4 + 4 * plane);        // [bpc_pad][MROWS]
   float* red = (float*)(cinit + bpc_pad * MROWS);     // [wnc][ksc][MROWS][4]
 
+  MGN_STAMP_INIT();
   MGN_STAMP(0);
+  MGN_STAMP_WALL(13);
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   // everything derived from the wave index is wave-uniform: keep it in scalar registers
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -344,6 +359,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
       }
     }
     MGN_STAMP(12);
+    MGN_STAMP_WALL(14);
     return;
   }
 #pragma unroll
@@ -366,6 +382,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
     }
   }
   MGN_STAMP(12);
+  MGN_STAMP_WALL(14);
 }
 
 struct MfmaGemvPlan {
@@ -415,7 +432,7 @@ int launch_steps(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
     big_lds_enabled = true;
   }
   hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, x.w, (const float*)x.a, x.d, x.c, x.m,
-                     p.ksc);
+                     p.ksc MGN_TRACE_ARG);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

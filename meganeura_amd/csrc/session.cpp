@@ -336,6 +336,7 @@ Session::~Session() { release(); }
 void Session::release() {
   if (!ctx_) return;
   (void)mgn_sync(ctx_);  // Drop waits for the GPU first (src/runtime.rs:4339-4345)
+  drop_graph();
   for (mgn_buf* b : buffers_) mgn_buf_free(ctx_, b);
   for (mgn_weight* w : weights_) mgn_weight_free(ctx_, w);
   buffers_.clear();
@@ -348,6 +349,7 @@ void Session::upload_weight(int buf, const WeightBufferInfo& info, const float* 
   mgn_weight* fresh = nullptr;
   const mgn_fmt fmt = info.fmt == WeightFormat::Q4 ? MGN_FMT_Q4 : MGN_FMT_Q8;
   check(mgn_weight_create(ctx_, fmt, data, info.rows, info.cols, &fresh), "mgn_weight_create");
+  drop_graph();  // a captured step holds the old handle's addresses
   mgn_weight_free(ctx_, weights_[buf]);  // waits for in-flight work that may still read it
   weights_[buf] = fresh;
 }
@@ -411,7 +413,66 @@ void Session::set_input(const std::string& name, const float* data, size_t len) 
 
 // src/runtime.rs:2843-2959: replay the dispatch list on the stream; returns after
 // submission.  Stream order stands in for the barriers between dependency groups.
+// src/runtime.rs:2843-2959 submits the whole plan as one command buffer; the equivalent here
+// is one captured graph.  Kernel nodes only: nothing on this path records a memset.
 void Session::step() {
+  if (exec_) {
+    hipError_t e = hipGraphLaunch(exec_, ctx_->stream);
+    if (e != hipSuccess) throw std::runtime_error(std::string("hipGraphLaunch: ") + hipGetErrorString(e));
+    return;
+  }
+  if (!graph_wanted_ || eager_steps_ == 0) {
+    // the first step also lets every kernel variant do its one-time attribute setup
+    run_dispatches();
+    eager_steps_++;
+    return;
+  }
+  hipError_t e = hipStreamBeginCapture(ctx_->stream, hipStreamCaptureModeThreadLocal);
+  if (e != hipSuccess) {
+    graph_wanted_ = false;
+    run_dispatches();
+    return;
+  }
+  std::exception_ptr failure;
+  try {
+    run_dispatches();
+  } catch (...) {
+    failure = std::current_exception();
+  }
+  e = hipStreamEndCapture(ctx_->stream, &graph_);
+  if (failure) {
+    drop_graph();
+    graph_wanted_ = false;
+    std::rethrow_exception(failure);
+  }
+  if (e == hipSuccess) e = hipGraphInstantiate(&exec_, graph_, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    // capture is an optimisation: fall back to plain launches for good
+    (void)hipGetLastError();
+    drop_graph();
+    graph_wanted_ = false;
+    run_dispatches();
+    return;
+  }
+  e = hipGraphLaunch(exec_, ctx_->stream);
+  if (e != hipSuccess) throw std::runtime_error(std::string("hipGraphLaunch: ") + hipGetErrorString(e));
+}
+
+void Session::set_graph_replay(bool on) {
+  graph_wanted_ = on;
+  if (!on) drop_graph();
+}
+
+void Session::drop_graph() {
+  if (exec_ || graph_) (void)mgn_sync(ctx_);
+  if (exec_) (void)hipGraphExecDestroy(exec_);
+  if (graph_) (void)hipGraphDestroy(graph_);
+  exec_ = nullptr;
+  graph_ = nullptr;
+  eager_steps_ = 0;
+}
+
+void Session::run_dispatches() {
   for (const Dispatch& d : plan_.dispatches) {
     float* out = (float*)buffers_[d.output_buffer]->ptr;
     auto fin = [&](size_t i) { return (const float*)buffers_[d.input_buffers[i]]->ptr; };
@@ -618,6 +679,10 @@ mgn_status mgn_session_set_input(mgn_session* s, const char* name, const float* 
 }
 mgn_status mgn_session_step(mgn_session* s) { return session_call(s, [&] { s->s->step(); }); }
 mgn_status mgn_session_wait(mgn_session* s) { return session_call(s, [&] { s->s->wait(); }); }
+mgn_status mgn_session_set_graph_replay(mgn_session* s, int enable) {
+  return session_call(s, [&] { s->s->set_graph_replay(enable != 0); });
+}
+int mgn_session_graph_active(const mgn_session* s) { return s && s->s && s->s->graph_active() ? 1 : 0; }
 mgn_status mgn_session_read_output(mgn_session* s, float* out, size_t len) {
   if (!out) return MGN_EINVAL;
   return session_call(s, [&] { s->s->read_output(out, len); });

@@ -9,6 +9,9 @@
 #include <vector>
 
 #include "mgn_internal.h"
+
+struct ihipGraph;
+struct hipGraphExec;
 #include "../../include/mgn_session.h"
 
 namespace mgn {
@@ -138,6 +141,11 @@ class Session {
   void set_parameter(const std::string& name, const float* data, size_t len);
   void set_input(const std::string& name, const float* data, size_t len);
   void step();
+  // Replay steps as one captured HIP graph (default on): the first step after the set of
+  // weight handles changed runs launch by launch, the next one is captured, later ones
+  // are a single graph launch.  Results are identical; only launch overhead changes.
+  void set_graph_replay(bool on);
+  bool graph_active() const { return exec_ != nullptr; }
   void wait();
   void read_output(float* out, size_t len) { read_output_by_index(0, out, len); }
   void read_output_by_index(size_t index, float* out, size_t len);
@@ -147,11 +155,17 @@ class Session {
   void upload_weight(int buf, const WeightBufferInfo& info, const float* data);
   void check(mgn_status st, const char* what);
   void release();
+  void run_dispatches();
+  void drop_graph();
   ExecutionPlan plan_;
   mgn_ctx* ctx_ = nullptr;
   std::vector<mgn_buf*> buffers_;        // f32 buffers (null for quantized params)
   std::vector<mgn_weight*> weights_;     // quantized params (null otherwise)
   std::map<int, std::vector<float>> weight_staging_;  // src/runtime.rs:2373-2376
+  bool graph_wanted_ = true;
+  int eager_steps_ = 0;  // launch-by-launch steps since the weight handles last changed
+  ihipGraph* graph_ = nullptr;    // hipGraph_t
+  hipGraphExec* exec_ = nullptr;  // hipGraphExec_t
 };
 
 // build_inference_session (src/train.rs:380-389): optimize -> compile -> Session.

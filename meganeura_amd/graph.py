@@ -149,6 +149,17 @@ class Session:
     def wait(self):
         self._check(self.lib.mgn_session_wait(self.h))
 
+    def set_graph_replay(self, enable):
+        """Steps replay one captured HIP graph (default) or launch dispatch by dispatch."""
+        self._check(self.lib.mgn_session_set_graph_replay(self.h, 1 if enable else 0))
+
+    def graph_active(self):
+        return bool(self.lib.mgn_session_graph_active(self.h))
+
+    def context(self):
+        """The session's context as a capi.Context view (timers, sync); not owned."""
+        return capi.Context.borrowed(self.lib.mgn_session_ctx(self.h))
+
     def read_output(self, length):
         out = np.empty(length, dtype=np.float32)
         self._check(self.lib.mgn_session_read_output(self.h, out.ctypes.data_as(C.c_void_p), length))

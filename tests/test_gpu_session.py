@@ -162,3 +162,74 @@ def test_f32_weight_matmul_is_refused():
     g.set_outputs([g.matmul(a, b)])
     with pytest.raises(capi.MgnError, match="quantized path"):
         build_inference_session(g)
+
+
+def _decode_layer_graph(hidden, inter, fmt_param):
+    """SmolLM2-style decode layer without the attention core (models/smollm2.rs:340-414):
+    norm -> q/k/v projections; o-projection + residual; norm -> gate, up -> swiglu -> down + residual."""
+    g = Graph()
+    x = g.input("x", [1, hidden])
+    attn = g.input("attn", [1, hidden])
+    n1 = g.rms_norm(x, g.parameter("norm1", [hidden]), 1e-5)
+    q = g.matmul(n1, fmt_param(g, "wq", [hidden, hidden]))
+    kk = g.matmul(n1, fmt_param(g, "wk", [hidden, hidden // 3]))
+    v = g.matmul(n1, fmt_param(g, "wv", [hidden, hidden // 3]))
+    h = g.add(g.matmul(attn, fmt_param(g, "wo", [hidden, hidden])), x)
+    n2 = g.rms_norm(h, g.parameter("norm2", [hidden]), 1e-5)
+    gate = g.matmul(n2, fmt_param(g, "wg", [hidden, inter]))
+    up = g.matmul(n2, fmt_param(g, "wu", [hidden, inter]))
+    out = g.add(g.matmul(g.swiglu(gate, up), fmt_param(g, "wd", [inter, hidden])), h)
+    g.set_outputs([out, q, kk, v])
+    return g
+
+
+def test_graph_replay_matches_individual_launches(orc):
+    """A step replayed as one captured HIP graph gives the same bits as the same step
+    launched dispatch by dispatch: replayed several times, with fresh inputs, eager work and
+    synchronisation in between."""
+    hidden, inter = 576, 1536
+    g = _decode_layer_graph(hidden, inter, lambda gr, name, shape: gr.parameter_q4(name, shape))
+    sess = build_inference_session(g)
+    shapes = {"wq": (hidden, hidden), "wk": (hidden, hidden // 3), "wv": (hidden, hidden // 3), "wo": (hidden, hidden),
+              "wg": (hidden, inter), "wu": (hidden, inter), "wd": (inter, hidden)}
+    for i, (name, (k, n)) in enumerate(shapes.items()):
+        sess.set_parameter(name, synth.normal(300 + i, k * n, 0.02))
+    sess.set_parameter("norm1", 1.0 + 0.1 * synth.normal(310, hidden, 1.0))
+    sess.set_parameter("norm2", 1.0 + 0.1 * synth.normal(311, hidden, 1.0))
+    sizes = [hidden, hidden, hidden // 3, hidden // 3]
+
+    def run(seed):
+        sess.set_input("x", synth.normal(seed, hidden, 1.0))
+        sess.set_input("attn", synth.normal(seed + 1000, hidden, 1.0))
+        sess.step()
+        sess.wait()
+        return [sess.read_output_by_index(i, n) for i, n in enumerate(sizes)]
+
+    sess.set_graph_replay(False)
+    want = {seed: run(seed) for seed in (1, 2, 3)}
+    assert not sess.graph_active()
+    sess.set_graph_replay(True)
+    run(2)                      # every kernel has run before: captured right away
+    assert sess.graph_active()
+    scratch = capi.Context(0)   # unrelated eager work on the same device between replays
+    for it in range(9):
+        seed = 1 + it % 3
+        got = run(seed)
+        for a, b in zip(got, want[seed]):
+            assert (a.view(np.uint32) == b.view(np.uint32)).all(), f"replay {it} differs from the eager step"
+        buf = scratch.upload(synth.normal(50 + it, 4096, 1.0))
+        scratch.sync()
+        buf.free()
+    scratch.close()
+    # a new weight invalidates the captured step; the next steps run eagerly, then re-capture
+    sess.set_parameter("wq", synth.normal(400, hidden * hidden, 0.02))
+    assert not sess.graph_active()
+    first = run(1)              # launch by launch
+    assert not sess.graph_active()
+    second = run(1)             # captured here
+    assert sess.graph_active()
+    third = run(1)
+    for a, b, c in zip(first, second, third):
+        assert (a.view(np.uint32) == b.view(np.uint32)).all() and (a.view(np.uint32) == c.view(np.uint32)).all()
+    assert (first[0].view(np.uint32) != want[1][1].view(np.uint32)).any()  # q really uses the new weight
+    sess.close()
