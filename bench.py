@@ -125,6 +125,55 @@ class Workload:
             self.d.free()
 
 
+def decode_layer_times(steps, warmup):
+    """C2 as the reference runs it: one SmolLM2-135M decode layer's matmuls through the
+    Graph/Session surface (models/smollm2.rs:340-414 without the attention core): rms_norm,
+    q/k/v, o-projection + residual, rms_norm, gate||up as one fused matmul, SwiGLU, down +
+    residual -- 9 dispatches after the optimizer's fusions.  Returns microseconds per layer
+    step, launched dispatch by dispatch and replayed as one captured graph."""
+    from meganeura_amd import capi, synth
+    from meganeura_amd.graph import Graph, build_inference_session
+
+    hidden, kv, inter = 576, 192, 1536
+    g = Graph()
+    x = g.input("x", [1, hidden])
+    attn = g.input("attn", [1, hidden])
+    n1 = g.rms_norm(x, g.parameter("norm1", [hidden]), 1e-5)
+    q = g.matmul(n1, g.parameter_q4("wq", [hidden, hidden]))
+    k = g.matmul(n1, g.parameter_q4("wk", [hidden, kv]))
+    v = g.matmul(n1, g.parameter_q4("wv", [hidden, kv]))
+    h = g.add(g.matmul(attn, g.parameter_q4("wo", [hidden, hidden])), x)
+    n2 = g.rms_norm(h, g.parameter("norm2", [hidden]), 1e-5)
+    gate = g.matmul(n2, g.parameter_q4("wg", [hidden, inter]))
+    up = g.matmul(n2, g.parameter_q4("wu", [hidden, inter]))
+    out = g.add(g.matmul(g.swiglu(gate, up), g.parameter_q4("wd", [inter, hidden])), h)
+    g.set_outputs([out, q, k, v])
+    sess = build_inference_session(g)
+    shapes = {"wq": (hidden, hidden), "wk": (hidden, kv), "wv": (hidden, kv), "wo": (hidden, hidden),
+              "wg": (hidden, inter), "wu": (hidden, inter), "wd": (inter, hidden)}
+    for i, (name, (kk, nn)) in enumerate(shapes.items()):
+        sess.set_parameter(name, synth.weights(2, kk, nn, which=i))
+    sess.set_parameter("norm1", np.ones(hidden, np.float32))
+    sess.set_parameter("norm2", np.ones(hidden, np.float32))
+    sess.set_input("x", synth.activations(2, 1, hidden, which=0))
+    sess.set_input("attn", synth.activations(2, 1, hidden, which=1))
+    ctx = sess.context()
+    res = {"dispatches": len(sess.plan())}
+    for label, replay in (("launches", False), ("graph", True)):
+        sess.set_graph_replay(replay)
+        for _ in range(warmup + 2):
+            sess.step()
+        ctx.sync()
+        ctx.timer_start()
+        for _ in range(steps):
+            sess.step()
+        ms = ctx.timer_stop()
+        ctx.sync()
+        res[label + "_us_per_layer"] = ms * 1e3 / steps
+    sess.close()
+    return res
+
+
 def cpu_baseline(wl, budget_s=20.0):
     """The reference's tiled dequant-on-load algorithm restated for the CPU
     (oracle/mgn_oracle.c: orc_matmul_q_tiled), one OpenMP task per workgroup, on
@@ -257,6 +306,9 @@ def main():
             row["cold_pct_hbm"] = 100.0 * row["cold_GBs"] / HBM_PEAK_GBS
             rows.append(row)
             print(json.dumps(row), file=sys.stderr, flush=True)
+        layer = {"workload": "c2_q4_decode_layer_session", **decode_layer_times(max(50, args.steps // 2), args.warmup)}
+        rows.append(layer)
+        print(json.dumps(layer), file=sys.stderr, flush=True)
         out_dir = os.path.join(ROOT, "gpurun_out")
         if os.path.isdir(out_dir):
             with open(os.path.join(out_dir, "bench_sweep.json"), "w") as f:

@@ -141,9 +141,10 @@ class Session {
   void set_parameter(const std::string& name, const float* data, size_t len);
   void set_input(const std::string& name, const float* data, size_t len);
   void step();
-  // Replay steps as one captured HIP graph (default on): the first step after the set of
-  // weight handles changed runs launch by launch, the next one is captured, later ones
-  // are a single graph launch.  Results are identical; only launch overhead changes.
+  // Replay steps as one captured HIP graph (off by default): the first step after the set
+  // of weight handles changed runs launch by launch, the next one is captured, later ones
+  // are a single graph launch.  Results are identical; only launch overhead changes --
+  // less host work per step, but measured slower on the GPU side for chains of tiny kernels.
   void set_graph_replay(bool on);
   bool graph_active() const { return exec_ != nullptr; }
   void wait();
@@ -162,7 +163,7 @@ class Session {
   std::vector<mgn_buf*> buffers_;        // f32 buffers (null for quantized params)
   std::vector<mgn_weight*> weights_;     // quantized params (null otherwise)
   std::map<int, std::vector<float>> weight_staging_;  // src/runtime.rs:2373-2376
-  bool graph_wanted_ = true;
+  bool graph_wanted_ = false;
   int eager_steps_ = 0;  // launch-by-launch steps since the weight handles last changed
   ihipGraph* graph_ = nullptr;    // hipGraph_t
   hipGraphExec* exec_ = nullptr;  // hipGraphExec_t

@@ -224,6 +224,7 @@ def test_graph_replay_matches_individual_launches(orc):
     # a new weight invalidates the captured step; the next steps run eagerly, then re-capture
     sess.set_parameter("wq", synth.normal(400, hidden * hidden, 0.02))
     assert not sess.graph_active()
+    sess.set_graph_replay(True)
     first = run(1)              # launch by launch
     assert not sess.graph_active()
     second = run(1)             # captured here
