@@ -40,8 +40,6 @@
 // of a column are summed once per column quad.  The activations' A operands
 // are prepared once per workgroup in LDS, laid out so that consecutive lanes
 // read consecutive 16-byte chunks.
-#include <cstdlib>
-
 #include "kernels_common.hip.h"
 
 #ifdef MGN_TRACE
@@ -181,7 +179,9 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 // STEPS block loads up front and then runs straight-line code: with no branch around a
 // load the compiler's wait counts are exact, so step s starts as soon as its own block
 // has arrived while the later ones are still in flight.
-template <int FMT, int MROWS, int STEPS>
+// QPW > 1 (short K, many columns): a wave takes QPW consecutive quads, so that it still has
+// QPW * STEPS block loads to keep in flight and the workgroup count stays near the CU count.
+template <int FMT, int MROWS, int STEPS, int QPW>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const float* __restrict__ a,
                                                          const float* __restrict__ dres, float* __restrict__ c,
                                                          uint32_t m, uint32_t ksc MGN_TRACE_PARAM) {
@@ -203,9 +203,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t ks = wave % ksc, wn = wave / ksc;
   const uint32_t b = lane >> 2, i = lane & 3;
-  const uint32_t quad0 = blockIdx.x * wnc;
+  const uint32_t quad0 = blockIdx.x * wnc * QPW;
   const uint32_t nquads = (w.n + 3) / 4;
-  const uint32_t quad = quad0 + wn;
+  const uint32_t quad = quad0 + wn * QPW;  // first of this wave's QPW quads
   const uint32_t steps_total = bpc_pad / 16;
   const uint32_t step_begin = ks * STEPS;
   // a wave past the last K step (or past the last quad) keeps running on the zero block:
@@ -236,15 +236,17 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   // Weight blocks: kDepth loads run ahead of the step that consumes them.  That is enough
   // to keep the memory system busy; issuing every load up front would only park the wave
   // in the load queue (which drains at HBM speed) before it could prepare any activations.
-  Raw<FMT> blk[STEPS];
+  // load t = q * STEPS + s: K step s of the wave's quad q
+  constexpr int TS = STEPS * QPW;
+  Raw<FMT> blk[TS];
   const uint32_t wbase = (quad * 4 + i) * bpc + kb_first;
-  const bool n_ok = wave_live && quad * 4 + i < w.n;
-  auto fetch = [&](int s) {
-    const bool ok = n_ok && step_begin + s < steps_total && kb_first + s * 16 < bpc;
-    blk[s].load(w, ok ? wbase + s * 16 : zero_block);
+  auto fetch = [&](int t) {
+    const int q = t / STEPS, s = t % STEPS;
+    const bool ok = wave_live && (quad + q) * 4 + i < w.n && step_begin + s < steps_total && kb_first + s * 16 < bpc;
+    blk[t].load(w, ok ? wbase + q * 4 * bpc + s * 16 : zero_block);
   };
 #pragma unroll
-  for (int s = 0; s < STEPS && s < kDepth; s++) fetch(s);
+  for (int t = 0; t < TS && t < kDepth; t++) fetch(t);
   for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += blockDim.x) red[t] = 0.0f;
   MGN_STAMP(1);
 
@@ -288,15 +290,18 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   // in LDS) and the D entries they produce are never looked at.
   const char* xa_lane = (const char*)xa + ((kb_first * NJ) + (i % NJ)) * 16;
   const char* ci_lane = (const char*)cinit + kb_first * MROWS * 8;
-  float acc[MROWS];  // lane (b, j): sum over this lane's K blocks for column 4*quad+j, per row
+  float acc[QPW][MROWS];  // lane (b, j): sum over this lane's K blocks for column 4*(quad+q)+j, per row
 #pragma unroll
-  for (int r = 0; r < MROWS; r++) acc[r] = 0.0f;
+  for (int q = 0; q < QPW; q++)
 #pragma unroll
-  for (int s = 0; s < STEPS; s++) {
+    for (int r = 0; r < MROWS; r++) acc[q][r] = 0.0f;
+#pragma unroll
+  for (int t = 0; t < TS; t++) {
+    const int s = t % STEPS, q = t / STEPS;
     // steps past the end of K multiply the zero block; keep their LDS reads in range
     const uint32_t so = (step_begin + s < steps_total) ? (uint32_t)s : 0u;
-    if (s + kDepth < STEPS) fetch(s + kDepth);
-    const Raw<FMT>& cur = blk[s];
+    if (t + kDepth < TS) fetch(t + kDepth);
+    const Raw<FMT>& cur = blk[t];
     // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks
     uint4 ax[4];
 #pragma unroll
@@ -340,22 +345,25 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
         const float mneg = __fmaf_rn(-0.125f, half_bits_to_float(cur.meta >> 16), -dscale);
         v = __fmaf_rn(mneg, ci[r].x, v);
       }
-      acc[r] = __fmaf_rn(v, ci[r].y, acc[r]);
+      acc[q][r] = __fmaf_rn(v, ci[r].y, acc[q][r]);
     }
-    if (s == 0) MGN_STAMP(7);
-    if (s == 3) MGN_STAMP(8);
+    if (t == 0) MGN_STAMP(7);
+    if (t == 3) MGN_STAMP(8);
   }
   MGN_STAMP(9);
   // ---- sum the 16 lanes of each column ----
-  if (ksc == 1) {
-    // no K split: lanes 0..3 hold the four finished columns of this wave's quad
+  if (QPW > 1 || ksc == 1) {
+    // no K split (always the case with QPW > 1): lanes 0..3 hold the four finished columns of a quad
 #pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      const float tot = sum_over_blocks(acc[r]);
-      const uint32_t n = quad * 4 + lane;
-      if (lane < 4 && wave_live && (uint32_t)r < m && n < w.n) {
-        const size_t o = (size_t)r * w.n + n;
-        c[o] = dres ? tot + dres[o] : tot;
+    for (int q = 0; q < QPW; q++) {
+#pragma unroll
+      for (int r = 0; r < MROWS; r++) {
+        const float tot = sum_over_blocks(acc[q][r]);
+        const uint32_t n = (quad + q) * 4 + lane;
+        if (lane < 4 && wave_live && (uint32_t)r < m && n < w.n) {
+          const size_t o = (size_t)r * w.n + n;
+          c[o] = dres ? tot + dres[o] : tot;
+        }
       }
     }
     MGN_STAMP(12);
@@ -364,7 +372,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   }
 #pragma unroll
   for (int r = 0; r < MROWS; r++) {
-    const float tot = sum_over_blocks(acc[r]);
+    const float tot = sum_over_blocks(acc[0][r]);
     if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot;
   }
   MGN_STAMP(10);
@@ -386,7 +394,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
 }
 
 struct MfmaGemvPlan {
-  uint32_t ksc, wnc, steps, grid;
+  uint32_t ksc, wnc, steps, qpw, grid;
   size_t lds;
 };
 
@@ -405,16 +413,21 @@ bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, MfmaGem
   while (ksc < 16 && nquads * ksc < want_waves && (steps_total + ksc) / (ksc + 1) >= 2) ksc++;
   p.steps = (steps_total + ksc - 1) / ksc;
   p.ksc = (steps_total + p.steps - 1) / p.steps;  // drop splits that would get no step
-  // quads per workgroup: spread the quads evenly over the CUs (one workgroup per CU when
+  // quads per wave: with a short K and very many columns a wave takes several quads, as
+  // long as that leaves at least 8 waves per CU
+  p.qpw = 1;
+  if (p.ksc == 1)
+    while (p.qpw < 4 && p.steps * p.qpw * 2 <= kMaxSteps && nquads / (p.qpw * 2) >= (uint32_t)num_cus * 8) p.qpw *= 2;
+  // waves per workgroup: spread the quads evenly over the CUs (one workgroup per CU when
   // there is enough work), so the activations are prepared as few times as possible
   const uint32_t max_wnc = 16 / p.ksc;
-  p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (nquads + num_cus - 1) / num_cus));
-  if (const char* e = getenv("MGN_DEV_WNC")) p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (uint32_t)atoi(e)));
+  const uint32_t wave_quads = (nquads + p.qpw - 1) / p.qpw;  // quad groups = waves with work
+  p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (wave_quads + num_cus - 1) / num_cus));
   // enough threads to prepare the activations (waves without a quad only help there)
   const uint32_t prep_waves = (bpc_pad * 4 + kMaxTasks * 64 - 1) / (kMaxTasks * 64);
   p.wnc = std::max<uint32_t>(p.wnc, (prep_waves + p.ksc - 1) / p.ksc);
   if (p.wnc > max_wnc) return false;
-  p.grid = (nquads + p.wnc - 1) / p.wnc;
+  p.grid = (wave_quads + p.wnc - 1) / p.wnc;
   const size_t nj = 2 * mrows;
   p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 8 + (size_t)p.wnc * p.ksc * mrows * 16 + 64;
   if (p.lds > 150 * 1024) return false;
@@ -422,9 +435,9 @@ bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, MfmaGem
   return true;
 }
 
-template <int FMT, int MROWS, int STEPS>
+template <int FMT, int MROWS, int STEPS, int QPW>
 int launch_steps(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS>;
+  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW>;
   static bool big_lds_enabled = false;
   if (p.lds > 64 * 1024 && !big_lds_enabled) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -441,15 +454,21 @@ template <int FMT, int MROWS>
 int launch_t(ihipStream_t* s, const LaunchArgs& x) {
   MfmaGemvPlan p;
   if (!plan_mfma_gemv(x.w.k, x.w.n, MROWS, x.num_cus, &p)) return (int)hipErrorInvalidValue;
-  switch (p.steps) {
-    case 1: return launch_steps<FMT, MROWS, 1>(s, x, p);
-    case 2: return launch_steps<FMT, MROWS, 2>(s, x, p);
-    case 3: return launch_steps<FMT, MROWS, 3>(s, x, p);
-    case 4: return launch_steps<FMT, MROWS, 4>(s, x, p);
-    case 5: return launch_steps<FMT, MROWS, 5>(s, x, p);
-    case 6: return launch_steps<FMT, MROWS, 6>(s, x, p);
-    case 7: return launch_steps<FMT, MROWS, 7>(s, x, p);
-    case 8: return launch_steps<FMT, MROWS, 8>(s, x, p);
+  switch (p.steps * 8 + p.qpw) {
+    case 1 * 8 + 1: return launch_steps<FMT, MROWS, 1, 1>(s, x, p);
+    case 1 * 8 + 2: return launch_steps<FMT, MROWS, 1, 2>(s, x, p);
+    case 1 * 8 + 4: return launch_steps<FMT, MROWS, 1, 4>(s, x, p);
+    case 2 * 8 + 1: return launch_steps<FMT, MROWS, 2, 1>(s, x, p);
+    case 2 * 8 + 2: return launch_steps<FMT, MROWS, 2, 2>(s, x, p);
+    case 2 * 8 + 4: return launch_steps<FMT, MROWS, 2, 4>(s, x, p);
+    case 3 * 8 + 1: return launch_steps<FMT, MROWS, 3, 1>(s, x, p);
+    case 3 * 8 + 2: return launch_steps<FMT, MROWS, 3, 2>(s, x, p);
+    case 4 * 8 + 1: return launch_steps<FMT, MROWS, 4, 1>(s, x, p);
+    case 4 * 8 + 2: return launch_steps<FMT, MROWS, 4, 2>(s, x, p);
+    case 5 * 8 + 1: return launch_steps<FMT, MROWS, 5, 1>(s, x, p);
+    case 6 * 8 + 1: return launch_steps<FMT, MROWS, 6, 1>(s, x, p);
+    case 7 * 8 + 1: return launch_steps<FMT, MROWS, 7, 1>(s, x, p);
+    case 8 * 8 + 1: return launch_steps<FMT, MROWS, 8, 1>(s, x, p);
     default: return (int)hipErrorInvalidValue;
   }
 }
