@@ -130,7 +130,8 @@ def decode_layer_times(steps, warmup):
     Graph/Session surface (models/smollm2.rs:340-414 without the attention core): rms_norm,
     q/k/v, o-projection + residual, rms_norm, gate||up as one fused matmul, SwiGLU, down +
     residual -- 9 dispatches after the optimizer's fusions.  Returns microseconds per layer
-    step, launched dispatch by dispatch and replayed as one captured graph."""
+    step: every dispatch its own launch, norms and SwiGLU folded into the matmuls (the
+    default), and the folded step replayed as one captured graph."""
     from meganeura_amd import capi, synth
     from meganeura_amd.graph import Graph, build_inference_session
 
@@ -159,8 +160,10 @@ def decode_layer_times(steps, warmup):
     sess.set_input("attn", synth.activations(2, 1, hidden, which=1))
     ctx = sess.context()
     res = {"dispatches": len(sess.plan())}
-    for label, replay in (("launches", False), ("graph", True)):
+    for label, fusion, replay in (("unfused", False, False), ("fused", True, False), ("fused_graph", True, True)):
+        sess.set_fusion(fusion)
         sess.set_graph_replay(replay)
+        res[label + "_launches"] = sess.num_launches()
         for _ in range(warmup + 2):
             sess.step()
         ctx.sync()

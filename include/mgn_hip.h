@@ -37,7 +37,8 @@ typedef enum mgn_status {
   MGN_ENOMEM = 2,    /* host or device allocation failed */
   MGN_EHIP = 3,      /* a HIP runtime call failed; see mgn_last_error */
   MGN_ENOTFOUND = 4, /* unknown name (session layer) */
-  MGN_ENODEVICE = 5  /* no usable gfx950 device */
+  MGN_ENODEVICE = 5, /* no usable gfx950 device */
+  MGN_EUNSUPPORTED = 6 /* a fused entry point asked for a shape its kernel does not serve */
 } mgn_status;
 
 /* compile::WeightFormat::{Q4,Q8} (src/compile.rs:8-29), graph::DType::{Q4_0,Q8_0}
@@ -139,6 +140,20 @@ mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, con
  * reference, src/runtime.rs:1634). */
 mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w,
                              const mgn_buf* d, mgn_buf* c, uint32_t m);
+
+/* Two neighbours of the decode-time matmul folded into its activation staging, each
+ * standing in for a dispatch pair of the reference's plan (M <= 2, f32 activations):
+ *   RmsNorm then MatMul[Gemv][Add]   (src/shaders/rms_norm.wgsl:1-57; models/smollm2.rs:340-341,396):
+ *     C = (x * rsqrt(mean(x^2) + eps) * norm_weight) x W (+ D), x[M,K], norm_weight[K];
+ *   SwiGLUConcat then MatMul[Gemv][Add]   (src/shaders/swiglu_concat.wgsl:20-32; compile.rs:1814-1830):
+ *     C = (gate * sigmoid(gate) * up) x W (+ D), gate_up[M,2K] = gate | up.
+ * MGN_EUNSUPPORTED when the shape is not served by the kernel that can fuse (run the two
+ * dispatches separately then); mgn_matmul_q_can_fuse tells beforehand (1 = yes). */
+mgn_status mgn_matmul_q_rms_norm(mgn_ctx* ctx, const mgn_buf* x, const mgn_buf* norm_weight, float eps,
+                                 const mgn_weight* w, const mgn_buf* d, mgn_buf* c, uint32_t m);
+mgn_status mgn_matmul_q_swiglu(mgn_ctx* ctx, const mgn_buf* gate_up, const mgn_weight* w,
+                               const mgn_buf* d, mgn_buf* c, uint32_t m);
+int mgn_matmul_q_can_fuse(mgn_ctx* ctx, const mgn_weight* w, uint32_t m);
 
 /* ---- GPU timing on the context's stream: Session::set_profiling +
  *      dump_gpu_timings (src/runtime.rs:1965, 2798-2832) reduced to one

@@ -91,6 +91,14 @@ mgn_status mgn_session_wait(mgn_session* s);
  * mgn_session_graph_active reports whether the next step will be a graph replay (1) or
  * individual launches (0). */
 mgn_status mgn_session_set_graph_replay(mgn_session* s, int enable);
+/* Launch-level fusion (on by default): an RmsNorm or SwiGLUConcat dispatch whose output is
+ * read only by batch-1/2 quantized matmuls is not launched; those matmuls apply it while
+ * staging their activations (mgn_matmul_q_rms_norm / mgn_matmul_q_swiglu).  The plan and
+ * mgn_session_dispatch_info keep the reference's dispatch list (src/compile.rs:494-528);
+ * mgn_session_num_launches reports how many kernels a step really launches.  The folded
+ * dispatch's own output buffer is then never written. */
+mgn_status mgn_session_set_fusion(mgn_session* s, int enable);
+size_t mgn_session_num_launches(mgn_session* s);
 int mgn_session_graph_active(const mgn_session* s);
 /* Session::read_output / read_output_by_index (src/runtime.rs:2612-2638). */
 mgn_status mgn_session_read_output(mgn_session* s, float* out, size_t len);

@@ -11,7 +11,7 @@ import numpy as np
 _DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_DIR, "libmgn_hip.so")
 
-OK, EINVAL, ENOMEM, EHIP, ENOTFOUND, ENODEVICE = range(6)
+OK, EINVAL, ENOMEM, EHIP, ENOTFOUND, ENODEVICE, EUNSUPPORTED = range(7)
 FMT_Q4, FMT_Q8 = 0, 1
 ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA = range(5)
 
@@ -22,7 +22,7 @@ HIP_SYMBOLS = [
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_matmul_q",
-    "mgn_matmul_q_f16a", "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
+    "mgn_matmul_q_f16a", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [
     "mgn_graph_new", "mgn_graph_free", "mgn_graph_last_error", "mgn_graph_input", "mgn_graph_parameter",
@@ -32,7 +32,7 @@ SESSION_SYMBOLS = [
     "mgn_session_num_dispatches", "mgn_session_dispatch_info", "mgn_session_set_parameter",
     "mgn_session_set_input", "mgn_session_step", "mgn_session_wait", "mgn_session_read_output",
     "mgn_session_read_output_by_index", "mgn_session_ctx", "mgn_session_set_graph_replay",
-    "mgn_session_graph_active",
+    "mgn_session_graph_active", "mgn_session_set_fusion", "mgn_session_num_launches",
 ]
 
 
@@ -91,6 +91,9 @@ def load():
         "mgn_weight_export_ref": (C.c_int, [vp, vp, vp]),
         "mgn_matmul_q": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_f16a": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
+        "mgn_matmul_q_rms_norm": (C.c_int, [vp, vp, vp, C.c_float, vp, vp, vp, C.c_uint32]),
+        "mgn_matmul_q_swiglu": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
+        "mgn_matmul_q_can_fuse": (C.c_int, [vp, vp, C.c_uint32]),
         "mgn_timer_start": (C.c_int, [vp]),
         "mgn_timer_stop": (C.c_int, [vp, C.POINTER(C.c_float)]),
         "mgn_version": (C.c_char_p, []),
@@ -122,6 +125,8 @@ def load():
         "mgn_session_ctx": (vp, [vp]),
         "mgn_session_set_graph_replay": (C.c_int, [vp, C.c_int]),
         "mgn_session_graph_active": (C.c_int, [vp]),
+        "mgn_session_set_fusion": (C.c_int, [vp, C.c_int]),
+        "mgn_session_num_launches": (sz, [vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -245,6 +250,17 @@ class Context:
 
     def matmul_q_f16a(self, a, w, c, m, d=None):
         self.check(self.lib.mgn_matmul_q_f16a(self.h, a.h, w.h, d.h if d is not None else None, c.h, m))
+
+    def matmul_q_rms_norm(self, x, norm_weight, eps, w, c, m, d=None):
+        """C = rms_norm(x; norm_weight, eps) x W (+ D) in one launch."""
+        self.check(self.lib.mgn_matmul_q_rms_norm(self.h, x.h, norm_weight.h, eps, w.h, d.h if d is not None else None, c.h, m))
+
+    def matmul_q_swiglu(self, gate_up, w, c, m, d=None):
+        """C = (silu(gate) * up) x W (+ D) in one launch; gate_up is [m, 2K]."""
+        self.check(self.lib.mgn_matmul_q_swiglu(self.h, gate_up.h, w.h, d.h if d is not None else None, c.h, m))
+
+    def can_fuse(self, w, m):
+        return bool(self.lib.mgn_matmul_q_can_fuse(self.h, w.h, m))
 
 
 class Buffer:

@@ -111,6 +111,17 @@ __device__ __forceinline__ float sum_over_blocks(float v) {
   return v;
 }
 
+// src/shaders/swiglu_concat.wgsl:20-32: silu(gate) * up with sig = 1 / (1 + exp(-gate))
+__device__ __forceinline__ float swiglu_act(float gate, float up) {
+  const float sig = 1.0f / (1.0f + expf(-gate));
+  return gate * sig * up;
+}
+
+struct GemvPrologue {
+  const float* norm_weight;  // [K], kProRmsNorm
+  float eps;
+};
+
 template <int FMT>
 struct Raw;
 template <>
@@ -181,10 +192,14 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 // has arrived while the later ones are still in flight.
 // QPW > 1 (short K, many columns): a wave takes QPW consecutive quads, so that it still has
 // QPW * STEPS block loads to keep in flight and the workgroup count stays near the CU count.
-template <int FMT, int MROWS, int STEPS, int QPW>
+// PRO: what the activations go through on their way into LDS, in place of a kernel of its own:
+//   kProNone     a[m, K] as is;
+//   kProRmsNorm  a[m, K] * rsqrt(mean(a^2) + eps) * norm_weight[K]   (src/shaders/rms_norm.wgsl:1-57);
+//   kProSwiglu   a[m, 2K] = gate | up  ->  gate * sigmoid(gate) * up  (src/shaders/swiglu_concat.wgsl:20-32).
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const float* __restrict__ a,
                                                          const float* __restrict__ dres, float* __restrict__ c,
-                                                         uint32_t m, uint32_t ksc MGN_TRACE_PARAM) {
+                                                         uint32_t m, uint32_t ksc, GemvPrologue pro MGN_TRACE_PARAM) {
   constexpr int NJ = 2 * MROWS;
   extern __shared__ uint4 lds4[];
   const uint32_t bpc = w.k / 32;
@@ -194,6 +209,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   uint4* xa = lds4;                                   // [4][plane]
   float2* cinit = (float2*)(lds4 + 4 * plane);        // [bpc_pad][MROWS]
   float* red = (float*)(cinit + bpc_pad * MROWS);     // [wnc][ksc][MROWS][4]
+  float* nrm = red + wnc * ksc * MROWS * 4;           // [16 waves][MROWS] sums of squares (kProRmsNorm)
 
   MGN_STAMP_INIT();
   MGN_STAMP(0);
@@ -220,6 +236,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   // One task = 8 consecutive activations of one row = one A chunk; the 4 tasks of a K
   // block sit in one lane quad.  A thread holds at most kMaxTasks tasks in registers.
   float4 xraw[kMaxTasks][MROWS][2];
+  float4 xup[PRO == kProSwiglu ? kMaxTasks : 1][MROWS][2];   // the "up" halves
+  float4 gw[PRO == kProRmsNorm ? kMaxTasks : 1][2];          // norm weights of the task's 8 columns
+  const uint32_t a_stride = PRO == kProSwiglu ? 2 * w.k : w.k;
 #pragma unroll
   for (int tt = 0; tt < kMaxTasks; tt++) {
     const uint32_t t = tid + tt * blockDim.x, kb = t >> 2, ch = t & 3;
@@ -228,9 +247,19 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
     for (int r = 0; r < MROWS; r++) {
       // always load (from element 0 when there is nothing to load) and zero afterwards
       const bool ok = live && (uint32_t)r < m;
-      const float4* src = (const float4*)(a + (ok ? (size_t)r * w.k + (size_t)kb * 32 + ch * 8 : (size_t)0));
+      const float4* src = (const float4*)(a + (ok ? (size_t)r * a_stride + (size_t)kb * 32 + ch * 8 : (size_t)0));
       xraw[tt][r][0] = src[0];
       xraw[tt][r][1] = src[1];
+      if constexpr (PRO == kProSwiglu) {
+        const float4* up = (const float4*)(a + (ok ? (size_t)r * a_stride + w.k + (size_t)kb * 32 + ch * 8 : (size_t)0));
+        xup[tt][r][0] = up[0];
+        xup[tt][r][1] = up[1];
+      }
+    }
+    if constexpr (PRO == kProRmsNorm) {
+      const float4* gp = (const float4*)(pro.norm_weight + (live ? (size_t)kb * 32 + ch * 8 : (size_t)0));
+      gw[tt][0] = gp[0];
+      gw[tt][1] = gp[1];
     }
   }
   // Weight blocks: kDepth loads run ahead of the step that consumes them.  That is enough
@@ -249,6 +278,59 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   for (int t = 0; t < TS && t < kDepth; t++) fetch(t);
   for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += blockDim.x) red[t] = 0.0f;
   MGN_STAMP(1);
+
+  // ---- fused prologue: turn the raw loads into the matmul's activations ----
+  if constexpr (PRO == kProSwiglu) {
+#pragma unroll
+    for (int tt = 0; tt < kMaxTasks; tt++)
+#pragma unroll
+      for (int r = 0; r < MROWS; r++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const float4 g4 = xraw[tt][r][h], u4 = xup[tt][r][h];
+          xraw[tt][r][h] = make_float4(swiglu_act(g4.x, u4.x), swiglu_act(g4.y, u4.y), swiglu_act(g4.z, u4.z),
+                                       swiglu_act(g4.w, u4.w));
+        }
+  }
+  if constexpr (PRO == kProRmsNorm) {
+    // row sums of squares: per thread, per wave (DPP), then across the waves through LDS
+    float ss[MROWS];
+#pragma unroll
+    for (int r = 0; r < MROWS; r++) {
+      ss[r] = 0.0f;
+#pragma unroll
+      for (int tt = 0; tt < kMaxTasks; tt++) {
+        const uint32_t kb = (tid + tt * blockDim.x) >> 2;
+        if (kb < bpc && (uint32_t)r < m) {
+#pragma unroll
+          for (int h = 0; h < 2; h++) {
+            const float4 v = xraw[tt][r][h];
+            ss[r] = __fmaf_rn(v.x, v.x, ss[r]);
+            ss[r] = __fmaf_rn(v.y, v.y, ss[r]);
+            ss[r] = __fmaf_rn(v.z, v.z, ss[r]);
+            ss[r] = __fmaf_rn(v.w, v.w, ss[r]);
+          }
+        }
+      }
+      ss[r] = group_sum<64>(ss[r]);
+      if (lane == 0) nrm[wave * MROWS + r] = ss[r];
+    }
+    lds_barrier();
+    const uint32_t nwv = blockDim.x >> 6;
+#pragma unroll
+    for (int r = 0; r < MROWS; r++) {
+      float tot = 0.0f;
+      for (uint32_t wv = 0; wv < nwv; wv++) tot += nrm[wv * MROWS + r];
+      const float rstd = 1.0f / sqrtf(tot / (float)w.k + pro.eps);
+#pragma unroll
+      for (int tt = 0; tt < kMaxTasks; tt++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const float4 v = xraw[tt][r][h], g4 = gw[tt][h];
+          xraw[tt][r][h] = make_float4(v.x * rstd * g4.x, v.y * rstd * g4.y, v.z * rstd * g4.z, v.w * rstd * g4.w);
+        }
+    }
+  }
 
   // ---- activations -> LDS (once per workgroup) ----
 #pragma unroll
@@ -400,7 +482,7 @@ struct MfmaGemvPlan {
 
 constexpr uint32_t kMaxSteps = 8;  // blocks a lane holds in flight: 8 x 20 B (Q4) or 8 x 34 B (Q8)
 
-bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, MfmaGemvPlan* out) {
+bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, bool fused_prologue, MfmaGemvPlan* out) {
   const uint32_t bpc = k / 32, bpc_pad = (bpc + 15) & ~15u;
   const uint32_t steps_total = bpc_pad / 16;
   const uint32_t nquads = (n + 3) / 4;
@@ -416,7 +498,7 @@ bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, MfmaGem
   // quads per wave: with a short K and very many columns a wave takes several quads, as
   // long as that leaves at least 8 waves per CU
   p.qpw = 1;
-  if (p.ksc == 1)
+  if (p.ksc == 1 && !fused_prologue)
     while (p.qpw < 4 && p.steps * p.qpw * 2 <= kMaxSteps && nquads / (p.qpw * 2) >= (uint32_t)num_cus * 8) p.qpw *= 2;
   // waves per workgroup: spread the quads evenly over the CUs (one workgroup per CU when
   // there is enough work), so the activations are prepared as few times as possible
@@ -429,31 +511,43 @@ bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, MfmaGem
   if (p.wnc > max_wnc) return false;
   p.grid = (wave_quads + p.wnc - 1) / p.wnc;
   const size_t nj = 2 * mrows;
-  p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 8 + (size_t)p.wnc * p.ksc * mrows * 16 + 64;
+  p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 8 + (size_t)p.wnc * p.ksc * mrows * 16 +
+          16 * mrows * 4 + 64;
   if (p.lds > 150 * 1024) return false;
   *out = p;
   return true;
 }
 
-template <int FMT, int MROWS, int STEPS, int QPW>
-int launch_steps(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW>;
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
+int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
+  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO>;
   static bool big_lds_enabled = false;
   if (p.lds > 64 * 1024 && !big_lds_enabled) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) return (int)e;
     big_lds_enabled = true;
   }
+  const GemvPrologue pro{x.pro_weight, x.pro_eps};
   hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, x.w, (const float*)x.a, x.d, x.c, x.m,
-                     p.ksc MGN_TRACE_ARG);
+                     p.ksc, pro MGN_TRACE_ARG);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
+}
+
+template <int FMT, int MROWS, int STEPS, int QPW>
+int launch_steps(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
+  if constexpr (QPW == 1) {  // fused prologues come with one quad per wave only
+    if (x.pro_kind == kProRmsNorm) return launch_pro<FMT, MROWS, STEPS, QPW, kProRmsNorm>(s, x, p);
+    if (x.pro_kind == kProSwiglu) return launch_pro<FMT, MROWS, STEPS, QPW, kProSwiglu>(s, x, p);
+  }
+  if (x.pro_kind != kProNone) return (int)hipErrorInvalidValue;
+  return launch_pro<FMT, MROWS, STEPS, QPW, kProNone>(s, x, p);
 }
 
 template <int FMT, int MROWS>
 int launch_t(ihipStream_t* s, const LaunchArgs& x) {
   MfmaGemvPlan p;
-  if (!plan_mfma_gemv(x.w.k, x.w.n, MROWS, x.num_cus, &p)) return (int)hipErrorInvalidValue;
+  if (!plan_mfma_gemv(x.w.k, x.w.n, MROWS, x.num_cus, x.pro_kind != kProNone, &p)) return (int)hipErrorInvalidValue;
   switch (p.steps * 8 + p.qpw) {
     case 1 * 8 + 1: return launch_steps<FMT, MROWS, 1, 1>(s, x, p);
     case 1 * 8 + 2: return launch_steps<FMT, MROWS, 1, 2>(s, x, p);
@@ -478,7 +572,7 @@ int launch_t(ihipStream_t* s, const LaunchArgs& x) {
 bool gemv_mfma_supported(const LaunchArgs& x) {
   if (x.a_is_f16 || x.m == 0 || x.m > 2) return false;
   MfmaGemvPlan p;
-  return plan_mfma_gemv(x.w.k, x.w.n, x.m, x.num_cus, &p);
+  return plan_mfma_gemv(x.w.k, x.w.n, x.m, x.num_cus, x.pro_kind != kProNone, &p);
 }
 
 int launch_matmul_gemv_mfma(ihipStream_t* s, const LaunchArgs& x) {

@@ -353,18 +353,34 @@ mgn_status mgn_weight_export_ref(mgn_ctx* ctx, const mgn_weight* w, uint8_t* out
 // ---- matmul ----
 
 static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, const mgn_weight* w, const mgn_buf* d,
-                              mgn_buf* c, uint32_t m) {
+                              mgn_buf* c, uint32_t m, int pro_kind = mgn::kProNone, const mgn_buf* norm_weight = nullptr,
+                              float eps = 0.0f) {
   if (!ctx || !a || !w || !c) return fail(ctx, MGN_EINVAL, "null argument");
   if (m == 0) return MGN_OK;
   const size_t k = w->rows, n = w->cols;
   const size_t a_elem = a_is_f16 ? 2 : 4;
-  if (a->bytes / a_elem < (size_t)m * k) return fail(ctx, MGN_EINVAL, "A is smaller than m*K elements");
+  const size_t a_cols = pro_kind == mgn::kProSwiglu ? 2 * k : k;
+  if (a->bytes / a_elem < (size_t)m * a_cols) return fail(ctx, MGN_EINVAL, "A is smaller than its m rows");
+  if (pro_kind == mgn::kProRmsNorm && (!norm_weight || norm_weight->bytes / 4 < k))
+    return fail(ctx, MGN_EINVAL, "norm weight is missing or shorter than K floats");
   if (c->bytes / 4 < (size_t)m * n) return fail(ctx, MGN_EINVAL, "C is smaller than m*N floats");
   if (d && d->bytes / 4 < (size_t)m * n) return fail(ctx, MGN_EINVAL, "D is smaller than m*N floats");
   if (c->ptr == a->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
-  mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus,
-                    ctx->scratch,  ctx->scratch_bytes, ctx->counters, ctx->n_counters};
+  mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus};
+  x.scratch = ctx->scratch;
+  x.scratch_bytes = ctx->scratch_bytes;
+  x.counters = ctx->counters;
+  x.n_counters = ctx->n_counters;
+  x.pro_kind = pro_kind;
+  x.pro_weight = norm_weight ? (const float*)norm_weight->ptr : nullptr;
+  x.pro_eps = eps;
   mgn_route route = ctx->route;
+  if (pro_kind != mgn::kProNone) {
+    // only the MFMA GEMV stages its activations in a way a prologue can ride on
+    if (a_is_f16 || !mgn::gemv_mfma_supported(x) || (route != MGN_ROUTE_AUTO && route != MGN_ROUTE_GEMV_MFMA))
+      return fail(ctx, MGN_EUNSUPPORTED, "fused prologue needs the GEMV_MFMA route (f32 activations, M <= 2)");
+    route = MGN_ROUTE_GEMV_MFMA;
+  }
   if (route == MGN_ROUTE_AUTO) {
     if (mgn::gemv_mfma_supported(x)) route = MGN_ROUTE_GEMV_MFMA;
     else if (mgn::gemm_mfma_supported(x)) route = MGN_ROUTE_GEMM_MFMA;
@@ -396,6 +412,23 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
 mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
                         uint32_t m) {
   return matmul_impl(ctx, a, false, w, d, c, m);
+}
+
+mgn_status mgn_matmul_q_rms_norm(mgn_ctx* ctx, const mgn_buf* x, const mgn_buf* norm_weight, float eps,
+                                 const mgn_weight* w, const mgn_buf* d, mgn_buf* c, uint32_t m) {
+  return matmul_impl(ctx, x, false, w, d, c, m, mgn::kProRmsNorm, norm_weight, eps);
+}
+
+mgn_status mgn_matmul_q_swiglu(mgn_ctx* ctx, const mgn_buf* gate_up, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
+                               uint32_t m) {
+  return matmul_impl(ctx, gate_up, false, w, d, c, m, mgn::kProSwiglu);
+}
+
+int mgn_matmul_q_can_fuse(mgn_ctx* ctx, const mgn_weight* w, uint32_t m) {
+  if (!ctx || !w || m == 0) return 0;
+  mgn::LaunchArgs x{view_of(w), nullptr, nullptr, nullptr, m, false, ctx->num_cus};
+  x.pro_kind = mgn::kProRmsNorm;
+  return (ctx->route == MGN_ROUTE_AUTO || ctx->route == MGN_ROUTE_GEMV_MFMA) && mgn::gemv_mfma_supported(x) ? 1 : 0;
 }
 
 mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,

@@ -35,6 +35,8 @@ struct WeightView {
   int fmt;        // mgn_fmt
 };
 
+enum { kProNone = 0, kProRmsNorm = 1, kProSwiglu = 2 };
+
 struct LaunchArgs {
   WeightView w;
   const void* a;   // [m, k] f32 or f16
@@ -43,6 +45,10 @@ struct LaunchArgs {
   uint32_t m;
   bool a_is_f16;
   int num_cus;
+  // fused prologue (GEMV-MFMA route only): what `a` goes through before the matmul
+  int pro_kind = 0;                   // kProNone / kProRmsNorm / kProSwiglu
+  const float* pro_weight = nullptr;  // norm weight [K]
+  float pro_eps = 0.0f;
   // context-owned workspace for kernels that split K across workgroups
   void* scratch = nullptr;
   size_t scratch_bytes = 0;

@@ -350,6 +350,7 @@ void Session::upload_weight(int buf, const WeightBufferInfo& info, const float* 
   const mgn_fmt fmt = info.fmt == WeightFormat::Q4 ? MGN_FMT_Q4 : MGN_FMT_Q8;
   check(mgn_weight_create(ctx_, fmt, data, info.rows, info.cols, &fresh), "mgn_weight_create");
   drop_graph();  // a captured step holds the old handle's addresses
+  launches_planned_ = false;
   mgn_weight_free(ctx_, weights_[buf]);  // waits for in-flight work that may still read it
   weights_[buf] = fresh;
 }
@@ -472,8 +473,62 @@ void Session::drop_graph() {
   eager_steps_ = 0;
 }
 
+void Session::set_fusion(bool on) {
+  if (on == fusion_wanted_) return;
+  fusion_wanted_ = on;
+  launches_planned_ = false;
+  drop_graph();
+}
+
+size_t Session::num_launches() {
+  plan_launches();
+  size_t n = 0;
+  for (char sk : skipped_) n += sk ? 0 : 1;
+  return n;
+}
+
+// Which RmsNorm / SwiGLUConcat dispatches disappear into the matmuls that read them
+// (models/smollm2.rs:340-341,396: norm -> q/k/v and norm -> gate/up; compile.rs:1814-1830:
+// swiglu_concat -> down).  A producer is folded only if every reader of its output is a
+// decode matmul taking it as the activation operand and served by the fusing kernel.
+void Session::plan_launches() {
+  if (launches_planned_) return;
+  const size_t nd = plan_.dispatches.size();
+  fused_.assign(nd, Fused{});
+  skipped_.assign(nd, 0);
+  launches_planned_ = true;
+  if (!fusion_wanted_) return;
+  std::vector<std::vector<int>> readers(plan_.buffers.size());
+  for (size_t i = 0; i < nd; i++)
+    for (int b : plan_.dispatches[i].input_buffers) readers[b].push_back((int)i);
+  std::vector<char> is_output(plan_.buffers.size(), 0);
+  for (int b : plan_.output_buffers) is_output[b] = 1;
+  for (size_t pi = 0; pi < nd; pi++) {
+    const Dispatch& p = plan_.dispatches[pi];
+    const bool norm = p.shader == MGN_SHADER_RMS_NORM, swi = p.shader == MGN_SHADER_SWIGLU_CONCAT;
+    if (!norm && !swi) continue;
+    const int out = p.output_buffer;
+    if (is_output[out] || readers[out].empty()) continue;
+    const uint32_t width = p.params[1];  // columns of the produced activation
+    bool ok = true;
+    for (int ci : readers[out]) {
+      const Dispatch& c = plan_.dispatches[ci];
+      mgn_weight* w = is_matmul(c.shader) ? weights_[c.input_buffers[1]] : nullptr;
+      ok = ok && (size_t)ci > pi && w && c.input_buffers[0] == out && c.params[1] == width &&
+           (c.input_buffers.size() < 3 || c.input_buffers[2] != out) && fused_[ci].kind == 0 &&
+           mgn_matmul_q_can_fuse(ctx_, w, c.params[0]) == 1;
+    }
+    if (!ok) continue;
+    skipped_[pi] = 1;
+    for (int ci : readers[out]) fused_[ci] = Fused{norm ? kProRmsNorm : kProSwiglu, (int)pi};
+  }
+}
+
 void Session::run_dispatches() {
-  for (const Dispatch& d : plan_.dispatches) {
+  plan_launches();
+  for (size_t di = 0; di < plan_.dispatches.size(); di++) {
+    if (skipped_[di]) continue;
+    const Dispatch& d = plan_.dispatches[di];
     float* out = (float*)buffers_[d.output_buffer]->ptr;
     auto fin = [&](size_t i) { return (const float*)buffers_[d.input_buffers[i]]->ptr; };
     int rc = 0;
@@ -485,8 +540,20 @@ void Session::run_dispatches() {
         mgn_weight* w = weights_[d.input_buffers[1]];
         if (!w) throw std::runtime_error("quantized parameter was never set");
         const mgn_buf* addend = d.input_buffers.size() > 2 ? buffers_[d.input_buffers[2]] : nullptr;
-        check(mgn_matmul_q(ctx_, buffers_[d.input_buffers[0]], w, addend, buffers_[d.output_buffer], d.params[0]),
-              "mgn_matmul_q");
+        const Fused& f = fused_[di];
+        if (f.kind == kProRmsNorm) {
+          const Dispatch& p = plan_.dispatches[f.producer];
+          check(mgn_matmul_q_rms_norm(ctx_, buffers_[p.input_buffers[0]], buffers_[p.input_buffers[1]], p.eps, w, addend,
+                                      buffers_[d.output_buffer], d.params[0]),
+                "mgn_matmul_q_rms_norm");
+        } else if (f.kind == kProSwiglu) {
+          const Dispatch& p = plan_.dispatches[f.producer];
+          check(mgn_matmul_q_swiglu(ctx_, buffers_[p.input_buffers[0]], w, addend, buffers_[d.output_buffer], d.params[0]),
+                "mgn_matmul_q_swiglu");
+        } else {
+          check(mgn_matmul_q(ctx_, buffers_[d.input_buffers[0]], w, addend, buffers_[d.output_buffer], d.params[0]),
+                "mgn_matmul_q");
+        }
         break;
       }
       case MGN_SHADER_ADD:
@@ -681,6 +748,14 @@ mgn_status mgn_session_step(mgn_session* s) { return session_call(s, [&] { s->s-
 mgn_status mgn_session_wait(mgn_session* s) { return session_call(s, [&] { s->s->wait(); }); }
 mgn_status mgn_session_set_graph_replay(mgn_session* s, int enable) {
   return session_call(s, [&] { s->s->set_graph_replay(enable != 0); });
+}
+mgn_status mgn_session_set_fusion(mgn_session* s, int enable) {
+  return session_call(s, [&] { s->s->set_fusion(enable != 0); });
+}
+size_t mgn_session_num_launches(mgn_session* s) {
+  size_t n = 0;
+  if (s && s->s) (void)session_call(s, [&] { n = s->s->num_launches(); });
+  return n;
 }
 int mgn_session_graph_active(const mgn_session* s) { return s && s->s && s->s->graph_active() ? 1 : 0; }
 mgn_status mgn_session_read_output(mgn_session* s, float* out, size_t len) {

@@ -146,6 +146,10 @@ class Session {
   // are a single graph launch.  Results are identical; only launch overhead changes --
   // less host work per step, but measured slower on the GPU side for chains of tiny kernels.
   void set_graph_replay(bool on);
+  // Fold RmsNorm / SwiGLUConcat dispatches into the decode matmuls that consume them
+  // (default on).  The plan keeps the reference's dispatch list; only the launches differ.
+  void set_fusion(bool on);
+  size_t num_launches();  // kernel launches one step makes with the current settings
   bool graph_active() const { return exec_ != nullptr; }
   void wait();
   void read_output(float* out, size_t len) { read_output_by_index(0, out, len); }
@@ -158,6 +162,15 @@ class Session {
   void release();
   void run_dispatches();
   void drop_graph();
+  void plan_launches();
+  struct Fused {
+    int kind = 0;       // kProNone / kProRmsNorm / kProSwiglu
+    int producer = -1;  // the folded-in dispatch
+  };
+  std::vector<Fused> fused_;     // per dispatch (matmuls only)
+  std::vector<char> skipped_;    // per dispatch: folded into its consumers
+  bool launches_planned_ = false;
+  bool fusion_wanted_ = true;
   ExecutionPlan plan_;
   mgn_ctx* ctx_ = nullptr;
   std::vector<mgn_buf*> buffers_;        // f32 buffers (null for quantized params)

@@ -153,6 +153,13 @@ class Session:
         """Steps replay one captured HIP graph (default) or launch dispatch by dispatch."""
         self._check(self.lib.mgn_session_set_graph_replay(self.h, 1 if enable else 0))
 
+    def set_fusion(self, enable):
+        """Fold RmsNorm / SwiGLUConcat dispatches into the decode matmuls reading them (default on)."""
+        self._check(self.lib.mgn_session_set_fusion(self.h, 1 if enable else 0))
+
+    def num_launches(self):
+        return int(self.lib.mgn_session_num_launches(self.h))
+
     def graph_active(self):
         return bool(self.lib.mgn_session_graph_active(self.h))
 

@@ -210,3 +210,67 @@ def test_split_k_is_repeatable(ctx, orc, fmt):
             b.free()
         c.free()
         wt.free()
+
+
+def _rms_norm_f32(x, g, eps):
+    # src/shaders/rms_norm.wgsl:1-57 in f32: x * rsqrt(mean(x^2) + eps) * weight
+    ms = (x.astype(np.float64) ** 2).mean(1, keepdims=True)
+    r = (1.0 / np.sqrt(ms + eps)).astype(np.float32)
+    return (x * r) * g
+
+
+def _swiglu_f32(gate_up):
+    k = gate_up.shape[1] // 2
+    gate, up = gate_up[:, :k], gate_up[:, k:]
+    sig = (1.0 / (1.0 + np.exp(-gate.astype(np.float64)))).astype(np.float32)
+    return gate * sig * up
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m,k,n,resid", [(1, 576, 576, False), (1, 576, 3072, False), (2, 576, 192, True),
+                                         (1, 4096, 1024, True), (1, 1536, 576, True)])
+def test_fused_prologues(ctx, orc, fmt, m, k, n, resid):
+    """rms_norm -> matmul and swiglu_concat -> matmul in one launch, against the two steps
+    done separately on the CPU (pointwise op in f32 with numpy, then the oracle's matmul)."""
+    w = synth.normal(500 + k + n, k * n, 0.02).reshape(k, n)
+    packed = orc.quantize(fmt, w)
+    wt = ctx.weight(fmt, w)
+    assert ctx.can_fuse(wt, m)
+    d = synth.normal(501, m * n, 1.0).reshape(m, n) if resid else None
+    dbuf = ctx.upload(d) if resid else None
+    c = ctx.buffer(m * n * 4)
+    # rms_norm
+    x = synth.normal(502 + m, m * k, 3.0).reshape(m, k)
+    g = 1.0 + 0.25 * synth.normal(503, k, 1.0)
+    xb, gb = ctx.upload(x), ctx.upload(g)
+    ctx.matmul_q_rms_norm(xb, gb, 1e-5, wt, c, m, dbuf)
+    got = c.download(np.float32, m * n).reshape(m, n)
+    orc.assert_close(got, orc.matmul_packed(fmt, _rms_norm_f32(x, g, 1e-5), packed, n, d), REL, ABS)
+    # swiglu over gate | up
+    gu = synth.normal(504 + m, m * 2 * k, 1.5).reshape(m, 2 * k)
+    gub = ctx.upload(gu)
+    ctx.matmul_q_swiglu(gub, wt, c, m, dbuf)
+    got = c.download(np.float32, m * n).reshape(m, n)
+    orc.assert_close(got, orc.matmul_packed(fmt, _swiglu_f32(gu), packed, n, d), REL, ABS)
+    for b in (xb, gb, gub, c) + ((dbuf,) if resid else ()):
+        b.free()
+    wt.free()
+
+
+def test_fused_prologue_is_refused_where_it_cannot_run(ctx):
+    k, n = 576, 64
+    wt = ctx.weight(Q4, synth.normal(510, k * n, 0.02).reshape(k, n))
+    x = ctx.upload(synth.normal(511, 8 * k, 1.0))
+    g = ctx.upload(np.ones(k, np.float32))
+    c = ctx.buffer(8 * n * 4)
+    assert not ctx.can_fuse(wt, 8)
+    with pytest.raises(capi.MgnError) as e:
+        ctx.matmul_q_rms_norm(x, g, 1e-5, wt, c, 8)
+    assert e.value.status == capi.EUNSUPPORTED
+    short = ctx.upload(np.ones(k - 1, np.float32))
+    with pytest.raises(capi.MgnError) as e:
+        ctx.matmul_q_rms_norm(x, short, 1e-5, wt, c, 1)
+    assert e.value.status == capi.EINVAL
+    for b in (x, g, c, short):
+        b.free()
+    wt.free()

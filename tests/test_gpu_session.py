@@ -234,3 +234,57 @@ def test_graph_replay_matches_individual_launches(orc):
         assert (a.view(np.uint32) == b.view(np.uint32)).all() and (a.view(np.uint32) == c.view(np.uint32)).all()
     assert (first[0].view(np.uint32) != want[1][1].view(np.uint32)).any()  # q really uses the new weight
     sess.close()
+
+
+def test_decode_layer_fuses_norm_and_swiglu_into_the_matmuls(orc):
+    """9 dispatches in the plan, 6 kernel launches per step: both norms and the SwiGLU ride on
+    the matmuls that read them.  Same numbers as the unfused step within the matmul bar."""
+    hidden, inter = 576, 1536
+    g = _decode_layer_graph(hidden, inter, lambda gr, name, shape: gr.parameter_q4(name, shape))
+    sess = build_inference_session(g)
+    shapes = {"wq": (hidden, hidden), "wk": (hidden, hidden // 3), "wv": (hidden, hidden // 3), "wo": (hidden, hidden),
+              "wg": (hidden, inter), "wu": (hidden, inter), "wd": (inter, hidden)}
+    for i, (name, (k, n)) in enumerate(shapes.items()):
+        sess.set_parameter(name, synth.normal(600 + i, k * n, 0.02))
+    sess.set_parameter("norm1", 1.0 + 0.1 * synth.normal(610, hidden, 1.0))
+    sess.set_parameter("norm2", 1.0 + 0.1 * synth.normal(611, hidden, 1.0))
+    sess.set_input("x", synth.normal(612, hidden, 1.0))
+    sess.set_input("attn", synth.normal(613, hidden, 1.0))
+    sizes = [hidden, hidden, hidden // 3, hidden // 3]
+    plan = [d.shader for d in sess.plan()]
+    assert len(plan) == 9 and plan.count(ShaderEntry.RmsNorm) == 2 and plan.count(ShaderEntry.SwiGLUConcat) == 1
+    assert sess.num_launches() == 6
+    sess.step()
+    sess.wait()
+    fused = [sess.read_output_by_index(i, n) for i, n in enumerate(sizes)]
+    sess.set_fusion(False)
+    assert sess.num_launches() == 9
+    sess.step()
+    sess.wait()
+    plain = [sess.read_output_by_index(i, n) for i, n in enumerate(sizes)]
+    for a, b in zip(fused, plain):
+        assert np.isfinite(a).all()
+        orc.assert_close(a, b, 1e-3, 1e-4)
+    sess.close()
+
+
+def test_norm_with_another_reader_is_not_folded():
+    # the normed activations are also an output: the RmsNorm dispatch must run on its own
+    hidden = 576
+    g = Graph()
+    x = g.input("x", [1, hidden])
+    n1 = g.rms_norm(x, g.parameter("norm", [hidden]), 1e-5)
+    q = g.matmul(n1, g.parameter_q4("wq", [hidden, hidden]))
+    g.set_outputs([q, n1])
+    sess = build_inference_session(g)
+    sess.set_parameter("wq", synth.normal(620, hidden * hidden, 0.02))
+    sess.set_parameter("norm", np.ones(hidden, np.float32))
+    assert sess.num_launches() == 2
+    xv = synth.normal(621, hidden, 2.0)
+    sess.set_input("x", xv)
+    sess.step()
+    sess.wait()
+    got = sess.read_output_by_index(1, hidden)
+    want = xv / np.sqrt((xv.astype(np.float64) ** 2).mean() + 1e-5)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    sess.close()
