@@ -155,6 +155,24 @@ mgn_status mgn_matmul_q_swiglu(mgn_ctx* ctx, const mgn_buf* gate_up, const mgn_w
                                const mgn_buf* d, mgn_buf* c, uint32_t m);
 int mgn_matmul_q_can_fuse(mgn_ctx* ctx, const mgn_weight* w, uint32_t m);
 
+/* One launch for up to three decode matmuls that read the same activations (the q, k and v
+ * projections: three MatMulGemv dispatches on one normed x, models/smollm2.rs:340-348), with the
+ * same optional prologue.  Weights must share K and the format; each item has its own output
+ * and optional residual.  C_j = prologue(A) x W_j (+ D_j).  Same availability rule and error
+ * as the fused entries above. */
+typedef enum mgn_prologue {
+  MGN_PROLOGUE_NONE = 0,
+  MGN_PROLOGUE_RMS_NORM = 1, /* A = x[M,K], with norm_weight[K] and eps */
+  MGN_PROLOGUE_SWIGLU = 2    /* A = gate_up[M,2K] */
+} mgn_prologue;
+typedef struct mgn_matmul_item {
+  const mgn_weight* w;
+  const mgn_buf* d; /* may be null */
+  mgn_buf* c;
+} mgn_matmul_item;
+mgn_status mgn_matmul_q_batch(mgn_ctx* ctx, const mgn_buf* a, mgn_prologue prologue, const mgn_buf* norm_weight,
+                              float eps, const mgn_matmul_item* items, size_t count, uint32_t m);
+
 /* ---- GPU timing on the context's stream: Session::set_profiling +
  *      dump_gpu_timings (src/runtime.rs:1965, 2798-2832) reduced to one
  *      start/stop pair of HIP events. */

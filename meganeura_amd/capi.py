@@ -22,7 +22,8 @@ HIP_SYMBOLS = [
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_matmul_q",
-    "mgn_matmul_q_f16a", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
+    "mgn_matmul_q_f16a", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
+    "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [
     "mgn_graph_new", "mgn_graph_free", "mgn_graph_last_error", "mgn_graph_input", "mgn_graph_parameter",
@@ -34,6 +35,13 @@ SESSION_SYMBOLS = [
     "mgn_session_read_output_by_index", "mgn_session_ctx", "mgn_session_set_graph_replay",
     "mgn_session_graph_active", "mgn_session_set_fusion", "mgn_session_num_launches",
 ]
+
+
+class MatmulItem(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("d", C.c_void_p), ("c", C.c_void_p)]
+
+
+PROLOGUE_NONE, PROLOGUE_RMS_NORM, PROLOGUE_SWIGLU = range(3)
 
 
 class DispatchInfo(C.Structure):
@@ -94,6 +102,7 @@ def load():
         "mgn_matmul_q_rms_norm": (C.c_int, [vp, vp, vp, C.c_float, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_swiglu": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_can_fuse": (C.c_int, [vp, vp, C.c_uint32]),
+        "mgn_matmul_q_batch": (C.c_int, [vp, vp, C.c_int, vp, C.c_float, C.POINTER(MatmulItem), sz, C.c_uint32]),
         "mgn_timer_start": (C.c_int, [vp]),
         "mgn_timer_stop": (C.c_int, [vp, C.POINTER(C.c_float)]),
         "mgn_version": (C.c_char_p, []),
@@ -258,6 +267,14 @@ class Context:
     def matmul_q_swiglu(self, gate_up, w, c, m, d=None):
         """C = (silu(gate) * up) x W (+ D) in one launch; gate_up is [m, 2K]."""
         self.check(self.lib.mgn_matmul_q_swiglu(self.h, gate_up.h, w.h, d.h if d is not None else None, c.h, m))
+
+    def matmul_q_batch(self, a, items, m, prologue=PROLOGUE_NONE, norm_weight=None, eps=0.0):
+        """items: (weight, c, d-or-None) tuples sharing the activations `a`; one launch."""
+        arr = (MatmulItem * len(items))()
+        for j, (w, c, d) in enumerate(items):
+            arr[j].w, arr[j].c, arr[j].d = w.h, c.h, (d.h if d is not None else None)
+        self.check(self.lib.mgn_matmul_q_batch(self.h, a.h, prologue, norm_weight.h if norm_weight is not None else None,
+                                               eps, arr, len(items), m))
 
     def can_fuse(self, w, m):
         return bool(self.lib.mgn_matmul_q_can_fuse(self.h, w.h, m))

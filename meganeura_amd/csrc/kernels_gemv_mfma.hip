@@ -117,6 +117,21 @@ __device__ __forceinline__ float swiglu_act(float gate, float up) {
   return gate * sig * up;
 }
 
+// Up to three weights that share K, the format and the activations, served by one launch
+// (the q, k and v projections of a decode layer): their column quads are numbered one
+// after the other and every wave looks up which weight its quad belongs to.
+constexpr int kMaxBatch = 3;
+struct GemvBatch {
+  WeightView w[kMaxBatch];
+  const float* d[kMaxBatch];
+  float* c[kMaxBatch];
+  uint32_t first_quad[kMaxBatch];  // [0] = 0; unused entries 0xFFFFFFFF
+};
+template <typename T>
+__device__ __forceinline__ T pick3(uint32_t idx, T a0, T a1, T a2) {
+  return idx == 0 ? a0 : idx == 1 ? a1 : a2;
+}
+
 struct GemvPrologue {
   const float* norm_weight;  // [K], kProRmsNorm
   float eps;
@@ -197,11 +212,23 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 //   kProRmsNorm  a[m, K] * rsqrt(mean(a^2) + eps) * norm_weight[K]   (src/shaders/rms_norm.wgsl:1-57);
 //   kProSwiglu   a[m, 2K] = gate | up  ->  gate * sigmoid(gate) * up  (src/shaders/swiglu_concat.wgsl:20-32).
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
-__global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const float* __restrict__ a,
-                                                         const float* __restrict__ dres, float* __restrict__ c,
-                                                         uint32_t m, uint32_t ksc, GemvPrologue pro MGN_TRACE_PARAM) {
+__global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const float* __restrict__ a, uint32_t m,
+                                                         uint32_t ksc, GemvPrologue pro MGN_TRACE_PARAM) {
   constexpr int NJ = 2 * MROWS;
   extern __shared__ uint4 lds4[];
+  // this wave's weight: the one whose quad range holds the wave's (first) quad
+  const uint32_t wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t gquad_u = (blockIdx.x * ((blockDim.x >> 6) / ksc) + wave_u / ksc) * QPW;
+  const uint32_t widx = (gquad_u >= bt.first_quad[1] ? 1u : 0u) + (gquad_u >= bt.first_quad[2] ? 1u : 0u);
+  WeightView w;
+  w.meta = pick3(widx, bt.w[0].meta, bt.w[1].meta, bt.w[2].meta);
+  w.quants = pick3(widx, bt.w[0].quants, bt.w[1].quants, bt.w[2].quants);
+  w.n = pick3(widx, bt.w[0].n, bt.w[1].n, bt.w[2].n);
+  w.k = bt.w[0].k;
+  w.fmt = FMT;
+  const float* const dres = pick3(widx, bt.d[0], bt.d[1], bt.d[2]);
+  float* const c = pick3(widx, bt.c[0], bt.c[1], bt.c[2]);
+  const uint32_t quad_base = pick3(widx, 0u, bt.first_quad[1], bt.first_quad[2]);  // first quad of that weight
   const uint32_t bpc = w.k / 32;
   const uint32_t bpc_pad = (bpc + 15) & ~15u;
   const uint32_t plane = bpc_pad * NJ;
@@ -219,9 +246,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t ks = wave % ksc, wn = wave / ksc;
   const uint32_t b = lane >> 2, i = lane & 3;
-  const uint32_t quad0 = blockIdx.x * wnc * QPW;
+  const uint32_t quad0 = blockIdx.x * wnc * QPW;  // first quad of the workgroup, numbered over the whole batch
   const uint32_t nquads = (w.n + 3) / 4;
-  const uint32_t quad = quad0 + wn * QPW;  // first of this wave's QPW quads
+  const uint32_t quad = quad0 + wn * QPW - quad_base;  // first of this wave's QPW quads, within its weight
   const uint32_t steps_total = bpc_pad / 16;
   const uint32_t step_begin = ks * STEPS;
   // a wave past the last K step (or past the last quad) keeps running on the zero block:
@@ -463,12 +490,17 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(WeightView w, const flo
   // ---- combine the K splits, add the residual, store ----
   for (uint32_t t = tid; t < wnc * MROWS * 4; t += blockDim.x) {
     const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
-    const uint32_t n = (quad0 + ql) * 4 + col;
-    if (r < m && n < w.n) {
+    // the quads of a workgroup may belong to different weights of the batch
+    const uint32_t gq = quad0 + ql;
+    const uint32_t wi = (gq >= bt.first_quad[1] ? 1u : 0u) + (gq >= bt.first_quad[2] ? 1u : 0u);
+    const uint32_t wn_cols = pick3(wi, bt.w[0].n, bt.w[1].n, bt.w[2].n);
+    const uint32_t n = (gq - pick3(wi, 0u, bt.first_quad[1], bt.first_quad[2])) * 4 + col;
+    if (r < m && n < wn_cols) {
       float v = 0.0f;
       for (uint32_t s = 0; s < ksc; s++) v += red[((ql * ksc + s) * MROWS + r) * 4 + col];
-      const size_t o = (size_t)r * w.n + n;
-      c[o] = dres ? v + dres[o] : v;
+      const size_t o = (size_t)r * wn_cols + n;
+      const float* const dd = pick3(wi, bt.d[0], bt.d[1], bt.d[2]);
+      pick3(wi, bt.c[0], bt.c[1], bt.c[2])[o] = dd ? v + dd[o] : v;
     }
   }
   MGN_STAMP(12);
@@ -482,10 +514,11 @@ struct MfmaGemvPlan {
 
 constexpr uint32_t kMaxSteps = 8;  // blocks a lane holds in flight: 8 x 20 B (Q4) or 8 x 34 B (Q8)
 
-bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, bool fused_prologue, MfmaGemvPlan* out) {
+// `nquads`: column quads over all weights of the launch; `one_quad_per_wave`: fused prologues
+// and batches of several weights come with QPW = 1 only.
+bool plan_mfma_gemv(uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bool one_quad_per_wave, MfmaGemvPlan* out) {
   const uint32_t bpc = k / 32, bpc_pad = (bpc + 15) & ~15u;
   const uint32_t steps_total = bpc_pad / 16;
-  const uint32_t nquads = (n + 3) / 4;
   MfmaGemvPlan p{};
   // K splits: at least enough that a wave's share fits in its registers; more when there
   // are too few column quads to give every CU a handful of waves
@@ -498,7 +531,7 @@ bool plan_mfma_gemv(uint32_t k, uint32_t n, uint32_t mrows, int num_cus, bool fu
   // quads per wave: with a short K and very many columns a wave takes several quads, as
   // long as that leaves at least 8 waves per CU
   p.qpw = 1;
-  if (p.ksc == 1 && !fused_prologue)
+  if (p.ksc == 1 && !one_quad_per_wave)
     while (p.qpw < 4 && p.steps * p.qpw * 2 <= kMaxSteps && nquads / (p.qpw * 2) >= (uint32_t)num_cus * 8) p.qpw *= 2;
   // waves per workgroup: spread the quads evenly over the CUs (one workgroup per CU when
   // there is enough work), so the activations are prepared as few times as possible
@@ -528,8 +561,22 @@ int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
     big_lds_enabled = true;
   }
   const GemvPrologue pro{x.pro_weight, x.pro_eps};
-  hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, x.w, (const float*)x.a, x.d, x.c, x.m,
-                     p.ksc, pro MGN_TRACE_ARG);
+  GemvBatch bt{};
+  uint32_t quads = 0;
+  for (int j = 0; j < kMaxBatch; j++) {
+    if (j == 0 || j <= x.n_more) {
+      bt.w[j] = j == 0 ? x.w : x.more[j - 1].w;
+      bt.d[j] = j == 0 ? x.d : x.more[j - 1].d;
+      bt.c[j] = j == 0 ? x.c : x.more[j - 1].c;
+      bt.first_quad[j] = quads;
+      quads += (bt.w[j].n + 3) / 4;
+    } else {
+      bt.w[j] = x.w;
+      bt.first_quad[j] = 0xFFFFFFFFu;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, bt, (const float*)x.a, x.m, p.ksc,
+                     pro MGN_TRACE_ARG);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }
@@ -544,10 +591,17 @@ int launch_steps(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
   return launch_pro<FMT, MROWS, STEPS, QPW, kProNone>(s, x, p);
 }
 
+uint32_t total_quads(const LaunchArgs& x) {
+  uint32_t q = (x.w.n + 3) / 4;
+  for (int j = 0; j < x.n_more; j++) q += (x.more[j].w.n + 3) / 4;
+  return q;
+}
+
 template <int FMT, int MROWS>
 int launch_t(ihipStream_t* s, const LaunchArgs& x) {
   MfmaGemvPlan p;
-  if (!plan_mfma_gemv(x.w.k, x.w.n, MROWS, x.num_cus, x.pro_kind != kProNone, &p)) return (int)hipErrorInvalidValue;
+  if (!plan_mfma_gemv(x.w.k, total_quads(x), MROWS, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p))
+    return (int)hipErrorInvalidValue;
   switch (p.steps * 8 + p.qpw) {
     case 1 * 8 + 1: return launch_steps<FMT, MROWS, 1, 1>(s, x, p);
     case 1 * 8 + 2: return launch_steps<FMT, MROWS, 1, 2>(s, x, p);
@@ -572,7 +626,10 @@ int launch_t(ihipStream_t* s, const LaunchArgs& x) {
 bool gemv_mfma_supported(const LaunchArgs& x) {
   if (x.a_is_f16 || x.m == 0 || x.m > 2) return false;
   MfmaGemvPlan p;
-  return plan_mfma_gemv(x.w.k, x.w.n, x.m, x.num_cus, x.pro_kind != kProNone, &p);
+  for (int j = 0; j < x.n_more; j++)
+    if (x.more[j].w.k != x.w.k || x.more[j].w.fmt != x.w.fmt) return false;
+  if (x.n_more < 0 || x.n_more > kMaxBatch - 1) return false;
+  return plan_mfma_gemv(x.w.k, total_quads(x), x.m, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p);
 }
 
 int launch_matmul_gemv_mfma(ihipStream_t* s, const LaunchArgs& x) {

@@ -424,6 +424,41 @@ mgn_status mgn_matmul_q_swiglu(mgn_ctx* ctx, const mgn_buf* gate_up, const mgn_w
   return matmul_impl(ctx, gate_up, false, w, d, c, m, mgn::kProSwiglu);
 }
 
+mgn_status mgn_matmul_q_batch(mgn_ctx* ctx, const mgn_buf* a, mgn_prologue prologue, const mgn_buf* norm_weight, float eps,
+                              const mgn_matmul_item* items, size_t count, uint32_t m) {
+  if (!ctx || !a || !items) return fail(ctx, MGN_EINVAL, "null argument");
+  if (count == 0 || count > 3) return fail(ctx, MGN_EINVAL, "a batch holds 1 to 3 matmuls");
+  if (prologue < MGN_PROLOGUE_NONE || prologue > MGN_PROLOGUE_SWIGLU) return fail(ctx, MGN_EINVAL, "unknown prologue");
+  if (m == 0) return MGN_OK;
+  for (size_t j = 0; j < count; j++)
+    if (!items[j].w || !items[j].c) return fail(ctx, MGN_EINVAL, "null weight or output in the batch");
+  const mgn_weight* w0 = items[0].w;
+  const size_t k = w0->rows;
+  const size_t a_cols = prologue == MGN_PROLOGUE_SWIGLU ? 2 * k : k;
+  if (a->bytes / 4 < (size_t)m * a_cols) return fail(ctx, MGN_EINVAL, "A is smaller than its m rows");
+  if (prologue == MGN_PROLOGUE_RMS_NORM && (!norm_weight || norm_weight->bytes / 4 < k))
+    return fail(ctx, MGN_EINVAL, "norm weight is missing or shorter than K floats");
+  mgn::LaunchArgs x{view_of(w0), a->ptr, items[0].d ? (const float*)items[0].d->ptr : nullptr, (float*)items[0].c->ptr, m,
+                    false, ctx->num_cus};
+  for (size_t j = 0; j < count; j++) {
+    const mgn_matmul_item& it = items[j];
+    if (it.w->rows != k || it.w->fmt != w0->fmt) return fail(ctx, MGN_EINVAL, "batched weights must share K and the format");
+    if (it.c->bytes / 4 < (size_t)m * it.w->cols) return fail(ctx, MGN_EINVAL, "C is smaller than m*N floats");
+    if (it.d && it.d->bytes / 4 < (size_t)m * it.w->cols) return fail(ctx, MGN_EINVAL, "D is smaller than m*N floats");
+    if (it.c->ptr == a->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
+    if (j > 0) x.more[j - 1] = {view_of(it.w), it.d ? (const float*)it.d->ptr : nullptr, (float*)it.c->ptr};
+  }
+  x.n_more = (int)count - 1;
+  x.pro_kind = (int)prologue;
+  x.pro_weight = norm_weight ? (const float*)norm_weight->ptr : nullptr;
+  x.pro_eps = eps;
+  if ((ctx->route != MGN_ROUTE_AUTO && ctx->route != MGN_ROUTE_GEMV_MFMA) || !mgn::gemv_mfma_supported(x))
+    return fail(ctx, MGN_EUNSUPPORTED, "batched matmul needs the GEMV_MFMA route (f32 activations, M <= 2)");
+  const int rc = mgn::launch_matmul_gemv_mfma(ctx->stream, x);
+  if (rc != 0) return hip_fail(ctx, "kernel launch", (hipError_t)rc);
+  return MGN_OK;
+}
+
 int mgn_matmul_q_can_fuse(mgn_ctx* ctx, const mgn_weight* w, uint32_t m) {
   if (!ctx || !w || m == 0) return 0;
   mgn::LaunchArgs x{view_of(w), nullptr, nullptr, nullptr, m, false, ctx->num_cus};

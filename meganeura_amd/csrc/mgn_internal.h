@@ -45,6 +45,15 @@ struct LaunchArgs {
   uint32_t m;
   bool a_is_f16;
   int num_cus;
+  // further weights served by the same launch (GEMV-MFMA route only): same K, format and
+  // activations, each with its own output and optional residual
+  struct More {
+    WeightView w;
+    const float* d;
+    float* c;
+  };
+  More more[2] = {};
+  int n_more = 0;
   // fused prologue (GEMV-MFMA route only): what `a` goes through before the matmul
   int pro_kind = 0;                   // kProNone / kProRmsNorm / kProSwiglu
   const float* pro_weight = nullptr;  // norm weight [K]

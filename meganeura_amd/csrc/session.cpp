@@ -520,7 +520,38 @@ void Session::plan_launches() {
     }
     if (!ok) continue;
     skipped_[pi] = 1;
-    for (int ci : readers[out]) fused_[ci] = Fused{norm ? kProRmsNorm : kProSwiglu, (int)pi};
+    for (int ci : readers[out]) {
+      fused_[ci].kind = norm ? kProRmsNorm : kProSwiglu;
+      fused_[ci].producer = (int)pi;
+    }
+  }
+  // Sibling decode matmuls: same activations (and prologue), same K and format.  The later
+  // ones move up to the first one's launch, which is legal when whatever else they read (the
+  // residual) already exists at that point.
+  std::vector<int> producer_of(plan_.buffers.size(), -1);
+  for (size_t i = 0; i < nd; i++) producer_of[plan_.dispatches[i].output_buffer] = (int)i;
+  auto batchable = [&](size_t i) {
+    const Dispatch& d = plan_.dispatches[i];
+    if (skipped_[i] || !is_matmul(d.shader)) return false;
+    mgn_weight* w = weights_[d.input_buffers[1]];
+    return w && mgn_matmul_q_can_fuse(ctx_, w, d.params[0]) == 1;
+  };
+  for (size_t i = 0; i < nd; i++) {
+    if (!batchable(i)) continue;
+    const Dispatch& di = plan_.dispatches[i];
+    int found = 0;
+    for (size_t j = i + 1; j < nd && found < 2; j++) {
+      if (!batchable(j)) continue;
+      const Dispatch& dj = plan_.dispatches[j];
+      const bool same_src = dj.input_buffers[0] == di.input_buffers[0] && fused_[j].kind == fused_[i].kind &&
+                            fused_[j].producer == fused_[i].producer;
+      const bool same_shape = dj.params[0] == di.params[0] && dj.params[1] == di.params[1] &&
+                              dj.weight_format == di.weight_format;
+      const bool addend_ready = dj.input_buffers.size() < 3 || producer_of[dj.input_buffers[2]] < (int)i;
+      if (!same_src || !same_shape || !addend_ready) continue;
+      fused_[i].more[found++] = (int)j;
+      skipped_[j] = 1;
+    }
   }
 }
 
@@ -541,7 +572,22 @@ void Session::run_dispatches() {
         if (!w) throw std::runtime_error("quantized parameter was never set");
         const mgn_buf* addend = d.input_buffers.size() > 2 ? buffers_[d.input_buffers[2]] : nullptr;
         const Fused& f = fused_[di];
-        if (f.kind == kProRmsNorm) {
+        if (f.more[0] >= 0) {
+          mgn_matmul_item items[3] = {{w, addend, buffers_[d.output_buffer]}, {}, {}};
+          size_t count = 1;
+          for (int sib : f.more) {
+            if (sib < 0) continue;
+            const Dispatch& sd = plan_.dispatches[sib];
+            items[count++] = {weights_[sd.input_buffers[1]],
+                              sd.input_buffers.size() > 2 ? buffers_[sd.input_buffers[2]] : nullptr,
+                              buffers_[sd.output_buffer]};
+          }
+          const Dispatch* p = f.kind != kProNone ? &plan_.dispatches[f.producer] : nullptr;
+          const mgn_buf* act = p ? buffers_[p->input_buffers[0]] : buffers_[d.input_buffers[0]];
+          const mgn_buf* nw = f.kind == kProRmsNorm ? buffers_[p->input_buffers[1]] : nullptr;
+          check(mgn_matmul_q_batch(ctx_, act, (mgn_prologue)f.kind, nw, p ? p->eps : 0.0f, items, count, d.params[0]),
+                "mgn_matmul_q_batch");
+        } else if (f.kind == kProRmsNorm) {
           const Dispatch& p = plan_.dispatches[f.producer];
           check(mgn_matmul_q_rms_norm(ctx_, buffers_[p.input_buffers[0]], buffers_[p.input_buffers[1]], p.eps, w, addend,
                                       buffers_[d.output_buffer], d.params[0]),

@@ -146,8 +146,8 @@ class Session {
   // are a single graph launch.  Results are identical; only launch overhead changes --
   // less host work per step, but measured slower on the GPU side for chains of tiny kernels.
   void set_graph_replay(bool on);
-  // Fold RmsNorm / SwiGLUConcat dispatches into the decode matmuls that consume them
-  // (default on).  The plan keeps the reference's dispatch list; only the launches differ.
+  // Fold RmsNorm / SwiGLUConcat dispatches into the decode matmuls that consume them and
+  // serve sibling decode matmuls (same activations, e.g. q/k/v) with one launch (default on).  The plan keeps the reference's dispatch list; only the launches differ.
   void set_fusion(bool on);
   size_t num_launches();  // kernel launches one step makes with the current settings
   bool graph_active() const { return exec_ != nullptr; }
@@ -164,8 +164,9 @@ class Session {
   void drop_graph();
   void plan_launches();
   struct Fused {
-    int kind = 0;       // kProNone / kProRmsNorm / kProSwiglu
-    int producer = -1;  // the folded-in dispatch
+    int kind = 0;          // kProNone / kProRmsNorm / kProSwiglu
+    int producer = -1;     // the folded-in dispatch
+    int more[2] = {-1, -1};  // sibling matmuls (same activations) served by this dispatch's launch
   };
   std::vector<Fused> fused_;     // per dispatch (matmuls only)
   std::vector<char> skipped_;    // per dispatch: folded into its consumers

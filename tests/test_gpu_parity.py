@@ -274,3 +274,47 @@ def test_fused_prologue_is_refused_where_it_cannot_run(ctx):
     for b in (x, g, c, short):
         b.free()
     wt.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m,k,ns", [(1, 576, (576, 192, 192)), (2, 576, (64, 6)), (1, 4096, (1024, 132, 4096)), (1, 64, (8, 4, 12))])
+def test_batched_matmuls_share_one_launch(ctx, orc, fmt, m, k, ns):
+    """Up to three weights on the same activations in one launch (q, k, v), with and without
+    a prologue and residuals.  The K split is planned for the whole batch, so the summation
+    order may differ from the single-weight launch: compared at the matmul bar, not bitwise."""
+    x = synth.normal(700 + k, m * k, 1.0).reshape(m, k)
+    xb = ctx.upload(x)
+    ws = [synth.normal(701 + j, k * n, 0.02).reshape(k, n) for j, n in enumerate(ns)]
+    wts = [ctx.weight(fmt, w) for w in ws]
+    ds = [synth.normal(710 + j, m * n, 1.0).reshape(m, n) if j == 1 else None for j, n in enumerate(ns)]
+    dbs = [ctx.upload(d) if d is not None else None for d in ds]
+    cs = [ctx.buffer(m * n * 4) for n in ns]
+    single = ctx.buffer(m * max(ns) * 4)
+    ctx.set_route(capi.ROUTE_GEMV_MFMA)
+    try:
+        ctx.matmul_q_batch(xb, list(zip(wts, cs, dbs)), m)
+        for j, n in enumerate(ns):
+            got = cs[j].download(np.float32, m * n).reshape(m, n)
+            orc.assert_close(got, orc.matmul_packed(fmt, x, orc.quantize(fmt, ws[j]), n, ds[j]), REL, ABS)
+            ctx.matmul_q(xb, wts[j], single, m, dbs[j])
+            orc.assert_close(single.download(np.float32, m * n).reshape(m, n), got, REL, ABS)
+        # with the norm folded in
+        g = ctx.upload(1.0 + 0.25 * synth.normal(720, k, 1.0))
+        ctx.matmul_q_batch(xb, list(zip(wts, cs, dbs)), m, capi.PROLOGUE_RMS_NORM, g, 1e-5)
+        for j, n in enumerate(ns):
+            got = cs[j].download(np.float32, m * n)
+            ctx.matmul_q_rms_norm(xb, g, 1e-5, wts[j], single, m, dbs[j])
+            orc.assert_close(single.download(np.float32, m * n), got, REL, ABS)
+        g.free()
+    finally:
+        ctx.set_route(capi.ROUTE_AUTO)
+    # different K in one batch is an argument error
+    other = ctx.weight(fmt, synth.normal(730, 2 * k * 8, 0.02).reshape(2 * k, 8))
+    with pytest.raises(capi.MgnError) as e:
+        ctx.matmul_q_batch(xb, [(wts[0], cs[0], None), (other, cs[1], None)], m)
+    assert e.value.status == capi.EINVAL
+    other.free()
+    for b in [xb, single] + cs + [d for d in dbs if d is not None]:
+        b.free()
+    for w in wts:
+        w.free()
