@@ -208,8 +208,8 @@ def cpu_baseline(wl, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
     ap.add_argument("--sweep", action="store_true", help="also measure every configuration (stderr)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
