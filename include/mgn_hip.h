@@ -111,6 +111,17 @@ mgn_status mgn_weight_create(mgn_ctx* ctx, mgn_fmt fmt, const float* w, size_t r
  * back into a Q4/Q8 buffer, src/runtime.rs:4256-4265). */
 mgn_status mgn_weight_create_packed(mgn_ctx* ctx, mgn_fmt fmt, const uint8_t* packed, size_t rows,
                                     size_t cols, mgn_weight** out);
+/* A weight stored [N, K] row-major: the B operand of Graph::matmul_bt (src/graph.rs:809-817,
+ * lowering src/compile.rs:1447-1485), which is how weight-tied lm_heads keep their embedding
+ * table (models/smollm2.rs:413-414).  Blocks run along K -- contiguous in this storage -- so
+ * the result is the same weight, byte for byte, as mgn_weight_create on the transposed [K, N]
+ * matrix, and C = A x B^T is then mgn_matmul_q with it.  (The reference's set_parameter blocks
+ * such a parameter along shape[0] = N while its shader reads it along K, src/compile.rs:1233-1239;
+ * that inconsistency is not reproduced.)  mgn_quantize_ref_nk is the host-only form; its
+ * output has the reference byte layout for rows = K, cols = N. */
+mgn_status mgn_quantize_ref_nk(mgn_fmt fmt, const float* w_nk, size_t n_rows, size_t k_cols, uint8_t* out);
+mgn_status mgn_weight_create_nk(mgn_ctx* ctx, mgn_fmt fmt, const float* w_nk, size_t n_rows, size_t k_cols,
+                                mgn_weight** out);
 /* Same from an f32 [rows, cols] matrix already on the device: the block
  * quantizer runs as a kernel, bit-exact with mgn_quantize_ref. */
 mgn_status mgn_weight_create_device(mgn_ctx* ctx, mgn_fmt fmt, const mgn_buf* w_f32, size_t rows,

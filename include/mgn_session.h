@@ -33,7 +33,9 @@ typedef enum mgn_shader {
   MGN_SHADER_ADD = 4,
   MGN_SHADER_SWIGLU = 5,
   MGN_SHADER_SWIGLU_CONCAT = 6,
-  MGN_SHADER_RMS_NORM = 7
+  MGN_SHADER_RMS_NORM = 7,
+  MGN_SHADER_MATMUL_BT = 8,      /* ShaderEntry::MatMulBT:     C = A x B^T, B stored [N, K] */
+  MGN_SHADER_MATMUL_GEMV_BT = 9  /* ShaderEntry::MatMulGemvBT: its M = 1 form */
 } mgn_shader;
 
 /* compile::Dispatch (src/compile.rs:435-488), the fields this path uses.
@@ -41,7 +43,7 @@ typedef enum mgn_shader {
 typedef struct mgn_dispatch_info {
   int32_t shader;          /* mgn_shader */
   uint32_t workgroups[3];  /* the grid the reference would launch */
-  uint32_t params[4];      /* [m, k, n, 0] for matmuls */
+  uint32_t params[4];      /* [m, k, n, 0] for matmuls, [m, n, k, 0] for the BT forms */
   int32_t weight_format;
 } mgn_dispatch_info;
 
@@ -56,6 +58,9 @@ int32_t mgn_graph_parameter(mgn_graph* g, const char* name, size_t rows, size_t 
 int32_t mgn_graph_parameter_q4(mgn_graph* g, const char* name, size_t rows, size_t cols);
 int32_t mgn_graph_parameter_q8(mgn_graph* g, const char* name, size_t rows, size_t cols);
 int32_t mgn_graph_matmul(mgn_graph* g, int32_t a, int32_t b);
+/* Graph::matmul_bt (src/graph.rs:809-817): a[M,K], b[N,K] -> [M,N].  With a quantized b the
+ * parameter is blocked along K (see mgn_weight_create_nk). */
+int32_t mgn_graph_matmul_bt(mgn_graph* g, int32_t a, int32_t b);
 int32_t mgn_graph_add(mgn_graph* g, int32_t a, int32_t b);
 int32_t mgn_graph_swiglu(mgn_graph* g, int32_t gate, int32_t up);
 int32_t mgn_graph_rms_norm(mgn_graph* g, int32_t x, int32_t weight, float eps);

@@ -20,14 +20,14 @@ HIP_SYMBOLS = [
     "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync", "mgn_ctx_set_route",
     "mgn_buf_alloc", "mgn_buf_free", "mgn_buf_size", "mgn_buf_device_ptr", "mgn_buf_upload",
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
-    "mgn_weight_create", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
+    "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_matmul_q",
     "mgn_matmul_q_f16a", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
     "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [
     "mgn_graph_new", "mgn_graph_free", "mgn_graph_last_error", "mgn_graph_input", "mgn_graph_parameter",
-    "mgn_graph_parameter_q4", "mgn_graph_parameter_q8", "mgn_graph_matmul", "mgn_graph_add",
+    "mgn_graph_parameter_q4", "mgn_graph_parameter_q8", "mgn_graph_matmul", "mgn_graph_matmul_bt", "mgn_graph_add",
     "mgn_graph_swiglu", "mgn_graph_rms_norm", "mgn_graph_set_outputs", "mgn_graph_compile",
     "mgn_build_inference_session", "mgn_session_free", "mgn_session_last_error",
     "mgn_session_num_dispatches", "mgn_session_dispatch_info", "mgn_session_set_parameter",
@@ -91,6 +91,8 @@ def load():
         "mgn_quantize_ref": (C.c_int, [C.c_int, vp, sz, sz, vp]),
         "mgn_dequantize_ref": (C.c_int, [C.c_int, vp, sz, sz, vp]),
         "mgn_weight_create": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
+        "mgn_weight_create_nk": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
+        "mgn_quantize_ref_nk": (C.c_int, [C.c_int, vp, sz, sz, vp]),
         "mgn_weight_create_packed": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
         "mgn_weight_create_device": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
         "mgn_weight_free": (None, [vp, vp]),
@@ -115,6 +117,7 @@ def load():
         "mgn_graph_parameter_q4": (C.c_int32, [vp, C.c_char_p, sz, sz]),
         "mgn_graph_parameter_q8": (C.c_int32, [vp, C.c_char_p, sz, sz]),
         "mgn_graph_matmul": (C.c_int32, [vp, C.c_int32, C.c_int32]),
+        "mgn_graph_matmul_bt": (C.c_int32, [vp, C.c_int32, C.c_int32]),
         "mgn_graph_add": (C.c_int32, [vp, C.c_int32, C.c_int32]),
         "mgn_graph_swiglu": (C.c_int32, [vp, C.c_int32, C.c_int32]),
         "mgn_graph_rms_norm": (C.c_int32, [vp, C.c_int32, C.c_int32, C.c_float]),
@@ -162,6 +165,17 @@ def quantize_ref(fmt, w):
     st = load().mgn_quantize_ref(fmt, _ptr(w), rows, cols, _ptr(out))
     if st != OK:
         raise MgnError(st, "quantize_ref: rows (K dim) must be a multiple of 32")
+    return out
+
+
+def quantize_ref_nk(fmt, w_nk):
+    """Packed bytes (reference layout for rows = K, cols = N) of a weight stored [N, K]."""
+    w_nk = np.ascontiguousarray(w_nk, dtype=np.float32)
+    n, k = w_nk.shape
+    out = np.zeros(packed_size(fmt, k, n), dtype=np.uint8)
+    st = load().mgn_quantize_ref_nk(fmt, _ptr(w_nk), n, k, _ptr(out))
+    if st != OK:
+        raise MgnError(st, "quantize_ref_nk: K must be a multiple of 32")
     return out
 
 
@@ -241,6 +255,13 @@ class Context:
         h = C.c_void_p()
         self.check(self.lib.mgn_weight_create(self.h, fmt, _ptr(w), w.shape[0], w.shape[1], C.byref(h)))
         return Weight(self, h, fmt, w.shape[0], w.shape[1])
+
+    def weight_nk(self, fmt, w_nk):
+        """Weight from an [N, K] matrix (matmul_bt operand); the handle is a [K, N] weight."""
+        w_nk = np.ascontiguousarray(w_nk, dtype=np.float32)
+        h = C.c_void_p()
+        self.check(self.lib.mgn_weight_create_nk(self.h, fmt, _ptr(w_nk), w_nk.shape[0], w_nk.shape[1], C.byref(h)))
+        return Weight(self, h, fmt, w_nk.shape[1], w_nk.shape[0])
 
     def weight_from_packed(self, fmt, packed, rows, cols):
         packed = np.ascontiguousarray(packed, dtype=np.uint8)

@@ -40,6 +40,8 @@
 // of a column are summed once per column quad.  The activations' A operands
 // are prepared once per workgroup in LDS, laid out so that consecutive lanes
 // read consecutive 16-byte chunks.
+#include <cstdlib>
+
 #include "kernels_common.hip.h"
 
 #ifdef MGN_TRACE
@@ -538,6 +540,9 @@ bool plan_mfma_gemv(uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bo
   const uint32_t max_wnc = 16 / p.ksc;
   const uint32_t wave_quads = (nquads + p.qpw - 1) / p.qpw;  // quad groups = waves with work
   p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (wave_quads + num_cus - 1) / num_cus));
+#ifdef MGN_TRACE  // development build only: force the waves per workgroup
+  if (const char* e = getenv("MGN_DEV_WNC")) p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (uint32_t)atoi(e)));
+#endif
   // enough threads to prepare the activations (waves without a quad only help there)
   const uint32_t prep_waves = (bpc_pad * 4 + kMaxTasks * 64 - 1) / (kMaxTasks * 64);
   p.wnc = std::max<uint32_t>(p.wnc, (prep_waves + p.ksc - 1) / p.ksc);

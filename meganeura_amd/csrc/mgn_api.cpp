@@ -224,6 +224,15 @@ mgn_status mgn_quantize_ref(mgn_fmt fmt, const float* w, size_t rows, size_t col
   return MGN_OK;
 }
 
+mgn_status mgn_quantize_ref_nk(mgn_fmt fmt, const float* w_nk, size_t n_rows, size_t k_cols, uint8_t* out) {
+  if (!valid_fmt(fmt) || k_cols % 32 != 0) return MGN_EINVAL;
+  if (n_rows == 0 || k_cols == 0) return MGN_OK;
+  if (!w_nk || !out) return MGN_EINVAL;
+  if (fmt == MGN_FMT_Q4) mgn::quantize_q4_host_nk(w_nk, n_rows, k_cols, out);
+  else mgn::quantize_q8_host_nk(w_nk, n_rows, k_cols, out);
+  return MGN_OK;
+}
+
 mgn_status mgn_dequantize_ref(mgn_fmt fmt, const uint8_t* in, size_t rows, size_t cols, float* out) {
   if (!valid_fmt(fmt) || rows % 32 != 0) return MGN_EINVAL;
   if (rows == 0 || cols == 0) return MGN_OK;
@@ -279,6 +288,23 @@ mgn_status mgn_weight_create(mgn_ctx* ctx, mgn_fmt fmt, const float* wdata, size
   }
   mgn_quantize_ref(fmt, wdata, rows, cols, packed.data());
   return mgn_weight_create_packed(ctx, fmt, packed.data(), rows, cols, out);
+}
+
+mgn_status mgn_weight_create_nk(mgn_ctx* ctx, mgn_fmt fmt, const float* w_nk, size_t n_rows, size_t k_cols,
+                                mgn_weight** out) {
+  if (!ctx || !out || !w_nk) return fail(ctx, MGN_EINVAL, "null argument");
+  *out = nullptr;
+  if (!valid_fmt(fmt)) return fail(ctx, MGN_EINVAL, "unknown weight format");
+  if (k_cols % 32 != 0) return fail(ctx, MGN_EINVAL, "quantized weights require the K dim to be a multiple of 32");
+  if (n_rows == 0 || k_cols == 0) return fail(ctx, MGN_EINVAL, "empty weight");
+  std::vector<uint8_t> packed;
+  try {
+    packed.resize(mgn_packed_size(fmt, k_cols, n_rows));
+  } catch (const std::bad_alloc&) {
+    return fail(ctx, MGN_ENOMEM, "out of host memory");
+  }
+  mgn_quantize_ref_nk(fmt, w_nk, n_rows, k_cols, packed.data());
+  return mgn_weight_create_packed(ctx, fmt, packed.data(), k_cols, n_rows, out);
 }
 
 mgn_status mgn_weight_create_device(mgn_ctx* ctx, mgn_fmt fmt, const mgn_buf* w_f32, size_t rows, size_t cols,

@@ -16,6 +16,8 @@ uint16_t f32_to_f16_bits(float f);
 float f16_bits_to_f32(uint16_t h);
 void quantize_q4_host(const float* w, size_t rows, size_t cols, uint8_t* out);
 void quantize_q8_host(const float* w, size_t rows, size_t cols, uint8_t* out);
+void quantize_q4_host_nk(const float* w_nk, size_t n_rows, size_t k_cols, uint8_t* out);
+void quantize_q8_host_nk(const float* w_nk, size_t n_rows, size_t k_cols, uint8_t* out);
 void dequantize_q4_host(const uint8_t* in, size_t rows, size_t cols, float* out);
 void dequantize_q8_host(const uint8_t* in, size_t rows, size_t cols, float* out);
 

@@ -127,6 +127,61 @@ void quantize_q4_host(const float* w, size_t rows, size_t cols, uint8_t* out) {
   });
 }
 
+// The same encoders for a weight stored [N, K] row-major (the B operand of matmul_bt,
+// src/graph.rs:809-817): block (n, kb) covers w_nk[n][kb*32 .. kb*32+31], contiguous in
+// memory, and lands where quantizing the transposed [K, N] matrix would put it.
+void quantize_q4_host_nk(const float* w_nk, size_t n_rows, size_t k_cols, uint8_t* out) {
+  const size_t bpc = k_cols / 32, nb = bpc * n_rows;
+  uint8_t* dm_base = out;
+  uint8_t* q_base = out + nb * 4;
+  parallel_rows(n_rows, [&](size_t n) {
+    for (size_t blk = 0; blk < bpc; blk++) {
+      const float* v = w_nk + n * k_cols + blk * 32;
+      float bmin = INFINITY, bmax = -INFINITY;
+      for (int i = 0; i < 32; i++) {
+        if (v[i] < bmin) bmin = v[i];
+        if (v[i] > bmax) bmax = v[i];
+      }
+      const float d = bmax > bmin ? (bmax - bmin) / 15.0f : 1.0f;
+      const float m = bmin;
+      const float d_inv = d > 0.0f ? 1.0f / d : 0.0f;
+      const size_t b = n * bpc + blk;
+      const uint32_t dm = uint32_t(f32_to_f16_bits(d)) | (uint32_t(f32_to_f16_bits(m)) << 16);
+      std::memcpy(dm_base + b * 4, &dm, 4);
+      uint8_t* q = q_base + b * 16;
+      for (int j = 0; j < 16; j++) {
+        float t0 = clamp_keep_nan(std::round((v[2 * j] - m) * d_inv), 0.0f, 15.0f);
+        float t1 = clamp_keep_nan(std::round((v[2 * j + 1] - m) * d_inv), 0.0f, 15.0f);
+        uint8_t n0 = t0 != t0 ? 0 : uint8_t(t0), n1 = t1 != t1 ? 0 : uint8_t(t1);
+        q[j] = uint8_t(n0 | (n1 << 4));
+      }
+    }
+  });
+}
+
+void quantize_q8_host_nk(const float* w_nk, size_t n_rows, size_t k_cols, uint8_t* out) {
+  const size_t bpc = k_cols / 32;
+  parallel_rows(n_rows, [&](size_t n) {
+    for (size_t blk = 0; blk < bpc; blk++) {
+      const float* v = w_nk + n * k_cols + blk * 32;
+      float amax = 0.0f;
+      for (int i = 0; i < 32; i++) {
+        float a = std::fabs(v[i]);
+        if (a > amax) amax = a;
+      }
+      const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+      const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+      uint8_t* p = out + (n * bpc + blk) * 36;
+      const uint32_t head = f32_to_f16_bits(scale);  // pad bytes 2..3 stay zero
+      std::memcpy(p, &head, 4);
+      for (int i = 0; i < 32; i++) {
+        float t = clamp_keep_nan(std::round(v[i] * inv), -128.0f, 127.0f);
+        p[4 + i] = uint8_t(int8_t(t != t ? 0 : int(t)));
+      }
+    }
+  });
+}
+
 void quantize_q8_host(const float* w, size_t rows, size_t cols, uint8_t* out) {
   const size_t bpc = rows / 32;
   parallel_rows(bpc, [&](size_t blk) {

@@ -54,6 +54,15 @@ NodeId Graph::matmul(NodeId a, NodeId b) {
   return add_raw_node(Op::MatMul, {a, b}, TensorType{{as[0], bs[1]}, DType::F32});
 }
 
+// src/graph.rs:809-817
+NodeId Graph::matmul_bt(NodeId a, NodeId b) {
+  const auto& as = node(a).ty.shape;
+  const auto& bs = node(b).ty.shape;
+  if (as.size() != 2 || bs.size() != 2) throw GraphError("matmul_bt requires 2D tensors");
+  if (as[1] != bs[1]) throw GraphError("MatMulBT: K dimensions must match");
+  return add_raw_node(Op::MatMulBT, {a, b}, TensorType{{as[0], bs[0]}, DType::F32});
+}
+
 // src/graph.rs:821-827
 NodeId Graph::add(NodeId a, NodeId b) {
   if (node(a).ty.shape != node(b).ty.shape) throw GraphError("add requires matching shapes");
@@ -226,6 +235,23 @@ ExecutionPlan compile(const Graph& g) {
       plan.input_buffers.push_back({nd.name, buf});
     }
   }
+  // a quantized parameter read by matmul_bt is blocked along its second dimension
+  for (const Node& nd : g.nodes()) {
+    if (nd.op != Op::MatMul && nd.op != Op::MatMulBT && nd.op != Op::FusedMatMulAdd) continue;
+    auto it = node_buf.find(nd.inputs[1]);
+    if (it == node_buf.end()) continue;
+    auto wb = plan.weight_buffers.find(it->second);
+    if (wb == plan.weight_buffers.end()) continue;
+    if (nd.op == Op::MatMulBT) wb->second.nk = true;
+  }
+  for (const Node& nd : g.nodes()) {
+    if (nd.op != Op::MatMul && nd.op != Op::FusedMatMulAdd) continue;
+    auto it = node_buf.find(nd.inputs[1]);
+    if (it == node_buf.end()) continue;
+    auto wb = plan.weight_buffers.find(it->second);
+    if (wb != plan.weight_buffers.end() && wb->second.nk)
+      throw GraphError("a quantized parameter cannot feed both matmul and matmul_bt: its blocks run along one dimension only");
+  }
   for (const DerivedParam& dp : g.derived_params) {
     for (const auto& pb : plan.param_buffers)
       if (pb.first == dp.name) plan.derived_params.push_back({pb.second, dp.sources, dp.rows});
@@ -263,6 +289,24 @@ ExecutionPlan compile(const Graph& g) {
         d.input_buffers = {buf_of(nd.inputs[0]), buf_of(nd.inputs[1])};
         if (fused) d.input_buffers.push_back(buf_of(nd.inputs[2]));
         d.params[0] = m, d.params[1] = k, d.params[2] = n, d.params[3] = 0;
+        d.weight_format = weight_format_from(bn.ty.dtype);
+        break;
+      }
+      case Op::MatMulBT: {
+        // src/compile.rs:1447-1485: M == 1 and K % 4 == 0 take the GEMV-BT entry with grid
+        // [N,1,1]; everything else the 64x64 tiled one.  Parameter order [m, n, k, 0].
+        const auto& as = g.node(nd.inputs[0]).ty.shape;
+        const Node& bn = g.node(nd.inputs[1]);
+        const uint32_t m = (uint32_t)as[0], k = (uint32_t)as[1], n = (uint32_t)bn.ty.shape[0];
+        if (m == 1 && k % 4 == 0) {
+          d.shader = MGN_SHADER_MATMUL_GEMV_BT;
+          d.workgroups[0] = n, d.workgroups[1] = 1, d.workgroups[2] = 1;
+        } else {
+          d.shader = MGN_SHADER_MATMUL_BT;
+          d.workgroups[0] = (n + 63) / 64, d.workgroups[1] = (m + 63) / 64, d.workgroups[2] = 1;
+        }
+        d.input_buffers = {buf_of(nd.inputs[0]), buf_of(nd.inputs[1])};
+        d.params[0] = m, d.params[1] = n, d.params[2] = k, d.params[3] = 0;
         d.weight_format = weight_format_from(bn.ty.dtype);
         break;
       }
@@ -308,7 +352,10 @@ void Session::check(mgn_status st, const char* what) {
   if (st != MGN_OK) throw std::runtime_error(std::string(what) + ": " + mgn_last_error(ctx_));
 }
 
-static bool is_matmul(mgn_shader s) { return s <= MGN_SHADER_MATMUL_GEMV_ADD; }
+static bool is_bt(mgn_shader s) { return s == MGN_SHADER_MATMUL_BT || s == MGN_SHADER_MATMUL_GEMV_BT; }
+static bool is_matmul(mgn_shader s) { return s <= MGN_SHADER_MATMUL_GEMV_ADD || is_bt(s); }
+// K of a matmul dispatch: params are [m, k, n, 0], or [m, n, k, 0] for the BT forms
+static uint32_t matmul_k(const Dispatch& d) { return is_bt(d.shader) ? d.params[2] : d.params[1]; }
 
 Session::Session(ExecutionPlan plan, int device_id) : plan_(std::move(plan)) {
   // This backend serves matmuls whose weight is quantized; a plain f32 weight
@@ -348,7 +395,8 @@ void Session::release() {
 void Session::upload_weight(int buf, const WeightBufferInfo& info, const float* data) {
   mgn_weight* fresh = nullptr;
   const mgn_fmt fmt = info.fmt == WeightFormat::Q4 ? MGN_FMT_Q4 : MGN_FMT_Q8;
-  check(mgn_weight_create(ctx_, fmt, data, info.rows, info.cols, &fresh), "mgn_weight_create");
+  if (info.nk) check(mgn_weight_create_nk(ctx_, fmt, data, info.rows, info.cols, &fresh), "mgn_weight_create_nk");
+  else check(mgn_weight_create(ctx_, fmt, data, info.rows, info.cols, &fresh), "mgn_weight_create");
   drop_graph();  // a captured step holds the old handle's addresses
   launches_planned_ = false;
   mgn_weight_free(ctx_, weights_[buf]);  // waits for in-flight work that may still read it
@@ -514,7 +562,7 @@ void Session::plan_launches() {
     for (int ci : readers[out]) {
       const Dispatch& c = plan_.dispatches[ci];
       mgn_weight* w = is_matmul(c.shader) ? weights_[c.input_buffers[1]] : nullptr;
-      ok = ok && (size_t)ci > pi && w && c.input_buffers[0] == out && c.params[1] == width &&
+      ok = ok && (size_t)ci > pi && w && c.input_buffers[0] == out && is_matmul(c.shader) && matmul_k(c) == width &&
            (c.input_buffers.size() < 3 || c.input_buffers[2] != out) && fused_[ci].kind == 0 &&
            mgn_matmul_q_can_fuse(ctx_, w, c.params[0]) == 1;
     }
@@ -545,7 +593,7 @@ void Session::plan_launches() {
       const Dispatch& dj = plan_.dispatches[j];
       const bool same_src = dj.input_buffers[0] == di.input_buffers[0] && fused_[j].kind == fused_[i].kind &&
                             fused_[j].producer == fused_[i].producer;
-      const bool same_shape = dj.params[0] == di.params[0] && dj.params[1] == di.params[1] &&
+      const bool same_shape = dj.params[0] == di.params[0] && matmul_k(dj) == matmul_k(di) &&
                               dj.weight_format == di.weight_format;
       const bool addend_ready = dj.input_buffers.size() < 3 || producer_of[dj.input_buffers[2]] < (int)i;
       if (!same_src || !same_shape || !addend_ready) continue;
@@ -567,7 +615,9 @@ void Session::run_dispatches() {
       case MGN_SHADER_MATMUL:
       case MGN_SHADER_MATMUL_GEMV:
       case MGN_SHADER_FUSED_MATMUL_ADD:
-      case MGN_SHADER_MATMUL_GEMV_ADD: {
+      case MGN_SHADER_MATMUL_GEMV_ADD:
+      case MGN_SHADER_MATMUL_BT:
+      case MGN_SHADER_MATMUL_GEMV_BT: {
         mgn_weight* w = weights_[d.input_buffers[1]];
         if (!w) throw std::runtime_error("quantized parameter was never set");
         const mgn_buf* addend = d.input_buffers.size() > 2 ? buffers_[d.input_buffers[2]] : nullptr;
@@ -715,6 +765,9 @@ int32_t mgn_graph_parameter_q8(mgn_graph* g, const char* name, size_t rows, size
 }
 int32_t mgn_graph_matmul(mgn_graph* g, int32_t a, int32_t b) {
   return graph_node(g, [&] { return g->g.matmul((mgn::NodeId)a, (mgn::NodeId)b); });
+}
+int32_t mgn_graph_matmul_bt(mgn_graph* g, int32_t a, int32_t b) {
+  return graph_node(g, [&] { return g->g.matmul_bt((mgn::NodeId)a, (mgn::NodeId)b); });
 }
 int32_t mgn_graph_add(mgn_graph* g, int32_t a, int32_t b) {
   return graph_node(g, [&] { return g->g.add((mgn::NodeId)a, (mgn::NodeId)b); });

@@ -45,7 +45,7 @@ struct TensorType {
   }
 };
 
-enum class Op { Input, Parameter, MatMul, Add, SwiGLU, RmsNorm, FusedMatMulAdd, SwiGLUConcat, Nop };
+enum class Op { Input, Parameter, MatMul, Add, SwiGLU, RmsNorm, FusedMatMulAdd, SwiGLUConcat, Nop, MatMulBT };
 
 struct Node {
   NodeId id;
@@ -74,6 +74,7 @@ class Graph {
   NodeId parameter_q4(const std::string& name, std::vector<size_t> shape);
   NodeId parameter_q8(const std::string& name, std::vector<size_t> shape);
   NodeId matmul(NodeId a, NodeId b);
+  NodeId matmul_bt(NodeId a, NodeId b);
   NodeId add(NodeId a, NodeId b);
   NodeId swiglu(NodeId gate, NodeId up);
   NodeId rms_norm(NodeId x, NodeId weight, float eps);
@@ -110,7 +111,8 @@ struct Dispatch {
 // compile::ExecutionPlan (src/compile.rs:494-528), the fields this path uses.
 struct WeightBufferInfo {
   WeightFormat fmt;
-  size_t rows, cols;
+  size_t rows, cols;  // shape[0], shape[1] as declared
+  bool nk = false;    // read by matmul_bt: stored [N, K], blocked along K
 };
 struct ExecutionPlan {
   std::vector<size_t> buffers;  // byte sizes

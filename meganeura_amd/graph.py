@@ -27,6 +27,8 @@ class ShaderEntry(IntEnum):
     SwiGLU = 5
     SwiGLUConcat = 6
     RmsNorm = 7
+    MatMulBT = 8
+    MatMulGemvBT = 9
 
 
 class WeightFormat(IntEnum):
@@ -84,6 +86,10 @@ class Graph:
 
     def matmul(self, a, b):
         return self._node(self.lib.mgn_graph_matmul(self.h, a, b))
+
+    def matmul_bt(self, a, b):
+        """a[M,K] x b[N,K]^T (src/graph.rs:809-817)."""
+        return self._node(self.lib.mgn_graph_matmul_bt(self.h, a, b))
 
     def add(self, a, b):
         return self._node(self.lib.mgn_graph_add(self.h, a, b))

@@ -289,3 +289,29 @@ def test_norm_with_another_reader_is_not_folded():
     want = xv / np.sqrt((xv.astype(np.float64) ** 2).mean() + 1e-5)
     assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
     sess.close()
+
+
+@pytest.mark.parametrize("quant", ["q4", "q8"])
+@pytest.mark.parametrize("m,k,n", [(1, 576, 49152), (1, 64, 66), (6, 128, 200)])
+def test_matmul_bt_with_quantized_table(orc, quant, m, k, n):
+    """Weight-tied lm_head: logits = x @ embed^T with embed[vocab, hidden] quantized
+    (models/smollm2.rs:413-414).  The table is blocked along hidden (K), so the result is the
+    plain quantized matmul against embed^T."""
+    fmt = Q4 if quant == "q4" else Q8
+    g = Graph()
+    x = g.input("x", [m, k])
+    e = (g.parameter_q4 if quant == "q4" else g.parameter_q8)("embed", [n, k])
+    g.set_outputs([g.matmul_bt(x, e)])
+    sess = build_inference_session(g)
+    (d,) = sess.plan()
+    assert d.shader == (ShaderEntry.MatMulGemvBT if m == 1 else ShaderEntry.MatMulBT)
+    embed = synth.normal(900 + n, n * k, 0.02).reshape(n, k)
+    xv = synth.normal(901 + k, m * k, 1.0).reshape(m, k)
+    sess.set_parameter("embed", embed)
+    sess.set_input("x", xv)
+    sess.step()
+    sess.wait()
+    got = sess.read_output(m * n).reshape(m, n)
+    want = orc.matmul_packed(fmt, xv, orc.quantize(fmt, np.ascontiguousarray(embed.T)), n)
+    orc.assert_close(got, want, 1e-3, 1e-4)
+    sess.close()

@@ -172,3 +172,45 @@ def test_graph_builder_errors():
     with pytest.raises(ValueError, match="2D"):
         g.matmul(a, v)
     assert g.rms_norm(a, v, 1e-6) >= 0
+
+
+def test_nk_quantizer_equals_quantizing_the_transpose(orc):
+    """A weight stored [N, K] (matmul_bt operand) is blocked along K: the bytes are those of
+    the reference quantizer applied to the transposed [K, N] matrix."""
+    from meganeura_amd import capi, synth
+    for fmt in (0, 1):
+        for n, k in ((5, 64), (192, 576), (1, 32)):
+            w_nk = synth.normal(800 + n + k, n * k, 0.02).reshape(n, k)
+            w_nk[0, :32] = 0.25  # a constant block
+            got = capi.quantize_ref_nk(fmt, w_nk)
+            assert (got == orc.quantize(fmt, np.ascontiguousarray(w_nk.T))).all()
+    with pytest.raises(capi.MgnError):
+        capi.quantize_ref_nk(0, np.zeros((4, 48), np.float32))
+
+
+def test_matmul_bt_lowering_and_mixed_use():
+    # src/compile.rs:1447-1485: GemvBT at M = 1 and K % 4 == 0, params [m, n, k, 0]
+    from meganeura_amd.graph import Graph, ShaderEntry, WeightFormat
+    g = Graph()
+    x = g.input("x", [1, 576])
+    e = g.parameter_q4("embed", [49152, 576])
+    g.set_outputs([g.matmul_bt(x, e)])
+    (d,) = g.compile()
+    assert d.shader == ShaderEntry.MatMulGemvBT and d.workgroups == [49152, 1, 1]
+    assert d.params == [1, 49152, 576, 0] and d.weight_format == WeightFormat.Q4
+    g = Graph()
+    x = g.input("x", [6, 64])
+    e = g.parameter_q8("e", [70, 64])
+    g.set_outputs([g.matmul_bt(x, e)])
+    (d,) = g.compile()
+    assert d.shader == ShaderEntry.MatMulBT and d.workgroups == [2, 1, 1] and d.params == [6, 70, 64, 0]
+    with pytest.raises(ValueError, match="K dimensions must match"):
+        g2 = Graph()
+        g2.matmul_bt(g2.input("x", [1, 64]), g2.parameter_q4("e", [64, 32]))
+    # one quantized parameter, both orientations: its blocks can only run one way
+    g3 = Graph()
+    x = g3.input("x", [1, 64])
+    e = g3.parameter_q4("e", [64, 64])
+    g3.set_outputs([g3.matmul(x, e), g3.matmul_bt(x, e)])
+    with pytest.raises(ValueError, match="both matmul and matmul_bt"):
+        g3.compile()
