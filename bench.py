@@ -177,6 +177,31 @@ def decode_layer_times(steps, warmup):
     return res
 
 
+def quantizer_times(ctx, fmt=Q4, k=4096, n=14336):
+    """set_parameter's cost for one C5 weight (58.7 M elements): the host quantizer of the
+    library (threads over block rows; the reference's is a single-threaded scalar loop,
+    src/runtime.rs:2035-2102) and the bit-identical device kernel fed from a device buffer."""
+    from meganeura_amd import capi, synth
+
+    w = synth.weights(5, k, n)
+    t0 = time.perf_counter()
+    packed = capi.quantize_ref(fmt, w)
+    host_s = time.perf_counter() - t0
+    src = ctx.upload(w)
+    wt = ctx.weight_from_device(fmt, src, k, n)  # warm-up: allocation paths, kernel load
+    wt.free()
+    ctx.sync()
+    ctx.timer_start()
+    wt = ctx.weight_from_device(fmt, src, k, n)
+    dev_ms = ctx.timer_stop()
+    same = bool((wt.export_ref() == packed).all())
+    wt.free()
+    src.free()
+    return {"workload": f"quantize_{'q4' if fmt == Q4 else 'q8'}_{k}x{n}", "host_ms": host_s * 1e3,
+            "host_GBs_f32_in": w.nbytes / host_s / 1e9, "device_ms": dev_ms,
+            "device_GBs_f32_in": w.nbytes / (dev_ms * 1e-3) / 1e9, "device_bytes_equal_host": same}
+
+
 def cpu_baseline(wl, budget_s=20.0):
     """The reference's tiled dequant-on-load algorithm restated for the CPU
     (oracle/mgn_oracle.c: orc_matmul_q_tiled), one OpenMP task per workgroup, on
@@ -312,6 +337,10 @@ def main():
         layer = {"workload": "c2_q4_decode_layer_session", **decode_layer_times(max(50, args.steps // 2), args.warmup)}
         rows.append(layer)
         print(json.dumps(layer), file=sys.stderr, flush=True)
+        for fmt in (Q4, Q8):
+            row = quantizer_times(ctx, fmt)
+            rows.append(row)
+            print(json.dumps(row), file=sys.stderr, flush=True)
         out_dir = os.path.join(ROOT, "gpurun_out")
         if os.path.isdir(out_dir):
             with open(os.path.join(out_dir, "bench_sweep.json"), "w") as f:

@@ -135,6 +135,16 @@ mgn_status mgn_weight_dequantize(mgn_ctx* ctx, const mgn_weight* w, float* out_h
  * packed buffer, src/runtime.rs:4218-4226). */
 mgn_status mgn_weight_export_ref(mgn_ctx* ctx, const mgn_weight* w, uint8_t* out_packed);
 
+/* Pre-quantized weights on disk.  The reference's save_checkpoint writes a quantized
+ * parameter's packed bytes under an F32 label and load_checkpoint copies them back blindly
+ * (src/runtime.rs:4218-4226, 4256-4265); this is a tagged container instead: 40-byte
+ * little-endian header "MGNQ", version 1, format, rows, cols, payload size, then the
+ * reference-layout packed bytes, so a file is independent of the private device layout and a
+ * weight never has to be re-quantized at start-up.  Load: MGN_ENOTFOUND if the file cannot be
+ * opened, MGN_EINVAL for a foreign, truncated or inconsistent file. */
+mgn_status mgn_weight_save(mgn_ctx* ctx, const mgn_weight* w, const char* path);
+mgn_status mgn_weight_load(mgn_ctx* ctx, const char* path, mgn_weight** out);
+
 /* ---- the matmul itself
  * C[M,N] = A[M,K] x W (+ D[M,N] when d is not null).  A, C, D: f32 row-major
  * device buffers.  Stands in for the ShaderEntry::{MatMul, MatMulGemv,

@@ -21,7 +21,7 @@ HIP_SYMBOLS = [
     "mgn_buf_alloc", "mgn_buf_free", "mgn_buf_size", "mgn_buf_device_ptr", "mgn_buf_upload",
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
-    "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_matmul_q",
+    "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_weight_save", "mgn_weight_load", "mgn_matmul_q",
     "mgn_matmul_q_f16a", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
     "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
@@ -96,9 +96,11 @@ def load():
         "mgn_weight_create_packed": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
         "mgn_weight_create_device": (C.c_int, [vp, C.c_int, vp, sz, sz, C.POINTER(vp)]),
         "mgn_weight_free": (None, [vp, vp]),
-        "mgn_weight_info": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(sz), C.POINTER(sz)]),
         "mgn_weight_dequantize": (C.c_int, [vp, vp, vp]),
         "mgn_weight_export_ref": (C.c_int, [vp, vp, vp]),
+        "mgn_weight_save": (C.c_int, [vp, vp, C.c_char_p]),
+        "mgn_weight_load": (C.c_int, [vp, C.c_char_p, C.POINTER(vp)]),
+        "mgn_weight_info": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(sz), C.POINTER(sz)]),
         "mgn_matmul_q": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_f16a": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_rms_norm": (C.c_int, [vp, vp, vp, C.c_float, vp, vp, vp, C.c_uint32]),
@@ -263,6 +265,14 @@ class Context:
         self.check(self.lib.mgn_weight_create_nk(self.h, fmt, _ptr(w_nk), w_nk.shape[0], w_nk.shape[1], C.byref(h)))
         return Weight(self, h, fmt, w_nk.shape[1], w_nk.shape[0])
 
+    def load_weight(self, path):
+        """Weight from a file written by Weight.save."""
+        h = C.c_void_p()
+        self.check(self.lib.mgn_weight_load(self.h, str(path).encode(), C.byref(h)))
+        fmt, rows, cols = C.c_int(), C.c_size_t(), C.c_size_t()
+        self.lib.mgn_weight_info(h, C.byref(fmt), C.byref(rows), C.byref(cols))
+        return Weight(self, h, fmt.value, rows.value, cols.value)
+
     def weight_from_packed(self, fmt, packed, rows, cols):
         packed = np.ascontiguousarray(packed, dtype=np.uint8)
         assert packed.size == packed_size(fmt, rows, cols)
@@ -332,6 +342,10 @@ class Weight:
         out = np.empty((self.rows, self.cols), dtype=np.float32)
         self.ctx.check(self.ctx.lib.mgn_weight_dequantize(self.ctx.h, self.h, _ptr(out)))
         return out
+
+    def save(self, path):
+        """Write the weight (format, shape, reference-layout bytes) to a file."""
+        self.ctx.check(self.ctx.lib.mgn_weight_save(self.ctx.h, self.h, str(path).encode()))
 
     def export_ref(self):
         out = np.empty(packed_size(self.fmt, self.rows, self.cols), dtype=np.uint8)

@@ -376,6 +376,68 @@ mgn_status mgn_weight_export_ref(mgn_ctx* ctx, const mgn_weight* w, uint8_t* out
   return MGN_OK;
 }
 
+// ---- pre-quantized weights on disk ----
+// Header, little-endian: "MGNQ" | u32 version (1) | u32 fmt | u32 reserved (0) | u64 rows | u64 cols
+// | u64 payload bytes; then the reference-layout packed bytes (mgn_packed_size of them).
+
+namespace {
+struct QFileHeader {
+  char magic[4];
+  uint32_t version, fmt, reserved;
+  uint64_t rows, cols, payload;
+};
+static_assert(sizeof(QFileHeader) == 40, "header is 40 bytes, no padding");
+}  // namespace
+
+mgn_status mgn_weight_save(mgn_ctx* ctx, const mgn_weight* w, const char* path) {
+  if (!ctx || !w || !path) return fail(ctx, MGN_EINVAL, "null argument");
+  std::vector<uint8_t> packed;
+  try {
+    packed.resize(mgn_packed_size(w->fmt, w->rows, w->cols));
+  } catch (const std::bad_alloc&) {
+    return fail(ctx, MGN_ENOMEM, "out of host memory");
+  }
+  mgn_status st = mgn_weight_export_ref(ctx, w, packed.data());
+  if (st != MGN_OK) return st;
+  QFileHeader h{{'M', 'G', 'N', 'Q'}, 1u, (uint32_t)w->fmt, 0u, (uint64_t)w->rows, (uint64_t)w->cols, (uint64_t)packed.size()};
+  FILE* f = std::fopen(path, "wb");
+  if (!f) return fail(ctx, MGN_EINVAL, std::string("cannot open for writing: ") + path);
+  const bool ok = std::fwrite(&h, sizeof(h), 1, f) == 1 && std::fwrite(packed.data(), 1, packed.size(), f) == packed.size();
+  const bool closed = std::fclose(f) == 0;
+  if (!ok || !closed) return fail(ctx, MGN_EINVAL, std::string("short write: ") + path);
+  return MGN_OK;
+}
+
+mgn_status mgn_weight_load(mgn_ctx* ctx, const char* path, mgn_weight** out) {
+  if (!ctx || !path || !out) return fail(ctx, MGN_EINVAL, "null argument");
+  *out = nullptr;
+  FILE* f = std::fopen(path, "rb");
+  if (!f) return fail(ctx, MGN_ENOTFOUND, std::string("cannot open: ") + path);
+  QFileHeader h{};
+  mgn_status st = MGN_OK;
+  std::vector<uint8_t> packed;
+  if (std::fread(&h, sizeof(h), 1, f) != 1 || std::memcmp(h.magic, "MGNQ", 4) != 0) {
+    st = fail(ctx, MGN_EINVAL, std::string("not a quantized-weight file: ") + path);
+  } else if (h.version != 1) {
+    st = fail(ctx, MGN_EINVAL, "unknown quantized-weight file version " + std::to_string(h.version));
+  } else if (!valid_fmt((mgn_fmt)h.fmt) || h.rows == 0 || h.cols == 0 || h.rows % 32 != 0 ||
+             h.rows > 0xFFFFFFE0ull || h.cols > 0xFFFFFFFFull || (h.rows / 32) * h.cols >= 0x7FFFFFFFull ||
+             h.payload != mgn_packed_size((mgn_fmt)h.fmt, h.rows, h.cols)) {
+    st = fail(ctx, MGN_EINVAL, std::string("inconsistent header in ") + path);
+  } else {
+    try {
+      packed.resize(h.payload);
+    } catch (const std::bad_alloc&) {
+      st = fail(ctx, MGN_ENOMEM, "out of host memory");
+    }
+    if (st == MGN_OK && std::fread(packed.data(), 1, packed.size(), f) != packed.size())
+      st = fail(ctx, MGN_EINVAL, std::string("truncated file: ") + path);
+  }
+  std::fclose(f);
+  if (st != MGN_OK) return st;
+  return mgn_weight_create_packed(ctx, (mgn_fmt)h.fmt, packed.data(), h.rows, h.cols, out);
+}
+
 // ---- matmul ----
 
 static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, const mgn_weight* w, const mgn_buf* d,

@@ -318,3 +318,34 @@ def test_batched_matmuls_share_one_launch(ctx, orc, fmt, m, k, ns):
         b.free()
     for w in wts:
         w.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+def test_weight_file_round_trip(ctx, orc, fmt, tmp_path):
+    """save -> load gives the same weight byte for byte; foreign, truncated and inconsistent
+    files are refused with a status, never loaded."""
+    k, n = 576, 130
+    w = synth.normal(950 + fmt, k * n, 0.02).reshape(k, n)
+    wt = ctx.weight(fmt, w)
+    path = tmp_path / "w.mgnq"
+    wt.save(path)
+    raw = path.read_bytes()
+    assert raw[:4] == b"MGNQ" and len(raw) == 40 + len(orc.quantize(fmt, w))
+    assert (np.frombuffer(raw[40:], np.uint8) == orc.quantize(fmt, w)).all()
+    back = ctx.load_weight(path)
+    assert (back.fmt, back.rows, back.cols) == (fmt, k, n)
+    assert (back.export_ref() == wt.export_ref()).all()
+    x = synth.normal(951, k, 1.0).reshape(1, k)
+    assert (bits(run_matmul(ctx, fmt, x, back)) == bits(run_matmul(ctx, fmt, x, wt))).all()
+    back.free()
+    wt.free()
+    with pytest.raises(capi.MgnError) as e:
+        ctx.load_weight(tmp_path / "missing.mgnq")
+    assert e.value.status == capi.ENOTFOUND
+    for name, data in (("foreign", b"GGUF" + raw[4:]), ("truncated", raw[:-7]), ("version", raw[:4] + b"\x02\0\0\0" + raw[8:]),
+                       ("shape", raw[:16] + (k + 32).to_bytes(8, "little") + raw[24:])):
+        p = tmp_path / name
+        p.write_bytes(data)
+        with pytest.raises(capi.MgnError) as e:
+            ctx.load_weight(p)
+        assert e.value.status == capi.EINVAL, name
