@@ -52,7 +52,7 @@ typedef enum mgn_route {
   MGN_ROUTE_AUTO = 0,
   MGN_ROUTE_GENERIC = 1,   /* scalar f32 fallback, any M */
   MGN_ROUTE_GEMV_VALU = 2, /* streaming dequant-GEMV on the vector ALU, M <= 4 */
-  MGN_ROUTE_GEMV_MFMA = 3, /* streaming dequant-GEMV, raw quants x split-fp16 activations on MFMA, M <= 2 */
+  MGN_ROUTE_GEMV_MFMA = 3, /* streaming dequant-GEMV, raw quants x split-fp16 activations on MFMA, M <= 4 */
   MGN_ROUTE_GEMM_MFMA = 4  /* tiled dequant-GEMM on MFMA, larger M */
 } mgn_route;
 
@@ -163,7 +163,7 @@ mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weigh
                              const mgn_buf* d, mgn_buf* c, uint32_t m);
 
 /* Two neighbours of the decode-time matmul folded into its activation staging, each
- * standing in for a dispatch pair of the reference's plan (M <= 2, f32 activations):
+ * standing in for a dispatch pair of the reference's plan (M <= 4, f32 activations):
  *   RmsNorm then MatMul[Gemv][Add]   (src/shaders/rms_norm.wgsl:1-57; models/smollm2.rs:340-341,396):
  *     C = (x * rsqrt(mean(x^2) + eps) * norm_weight) x W (+ D), x[M,K], norm_weight[K];
  *   SwiGLUConcat then MatMul[Gemv][Add]   (src/shaders/swiglu_concat.wgsl:20-32; compile.rs:1814-1830):

@@ -1,4 +1,4 @@
-// Dequant-GEMV on the matrix cores for M <= 2 (decode): C[M,N] = A[M,K] x W (+ D).
+// Dequant-GEMV on the matrix cores for M <= 4 (decode): C[M,N] = A[M,K] x W (+ D).
 //
 // Why MFMA for a matrix-vector product: streaming a 4-bit weight at HBM speed
 // leaves about one vector instruction per four weights per lane; converting
@@ -216,7 +216,8 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const float* __restrict__ a, uint32_t m,
                                                          uint32_t ksc, GemvPrologue pro MGN_TRACE_PARAM) {
-  constexpr int NJ = 2 * MROWS;
+  constexpr int NJ = 2 * MROWS;       // A rows in LDS: hi and lo of every activation row
+  constexpr int NG = (MROWS + 1) / 2;  // groups of four A rows = MFMA chains per weight chunk
   extern __shared__ uint4 lds4[];
   // this wave's weight: the one whose quad range holds the wave's (first) quad
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -399,7 +400,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const flo
   // ---- the K walk: STEPS blocks per lane, straight-line ----
   // Lanes i >= NJ have no activation row of their own; they re-read row i % NJ (a broadcast
   // in LDS) and the D entries they produce are never looked at.
-  const char* xa_lane = (const char*)xa + ((kb_first * NJ) + (i % NJ)) * 16;
+  const char* xa_lane = (const char*)xa + ((kb_first * NJ) + (NJ < 4 ? i % NJ : i)) * 16;
   const char* ci_lane = (const char*)cinit + kb_first * MROWS * 8;
   float acc[QPW][MROWS];  // lane (b, j): sum over this lane's K blocks for column 4*(quad+q)+j, per row
 #pragma unroll
@@ -413,15 +414,21 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const flo
     const uint32_t so = (step_begin + s < steps_total) ? (uint32_t)s : 0u;
     if (t + kDepth < TS) fetch(t + kDepth);
     const Raw<FMT>& cur = blk[t];
-    // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks
-    uint4 ax[4];
+    // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks; with more than
+    // two activation rows a second group of four A rows (rows 2 and 3, hi and lo) follows
+    uint4 ax[NG][4];
 #pragma unroll
-    for (int ch = 0; ch < 4; ch++) ax[ch] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + ch * plane * 16);
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+      for (int ch = 0; ch < 4; ch++)
+        ax[g][ch] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + ch * plane * 16 + g * 64);
     float2 ci[MROWS];  // {chain start value, factor that undoes the operand and block scales}
 #pragma unroll
     for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_lane + so * (16 * MROWS * 8) + r * 8);
     // the centring term rides in as the chain's start value (rows 2r and 2r+1 add up later)
-    floatx4 dsum = {ci[0].x, 0.0f, MROWS > 1 ? ci[MROWS - 1].x : 0.0f, 0.0f};
+    floatx4 dsum[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) dsum[g] = floatx4{ci[2 * g].x, 0.0f, 2 * g + 1 < MROWS ? ci[2 * g + 1 < MROWS ? 2 * g + 1 : 0].x : 0.0f, 0.0f};
     if constexpr (FMT == MGN_FMT_Q4) {
       const uint32_t words[4] = {cur.q.x, cur.q.y, cur.q.z, cur.q.w};
 #pragma unroll
@@ -430,8 +437,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const flo
         const uint32_t wd = words[ch];
         const uint32_t e0 = (wd << 4) & 0x00F000F0u, o0 = wd & 0x00F000F0u;         // (n0,n4), (n1,n5)
         const uint32_t e1 = (wd >> 4) & 0x00F000F0u, o1 = (wd >> 8) & 0x00F000F0u;  // (n2,n6), (n3,n7)
-        dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[ch].x, ax[ch].y), as_half4(e0, e1), dsum, 0, 0, 0);
-        dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[ch].z, ax[ch].w), as_half4(o0, o1), dsum, 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+          dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[g][ch].x, ax[g][ch].y), as_half4(e0, e1), dsum[g], 0, 0, 0);
+          dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[g][ch].z, ax[g][ch].w), as_half4(o0, o1), dsum[g], 0, 0, 0);
+        }
       }
     } else {
       const uint32_t words[8] = {cur.q0.x, cur.q0.y, cur.q0.z, cur.q0.w, cur.q1.x, cur.q1.y, cur.q1.z, cur.q1.w};
@@ -442,15 +452,18 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const flo
           const uint32_t u8 = words[2 * ch + h] ^ 0x80808080u;  // q + 128 in every byte
           const uint32_t lo2 = __builtin_amdgcn_perm(0u, u8, 0x0c010c00u);  // (b0, b1) as fp16 mantissas
           const uint32_t hi2 = __builtin_amdgcn_perm(0u, u8, 0x0c030c02u);  // (b2, b3)
-          const half4 aop = h == 0 ? as_half4(ax[ch].x, ax[ch].y) : as_half4(ax[ch].z, ax[ch].w);
-          dsum = __builtin_amdgcn_mfma_f32_4x4x4f16(aop, as_half4(lo2, hi2), dsum, 0, 0, 0);
+#pragma unroll
+          for (int g = 0; g < NG; g++) {
+            const half4 aop = h == 0 ? as_half4(ax[g][ch].x, ax[g][ch].y) : as_half4(ax[g][ch].z, ax[g][ch].w);
+            dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(aop, as_half4(lo2, hi2), dsum[g], 0, 0, 0);
+          }
         }
       }
     }
     const float dscale = half_bits_to_float(cur.meta & 0xFFFFu);
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
-      float v = dscale * (dsum[2 * r] + dsum[2 * r + 1]);
+      float v = dscale * (dsum[r / 2][2 * (r % 2)] + dsum[r / 2][2 * (r % 2) + 1]);
       if constexpr (FMT == MGN_FMT_Q4) {
         // (m + 8 d) * S with S = -ci * operand_scale / 8: fold the -1/8 into the block constant
         const float mneg = __fmaf_rn(-0.125f, half_bits_to_float(cur.meta >> 16), -dscale);
@@ -629,17 +642,18 @@ int launch_t(ihipStream_t* s, const LaunchArgs& x) {
 }  // namespace
 
 bool gemv_mfma_supported(const LaunchArgs& x) {
-  if (x.a_is_f16 || x.m == 0 || x.m > 2) return false;
+  if (x.a_is_f16 || x.m == 0 || x.m > 4) return false;
   MfmaGemvPlan p;
   for (int j = 0; j < x.n_more; j++)
     if (x.more[j].w.k != x.w.k || x.more[j].w.fmt != x.w.fmt) return false;
   if (x.n_more < 0 || x.n_more > kMaxBatch - 1) return false;
-  return plan_mfma_gemv(x.w.k, total_quads(x), x.m, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p);
+  return plan_mfma_gemv(x.w.k, total_quads(x), x.m <= 2 ? x.m : 4, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p);
 }
 
 int launch_matmul_gemv_mfma(ihipStream_t* s, const LaunchArgs& x) {
-  if (x.w.fmt == MGN_FMT_Q4) return x.m == 1 ? launch_t<MGN_FMT_Q4, 1>(s, x) : launch_t<MGN_FMT_Q4, 2>(s, x);
-  return x.m == 1 ? launch_t<MGN_FMT_Q8, 1>(s, x) : launch_t<MGN_FMT_Q8, 2>(s, x);
+  if (x.w.fmt == MGN_FMT_Q4)
+    return x.m == 1 ? launch_t<MGN_FMT_Q4, 1>(s, x) : x.m == 2 ? launch_t<MGN_FMT_Q4, 2>(s, x) : launch_t<MGN_FMT_Q4, 4>(s, x);
+  return x.m == 1 ? launch_t<MGN_FMT_Q8, 1>(s, x) : x.m == 2 ? launch_t<MGN_FMT_Q8, 2>(s, x) : launch_t<MGN_FMT_Q8, 4>(s, x);
 }
 
 }  // namespace mgn

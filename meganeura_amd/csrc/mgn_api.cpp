@@ -466,7 +466,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   if (pro_kind != mgn::kProNone) {
     // only the MFMA GEMV stages its activations in a way a prologue can ride on
     if (a_is_f16 || !mgn::gemv_mfma_supported(x) || (route != MGN_ROUTE_AUTO && route != MGN_ROUTE_GEMV_MFMA))
-      return fail(ctx, MGN_EUNSUPPORTED, "fused prologue needs the GEMV_MFMA route (f32 activations, M <= 2)");
+      return fail(ctx, MGN_EUNSUPPORTED, "fused prologue needs the GEMV_MFMA route (f32 activations, M <= 4)");
     route = MGN_ROUTE_GEMV_MFMA;
   }
   if (route == MGN_ROUTE_AUTO) {
@@ -541,7 +541,7 @@ mgn_status mgn_matmul_q_batch(mgn_ctx* ctx, const mgn_buf* a, mgn_prologue prolo
   x.pro_weight = norm_weight ? (const float*)norm_weight->ptr : nullptr;
   x.pro_eps = eps;
   if ((ctx->route != MGN_ROUTE_AUTO && ctx->route != MGN_ROUTE_GEMV_MFMA) || !mgn::gemv_mfma_supported(x))
-    return fail(ctx, MGN_EUNSUPPORTED, "batched matmul needs the GEMV_MFMA route (f32 activations, M <= 2)");
+    return fail(ctx, MGN_EUNSUPPORTED, "batched matmul needs the GEMV_MFMA route (f32 activations, M <= 4)");
   const int rc = mgn::launch_matmul_gemv_mfma(ctx->stream, x);
   if (rc != 0) return hip_fail(ctx, "kernel launch", (hipError_t)rc);
   return MGN_OK;
