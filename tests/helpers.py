@@ -34,3 +34,31 @@ def gemv_parity_inputs(k, n, seed):
     s31 = np.uint32((seed * 31) & 0xFFFFFFFF)
     b = np.cos((j ^ s31).astype(np.float32) * np.float32(0.0007)).astype(np.float32)
     return a.reshape(1, k), b.reshape(k, n)
+
+
+def golden_vectors():
+    """Known-answer vectors of tests/golden/known_answers.json: (name, fmt, input [rows, cols] f32, entry)."""
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "known_answers.json")
+    with open(path) as f:
+        data = json.load(f)
+    out = []
+    for v in data["vectors"]:
+        w = np.array(v["input_f32_bits"], np.uint32).view(np.float32).reshape(v["rows"], v["cols"])
+        out.append((v["name"], Q4 if v["fmt"] == "q4" else Q8, w, v))
+    return out, data["f16"]
+
+
+def check_golden_packed(name, packed, entry):
+    """Compare packed bytes with a golden entry (whole bytes, or the prefix + named nibbles)."""
+    packed = np.asarray(packed, np.uint8)
+    if "packed_hex" in entry:
+        assert packed.tobytes().hex() == entry["packed_hex"], name
+    else:
+        prefix = bytes.fromhex(entry["packed_prefix_hex"])
+        assert packed[:len(prefix)].tobytes() == prefix, name
+        for idx, nib in entry["nibbles"].items():
+            i = int(idx)
+            byte = int(packed[4 + i // 2])
+            assert ((byte >> 4) if i % 2 else (byte & 0xF)) == nib, (name, i)

@@ -65,6 +65,20 @@ def test_device_weight_is_bit_exact(ctx, orc, fmt, shape):
     wt.free(); src.free()
 
 
+def test_device_quantizer_matches_golden_vectors(ctx):
+    from helpers import check_golden_packed, golden_vectors
+    vectors, _ = golden_vectors()
+    for name, fmt, w, entry in vectors:
+        src = ctx.upload(w)
+        for wt in (ctx.weight(fmt, w), ctx.weight_from_device(fmt, src, *w.shape)):
+            check_golden_packed(name, wt.export_ref(), entry)
+            deq = wt.dequantize().reshape(-1)
+            for idx, bits_ in entry.get("dequant_f32_bits", {}).items():
+                assert int(deq[int(idx)].view(np.uint32)) == bits_, name
+            wt.free()
+        src.free()
+
+
 @pytest.mark.parametrize("fmt", [Q4, Q8])
 def test_device_weight_extreme_scales(ctx, orc, fmt):
     # half-subnormal scales must decode as the half crate does (kept, not flushed),

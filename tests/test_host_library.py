@@ -214,3 +214,14 @@ def test_matmul_bt_lowering_and_mixed_use():
     g3.set_outputs([g3.matmul(x, e), g3.matmul_bt(x, e)])
     with pytest.raises(ValueError, match="both matmul and matmul_bt"):
         g3.compile()
+
+
+def test_host_quantizer_matches_golden_vectors():
+    from helpers import check_golden_packed, golden_vectors
+    vectors, _ = golden_vectors()
+    for name, fmt, w, entry in vectors:
+        packed = capi.quantize_ref(fmt, w)
+        check_golden_packed(name, packed, entry)
+        deq = capi.dequantize_ref(fmt, packed, *w.shape).reshape(-1)
+        for idx, bits_ in entry.get("dequant_f32_bits", {}).items():
+            assert int(deq[int(idx)].view(np.uint32)) == bits_, name

@@ -10,6 +10,22 @@ import pytest
 Q4, Q8 = 0, 1
 
 
+# ---- committed golden vectors ------------------------------------------------------
+
+def test_golden_vectors(orc):
+    from helpers import check_golden_packed, golden_vectors
+    vectors, f16 = golden_vectors()
+    assert len(vectors) >= 7
+    for name, fmt, w, entry in vectors:
+        packed = orc.quantize(fmt, w)
+        check_golden_packed(name, packed, entry)
+        deq = orc.dequantize(fmt, packed, *w.shape).reshape(-1)
+        for idx, bits_ in entry.get("dequant_f32_bits", {}).items():
+            assert int(deq[int(idx)].view(np.uint32)) == bits_, name
+    for bits_, val in f16["decode"].items():
+        assert orc.f16_bits_to_f32(int(bits_, 16)) == np.float32(val)
+
+
 # ---- f16 conversion ------------------------------------------------------------
 
 def test_f16_decode_reference_bit_patterns(orc):
