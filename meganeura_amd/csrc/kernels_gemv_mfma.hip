@@ -214,24 +214,33 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 //   kProRmsNorm  a[m, K] * rsqrt(mean(a^2) + eps) * norm_weight[K]   (src/shaders/rms_norm.wgsl:1-57);
 //   kProSwiglu   a[m, 2K] = gate | up  ->  gate * sigmoid(gate) * up  (src/shaders/swiglu_concat.wgsl:20-32).
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
-__global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const float* __restrict__ a, uint32_t m,
-                                                         uint32_t ksc, GemvPrologue pro MGN_TRACE_PARAM) {
+__global__ __launch_bounds__(1024) void gemv_mfma_kernel(
+    // The leading scalar arguments are what a wave needs before it can issue its first loads;
+    // they are declared first (and not inside a struct) so that the dispatcher can hand them
+    // over in registers (kernel-argument preload) instead of the wave fetching them from memory.
+    const float* __restrict__ a, uint32_t m, uint32_t ksc, uint32_t kdim, const float* __restrict__ norm_weight, float eps,
+    uint32_t first_quad1, uint32_t first_quad2, const void* __restrict__ meta0, const void* __restrict__ quants0, uint32_t n0,
+    GemvBatch bt MGN_TRACE_PARAM) {
+  const GemvPrologue pro{norm_weight, eps};
   constexpr int NJ = 2 * MROWS;       // A rows in LDS: hi and lo of every activation row
   constexpr int NG = (MROWS + 1) / 2;  // groups of four A rows = MFMA chains per weight chunk
   extern __shared__ uint4 lds4[];
   // this wave's weight: the one whose quad range holds the wave's (first) quad
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t gquad_u = (blockIdx.x * ((blockDim.x >> 6) / ksc) + wave_u / ksc) * QPW;
-  const uint32_t widx = (gquad_u >= bt.first_quad[1] ? 1u : 0u) + (gquad_u >= bt.first_quad[2] ? 1u : 0u);
+  const uint32_t widx = (gquad_u >= first_quad1 ? 1u : 0u) + (gquad_u >= first_quad2 ? 1u : 0u);
   WeightView w;
-  w.meta = pick3(widx, bt.w[0].meta, bt.w[1].meta, bt.w[2].meta);
-  w.quants = pick3(widx, bt.w[0].quants, bt.w[1].quants, bt.w[2].quants);
-  w.n = pick3(widx, bt.w[0].n, bt.w[1].n, bt.w[2].n);
-  w.k = bt.w[0].k;
+  w.meta = meta0;
+  w.quants = quants0;
+  w.n = n0;
+  if (widx != 0) {  // a later weight of a batch: its view comes from the argument block in memory
+    w.meta = widx == 1 ? bt.w[1].meta : bt.w[2].meta;
+    w.quants = widx == 1 ? bt.w[1].quants : bt.w[2].quants;
+    w.n = widx == 1 ? bt.w[1].n : bt.w[2].n;
+  }
+  w.k = kdim;
   w.fmt = FMT;
-  const float* const dres = pick3(widx, bt.d[0], bt.d[1], bt.d[2]);
-  float* const c = pick3(widx, bt.c[0], bt.c[1], bt.c[2]);
-  const uint32_t quad_base = pick3(widx, 0u, bt.first_quad[1], bt.first_quad[2]);  // first quad of that weight
+  const uint32_t quad_base = pick3(widx, 0u, first_quad1, first_quad2);  // first quad of that weight
   const uint32_t bpc = w.k / 32;
   const uint32_t bpc_pad = (bpc + 15) & ~15u;
   const uint32_t plane = bpc_pad * NJ;
@@ -486,6 +495,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const flo
         const uint32_t n = (quad + q) * 4 + lane;
         if (lane < 4 && wave_live && (uint32_t)r < m && n < w.n) {
           const size_t o = (size_t)r * w.n + n;
+          const float* const dres = pick3(widx, bt.d[0], bt.d[1], bt.d[2]);
+          float* const c = pick3(widx, bt.c[0], bt.c[1], bt.c[2]);
           c[o] = dres ? tot + dres[o] : tot;
         }
       }
@@ -507,9 +518,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(GemvBatch bt, const flo
     const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
     // the quads of a workgroup may belong to different weights of the batch
     const uint32_t gq = quad0 + ql;
-    const uint32_t wi = (gq >= bt.first_quad[1] ? 1u : 0u) + (gq >= bt.first_quad[2] ? 1u : 0u);
-    const uint32_t wn_cols = pick3(wi, bt.w[0].n, bt.w[1].n, bt.w[2].n);
-    const uint32_t n = (gq - pick3(wi, 0u, bt.first_quad[1], bt.first_quad[2])) * 4 + col;
+    const uint32_t wi = (gq >= first_quad1 ? 1u : 0u) + (gq >= first_quad2 ? 1u : 0u);
+    const uint32_t wn_cols = pick3(wi, n0, bt.w[1].n, bt.w[2].n);
+    const uint32_t n = (gq - pick3(wi, 0u, first_quad1, first_quad2)) * 4 + col;
     if (r < m && n < wn_cols) {
       float v = 0.0f;
       for (uint32_t s = 0; s < ksc; s++) v += red[((ql * ksc + s) * MROWS + r) * 4 + col];
@@ -578,7 +589,6 @@ int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
     if (e != hipSuccess) return (int)e;
     big_lds_enabled = true;
   }
-  const GemvPrologue pro{x.pro_weight, x.pro_eps};
   GemvBatch bt{};
   uint32_t quads = 0;
   for (int j = 0; j < kMaxBatch; j++) {
@@ -593,8 +603,9 @@ int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
       bt.first_quad[j] = 0xFFFFFFFFu;
     }
   }
-  hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, bt, (const float*)x.a, x.m, p.ksc,
-                     pro MGN_TRACE_ARG);
+  hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.m, p.ksc, x.w.k,
+                     x.pro_weight, x.pro_eps, bt.first_quad[1], bt.first_quad[2], x.w.meta, x.w.quants, x.w.n,
+                     bt MGN_TRACE_ARG);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }
