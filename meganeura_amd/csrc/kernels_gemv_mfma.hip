@@ -54,8 +54,18 @@ extern "C" int mgn_debug_set_trace(void* p) {
 }
 #define MGN_TRACE_PARAM , unsigned long long* trace_arg
 #define MGN_TRACE_ARG , g_gemv_trace_host
-#define MGN_STAMP_INIT() \
-  unsigned long long* const trace_base = trace_arg ? trace_arg + ((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 16 : nullptr
+// The first two stamps are taken into registers and written once the buffer pointer (an
+// argument that lives in memory) is first needed, so that tracing does not itself make the
+// wave wait for an argument fetch before its first loads.
+#define MGN_STAMP_INIT()                                              \
+  const unsigned long long trace_t0 = __builtin_readcyclecounter();   \
+  const unsigned long long trace_w0 = wall_clock64();                 \
+  unsigned long long trace_t1 = 0
+#define MGN_STAMP_EARLY() trace_t1 = __builtin_readcyclecounter()
+#define MGN_STAMP_FLUSH()                                                                                     \
+  unsigned long long* const trace_base =                                                                      \
+      trace_arg ? trace_arg + ((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 16 : nullptr;                  \
+  if (trace_base && (threadIdx.x & 63) == 0) trace_base[0] = trace_t0, trace_base[1] = trace_t1, trace_base[13] = trace_w0
 #define MGN_STAMP(slot)                                                                          \
   do {                                                                                           \
     if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = __builtin_readcyclecounter();   \
@@ -69,6 +79,8 @@ extern "C" int mgn_debug_set_trace(void* p) {
 #define MGN_TRACE_PARAM
 #define MGN_TRACE_ARG
 #define MGN_STAMP_INIT() do {} while (0)
+#define MGN_STAMP_EARLY() do {} while (0)
+#define MGN_STAMP_FLUSH() do {} while (0)
 #define MGN_STAMP(slot) do {} while (0)
 #endif
 
@@ -82,7 +94,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // fp16 bit patterns used as operands stand for value * 2^-kOperandShift
 template <int FMT>
 constexpr float operand_scale() { return FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f; }  // 2^20, 2^24
-constexpr int kMaxTasks = 2;  // activation chunks a thread prepares, per row
+constexpr int kMaxTasks = 2;  // activation chunks a thread prepares at most, per row
 #ifndef MGN_GEMV_DEPTH
 #define MGN_GEMV_DEPTH 3
 #endif
@@ -213,27 +225,34 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 //   kProNone     a[m, K] as is;
 //   kProRmsNorm  a[m, K] * rsqrt(mean(a^2) + eps) * norm_weight[K]   (src/shaders/rms_norm.wgsl:1-57);
 //   kProSwiglu   a[m, 2K] = gate | up  ->  gate * sigmoid(gate) * up  (src/shaders/swiglu_concat.wgsl:20-32).
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
+// TASKS: activation chunks per thread (1 when the workgroup has a thread for every chunk; the
+// prologue in front of the first weight load is then half as long).
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // The leading scalar arguments are what a wave needs before it can issue its first loads;
     // they are declared first (and not inside a struct) so that the dispatcher can hand them
     // over in registers (kernel-argument preload) instead of the wave fetching them from memory.
-    const float* __restrict__ a, uint32_t m, uint32_t ksc, uint32_t kdim, const float* __restrict__ norm_weight, float eps,
-    uint32_t first_quad1, uint32_t first_quad2, const void* __restrict__ meta0, const void* __restrict__ quants0, uint32_t n0,
-    GemvBatch bt MGN_TRACE_PARAM) {
+    // (three pointers and eight 32-bit values: the 14 dwords that can be preloaded)
+    const float* __restrict__ a, const void* __restrict__ meta0, const void* __restrict__ quants0, uint32_t m,
+    uint32_t ksc, uint32_t wnc, uint32_t kdim, uint32_t n0, uint32_t first_quad1, uint32_t first_quad2,
+    uint32_t ksc_recip,  // ceil(4096 / ksc): wave / ksc == (wave * ksc_recip) >> 12 for the 16 waves there can be
+    const float* __restrict__ norm_weight, float eps, GemvBatch bt MGN_TRACE_PARAM) {
+  MGN_STAMP_INIT();
   const GemvPrologue pro{norm_weight, eps};
   constexpr int NJ = 2 * MROWS;       // A rows in LDS: hi and lo of every activation row
   constexpr int NG = (MROWS + 1) / 2;  // groups of four A rows = MFMA chains per weight chunk
   extern __shared__ uint4 lds4[];
   // this wave's weight: the one whose quad range holds the wave's (first) quad
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t gquad_u = (blockIdx.x * ((blockDim.x >> 6) / ksc) + wave_u / ksc) * QPW;
+  const uint32_t nthreads = 64 * ksc * wnc;  // = blockDim.x, without reading it from memory
+  const uint32_t gquad_u = (blockIdx.x * wnc + ((wave_u * ksc_recip) >> 12)) * QPW;
   const uint32_t widx = (gquad_u >= first_quad1 ? 1u : 0u) + (gquad_u >= first_quad2 ? 1u : 0u);
   WeightView w;
   w.meta = meta0;
   w.quants = quants0;
   w.n = n0;
   if (widx != 0) {  // a later weight of a batch: its view comes from the argument block in memory
+    asm volatile("" ::: "memory");  // keep these loads (and the wait for them) inside the branch
     w.meta = widx == 1 ? bt.w[1].meta : bt.w[2].meta;
     w.quants = widx == 1 ? bt.w[1].quants : bt.w[2].quants;
     w.n = widx == 1 ? bt.w[1].n : bt.w[2].n;
@@ -244,19 +263,16 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   const uint32_t bpc = w.k / 32;
   const uint32_t bpc_pad = (bpc + 15) & ~15u;
   const uint32_t plane = bpc_pad * NJ;
-  const uint32_t nwaves = blockDim.x >> 6, wnc = nwaves / ksc;
+  const uint32_t nwaves = ksc * wnc;
   uint4* xa = lds4;                                   // [4][plane]
   float2* cinit = (float2*)(lds4 + 4 * plane);        // [bpc_pad][MROWS]
   float* red = (float*)(cinit + bpc_pad * MROWS);     // [wnc][ksc][MROWS][4]
   float* nrm = red + wnc * ksc * MROWS * 4;           // [16 waves][MROWS] sums of squares (kProRmsNorm)
 
-  MGN_STAMP_INIT();
-  MGN_STAMP(0);
-  MGN_STAMP_WALL(13);
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   // everything derived from the wave index is wave-uniform: keep it in scalar registers
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t ks = wave % ksc, wn = wave / ksc;
+  const uint32_t wn = (wave * ksc_recip) >> 12, ks = wave - wn * ksc;
   const uint32_t b = lane >> 2, i = lane & 3;
   const uint32_t quad0 = blockIdx.x * wnc * QPW;  // first quad of the workgroup, numbered over the whole batch
   const uint32_t nquads = (w.n + 3) / 4;
@@ -273,14 +289,14 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   // activation loads go first and the weight loads right behind them: the activation
   // prep below then waits for its own data only, while the weights stream in.
   // One task = 8 consecutive activations of one row = one A chunk; the 4 tasks of a K
-  // block sit in one lane quad.  A thread holds at most kMaxTasks tasks in registers.
-  float4 xraw[kMaxTasks][MROWS][2];
-  float4 xup[PRO == kProSwiglu ? kMaxTasks : 1][MROWS][2];   // the "up" halves
-  float4 gw[PRO == kProRmsNorm ? kMaxTasks : 1][2];          // norm weights of the task's 8 columns
+  // block sit in one lane quad.  A thread holds TASKS tasks in registers.
+  float4 xraw[TASKS][MROWS][2];
+  float4 xup[PRO == kProSwiglu ? TASKS : 1][MROWS][2];   // the "up" halves
+  float4 gw[PRO == kProRmsNorm ? TASKS : 1][2];          // norm weights of the task's 8 columns
   const uint32_t a_stride = PRO == kProSwiglu ? 2 * w.k : w.k;
 #pragma unroll
-  for (int tt = 0; tt < kMaxTasks; tt++) {
-    const uint32_t t = tid + tt * blockDim.x, kb = t >> 2, ch = t & 3;
+  for (int tt = 0; tt < TASKS; tt++) {
+    const uint32_t t = tid + tt * nthreads, kb = t >> 2, ch = t & 3;
     const bool live = kb < bpc;
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
@@ -315,13 +331,14 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   };
 #pragma unroll
   for (int t = 0; t < TS && t < kDepth; t++) fetch(t);
-  for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += blockDim.x) red[t] = 0.0f;
-  MGN_STAMP(1);
+  for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += nthreads) red[t] = 0.0f;
+  MGN_STAMP_EARLY();
+  MGN_STAMP_FLUSH();
 
   // ---- fused prologue: turn the raw loads into the matmul's activations ----
   if constexpr (PRO == kProSwiglu) {
 #pragma unroll
-    for (int tt = 0; tt < kMaxTasks; tt++)
+    for (int tt = 0; tt < TASKS; tt++)
 #pragma unroll
       for (int r = 0; r < MROWS; r++)
 #pragma unroll
@@ -338,8 +355,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     for (int r = 0; r < MROWS; r++) {
       ss[r] = 0.0f;
 #pragma unroll
-      for (int tt = 0; tt < kMaxTasks; tt++) {
-        const uint32_t kb = (tid + tt * blockDim.x) >> 2;
+      for (int tt = 0; tt < TASKS; tt++) {
+        const uint32_t kb = (tid + tt * nthreads) >> 2;
         if (kb < bpc && (uint32_t)r < m) {
 #pragma unroll
           for (int h = 0; h < 2; h++) {
@@ -355,14 +372,14 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       if (lane == 0) nrm[wave * MROWS + r] = ss[r];
     }
     lds_barrier();
-    const uint32_t nwv = blockDim.x >> 6;
+    const uint32_t nwv = nwaves;
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
       float tot = 0.0f;
       for (uint32_t wv = 0; wv < nwv; wv++) tot += nrm[wv * MROWS + r];
       const float rstd = 1.0f / sqrtf(tot / (float)w.k + pro.eps);
 #pragma unroll
-      for (int tt = 0; tt < kMaxTasks; tt++)
+      for (int tt = 0; tt < TASKS; tt++)
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           const float4 v = xraw[tt][r][h], g4 = gw[tt][h];
@@ -373,8 +390,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 
   // ---- activations -> LDS (once per workgroup) ----
 #pragma unroll
-  for (int tt = 0; tt < kMaxTasks; tt++) {
-    const uint32_t t = tid + tt * blockDim.x, kb = t >> 2, ch = t & 3;
+  for (int tt = 0; tt < TASKS; tt++) {
+    const uint32_t t = tid + tt * nthreads, kb = t >> 2, ch = t & 3;
     if (t < bpc_pad * 4) {  // whole waves take this branch together (bpc_pad * 4 is a multiple of 64)
 #pragma unroll
       for (int r = 0; r < MROWS; r++) {
@@ -514,7 +531,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   lds_barrier();
   MGN_STAMP(11);
   // ---- combine the K splits, add the residual, store ----
-  for (uint32_t t = tid; t < wnc * MROWS * 4; t += blockDim.x) {
+  for (uint32_t t = tid; t < wnc * MROWS * 4; t += nthreads) {
     const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
     // the quads of a workgroup may belong to different weights of the batch
     const uint32_t gq = quad0 + ql;
@@ -534,7 +551,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 }
 
 struct MfmaGemvPlan {
-  uint32_t ksc, wnc, steps, qpw, grid;
+  uint32_t ksc, wnc, steps, qpw, tasks, grid;
   size_t lds;
 };
 
@@ -572,6 +589,7 @@ bool plan_mfma_gemv(uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bo
   p.wnc = std::max<uint32_t>(p.wnc, (prep_waves + p.ksc - 1) / p.ksc);
   if (p.wnc > max_wnc) return false;
   p.grid = (wave_quads + p.wnc - 1) / p.wnc;
+  p.tasks = bpc_pad * 4 <= 64 * p.ksc * p.wnc ? 1 : 2;
   const size_t nj = 2 * mrows;
   p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 8 + (size_t)p.wnc * p.ksc * mrows * 16 +
           16 * mrows * 4 + 64;
@@ -580,9 +598,9 @@ bool plan_mfma_gemv(uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bo
   return true;
 }
 
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
-int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO>;
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS>
+int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
+  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS>;
   static bool big_lds_enabled = false;
   if (p.lds > 64 * 1024 && !big_lds_enabled) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -603,11 +621,18 @@ int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
       bt.first_quad[j] = 0xFFFFFFFFu;
     }
   }
-  hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.m, p.ksc, x.w.k,
-                     x.pro_weight, x.pro_eps, bt.first_quad[1], bt.first_quad[2], x.w.meta, x.w.quants, x.w.n,
+  hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants, x.m,
+                     p.ksc, p.wnc, x.w.k, x.w.n, bt.first_quad[1], bt.first_quad[2], (4096u + p.ksc - 1) / p.ksc, x.pro_weight,
+                     x.pro_eps,
                      bt MGN_TRACE_ARG);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
+}
+
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
+int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
+  return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1>(s, x, p)
+                      : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2>(s, x, p);
 }
 
 template <int FMT, int MROWS, int STEPS, int QPW>
