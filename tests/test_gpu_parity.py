@@ -363,3 +363,30 @@ def test_weight_file_round_trip(ctx, orc, fmt, tmp_path):
         with pytest.raises(capi.MgnError) as e:
             ctx.load_weight(p)
         assert e.value.status == capi.EINVAL, name
+
+
+def test_zero_rows_is_a_no_op(ctx):
+    wt = ctx.weight(Q4, synth.normal(970, 64 * 8, 0.02).reshape(64, 8))
+    a = ctx.buffer(4 * 64)
+    c = ctx.upload(np.full(8, 7.0, np.float32))
+    ctx.matmul_q(a, wt, c, 0)
+    ctx.matmul_q_f16a(a, wt, c, 0)
+    assert (c.download(np.float32, 8) == 7.0).all()
+    a.free(); c.free(); wt.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m,route", [(1, "gemv_mfma"), (4, "gemv_mfma"), (16, "gemm_mfma")])
+def test_activations_and_weights_with_a_large_mean(ctx, orc, fmt, m, route):
+    """All-positive activations against weights whose blocks sit far from zero: the format's
+    additive part (block minimum x sum of activations) and the scaled quant sums are then both
+    large and the kernels keep them in separate accumulators or centre them.  Checked against
+    the f64 product of the dequantized weights at the matmul bar."""
+    k, n = 8192, 160
+    x = np.abs(synth.normal(980 + m, m * k, 1.0)).reshape(m, k) + np.float32(0.5)
+    w = (synth.normal(981, k * n, 0.02) + np.float32(0.3)).reshape(k, n)
+    w[:, 1::2] -= np.float32(0.6)  # every other column far below zero
+    packed = orc.quantize(fmt, w)
+    want = orc.matmul_f64(x, orc.dequantize(fmt, packed, k, n))
+    got = run_matmul(ctx, fmt, x, w, ROUTES[route])
+    orc.assert_close(got, want, REL, ABS)
