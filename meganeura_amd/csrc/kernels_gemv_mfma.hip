@@ -1,681 +1,24 @@
-// Dequant-GEMV on the matrix cores for M <= 4 (decode): C[M,N] = A[M,K] x W (+ D).
-//
-// Why MFMA for a matrix-vector product: streaming a 4-bit weight at HBM speed
-// leaves about one vector instruction per four weights per lane; converting
-// every nibble to f32 and multiplying it on the vector ALU costs three times
-// that and makes the kernel ALU-bound.  Here the vector ALU only masks nibbles
-// into place (5 instructions per 8 weights); the multiply-adds run on
-// v_mfma_f32_4x4x4_16B_f16, whose 16 independent 4x4 blocks fit the problem.
-// With b = lane/4 the MFMA block and i, j = lane%4:
-//   lane (b, j) supplies column j of block b's B operand: four weights of ITS OWN
-//     quant block (output column 4q+j, K block kb0+b);
-//   lane (b, i) supplies row i of block b's A operand: four activations of K block
-//     kb0+b; row 0/1 = high/low half of an fp16 split of activation row 0, row
-//     2/3 the same for activation row 1;
-//   lane (b, j) receives D[i][j], i = 0..3: the dot products of its own weights
-//     with the four activation rows, so scaling by the block's d stays in-lane.
-// Eight such MFMAs cover one 32-element quant block per lane.
-//
-// Exactness.  A nibble n masked to bits 4-7 of an fp16 is the subnormal
-// n * 2^-20, and the matrix cores do not flush fp16 subnormals.  (Bits 0-3,
-// n * 2^-24, would save the shifts but is measurably worse: the MFMA datapath
-// aligns products by the operands' nominal exponents and drops low bits of
-// mantissas with many leading zeros.  Q8 bytes, q + 128 in bits 0-7, have few
-// leading zeros and are fine.)  Activations are split x = hi + lo into two fp16 after
-// scaling each 32-element K block by its own power of two (|x| < 2^12; the
-// scale needs only the block's four preparing lanes, no workgroup-wide
-// reduction), so products are exact in f32
-// and only the f32 accumulation rounds: the result carries ~21 bits of x, not
-// 11.  Per block the identity used is
-//   sum_k (n_k d + m) x_k = d * (sum_k n_k x_k - 8 S) + (m + 8 d) * S,  S = sum_k x_k :
-// the nibbles are centred (n - 8) so that neither term is large against the
-// result, and "- 8 S" enters as the MFMA chain's initial accumulator, i.e.
-// before anything is scaled or summed across blocks; accumulating
-// d * sum(n x) and m * sum(x) separately down a column would cancel
-// catastrophically.  Q8 bytes are biased to unsigned (q + 128) and the bias
-// leaves the same way (- 128 S as the initial accumulator).
-//
-// A wave owns four adjacent columns and walks K sixteen blocks at a time, so a
-// lane's accumulator stays in a register down the whole column; the 16 lanes
-// of a column are summed once per column quad.  The activations' A operands
-// are prepared once per workgroup in LDS, laid out so that consecutive lanes
-// read consecutive 16-byte chunks.
-#include <cstdlib>
-
-#include "kernels_common.hip.h"
+// The MFMA GEMV route: shape check and dispatch to the per-(format, rows) translation units.
+// The kernel template lives in kernels_gemv_mfma.hip.h; each kernels_gemv_mfma_<fmt>_m<rows>.hip
+// instantiates it for one weight format and one row count so that they compile in parallel.
+#include "kernels_gemv_mfma.hip.h"
 
 #ifdef MGN_TRACE
-// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.  The
-// buffer travels as a kernel argument, so a stamp is one clock read and one store.
-static unsigned long long* g_gemv_trace_host = nullptr;
+unsigned long long* g_gemv_trace_host = nullptr;
 extern "C" int mgn_debug_set_trace(void* p) {
   g_gemv_trace_host = (unsigned long long*)p;
   return 0;
 }
-#define MGN_TRACE_PARAM , unsigned long long* trace_arg
-#define MGN_TRACE_ARG , g_gemv_trace_host
-// The first two stamps are taken into registers and written once the buffer pointer (an
-// argument that lives in memory) is first needed, so that tracing does not itself make the
-// wave wait for an argument fetch before its first loads.
-#define MGN_STAMP_INIT()                                              \
-  const unsigned long long trace_t0 = __builtin_readcyclecounter();   \
-  const unsigned long long trace_w0 = wall_clock64();                 \
-  unsigned long long trace_t1 = 0
-#define MGN_STAMP_EARLY() trace_t1 = __builtin_readcyclecounter()
-#define MGN_STAMP_FLUSH()                                                                                     \
-  unsigned long long* const trace_base =                                                                      \
-      trace_arg ? trace_arg + ((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 16 : nullptr;                  \
-  if (trace_base && (threadIdx.x & 63) == 0) trace_base[0] = trace_t0, trace_base[1] = trace_t1, trace_base[13] = trace_w0
-#define MGN_STAMP(slot)                                                                          \
-  do {                                                                                           \
-    if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = __builtin_readcyclecounter();   \
-  } while (0)
-#define MGN_STAMP_WALL(slot)                                                        \
-  do {                                                                             \
-    if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = wall_clock64();  \
-  } while (0)
-#else
-#define MGN_STAMP_WALL(slot) do {} while (0)
-#define MGN_TRACE_PARAM
-#define MGN_TRACE_ARG
-#define MGN_STAMP_INIT() do {} while (0)
-#define MGN_STAMP_EARLY() do {} while (0)
-#define MGN_STAMP_FLUSH() do {} while (0)
-#define MGN_STAMP(slot) do {} while (0)
 #endif
 
 namespace mgn {
-namespace {
 
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
-// fp16 bit patterns used as operands stand for value * 2^-kOperandShift
-template <int FMT>
-constexpr float operand_scale() { return FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f; }  // 2^20, 2^24
-constexpr int kMaxTasks = 2;  // activation chunks a thread prepares at most, per row
-#ifndef MGN_GEMV_DEPTH
-#define MGN_GEMV_DEPTH 3
-#endif
-constexpr int kDepth = MGN_GEMV_DEPTH;  // weight blocks in flight per lane ahead of the one in use
-
-__device__ __forceinline__ half4 as_half4(uint32_t lo, uint32_t hi) {
-  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-  const u32x2 v = {lo, hi};
-  return __builtin_bit_cast(half4, v);
-}
-
-// two floats -> packed fp16 pair, truncating: the low halves computed from the
-// residual make up for the truncation
-__device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
-  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
-}
-__device__ __forceinline__ float half_lo(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[0]; }
-__device__ __forceinline__ float half_hi(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[1]; }
-
-constexpr int kRowRor4 = 0x124, kRowRor8 = 0x128;  // rotate right within a row of 16 lanes
-
-// sum over the 16 lanes sharing lane%4 (every such lane ends with the total)
-__device__ __forceinline__ float sum_over_blocks(float v) {
-  v += dpp_move<kRowRor4>(v);
-  v += dpp_move<kRowRor8>(v);
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  return v;
-}
-
-// src/shaders/swiglu_concat.wgsl:20-32: silu(gate) * up with sig = 1 / (1 + exp(-gate))
-__device__ __forceinline__ float swiglu_act(float gate, float up) {
-  const float sig = 1.0f / (1.0f + expf(-gate));
-  return gate * sig * up;
-}
-
-// Up to three weights that share K, the format and the activations, served by one launch
-// (the q, k and v projections of a decode layer): their column quads are numbered one
-// after the other and every wave looks up which weight its quad belongs to.
-constexpr int kMaxBatch = 3;
-struct GemvBatch {
-  WeightView w[kMaxBatch];
-  const float* d[kMaxBatch];
-  float* c[kMaxBatch];
-  uint32_t first_quad[kMaxBatch];  // [0] = 0; unused entries 0xFFFFFFFF
-};
-template <typename T>
-__device__ __forceinline__ T pick3(uint32_t idx, T a0, T a1, T a2) {
-  return idx == 0 ? a0 : idx == 1 ? a1 : a2;
-}
-
-struct GemvPrologue {
-  const float* norm_weight;  // [K], kProRmsNorm
-  float eps;
-};
-
-template <int FMT>
-struct Raw;
-template <>
-struct Raw<MGN_FMT_Q4> {
-  uint4 q;
-  uint32_t meta;
-  __device__ __forceinline__ void load(const WeightView& w, size_t b) {
-    q = stream_load_u128((const uint4*)w.quants + b);
-    meta = stream_load_u32((const uint32_t*)w.meta + b);
-  }
-};
-template <>
-struct Raw<MGN_FMT_Q8> {
-  uint4 q0, q1;
-  uint32_t meta;
-  __device__ __forceinline__ void load(const WeightView& w, size_t b) {
-    q0 = stream_load_u128((const uint4*)w.quants + b * 2);
-    q1 = stream_load_u128((const uint4*)w.quants + b * 2 + 1);
-    meta = stream_load_u16((const uint16_t*)w.meta + b);
-  }
-};
-
-// LDS image of the activations, per workgroup:
-//   chunk planes  xa[c][kb * NJ + j]  (uint4), c = 0..3: the A-operand rows of the two
-//                 MFMAs that consume elements 8c..8c+7 of K block kb; j = 2*row (high
-//                 halves) or 2*row + 1 (low halves);
-//   cinit[kb][row] = { -bias / operand_scale * S(kb, row), the chain's initial accumulator;
-//                      operand_scale / block scale, which undoes both scalings afterwards }.
-// Q4 pairs nibble k with k+4 in one fp16x2 mask, so the chunk is (x0,x4,x2,x6 | x1,x5,x3,x7).
-// Q8 bytes come out in natural order: (x0,x1,x2,x3 | x4,x5,x6,x7).
-template <int FMT>
-__device__ __forceinline__ void make_chunks(const float (&x)[8], uint4& hi, uint4& lo) {
-  float p[8];
-  if constexpr (FMT == MGN_FMT_Q4) {
-    p[0] = x[0], p[1] = x[4], p[2] = x[2], p[3] = x[6];
-    p[4] = x[1], p[5] = x[5], p[6] = x[3], p[7] = x[7];
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; i++) p[i] = x[i];
-  }
-  hi = make_uint4(pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7]));
-  const uint32_t h[4] = {hi.x, hi.y, hi.z, hi.w};
-  uint32_t l[4];
-#pragma unroll
-  for (int i = 0; i < 4; i++) l[i] = pack_rtz(p[2 * i] - half_lo(h[i]), p[2 * i + 1] - half_hi(h[i]));
-  lo = make_uint4(l[0], l[1], l[2], l[3]);
-}
-
-// Power of two that brings a block's largest magnitude below 2^12 (1 if the block
-// is all zero, tiny or not finite).  *inv gets the reciprocal.
-__device__ __forceinline__ float block_scale(float amax, float* inv) {
-  const uint32_t amax_bits = __builtin_bit_cast(uint32_t, amax);
-  const int e = (int)(amax_bits >> 23) - 127;  // floor(log2(amax)) for normal values
-  if (amax_bits == 0 || e >= 100 || e <= -100) {
-    *inv = 1.0f;
-    return 1.0f;
-  }
-  const int sh = 11 - e;  // amax * 2^sh in [2^11, 2^12)
-  *inv = __builtin_bit_cast(float, (uint32_t)(127 - sh) << 23);
-  return __builtin_bit_cast(float, (uint32_t)(127 + sh) << 23);
-}
-
-// blockDim.x = 64 * ksc * wnc.  Wave w: K split ks = w % ksc, quad slot wn = w / ksc.
-// The workgroup owns quads [blockIdx.x * wnc, +wnc); wave (ks, wn) takes quad wn and the
-// K steps [ks * STEPS, (ks+1) * STEPS) of 16 blocks each.  Every wave issues all of its
-// STEPS block loads up front and then runs straight-line code: with no branch around a
-// load the compiler's wait counts are exact, so step s starts as soon as its own block
-// has arrived while the later ones are still in flight.
-// QPW > 1 (short K, many columns): a wave takes QPW consecutive quads, so that it still has
-// QPW * STEPS block loads to keep in flight and the workgroup count stays near the CU count.
-// PRO: what the activations go through on their way into LDS, in place of a kernel of its own:
-//   kProNone     a[m, K] as is;
-//   kProRmsNorm  a[m, K] * rsqrt(mean(a^2) + eps) * norm_weight[K]   (src/shaders/rms_norm.wgsl:1-57);
-//   kProSwiglu   a[m, 2K] = gate | up  ->  gate * sigmoid(gate) * up  (src/shaders/swiglu_concat.wgsl:20-32).
-// TASKS: activation chunks per thread (1 when the workgroup has a thread for every chunk; the
-// prologue in front of the first weight load is then half as long).
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS>
-__global__ __launch_bounds__(1024) void gemv_mfma_kernel(
-    // The leading scalar arguments are what a wave needs before it can issue its first loads;
-    // they are declared first (and not inside a struct) so that the dispatcher can hand them
-    // over in registers (kernel-argument preload) instead of the wave fetching them from memory.
-    // (three pointers and eight 32-bit values: the 14 dwords that can be preloaded)
-    const float* __restrict__ a, const void* __restrict__ meta0, const void* __restrict__ quants0, uint32_t m,
-    uint32_t ksc, uint32_t wnc, uint32_t kdim, uint32_t n0, uint32_t first_quad1, uint32_t first_quad2,
-    uint32_t ksc_recip,  // ceil(4096 / ksc): wave / ksc == (wave * ksc_recip) >> 12 for the 16 waves there can be
-    const float* __restrict__ norm_weight, float eps, GemvBatch bt MGN_TRACE_PARAM) {
-  MGN_STAMP_INIT();
-  const GemvPrologue pro{norm_weight, eps};
-  constexpr int NJ = 2 * MROWS;       // A rows in LDS: hi and lo of every activation row
-  constexpr int NG = (MROWS + 1) / 2;  // groups of four A rows = MFMA chains per weight chunk
-  extern __shared__ uint4 lds4[];
-  // this wave's weight: the one whose quad range holds the wave's (first) quad
-  const uint32_t wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t nthreads = 64 * ksc * wnc;  // = blockDim.x, without reading it from memory
-  const uint32_t gquad_u = (blockIdx.x * wnc + ((wave_u * ksc_recip) >> 12)) * QPW;
-  const uint32_t widx = (gquad_u >= first_quad1 ? 1u : 0u) + (gquad_u >= first_quad2 ? 1u : 0u);
-  WeightView w;
-  w.meta = meta0;
-  w.quants = quants0;
-  w.n = n0;
-  if (widx != 0) {  // a later weight of a batch: its view comes from the argument block in memory
-    asm volatile("" ::: "memory");  // keep these loads (and the wait for them) inside the branch
-    w.meta = widx == 1 ? bt.w[1].meta : bt.w[2].meta;
-    w.quants = widx == 1 ? bt.w[1].quants : bt.w[2].quants;
-    w.n = widx == 1 ? bt.w[1].n : bt.w[2].n;
-  }
-  w.k = kdim;
-  w.fmt = FMT;
-  const uint32_t quad_base = pick3(widx, 0u, first_quad1, first_quad2);  // first quad of that weight
-  const uint32_t bpc = w.k / 32;
-  const uint32_t bpc_pad = (bpc + 15) & ~15u;
-  const uint32_t plane = bpc_pad * NJ;
-  const uint32_t nwaves = ksc * wnc;
-  uint4* xa = lds4;                                   // [4][plane]
-  float2* cinit = (float2*)(lds4 + 4 * plane);        // [bpc_pad][MROWS]
-  float* red = (float*)(cinit + bpc_pad * MROWS);     // [wnc][ksc][MROWS][4]
-  float* nrm = red + wnc * ksc * MROWS * 4;           // [16 waves][MROWS] sums of squares (kProRmsNorm)
-
-  const uint32_t tid = threadIdx.x, lane = tid & 63;
-  // everything derived from the wave index is wave-uniform: keep it in scalar registers
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t wn = (wave * ksc_recip) >> 12, ks = wave - wn * ksc;
-  const uint32_t b = lane >> 2, i = lane & 3;
-  const uint32_t quad0 = blockIdx.x * wnc * QPW;  // first quad of the workgroup, numbered over the whole batch
-  const uint32_t nquads = (w.n + 3) / 4;
-  const uint32_t quad = quad0 + wn * QPW - quad_base;  // first of this wave's QPW quads, within its weight
-  const uint32_t steps_total = bpc_pad / 16;
-  const uint32_t step_begin = ks * STEPS;
-  // a wave past the last K step (or past the last quad) keeps running on the zero block:
-  // it contributes nothing and clamps its LDS reads to step 0
-  const bool wave_live = step_begin < steps_total && quad < nquads;
-  const uint32_t kb_first = (wave_live ? step_begin : 0u) * 16 + b;  // this lane's K block at step 0
-  const uint32_t zero_block = bpc * w.n;  // an all-zero block behind the last real one
-
-  // Memory returns a wave's loads in issue order, so the (small, cache-resident)
-  // activation loads go first and the weight loads right behind them: the activation
-  // prep below then waits for its own data only, while the weights stream in.
-  // One task = 8 consecutive activations of one row = one A chunk; the 4 tasks of a K
-  // block sit in one lane quad.  A thread holds TASKS tasks in registers.
-  float4 xraw[TASKS][MROWS][2];
-  float4 xup[PRO == kProSwiglu ? TASKS : 1][MROWS][2];   // the "up" halves
-  float4 gw[PRO == kProRmsNorm ? TASKS : 1][2];          // norm weights of the task's 8 columns
-  const uint32_t a_stride = PRO == kProSwiglu ? 2 * w.k : w.k;
-#pragma unroll
-  for (int tt = 0; tt < TASKS; tt++) {
-    const uint32_t t = tid + tt * nthreads, kb = t >> 2, ch = t & 3;
-    const bool live = kb < bpc;
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      // always load (from element 0 when there is nothing to load) and zero afterwards
-      const bool ok = live && (uint32_t)r < m;
-      const float4* src = (const float4*)(a + (ok ? (size_t)r * a_stride + (size_t)kb * 32 + ch * 8 : (size_t)0));
-      xraw[tt][r][0] = src[0];
-      xraw[tt][r][1] = src[1];
-      if constexpr (PRO == kProSwiglu) {
-        const float4* up = (const float4*)(a + (ok ? (size_t)r * a_stride + w.k + (size_t)kb * 32 + ch * 8 : (size_t)0));
-        xup[tt][r][0] = up[0];
-        xup[tt][r][1] = up[1];
-      }
-    }
-    if constexpr (PRO == kProRmsNorm) {
-      const float4* gp = (const float4*)(pro.norm_weight + (live ? (size_t)kb * 32 + ch * 8 : (size_t)0));
-      gw[tt][0] = gp[0];
-      gw[tt][1] = gp[1];
-    }
-  }
-  // Weight blocks: kDepth loads run ahead of the step that consumes them.  That is enough
-  // to keep the memory system busy; issuing every load up front would only park the wave
-  // in the load queue (which drains at HBM speed) before it could prepare any activations.
-  // load t = q * STEPS + s: K step s of the wave's quad q
-  constexpr int TS = STEPS * QPW;
-  Raw<FMT> blk[TS];
-  const uint32_t wbase = (quad * 4 + i) * bpc + kb_first;
-  auto fetch = [&](int t) {
-    const int q = t / STEPS, s = t % STEPS;
-    const bool ok = wave_live && (quad + q) * 4 + i < w.n && step_begin + s < steps_total && kb_first + s * 16 < bpc;
-    blk[t].load(w, ok ? wbase + q * 4 * bpc + s * 16 : zero_block);
-  };
-#pragma unroll
-  for (int t = 0; t < TS && t < kDepth; t++) fetch(t);
-  for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += nthreads) red[t] = 0.0f;
-  MGN_STAMP_EARLY();
-  MGN_STAMP_FLUSH();
-
-  // ---- fused prologue: turn the raw loads into the matmul's activations ----
-  if constexpr (PRO == kProSwiglu) {
-#pragma unroll
-    for (int tt = 0; tt < TASKS; tt++)
-#pragma unroll
-      for (int r = 0; r < MROWS; r++)
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const float4 g4 = xraw[tt][r][h], u4 = xup[tt][r][h];
-          xraw[tt][r][h] = make_float4(swiglu_act(g4.x, u4.x), swiglu_act(g4.y, u4.y), swiglu_act(g4.z, u4.z),
-                                       swiglu_act(g4.w, u4.w));
-        }
-  }
-  if constexpr (PRO == kProRmsNorm) {
-    // row sums of squares: per thread, per wave (DPP), then across the waves through LDS
-    float ss[MROWS];
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      ss[r] = 0.0f;
-#pragma unroll
-      for (int tt = 0; tt < TASKS; tt++) {
-        const uint32_t kb = (tid + tt * nthreads) >> 2;
-        if (kb < bpc && (uint32_t)r < m) {
-#pragma unroll
-          for (int h = 0; h < 2; h++) {
-            const float4 v = xraw[tt][r][h];
-            ss[r] = __fmaf_rn(v.x, v.x, ss[r]);
-            ss[r] = __fmaf_rn(v.y, v.y, ss[r]);
-            ss[r] = __fmaf_rn(v.z, v.z, ss[r]);
-            ss[r] = __fmaf_rn(v.w, v.w, ss[r]);
-          }
-        }
-      }
-      ss[r] = group_sum<64>(ss[r]);
-      if (lane == 0) nrm[wave * MROWS + r] = ss[r];
-    }
-    lds_barrier();
-    const uint32_t nwv = nwaves;
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      float tot = 0.0f;
-      for (uint32_t wv = 0; wv < nwv; wv++) tot += nrm[wv * MROWS + r];
-      const float rstd = 1.0f / sqrtf(tot / (float)w.k + pro.eps);
-#pragma unroll
-      for (int tt = 0; tt < TASKS; tt++)
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const float4 v = xraw[tt][r][h], g4 = gw[tt][h];
-          xraw[tt][r][h] = make_float4(v.x * rstd * g4.x, v.y * rstd * g4.y, v.z * rstd * g4.z, v.w * rstd * g4.w);
-        }
-    }
-  }
-
-  // ---- activations -> LDS (once per workgroup) ----
-#pragma unroll
-  for (int tt = 0; tt < TASKS; tt++) {
-    const uint32_t t = tid + tt * nthreads, kb = t >> 2, ch = t & 3;
-    if (t < bpc_pad * 4) {  // whole waves take this branch together (bpc_pad * 4 is a multiple of 64)
-#pragma unroll
-      for (int r = 0; r < MROWS; r++) {
-        float4 v0 = xraw[tt][r][0], v1 = xraw[tt][r][1];
-        if (!(kb < bpc && (uint32_t)r < m)) v0 = v1 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        // block maximum over the quad's 32 values; NaN never wins fmaxf, an infinity
-        // does and switches scaling off
-        float am = fmaxf(fmaxf(fmaxf(fabsf(v0.x), fabsf(v0.y)), fmaxf(fabsf(v0.z), fabsf(v0.w))),
-                         fmaxf(fmaxf(fabsf(v1.x), fabsf(v1.y)), fmaxf(fabsf(v1.z), fabsf(v1.w))));
-        am = fmaxf(am, dpp_move<kDppQuadXor1>(am));
-        am = fmaxf(am, dpp_move<kDppQuadXor2>(am));
-        float inv;
-        const float scale = block_scale(am, &inv);
-        const float x[8] = {v0.x * scale, v0.y * scale, v0.z * scale, v0.w * scale,
-                            v1.x * scale, v1.y * scale, v1.z * scale, v1.w * scale};
-        uint4 hi, lo;
-        make_chunks<FMT>(x, hi, lo);
-        xa[ch * plane + kb * NJ + 2 * r] = hi;
-        xa[ch * plane + kb * NJ + 2 * r + 1] = lo;
-        float s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
-        s += dpp_move<kDppQuadXor1>(s);
-        s += dpp_move<kDppQuadXor2>(s);
-        constexpr float bias = FMT == MGN_FMT_Q4 ? 8.0f : 128.0f;
-        if (ch == 0) cinit[kb * MROWS + r] = make_float2(s * (-bias / operand_scale<FMT>()), inv * operand_scale<FMT>());
-      }
-    }
-  }
-  MGN_STAMP(5);
-  lds_barrier();
-  MGN_STAMP(6);
-
-  // ---- the K walk: STEPS blocks per lane, straight-line ----
-  // Lanes i >= NJ have no activation row of their own; they re-read row i % NJ (a broadcast
-  // in LDS) and the D entries they produce are never looked at.
-  const char* xa_lane = (const char*)xa + ((kb_first * NJ) + (NJ < 4 ? i % NJ : i)) * 16;
-  const char* ci_lane = (const char*)cinit + kb_first * MROWS * 8;
-  float acc[QPW][MROWS];  // lane (b, j): sum over this lane's K blocks for column 4*(quad+q)+j, per row
-#pragma unroll
-  for (int q = 0; q < QPW; q++)
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) acc[q][r] = 0.0f;
-#pragma unroll
-  for (int t = 0; t < TS; t++) {
-    const int s = t % STEPS, q = t / STEPS;
-    // steps past the end of K multiply the zero block; keep their LDS reads in range
-    const uint32_t so = (step_begin + s < steps_total) ? (uint32_t)s : 0u;
-    if (t + kDepth < TS) fetch(t + kDepth);
-    const Raw<FMT>& cur = blk[t];
-    // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks; with more than
-    // two activation rows a second group of four A rows (rows 2 and 3, hi and lo) follows
-    uint4 ax[NG][4];
-#pragma unroll
-    for (int g = 0; g < NG; g++)
-#pragma unroll
-      for (int ch = 0; ch < 4; ch++)
-        ax[g][ch] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + ch * plane * 16 + g * 64);
-    float2 ci[MROWS];  // {chain start value, factor that undoes the operand and block scales}
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_lane + so * (16 * MROWS * 8) + r * 8);
-    // the centring term rides in as the chain's start value (rows 2r and 2r+1 add up later)
-    floatx4 dsum[NG];
-#pragma unroll
-    for (int g = 0; g < NG; g++) dsum[g] = floatx4{ci[2 * g].x, 0.0f, 2 * g + 1 < MROWS ? ci[2 * g + 1 < MROWS ? 2 * g + 1 : 0].x : 0.0f, 0.0f};
-    if constexpr (FMT == MGN_FMT_Q4) {
-      const uint32_t words[4] = {cur.q.x, cur.q.y, cur.q.z, cur.q.w};
-#pragma unroll
-      for (int ch = 0; ch < 4; ch++) {
-        // every nibble pair goes to bits 4-7 / 20-23: n * 2^-20 in each fp16 half
-        const uint32_t wd = words[ch];
-        const uint32_t e0 = (wd << 4) & 0x00F000F0u, o0 = wd & 0x00F000F0u;         // (n0,n4), (n1,n5)
-        const uint32_t e1 = (wd >> 4) & 0x00F000F0u, o1 = (wd >> 8) & 0x00F000F0u;  // (n2,n6), (n3,n7)
-#pragma unroll
-        for (int g = 0; g < NG; g++) {
-          dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[g][ch].x, ax[g][ch].y), as_half4(e0, e1), dsum[g], 0, 0, 0);
-          dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[g][ch].z, ax[g][ch].w), as_half4(o0, o1), dsum[g], 0, 0, 0);
-        }
-      }
-    } else {
-      const uint32_t words[8] = {cur.q0.x, cur.q0.y, cur.q0.z, cur.q0.w, cur.q1.x, cur.q1.y, cur.q1.z, cur.q1.w};
-#pragma unroll
-      for (int ch = 0; ch < 4; ch++) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const uint32_t u8 = words[2 * ch + h] ^ 0x80808080u;  // q + 128 in every byte
-          const uint32_t lo2 = __builtin_amdgcn_perm(0u, u8, 0x0c010c00u);  // (b0, b1) as fp16 mantissas
-          const uint32_t hi2 = __builtin_amdgcn_perm(0u, u8, 0x0c030c02u);  // (b2, b3)
-#pragma unroll
-          for (int g = 0; g < NG; g++) {
-            const half4 aop = h == 0 ? as_half4(ax[g][ch].x, ax[g][ch].y) : as_half4(ax[g][ch].z, ax[g][ch].w);
-            dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(aop, as_half4(lo2, hi2), dsum[g], 0, 0, 0);
-          }
-        }
-      }
-    }
-    const float dscale = half_bits_to_float(cur.meta & 0xFFFFu);
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      float v = dscale * (dsum[r / 2][2 * (r % 2)] + dsum[r / 2][2 * (r % 2) + 1]);
-      if constexpr (FMT == MGN_FMT_Q4) {
-        // (m + 8 d) * S with S = -ci * operand_scale / 8: fold the -1/8 into the block constant
-        const float mneg = __fmaf_rn(-0.125f, half_bits_to_float(cur.meta >> 16), -dscale);
-        v = __fmaf_rn(mneg, ci[r].x, v);
-      }
-      acc[q][r] = __fmaf_rn(v, ci[r].y, acc[q][r]);
-    }
-    if (t == 0) MGN_STAMP(7);
-    if (t == 3) MGN_STAMP(8);
-  }
-  MGN_STAMP(9);
-  // ---- sum the 16 lanes of each column ----
-  if (QPW > 1 || ksc == 1) {
-    // no K split (always the case with QPW > 1): lanes 0..3 hold the four finished columns of a quad
-#pragma unroll
-    for (int q = 0; q < QPW; q++) {
-#pragma unroll
-      for (int r = 0; r < MROWS; r++) {
-        const float tot = sum_over_blocks(acc[q][r]);
-        const uint32_t n = (quad + q) * 4 + lane;
-        if (lane < 4 && wave_live && (uint32_t)r < m && n < w.n) {
-          const size_t o = (size_t)r * w.n + n;
-          const float* const dres = pick3(widx, bt.d[0], bt.d[1], bt.d[2]);
-          float* const c = pick3(widx, bt.c[0], bt.c[1], bt.c[2]);
-          c[o] = dres ? tot + dres[o] : tot;
-        }
-      }
-    }
-    MGN_STAMP(12);
-    MGN_STAMP_WALL(14);
-    return;
-  }
-#pragma unroll
-  for (int r = 0; r < MROWS; r++) {
-    const float tot = sum_over_blocks(acc[0][r]);
-    if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot;
-  }
-  MGN_STAMP(10);
-  lds_barrier();
-  MGN_STAMP(11);
-  // ---- combine the K splits, add the residual, store ----
-  for (uint32_t t = tid; t < wnc * MROWS * 4; t += nthreads) {
-    const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
-    // the quads of a workgroup may belong to different weights of the batch
-    const uint32_t gq = quad0 + ql;
-    const uint32_t wi = (gq >= first_quad1 ? 1u : 0u) + (gq >= first_quad2 ? 1u : 0u);
-    const uint32_t wn_cols = pick3(wi, n0, bt.w[1].n, bt.w[2].n);
-    const uint32_t n = (gq - pick3(wi, 0u, first_quad1, first_quad2)) * 4 + col;
-    if (r < m && n < wn_cols) {
-      float v = 0.0f;
-      for (uint32_t s = 0; s < ksc; s++) v += red[((ql * ksc + s) * MROWS + r) * 4 + col];
-      const size_t o = (size_t)r * wn_cols + n;
-      const float* const dd = pick3(wi, bt.d[0], bt.d[1], bt.d[2]);
-      pick3(wi, bt.c[0], bt.c[1], bt.c[2])[o] = dd ? v + dd[o] : v;
-    }
-  }
-  MGN_STAMP(12);
-  MGN_STAMP_WALL(14);
-}
-
-struct MfmaGemvPlan {
-  uint32_t ksc, wnc, steps, qpw, tasks, grid;
-  size_t lds;
-};
-
-constexpr uint32_t kMaxSteps = 8;  // blocks a lane holds in flight: 8 x 20 B (Q4) or 8 x 34 B (Q8)
-
-// `nquads`: column quads over all weights of the launch; `one_quad_per_wave`: fused prologues
-// and batches of several weights come with QPW = 1 only.
-bool plan_mfma_gemv(uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bool one_quad_per_wave, MfmaGemvPlan* out) {
-  const uint32_t bpc = k / 32, bpc_pad = (bpc + 15) & ~15u;
-  const uint32_t steps_total = bpc_pad / 16;
-  MfmaGemvPlan p{};
-  // K splits: at least enough that a wave's share fits in its registers; more when there
-  // are too few column quads to give every CU a handful of waves
-  uint32_t ksc = (steps_total + kMaxSteps - 1) / kMaxSteps;
-  if (ksc > 16) return false;
-  const uint32_t want_waves = (uint32_t)num_cus * 8;
-  while (ksc < 16 && nquads * ksc < want_waves && (steps_total + ksc) / (ksc + 1) >= 2) ksc++;
-  p.steps = (steps_total + ksc - 1) / ksc;
-  p.ksc = (steps_total + p.steps - 1) / p.steps;  // drop splits that would get no step
-  // quads per wave: with a short K and very many columns a wave takes several quads, as
-  // long as that leaves at least 8 waves per CU
-  p.qpw = 1;
-  if (p.ksc == 1 && !one_quad_per_wave)
-    while (p.qpw < 4 && p.steps * p.qpw * 2 <= kMaxSteps && nquads / (p.qpw * 2) >= (uint32_t)num_cus * 8) p.qpw *= 2;
-  // waves per workgroup: spread the quads evenly over the CUs (one workgroup per CU when
-  // there is enough work), so the activations are prepared as few times as possible
-  const uint32_t max_wnc = 16 / p.ksc;
-  const uint32_t wave_quads = (nquads + p.qpw - 1) / p.qpw;  // quad groups = waves with work
-  p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (wave_quads + num_cus - 1) / num_cus));
-#ifdef MGN_TRACE  // development build only: force the waves per workgroup
-  if (const char* e = getenv("MGN_DEV_WNC")) p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (uint32_t)atoi(e)));
-#endif
-  // enough threads to prepare the activations (waves without a quad only help there)
-  const uint32_t prep_waves = (bpc_pad * 4 + kMaxTasks * 64 - 1) / (kMaxTasks * 64);
-  p.wnc = std::max<uint32_t>(p.wnc, (prep_waves + p.ksc - 1) / p.ksc);
-  if (p.wnc > max_wnc) return false;
-  p.grid = (wave_quads + p.wnc - 1) / p.wnc;
-  p.tasks = bpc_pad * 4 <= 64 * p.ksc * p.wnc ? 1 : 2;
-  const size_t nj = 2 * mrows;
-  p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 8 + (size_t)p.wnc * p.ksc * mrows * 16 +
-          16 * mrows * 4 + 64;
-  if (p.lds > 150 * 1024) return false;
-  *out = p;
-  return true;
-}
-
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS>
-int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS>;
-  static bool big_lds_enabled = false;
-  if (p.lds > 64 * 1024 && !big_lds_enabled) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return (int)e;
-    big_lds_enabled = true;
-  }
-  GemvBatch bt{};
-  uint32_t quads = 0;
-  for (int j = 0; j < kMaxBatch; j++) {
-    if (j == 0 || j <= x.n_more) {
-      bt.w[j] = j == 0 ? x.w : x.more[j - 1].w;
-      bt.d[j] = j == 0 ? x.d : x.more[j - 1].d;
-      bt.c[j] = j == 0 ? x.c : x.more[j - 1].c;
-      bt.first_quad[j] = quads;
-      quads += (bt.w[j].n + 3) / 4;
-    } else {
-      bt.w[j] = x.w;
-      bt.first_quad[j] = 0xFFFFFFFFu;
-    }
-  }
-  hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants, x.m,
-                     p.ksc, p.wnc, x.w.k, x.w.n, bt.first_quad[1], bt.first_quad[2], (4096u + p.ksc - 1) / p.ksc, x.pro_weight,
-                     x.pro_eps,
-                     bt MGN_TRACE_ARG);
-  MGN_HIP_LAUNCH_CHECK();
-  return 0;
-}
-
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
-int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1>(s, x, p)
-                      : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2>(s, x, p);
-}
-
-template <int FMT, int MROWS, int STEPS, int QPW>
-int launch_steps(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  if constexpr (QPW == 1) {  // fused prologues come with one quad per wave only
-    if (x.pro_kind == kProRmsNorm) return launch_pro<FMT, MROWS, STEPS, QPW, kProRmsNorm>(s, x, p);
-    if (x.pro_kind == kProSwiglu) return launch_pro<FMT, MROWS, STEPS, QPW, kProSwiglu>(s, x, p);
-  }
-  if (x.pro_kind != kProNone) return (int)hipErrorInvalidValue;
-  return launch_pro<FMT, MROWS, STEPS, QPW, kProNone>(s, x, p);
-}
-
-uint32_t total_quads(const LaunchArgs& x) {
-  uint32_t q = (x.w.n + 3) / 4;
-  for (int j = 0; j < x.n_more; j++) q += (x.more[j].w.n + 3) / 4;
-  return q;
-}
-
-template <int FMT, int MROWS>
-int launch_t(ihipStream_t* s, const LaunchArgs& x) {
-  MfmaGemvPlan p;
-  if (!plan_mfma_gemv(x.w.k, total_quads(x), MROWS, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p))
-    return (int)hipErrorInvalidValue;
-  switch (p.steps * 8 + p.qpw) {
-    case 1 * 8 + 1: return launch_steps<FMT, MROWS, 1, 1>(s, x, p);
-    case 1 * 8 + 2: return launch_steps<FMT, MROWS, 1, 2>(s, x, p);
-    case 1 * 8 + 4: return launch_steps<FMT, MROWS, 1, 4>(s, x, p);
-    case 2 * 8 + 1: return launch_steps<FMT, MROWS, 2, 1>(s, x, p);
-    case 2 * 8 + 2: return launch_steps<FMT, MROWS, 2, 2>(s, x, p);
-    case 2 * 8 + 4: return launch_steps<FMT, MROWS, 2, 4>(s, x, p);
-    case 3 * 8 + 1: return launch_steps<FMT, MROWS, 3, 1>(s, x, p);
-    case 3 * 8 + 2: return launch_steps<FMT, MROWS, 3, 2>(s, x, p);
-    case 4 * 8 + 1: return launch_steps<FMT, MROWS, 4, 1>(s, x, p);
-    case 4 * 8 + 2: return launch_steps<FMT, MROWS, 4, 2>(s, x, p);
-    case 5 * 8 + 1: return launch_steps<FMT, MROWS, 5, 1>(s, x, p);
-    case 6 * 8 + 1: return launch_steps<FMT, MROWS, 6, 1>(s, x, p);
-    case 7 * 8 + 1: return launch_steps<FMT, MROWS, 7, 1>(s, x, p);
-    case 8 * 8 + 1: return launch_steps<FMT, MROWS, 8, 1>(s, x, p);
-    default: return (int)hipErrorInvalidValue;
-  }
-}
-
-}  // namespace
+int launch_gemv_mfma_q4_m1(ihipStream_t* s, const LaunchArgs& x);
+int launch_gemv_mfma_q4_m2(ihipStream_t* s, const LaunchArgs& x);
+int launch_gemv_mfma_q4_m4(ihipStream_t* s, const LaunchArgs& x);
+int launch_gemv_mfma_q8_m1(ihipStream_t* s, const LaunchArgs& x);
+int launch_gemv_mfma_q8_m2(ihipStream_t* s, const LaunchArgs& x);
+int launch_gemv_mfma_q8_m4(ihipStream_t* s, const LaunchArgs& x);
 
 bool gemv_mfma_supported(const LaunchArgs& x) {
   if (x.a_is_f16 || x.m == 0 || x.m > 4) return false;
@@ -688,8 +31,8 @@ bool gemv_mfma_supported(const LaunchArgs& x) {
 
 int launch_matmul_gemv_mfma(ihipStream_t* s, const LaunchArgs& x) {
   if (x.w.fmt == MGN_FMT_Q4)
-    return x.m == 1 ? launch_t<MGN_FMT_Q4, 1>(s, x) : x.m == 2 ? launch_t<MGN_FMT_Q4, 2>(s, x) : launch_t<MGN_FMT_Q4, 4>(s, x);
-  return x.m == 1 ? launch_t<MGN_FMT_Q8, 1>(s, x) : x.m == 2 ? launch_t<MGN_FMT_Q8, 2>(s, x) : launch_t<MGN_FMT_Q8, 4>(s, x);
+    return x.m == 1 ? launch_gemv_mfma_q4_m1(s, x) : x.m == 2 ? launch_gemv_mfma_q4_m2(s, x) : launch_gemv_mfma_q4_m4(s, x);
+  return x.m == 1 ? launch_gemv_mfma_q8_m1(s, x) : x.m == 2 ? launch_gemv_mfma_q8_m2(s, x) : launch_gemv_mfma_q8_m4(s, x);
 }
 
 }  // namespace mgn

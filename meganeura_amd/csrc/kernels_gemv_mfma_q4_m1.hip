@@ -1,0 +1,6 @@
+// MFMA GEMV kernels for Q4 weights and one activation row.
+#include "kernels_gemv_mfma.hip.h"
+
+namespace mgn {
+int launch_gemv_mfma_q4_m1(ihipStream_t* s, const LaunchArgs& x) { return launch_t<MGN_FMT_Q4, 1>(s, x); }
+}  // namespace mgn

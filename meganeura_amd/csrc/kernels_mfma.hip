@@ -613,7 +613,6 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
             bp.parts, bp.nch, bp.tpt, bp.colgroups * bp.parts * bp.grid_y);
 #endif
   if (best == 0 || (uint64_t)bp.colgroups * bp.parts > 0x7fffffffu) return false;
-  const uint32_t cb = 8 * bp.ksc;
   bp.lds = gemm_lds_bytes(x.w.fmt, bp.ksc, bp.wnc);
   *out = bp;
   return true;
