@@ -51,7 +51,7 @@ extern "C" int mgn_debug_set_trace_gemm(void* p) {
 }
 #define MGN_GSTAMP_INIT()                                                                                  \
   unsigned long long* const trace_base =                                                                   \
-      g.trace ? g.trace + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 16 : nullptr
+      g.trace ? g.trace + ((((size_t)blockIdx.z * g.colgroups + blockIdx.y) * g.parts + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 16 : nullptr
 #define MGN_GSTAMP(slot)                                                                  \
   do {                                                                                    \
     if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = __builtin_readcyclecounter(); \
@@ -113,14 +113,12 @@ constexpr int slice_stride(int fmt) { return fmt == MGN_FMT_Q4 ? 8 * 16 + 16 : 8
 typedef uint32_t u32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x2_unaligned __attribute__((ext_vector_type(2), aligned(2)));
 
-struct GemmArgs {
-  WeightView w;
-  const void* a;
+struct GemmTail {  // arguments first needed in the epilogue
   const float* dres;
   float* c;
   float* scratch;      // [parts][row tiles * ROWS][n] partial results when parts > 1
   uint32_t* counters;  // one arrival counter per (row tile, column group), zero between launches
-  uint32_t m, ksc, wnc, nch, parts, colgroups;
+  uint32_t row_tiles;
 #ifdef MGN_TRACE
   unsigned long long* trace;
 #endif
@@ -136,14 +134,39 @@ __device__ __forceinline__ uint4 f16_operand(uint4 v) {
   }
 }
 
-// grid = (column groups * parts, row tiles); blockDim.x = 64 * ksc * wnc, ksc in {1, 2}.
+// grid = (parts, column groups, row tiles); blockDim.x = 64 * ksc * wnc, ksc in {1, 2}.
 // A workgroup owns wnc column tiles of one row tile and K blocks
 // [part * nch * CB, (part + 1) * nch * CB); within a chunk wave (ks, wn) takes the
 // 8 blocks starting at 8 * ks.  While a chunk is being multiplied, the next chunk's
 // activations are in flight to registers and the weight ring is refilled one chunk ahead.
 // TPT = staging tasks per thread per chunk (one task = 8 consecutive k of one row).
+// The leading scalar arguments are the ones a wave needs before its first loads; as plain
+// scalars (not struct members) they can be handed over in registers at wave launch.
 template <int FMT, bool F32A, int TPT>
-__global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
+__global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__ a_arg, const void* __restrict__ meta_arg,
+                                                        const void* __restrict__ quants_arg, uint32_t m_arg, uint32_t ksc_arg,
+                                                        uint32_t wnc_arg, uint32_t nch_arg, uint32_t k_arg, uint32_t n_arg,
+                                                        uint32_t parts_arg, uint32_t colgroups_arg, GemmTail tail) {
+  // one view over both argument groups (the compiler keeps it in scalar registers)
+  struct {
+    WeightView w;
+    const void* a;
+    const float* dres;
+    float* c;
+    float* scratch;
+    uint32_t* counters;
+    uint32_t m, ksc, wnc, nch, parts, colgroups;
+#ifdef MGN_TRACE
+    unsigned long long* trace;
+#endif
+  } g;
+  g.w.meta = meta_arg, g.w.quants = quants_arg, g.w.k = k_arg, g.w.n = n_arg, g.w.fmt = FMT;
+  g.a = a_arg, g.m = m_arg, g.ksc = ksc_arg, g.wnc = wnc_arg, g.nch = nch_arg;
+  g.parts = parts_arg, g.colgroups = colgroups_arg;
+  g.dres = tail.dres, g.c = tail.c, g.scratch = tail.scratch, g.counters = tail.counters;
+#ifdef MGN_TRACE
+  g.trace = tail.trace;
+#endif
   constexpr int ROWS = F32A ? 16 : 32;  // real rows per tile
   constexpr int NI = F32A ? 8 : 16;     // result registers per lane
   constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;
@@ -159,15 +182,16 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
 
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t ks = wave % ksc, wn = wave / ksc;
+  const uint32_t ks = wave & (ksc - 1), wn = wave >> (ksc - 1);  // ksc is 1 or 2
   const uint32_t cl = lane & 31, gh = lane >> 5;
   const uint32_t bpc = w.k / 32;
   const uint32_t n_tiles = (w.n + 31) / 32;
-  const uint32_t cg = blockIdx.x / g.parts, part = blockIdx.x % g.parts;
+  const uint32_t cg = blockIdx.y, part = blockIdx.x;
+  const uint32_t nthreads = 64 * ksc * wnc;  // = blockDim.x
   const uint32_t col_tile = cg * wnc + wn;
   const uint32_t n = col_tile * 32 + cl;
   const bool n_ok = col_tile < n_tiles && n < w.n;
-  const uint32_t row0 = blockIdx.y * ROWS;
+  const uint32_t row0 = blockIdx.z * ROWS;
   const uint32_t zero_block = bpc * w.n;
   const uint32_t chunk0 = part * g.nch;  // first chunk of this workgroup
 
@@ -180,7 +204,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
   bool t_rowok[TPT], t_live[TPT];
 #pragma unroll
   for (int tt = 0; tt < TPT; tt++) {
-    const uint32_t t = tid + tt * blockDim.x;
+    const uint32_t t = tid + tt * nthreads;
     const uint32_t sub = t & 3, r = (t >> 2) % ROWS, lb = (t >> 2) / ROWS;
     t_lb[tt] = lb;
     t_r[tt] = r;
@@ -335,7 +359,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
   fetch_slice(chunk0, true);
   MGN_GSTAMP(1);
   // the additive operands' unused slots must read as zero for the whole kernel
-  for (uint32_t t = tid; t < 2 * s_stride; t += blockDim.x) simg[t] = make_uint4(0, 0, 0, 0);
+  for (uint32_t t = tid; t < 2 * s_stride; t += nthreads) simg[t] = make_uint4(0, 0, 0, 0);
   lds_barrier();
   stage(chunk0, 0);
   MGN_GSTAMP(2);
@@ -469,7 +493,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
     // (write-through stores, L2-coherent loads), with a single release fence per
     // workgroup; a fence in every wave plus an acquire on the reading side would write
     // back and invalidate the whole L2 hundreds of times.
-    const size_t plane = (size_t)gridDim.y * ROWS * w.n;  // floats per part
+    const size_t plane = (size_t)tail.row_tiles * ROWS * w.n;  // floats per part
     float* const mine = g.scratch + (size_t)part * plane + (size_t)row0 * w.n + n;
     if (writer) {
 #pragma unroll
@@ -482,7 +506,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
     MGN_GSTAMP(9);
     uint32_t* const flag = (uint32_t*)lds4;
     if (tid == 0) {
-      uint32_t* ctr = g.counters + blockIdx.y * g.colgroups + cg;
+      uint32_t* ctr = g.counters + blockIdx.z * g.colgroups + cg;
       // one device-scope release per workgroup: the barrier above ordered every wave's
       // stores before it, and it makes them visible to the other XCDs before the count
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
@@ -571,6 +595,7 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
       if (gemm_lds_bytes(x.w.fmt, ksc, wnc) > 160 * 1024) continue;
       if (wnc > n_tiles && wnc * ksc > 8 && wnc > 4) continue;  // idle waves only help staging up to a point
       const uint32_t colgroups = (n_tiles + wnc - 1) / wnc;
+      if (colgroups > 65535) continue;  // grid.y
       for (uint32_t nch = chunks; nch >= 1; nch--) {
         const uint32_t parts = (chunks + nch - 1) / nch;
         if ((chunks + parts - 1) / parts != nch) continue;  // same split, already seen
@@ -627,11 +652,13 @@ int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
     if (e != hipSuccess) return (int)e;
     big_lds_enabled = true;
   }
-  GemmArgs g{x.w, x.a, x.d, x.c, (float*)x.scratch, x.counters, x.m, p.ksc, p.wnc, p.nch, p.parts, p.colgroups};
+  GemmTail tail{x.d, x.c, (float*)x.scratch, x.counters, p.grid_y};
 #ifdef MGN_TRACE
-  g.trace = g_gemm_trace_host;
+  tail.trace = g_gemm_trace_host;
 #endif
-  hipLaunchKernelGGL(kern, dim3(p.colgroups * p.parts, p.grid_y), dim3(64 * p.ksc * p.wnc), p.lds, s, g);
+  if (p.colgroups > 65535 || p.grid_y > 65535) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups, p.grid_y), dim3(64 * p.ksc * p.wnc), p.lds, s, x.a, x.w.meta, x.w.quants,
+                     x.m, p.ksc, p.wnc, p.nch, x.w.k, x.w.n, p.parts, p.colgroups, tail);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }
