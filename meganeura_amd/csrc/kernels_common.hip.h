@@ -2,6 +2,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "mgn_internal.h"
 
 namespace mgn {
@@ -66,6 +68,19 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Kernels that use more than 64 KB of dynamic LDS need the limit raised once per kernel and
+// per device (the attribute belongs to the device's copy of the function).  `done` is a
+// per-kernel bit set over device ordinals.
+template <typename Kernel>
+inline int enable_big_lds(Kernel kern, int device, std::atomic<uint64_t>& done) {
+  const uint64_t bit = 1ull << (device & 63);
+  if (done.load(std::memory_order_acquire) & bit) return 0;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e != hipSuccess) return (int)e;
+  done.fetch_or(bit, std::memory_order_release);
+  return 0;
 }
 
 #define MGN_HIP_LAUNCH_CHECK()                      \

@@ -281,17 +281,13 @@ int launch_gemv_t(ihipStream_t* s, const LaunchArgs& x) {
   const uint32_t nw = 64 / p.kbw;
   const size_t lds = ((size_t)MR * (x.w.k / 32) * kXStride +
                       (p.kgc > 1 ? (size_t)p.kgc * MR * p.steps * nw * p.wnc : 0)) * sizeof(float);
-  // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+  // more than 64 KiB of dynamic LDS has to be allowed per kernel and device, once
 #define MGN_GEMV(KBW)                                                                                   \
   do {                                                                                                  \
     auto kern = gemv_kernel<FMT, KBW, MR, kUnroll>;                                                     \
-    static bool big_lds_enabled = false;                                                                \
-    if (lds > 64 * 1024 && !big_lds_enabled) {                                                          \
-      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                         160 * 1024);                                                   \
-      if (e != hipSuccess) return (int)e;                                                               \
-      big_lds_enabled = true;                                                                           \
-    }                                                                                                   \
+    static std::atomic<uint64_t> big_lds_done{0};                                                       \
+    if (lds > 64 * 1024)                                                                                \
+      if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;                               \
     hipLaunchKernelGGL(kern, grid, block, lds, s, x.w, (const float*)x.a, x.d, x.c, x.m, p.steps, p.kgc); \
   } while (0)
   switch (p.kbw) {

@@ -598,12 +598,9 @@ bool plan_mfma_gemv(uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bo
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS>
 int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
   auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS>;
-  static bool big_lds_enabled = false;
-  if (p.lds > 64 * 1024 && !big_lds_enabled) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return (int)e;
-    big_lds_enabled = true;
-  }
+  static std::atomic<uint64_t> big_lds_done{0};
+  if (p.lds > 64 * 1024)
+    if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
   GemvBatch bt{};
   uint32_t quads = 0;
   for (int j = 0; j < kMaxBatch; j++) {

@@ -646,12 +646,8 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
 template <int FMT, bool F32A, int TPT>
 int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
   auto kern = gemm_mfma_kernel<FMT, F32A, TPT>;
-  static bool big_lds_enabled = false;
-  if (!big_lds_enabled) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return (int)e;
-    big_lds_enabled = true;
-  }
+  static std::atomic<uint64_t> big_lds_done{0};
+  if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
   GemmTail tail{x.d, x.c, (float*)x.scratch, x.counters, p.grid_y};
 #ifdef MGN_TRACE
   tail.trace = g_gemm_trace_host;

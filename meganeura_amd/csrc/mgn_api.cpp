@@ -455,6 +455,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   if (d && d->bytes / 4 < (size_t)m * n) return fail(ctx, MGN_EINVAL, "D is smaller than m*N floats");
   if (c->ptr == a->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
   mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus};
+  x.device = ctx->device;
   x.scratch = ctx->scratch;
   x.scratch_bytes = ctx->scratch_bytes;
   x.counters = ctx->counters;
@@ -537,6 +538,7 @@ mgn_status mgn_matmul_q_batch(mgn_ctx* ctx, const mgn_buf* a, mgn_prologue prolo
     if (j > 0) x.more[j - 1] = {view_of(it.w), it.d ? (const float*)it.d->ptr : nullptr, (float*)it.c->ptr};
   }
   x.n_more = (int)count - 1;
+  x.device = ctx->device;
   x.pro_kind = (int)prologue;
   x.pro_weight = norm_weight ? (const float*)norm_weight->ptr : nullptr;
   x.pro_eps = eps;

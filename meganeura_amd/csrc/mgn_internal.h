@@ -47,6 +47,7 @@ struct LaunchArgs {
   uint32_t m;
   bool a_is_f16;
   int num_cus;
+  int device = 0;  // HIP device ordinal of the context
   // further weights served by the same launch (GEMV-MFMA route only): same K, format and
   // activations, each with its own output and optional residual
   struct More {
