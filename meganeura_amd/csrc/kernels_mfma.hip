@@ -673,6 +673,7 @@ int launch_fa(ihipStream_t* s, const LaunchArgs& x) {
 }  // namespace
 
 bool gemm_mfma_supported(const LaunchArgs& x) {
+  if (!x.w.mfma_gemm_range_ok) return false;  // a block minimum or scale too large for the fp16 operand
   GemmPlan p;
   return plan_gemm(x, &p);
 }

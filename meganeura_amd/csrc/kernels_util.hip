@@ -1,6 +1,8 @@
 // Layout and conversion kernels: device-side dequantize, the bit-exact block
 // quantizer, and conversion between the reference's Q8 byte layout and the
 // device layout.  None of these is on the per-token path.
+#include <algorithm>
+
 #include "kernels_common.hip.h"
 #include "session.h"
 
@@ -61,6 +63,25 @@ __global__ __launch_bounds__(256) void import_q8_kernel(const uint32_t* __restri
   scales[b] = (uint16_t)ref[b * 9];
 #pragma unroll
   for (int i = 0; i < 8; i++) quants[b * 8 + i] = ref[b * 9 + 1 + i];
+}
+
+// Largest |scale| and largest |min| over all blocks, as f32 bit patterns (for non-negative
+// floats the unsigned order is the numeric order, and inf / NaN sort above every finite value).
+// out[0], out[1] must be zero before the launch.
+__global__ __launch_bounds__(256) void scale_range_kernel(int fmt, const void* __restrict__ meta, size_t nb,
+                                                          uint32_t* __restrict__ out) {
+  uint32_t smax = 0, mmax = 0;
+  for (size_t b = (size_t)blockIdx.x * 256 + threadIdx.x; b < nb; b += (size_t)gridDim.x * 256) {
+    if (fmt == MGN_FMT_Q4) {
+      const uint32_t dm = ((const uint32_t*)meta)[b];
+      smax = max(smax, __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(dm & 0xFFFFu))));
+      mmax = max(mmax, __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(dm >> 16))));
+    } else {
+      smax = max(smax, __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(((const uint16_t*)meta)[b]))));
+    }
+  }
+  atomicMax(out, smax);
+  atomicMax(out + 1, mmax);
 }
 
 __device__ __forceinline__ float clamp_keep_nan(float v, float lo, float hi) {
@@ -213,6 +234,14 @@ int launch_export_q8(ihipStream_t* s, const WeightView& w, uint8_t* out_dev) {
   const size_t nb = (size_t)(w.k / 32) * w.n;
   hipLaunchKernelGGL(export_q8_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s,
                      (const uint16_t*)w.meta, (const uint32_t*)w.quants, nb, (uint32_t*)out_dev);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev) {
+  const size_t nb = (size_t)(w.k / 32) * w.n;
+  hipLaunchKernelGGL(scale_range_kernel, dim3((unsigned)std::min<size_t>((nb + 255) / 256, 4096)), dim3(256), 0, s, w.fmt,
+                     w.meta, nb, out2_dev);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

@@ -3,6 +3,7 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 #include <new>
 #include <string>
@@ -37,7 +38,7 @@ size_t quant_elem(mgn_fmt fmt) { return fmt == MGN_FMT_Q4 ? 16 : 32; }
 bool valid_fmt(mgn_fmt fmt) { return fmt == MGN_FMT_Q4 || fmt == MGN_FMT_Q8; }
 
 mgn::WeightView view_of(const mgn_weight* w) {
-  return mgn::WeightView{w->meta, w->quants, (uint32_t)w->rows, (uint32_t)w->cols, (int)w->fmt};
+  return mgn::WeightView{w->meta, w->quants, (uint32_t)w->rows, (uint32_t)w->cols, (int)w->fmt, w->mfma_gemm_range_ok};
 }
 
 // Device storage for a [rows, cols] weight, contents undefined.
@@ -78,6 +79,23 @@ mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn
   return MGN_OK;
 }
 
+// Looks at every block's scale (and minimum) once, right after a weight's blocks are on the
+// device, and records whether the tiled MFMA kernel may take this weight.  Synchronises.
+mgn_status scan_weight_range(mgn_ctx* ctx, mgn_weight* w) {
+  uint32_t* dev = (uint32_t*)((char*)ctx->scratch + ctx->scratch_bytes) + ctx->n_counters;  // two spare words
+  hipError_t e = hipMemsetAsync(dev, 0, 8, ctx->stream);
+  if (e == hipSuccess) e = (hipError_t)mgn::launch_scale_range(ctx->stream, view_of(w), dev);
+  uint32_t host[2] = {0, 0};
+  if (e == hipSuccess) e = hipMemcpyAsync(host, dev, 8, hipMemcpyDeviceToHost, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess) return hip_fail(ctx, "weight range scan", e);
+  float smax, mmax;
+  std::memcpy(&smax, &host[0], 4);
+  std::memcpy(&mmax, &host[1], 4);
+  w->mfma_gemm_range_ok = w->fmt == MGN_FMT_Q4 ? (mmax < 2047.0f && std::isfinite(smax)) : smax < 15.99f;
+  return MGN_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -109,8 +127,9 @@ mgn_status mgn_ctx_create(int device_id, mgn_ctx** out) {
   // workspace of the split-K matmul kernels: partial tiles, then 4096 arrival counters
   constexpr size_t kScratchBytes = (size_t)16 << 20;
   constexpr uint32_t kCounters = 4096;
-  if ((e = hipMalloc(&ctx->scratch, kScratchBytes + kCounters * sizeof(uint32_t))) != hipSuccess ||
-      (e = hipMemsetAsync((char*)ctx->scratch + kScratchBytes, 0, kCounters * sizeof(uint32_t), ctx->stream)) != hipSuccess) {
+  // (+ two words the weight range scan reduces into)
+  if ((e = hipMalloc(&ctx->scratch, kScratchBytes + (kCounters + 2) * sizeof(uint32_t))) != hipSuccess ||
+      (e = hipMemsetAsync((char*)ctx->scratch + kScratchBytes, 0, (kCounters + 2) * sizeof(uint32_t), ctx->stream)) != hipSuccess) {
     mgn_ctx_destroy(ctx);
     return hip_fail(nullptr, "workspace allocation", e);
   }
@@ -269,6 +288,11 @@ mgn_status mgn_weight_create_packed(mgn_ctx* ctx, mgn_fmt fmt, const uint8_t* pa
     mgn_weight_free(ctx, w);
     return hip_fail(ctx, "weight upload", e);
   }
+  st = scan_weight_range(ctx, w);
+  if (st != MGN_OK) {
+    mgn_weight_free(ctx, w);
+    return st;
+  }
   *out = w;
   return MGN_OK;
 }
@@ -322,6 +346,11 @@ mgn_status mgn_weight_create_device(mgn_ctx* ctx, mgn_fmt fmt, const mgn_buf* w_
   if (e != hipSuccess) {
     mgn_weight_free(ctx, w);
     return hip_fail(ctx, "quantize kernel", e);
+  }
+  st = scan_weight_range(ctx, w);
+  if (st != MGN_OK) {
+    mgn_weight_free(ctx, w);
+    return st;
   }
   *out = w;
   return MGN_OK;

@@ -35,6 +35,9 @@ struct WeightView {
   const void* quants;
   uint32_t k, n;  // rows, cols
   int fmt;        // mgn_fmt
+  // The tiled MFMA kernel feeds 32 * min (Q4) or 4096 * scale (Q8) to the matrix cores as
+  // fp16: true when every block of this weight keeps that finite (|min| < 2047, scale < 15.99).
+  bool mfma_gemm_range_ok = true;
 };
 
 enum { kProNone = 0, kProRmsNorm = 1, kProSwiglu = 2 };
@@ -72,6 +75,7 @@ struct LaunchArgs {
 int launch_dequantize(ihipStream_t* s, const WeightView& w, float* out_dev);  // out [k, n] f32
 int launch_export_q8(ihipStream_t* s, const WeightView& w, uint8_t* out_dev);  // 36-byte blocks
 int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* meta, void* quants);
+int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev);  // out: max |scale|, max |min| bits
 int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, uint32_t n, void* meta,
                     void* quants);
 int launch_matmul_generic(ihipStream_t* s, const LaunchArgs& a);
@@ -110,4 +114,5 @@ struct mgn_weight {
   void* meta = nullptr;    // into base
   void* quants = nullptr;  // into base, 256-byte aligned
   size_t meta_bytes = 0, quant_bytes = 0;
+  bool mfma_gemm_range_ok = true;  // see WeightView
 };

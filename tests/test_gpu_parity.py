@@ -390,3 +390,33 @@ def test_activations_and_weights_with_a_large_mean(ctx, orc, fmt, m, route):
     want = orc.matmul_f64(x, orc.dequantize(fmt, packed, k, n))
     got = run_matmul(ctx, fmt, x, w, ROUTES[route])
     orc.assert_close(got, want, REL, ABS)
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+def test_weights_outside_the_tiled_kernels_range_take_another_route(ctx, orc, fmt):
+    """The tiled MFMA kernel hands 32 x block-minimum (Q4) or 4096 x scale (Q8) to the matrix
+    cores as fp16.  A weight with a block beyond that is recognised when it is created: the
+    automatic route then avoids that kernel and the result is still the oracle's."""
+    m, k, n = 16, 256, 96
+    w = synth.normal(990 + fmt, k * n, 0.02).reshape(k, n)
+    w[32:64, 5] = np.linspace(-5000.0, -4990.0, 32, dtype=np.float32)   # block minimum -5000
+    w[64:96, 7] = np.linspace(-3000.0, 3000.0, 32, dtype=np.float32)    # Q8 scale 23.6
+    x = synth.normal(991, m * k, 1.0).reshape(m, k)
+    wt = ctx.weight(fmt, w)
+    want = orc.matmul_packed(fmt, x, orc.quantize(fmt, w), n)
+    got = run_matmul(ctx, fmt, x, wt)
+    assert np.isfinite(got).all()
+    orc.assert_close(got, want, REL, ABS)
+    with pytest.raises(capi.MgnError, match="does not support"):
+        run_matmul(ctx, fmt, x, wt, ROUTES["gemm_mfma"])
+    # batch-1 stays on the MFMA GEMV, which has no such limit
+    got1 = run_matmul(ctx, fmt, x[:1], wt, ROUTES["gemv_mfma"])
+    orc.assert_close(got1, want[:1], REL, ABS)
+    wt.free()
+    # same weight through the device quantizer and from packed bytes
+    src = ctx.upload(w)
+    for other in (ctx.weight_from_device(fmt, src, k, n), ctx.weight_from_packed(fmt, orc.quantize(fmt, w), k, n)):
+        with pytest.raises(capi.MgnError, match="does not support"):
+            run_matmul(ctx, fmt, x, other, ROUTES["gemm_mfma"])
+        other.free()
+    src.free()
