@@ -38,7 +38,9 @@ typedef enum mgn_status {
   MGN_EHIP = 3,      /* a HIP runtime call failed; see mgn_last_error */
   MGN_ENOTFOUND = 4, /* unknown name (session layer) */
   MGN_ENODEVICE = 5, /* no usable gfx950 device */
-  MGN_EUNSUPPORTED = 6 /* a fused entry point asked for a shape its kernel does not serve */
+  MGN_EUNSUPPORTED = 6, /* a fused entry point asked for a shape its kernel does not serve */
+  MGN_ERANGE = 7 /* reported by the next synchronising call: an f32 activation too large for the kernel
+                    that ran (|x| >= 65504 on the tiled MFMA route, M >= 5); outputs of that call are wrong */
 } mgn_status;
 
 /* compile::WeightFormat::{Q4,Q8} (src/compile.rs:8-29), graph::DType::{Q4_0,Q8_0}

@@ -118,6 +118,7 @@ struct GemmTail {  // arguments first needed in the epilogue
   float* c;
   float* scratch;      // [parts][row tiles * ROWS][n] partial results when parts > 1
   uint32_t* counters;  // one arrival counter per (row tile, column group), zero between launches
+  uint32_t* range_flag;  // host-visible: set when an f32 activation does not fit the fp16 pair
   uint32_t row_tiles;
 #ifdef MGN_TRACE
   unsigned long long* trace;
@@ -251,6 +252,10 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
 #pragma unroll
           for (int e = 0; e < 8; e++) p[e] = x[e];
         }
+        // hi + lo covers |x| < 65504 only (the conversion saturates silently beyond): say so
+        const float amax = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))),
+                                 fmaxf(fmaxf(fabsf(x[4]), fabsf(x[5])), fmaxf(fabsf(x[6]), fabsf(x[7]))));
+        if (!(amax < 65504.0f) && tail.range_flag) *tail.range_flag = 1u;
         const uint32_t hp[4] = {pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7])};
         float res[8], hs = 0.0f;
 #pragma unroll
@@ -648,7 +653,7 @@ int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
   auto kern = gemm_mfma_kernel<FMT, F32A, TPT>;
   static std::atomic<uint64_t> big_lds_done{0};
   if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
-  GemmTail tail{x.d, x.c, (float*)x.scratch, x.counters, p.grid_y};
+  GemmTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.range_flag, p.grid_y};
 #ifdef MGN_TRACE
   tail.trace = g_gemm_trace_host;
 #endif

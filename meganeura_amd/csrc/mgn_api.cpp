@@ -79,6 +79,15 @@ mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn
   return MGN_OK;
 }
 
+// After the stream has been synchronised: did a kernel meet activations outside its range?
+mgn_status check_range_flag(mgn_ctx* ctx) {
+  if (!ctx->range_flag_host || *(volatile uint32_t*)ctx->range_flag_host == 0) return MGN_OK;
+  *(volatile uint32_t*)ctx->range_flag_host = 0;
+  return fail(ctx, MGN_ERANGE,
+              "an f32 activation of magnitude >= 65504 reached the tiled MFMA kernel (M >= 5), which splits activations "
+              "into fp16 pairs: the affected outputs are wrong; select MGN_ROUTE_GENERIC for such data");
+}
+
 // Looks at every block's scale (and minimum) once, right after a weight's blocks are on the
 // device, and records whether the tiled MFMA kernel may take this weight.  Synchronises.
 mgn_status scan_weight_range(mgn_ctx* ctx, mgn_weight* w) {
@@ -136,6 +145,14 @@ mgn_status mgn_ctx_create(int device_id, mgn_ctx** out) {
   ctx->scratch_bytes = kScratchBytes;
   ctx->counters = (uint32_t*)((char*)ctx->scratch + kScratchBytes);
   ctx->n_counters = kCounters;
+  // one pinned, device-mapped word: a kernel that meets activations it cannot represent sets it
+  // and the next synchronising call reports MGN_ERANGE
+  if ((e = hipHostMalloc((void**)&ctx->range_flag_host, sizeof(uint32_t), hipHostMallocMapped)) != hipSuccess ||
+      (e = hipHostGetDevicePointer((void**)&ctx->range_flag_dev, ctx->range_flag_host, 0)) != hipSuccess) {
+    mgn_ctx_destroy(ctx);
+    return hip_fail(nullptr, "pinned flag allocation", e);
+  }
+  *ctx->range_flag_host = 0;
   *out = ctx;
   return MGN_OK;
 }
@@ -147,6 +164,7 @@ void mgn_ctx_destroy(mgn_ctx* ctx) {
     (void)hipStreamDestroy(ctx->stream);
   }
   if (ctx->scratch) (void)hipFree(ctx->scratch);
+  if (ctx->range_flag_host) (void)hipHostFree(ctx->range_flag_host);
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
   if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
   delete ctx;
@@ -157,7 +175,7 @@ const char* mgn_last_error(const mgn_ctx* ctx) { return ctx ? ctx->err.c_str() :
 mgn_status mgn_sync(mgn_ctx* ctx) {
   if (!ctx) return MGN_EINVAL;
   MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  return MGN_OK;
+  return check_range_flag(ctx);
 }
 
 mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route) {
@@ -216,7 +234,7 @@ mgn_status mgn_buf_download(mgn_ctx* ctx, const mgn_buf* buf, size_t offset, voi
   if (bytes == 0) return mgn_sync(ctx);
   MGN_HIP(ctx, hipMemcpyAsync(dst, (const char*)buf->ptr + offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
   MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
-  return MGN_OK;
+  return check_range_flag(ctx);
 }
 
 mgn_status mgn_buf_copy(mgn_ctx* ctx, mgn_buf* dst, const mgn_buf* src, size_t bytes) {
@@ -485,6 +503,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   if (c->ptr == a->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
   mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus};
   x.device = ctx->device;
+  x.range_flag = ctx->range_flag_dev;
   x.scratch = ctx->scratch;
   x.scratch_bytes = ctx->scratch_bytes;
   x.counters = ctx->counters;
@@ -603,7 +622,7 @@ mgn_status mgn_timer_stop(mgn_ctx* ctx, float* elapsed_ms) {
   MGN_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
   MGN_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
   MGN_HIP(ctx, hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
-  return MGN_OK;
+  return check_range_flag(ctx);
 }
 
 }  // extern "C"

@@ -69,6 +69,8 @@ struct LaunchArgs {
   size_t scratch_bytes = 0;
   uint32_t* counters = nullptr;  // all zero between launches
   uint32_t n_counters = 0;
+  // host-visible word a kernel sets when f32 activations leave the range it can represent
+  uint32_t* range_flag = nullptr;
 };
 
 // kernels.hip
@@ -99,6 +101,8 @@ struct mgn_ctx {
   size_t scratch_bytes = 0;
   uint32_t* counters = nullptr;
   uint32_t n_counters = 0;
+  uint32_t* range_flag_host = nullptr;  // pinned, mapped: written by kernels, read at sync points
+  uint32_t* range_flag_dev = nullptr;   // the same word as the device sees it
   std::string err;
 };
 

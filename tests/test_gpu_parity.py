@@ -420,3 +420,24 @@ def test_weights_outside_the_tiled_kernels_range_take_another_route(ctx, orc, fm
             run_matmul(ctx, fmt, x, other, ROUTES["gemm_mfma"])
         other.free()
     src.free()
+
+
+def test_activations_beyond_the_fp16_pair_are_reported(ctx, orc):
+    """An f32 activation >= 65504 cannot be split into an fp16 pair: the tiled kernel flags it
+    and the next synchronising call fails loudly instead of handing back wrong numbers.  The
+    generic route computes such data; batch-1..4 (MFMA GEMV) rescales per block and has no limit."""
+    m, k, n = 16, 256, 96
+    w = synth.normal(995, k * n, 0.02).reshape(k, n)
+    x = synth.normal(996, m * k, 1.0).reshape(m, k)
+    x[3, 17] = np.float32(2.0e5)
+    wt = ctx.weight(Q4, w)
+    want = orc.matmul_packed(Q4, x, orc.quantize(Q4, w), n)
+    with pytest.raises(capi.MgnError) as e:
+        run_matmul(ctx, Q4, x, wt, ROUTES["gemm_mfma"])
+    assert e.value.status == capi.ERANGE
+    ctx.sync()  # reported once; the context keeps working
+    orc.assert_close(run_matmul(ctx, Q4, x, wt, ROUTES["generic"]), want, REL, ABS)
+    orc.assert_close(run_matmul(ctx, Q4, x[:4], wt, ROUTES["gemv_mfma"]), want[:4], REL, ABS)
+    x[3, 17] = np.float32(60000.0)  # inside the range
+    orc.assert_close(run_matmul(ctx, Q4, x, wt, ROUTES["gemm_mfma"]), orc.matmul_packed(Q4, x, orc.quantize(Q4, w), n), REL, ABS)
+    wt.free()
