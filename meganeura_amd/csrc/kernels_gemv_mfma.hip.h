@@ -95,7 +95,7 @@ constexpr int kMaxTasks = 2;  // activation chunks a thread prepares at most, pe
 #ifndef MGN_GEMV_DEPTH
 #define MGN_GEMV_DEPTH 3
 #endif
-constexpr int kDepth = MGN_GEMV_DEPTH;  // weight blocks in flight per lane ahead of the one in use
+constexpr int kDepth = MGN_GEMV_DEPTH;
 
 __device__ __forceinline__ half4 as_half4(uint32_t lo, uint32_t hi) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -158,24 +158,51 @@ struct Raw<MGN_FMT_Q4> {
     q = stream_load_u128((const uint4*)w.quants + b);
     meta = stream_load_u32((const uint32_t*)w.meta + b);
   }
+  __device__ __forceinline__ void load_at(const char* pq, const char* pm) {
+    q = stream_load_u128(pq);
+    meta = stream_load_u32(pm);
+  }
 };
+// Q8: a lane does not fetch "its" 32-byte block with two 16-byte loads (each load instruction
+// would then touch only half of every cache line it brings in, and the line is fetched from
+// L2 twice).  Instead the 16 lanes of a column read 16 consecutive 16-byte pieces per load:
+// lane b gets half (b & 1) of K block kb0 + b/2 from the first load and the same half of
+// block kb0 + 8 + b/2 from the second.  Each half block carries its own scale and its own
+// MFMA chain; the A operands are read from LDS to match.
 template <>
 struct Raw<MGN_FMT_Q8> {
   uint4 q0, q1;
-  uint32_t meta;
-  __device__ __forceinline__ void load(const WeightView& w, size_t b) {
-    q0 = stream_load_u128((const uint4*)w.quants + b * 2);
-    q1 = stream_load_u128((const uint4*)w.quants + b * 2 + 1);
-    meta = stream_load_u16((const uint16_t*)w.meta + b);
+  uint32_t meta0, meta1;
+  __device__ __forceinline__ void load(const WeightView& w, size_t b0, size_t b1, uint32_t half) {
+    q0 = stream_load_u128((const uint4*)w.quants + b0 * 2 + half);
+    q1 = stream_load_u128((const uint4*)w.quants + b1 * 2 + half);
+    meta0 = stream_load_u16((const uint16_t*)w.meta + b0);
+    meta1 = stream_load_u16((const uint16_t*)w.meta + b1);
+  }
+  // pq, pm: this lane's half of block kb0 + b/2; the partner block is 8 blocks further on
+  __device__ __forceinline__ void load_at(const char* pq, const char* pm) {
+    q0 = stream_load_u128(pq);
+    q1 = stream_load_u128(pq + 8 * 32);
+    meta0 = stream_load_u16(pm);
+    meta1 = stream_load_u16(pm + 8 * 2);
   }
 };
+
+// LDS entries of the chain constants per K block: one for a Q4 block, one per half for Q8
+template <int FMT>
+constexpr uint32_t cinit_per_block() { return FMT == MGN_FMT_Q8 ? 2u : 1u; }
+// Padding (in 16-byte units) behind every chunk plane.  Q8 lanes of one LDS access read from
+// two planes at once (chunks 2h and 2h+1 of half h); the padding moves those onto different banks.
+template <int FMT>
+constexpr uint32_t plane_pad(uint32_t nj) { return FMT == MGN_FMT_Q8 ? (nj == 4 ? 4u : 2u) : 0u; }
 
 // LDS image of the activations, per workgroup:
 //   chunk planes  xa[c][kb * NJ + j]  (uint4), c = 0..3: the A-operand rows of the two
 //                 MFMAs that consume elements 8c..8c+7 of K block kb; j = 2*row (high
 //                 halves) or 2*row + 1 (low halves);
 //   cinit[kb][row] = { -bias / operand_scale * S(kb, row), the chain's initial accumulator;
-//                      operand_scale / block scale, which undoes both scalings afterwards }.
+//                      operand_scale / block scale, which undoes both scalings afterwards }
+//                 (Q8: cinit[kb][half][row], S over the 16 elements of that half).
 // Q4 pairs nibble k with k+4 in one fp16x2 mask, so the chunk is (x0,x4,x2,x6 | x1,x5,x3,x7).
 // Q8 bytes come out in natural order: (x0,x1,x2,x3 | x4,x5,x6,x7).
 template <int FMT>
@@ -224,7 +251,11 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 //   kProSwiglu   a[m, 2K] = gate | up  ->  gate * sigmoid(gate) * up  (src/shaders/swiglu_concat.wgsl:20-32).
 // TASKS: activation chunks per thread (1 when the workgroup has a thread for every chunk; the
 // prologue in front of the first weight load is then half as long).
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS>
+// EXACT: K is a multiple of 512 and the K splits share the steps evenly, so every step of every
+// live wave is a full one.  A lane's loads are then its base pointer plus a constant (no
+// address arithmetic or range checks per step), waves without a quad skip the walk, and only
+// the column index is clamped (for a last quad with fewer than four columns).
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // The leading scalar arguments are what a wave needs before it can issue its first loads;
     // they are declared first (and not inside a struct) so that the dispatcher can hand them
@@ -259,11 +290,12 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   const uint32_t quad_base = pick3(widx, 0u, first_quad1, first_quad2);  // first quad of that weight
   const uint32_t bpc = w.k / 32;
   const uint32_t bpc_pad = (bpc + 15) & ~15u;
-  const uint32_t plane = bpc_pad * NJ;
+  constexpr uint32_t CPB = cinit_per_block<FMT>();
+  const uint32_t plane = bpc_pad * NJ + plane_pad<FMT>(NJ);
   const uint32_t nwaves = ksc * wnc;
   uint4* xa = lds4;                                   // [4][plane]
-  float2* cinit = (float2*)(lds4 + 4 * plane);        // [bpc_pad][MROWS]
-  float* red = (float*)(cinit + bpc_pad * MROWS);     // [wnc][ksc][MROWS][4]
+  float2* cinit = (float2*)(lds4 + 4 * plane);        // [bpc_pad][CPB][MROWS]
+  float* red = (float*)(cinit + bpc_pad * CPB * MROWS);  // [wnc][ksc][MROWS][4]
   float* nrm = red + wnc * ksc * MROWS * 4;           // [16 waves][MROWS] sums of squares (kProRmsNorm)
 
   const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -321,13 +353,44 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   constexpr int TS = STEPS * QPW;
   Raw<FMT> blk[TS];
   const uint32_t wbase = (quad * 4 + i) * bpc + kb_first;
+  // Q8: first block of this lane's pair, see Raw<MGN_FMT_Q8>
+  const uint32_t kb8_first = (wave_live ? step_begin : 0u) * 16 + (b >> 1);
+  const uint32_t wbase8 = (quad * 4 + i) * bpc + kb8_first;
+  constexpr uint32_t QB = FMT == MGN_FMT_Q8 ? 32 : 16, MB = FMT == MGN_FMT_Q8 ? 2 : 4;  // bytes per block
+  const char* pq[QPW];
+  const char* pm[QPW];
+  if constexpr (EXACT) {
+#pragma unroll
+    for (int q = 0; q < QPW; q++) {
+      const uint32_t col = min((quad + q) * 4 + i, w.n - 1);
+      const uint32_t at = col * bpc + (FMT == MGN_FMT_Q8 ? kb8_first : kb_first);
+      pq[q] = (const char*)w.quants + (size_t)at * QB + (FMT == MGN_FMT_Q8 ? (b & 1) * 16 : 0);
+      pm[q] = (const char*)w.meta + (size_t)at * MB;
+    }
+  }
   auto fetch = [&](int t) {
     const int q = t / STEPS, s = t % STEPS;
-    const bool ok = wave_live && (quad + q) * 4 + i < w.n && step_begin + s < steps_total && kb_first + s * 16 < bpc;
-    blk[t].load(w, ok ? wbase + q * 4 * bpc + s * 16 : zero_block);
+    if constexpr (EXACT) {
+      blk[t].load_at(pq[q] + s * (16 * QB), pm[q] + s * (16 * MB));
+      return;
+    }
+    const bool col_ok = wave_live && (quad + q) * 4 + i < w.n && step_begin + s < steps_total;
+    if constexpr (FMT == MGN_FMT_Q8) {
+      const bool ok0 = col_ok && kb8_first + s * 16 < bpc, ok1 = col_ok && kb8_first + s * 16 + 8 < bpc;
+      const uint32_t at = wbase8 + q * 4 * bpc + s * 16;
+      blk[t].load(w, ok0 ? at : zero_block, ok1 ? at + 8 : zero_block, b & 1);
+    } else {
+      const bool ok = col_ok && kb_first + s * 16 < bpc;
+      blk[t].load(w, ok ? wbase + q * 4 * bpc + s * 16 : zero_block);
+    }
   };
+  // (EXACT: a wave without a quad issues these too, from the last column's blocks, and skips
+  // the walk; a branch around the loads would make every wave wait for them at the join)
 #pragma unroll
-  for (int t = 0; t < TS && t < kDepth; t++) fetch(t);
+  for (int t = 0; t < TS && t < kDepth; t++) {
+    fetch(t);
+    if constexpr (EXACT) __builtin_amdgcn_sched_barrier(0);  // in this order: step 0 waits for its own block only
+  }
   for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += nthreads) red[t] = 0.0f;
   MGN_STAMP_EARLY();
   MGN_STAMP_FLUSH();
@@ -410,9 +473,15 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         xa[ch * plane + kb * NJ + 2 * r + 1] = lo;
         float s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
         s += dpp_move<kDppQuadXor1>(s);
-        s += dpp_move<kDppQuadXor2>(s);
         constexpr float bias = FMT == MGN_FMT_Q4 ? 8.0f : 128.0f;
-        if (ch == 0) cinit[kb * MROWS + r] = make_float2(s * (-bias / operand_scale<FMT>()), inv * operand_scale<FMT>());
+        if constexpr (FMT == MGN_FMT_Q8) {
+          // chunks 0,1 and 2,3 are the two halves of the block
+          if ((ch & 1) == 0)
+            cinit[(kb * 2 + (ch >> 1)) * MROWS + r] = make_float2(s * (-bias / operand_scale<FMT>()), inv * operand_scale<FMT>());
+        } else {
+          s += dpp_move<kDppQuadXor2>(s);
+          if (ch == 0) cinit[kb * MROWS + r] = make_float2(s * (-bias / operand_scale<FMT>()), inv * operand_scale<FMT>());
+        }
       }
     }
   }
@@ -423,36 +492,49 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   // ---- the K walk: STEPS blocks per lane, straight-line ----
   // Lanes i >= NJ have no activation row of their own; they re-read row i % NJ (a broadcast
   // in LDS) and the D entries they produce are never looked at.
-  const char* xa_lane = (const char*)xa + ((kb_first * NJ) + (NJ < 4 ? i % NJ : i)) * 16;
-  const char* ci_lane = (const char*)cinit + kb_first * MROWS * 8;
+  const uint32_t jrow = NJ < 4 ? i % NJ : i;
+  // Q4: K block kb_first + 16 s.  Q8: half (b & 1) of blocks kb8_first + 16 s and + 8, i.e. chunks
+  // 2 (b & 1) and 2 (b & 1) + 1 of those blocks.
+  const char* xa_lane = FMT == MGN_FMT_Q8
+                            ? (const char*)xa + ((size_t)kb8_first * NJ + jrow + (size_t)2 * (b & 1) * plane) * 16
+                            : (const char*)xa + ((size_t)kb_first * NJ + jrow) * 16;
+  const char* ci_lane = FMT == MGN_FMT_Q8 ? (const char*)cinit + (size_t)(kb8_first * 2 + (b & 1)) * MROWS * 8
+                                          : (const char*)cinit + (size_t)kb_first * MROWS * 8;
   float acc[QPW][MROWS];  // lane (b, j): sum over this lane's K blocks for column 4*(quad+q)+j, per row
 #pragma unroll
   for (int q = 0; q < QPW; q++)
 #pragma unroll
     for (int r = 0; r < MROWS; r++) acc[q][r] = 0.0f;
+  if (!EXACT || wave_live) {
 #pragma unroll
   for (int t = 0; t < TS; t++) {
     const int s = t % STEPS, q = t / STEPS;
     // steps past the end of K multiply the zero block; keep their LDS reads in range
-    const uint32_t so = (step_begin + s < steps_total) ? (uint32_t)s : 0u;
-    if (t + kDepth < TS) fetch(t + kDepth);
+    const uint32_t so = (EXACT || step_begin + s < steps_total) ? (uint32_t)s : 0u;
+    if (t + kDepth < TS) {
+      // keep the load where it is written: one step's loads per step, kDepth steps ahead (with
+      // constant offsets the scheduler would otherwise gather the loads of several steps)
+      if constexpr (EXACT) __builtin_amdgcn_sched_barrier(0);
+      fetch(t + kDepth);
+      if constexpr (EXACT) __builtin_amdgcn_sched_barrier(0);
+    }
     const Raw<FMT>& cur = blk[t];
-    // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks; with more than
-    // two activation rows a second group of four A rows (rows 2 and 3, hi and lo) follows
-    uint4 ax[NG][4];
-#pragma unroll
-    for (int g = 0; g < NG; g++)
-#pragma unroll
-      for (int ch = 0; ch < 4; ch++)
-        ax[g][ch] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + ch * plane * 16 + g * 64);
-    float2 ci[MROWS];  // {chain start value, factor that undoes the operand and block scales}
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_lane + so * (16 * MROWS * 8) + r * 8);
-    // the centring term rides in as the chain's start value (rows 2r and 2r+1 add up later)
-    floatx4 dsum[NG];
-#pragma unroll
-    for (int g = 0; g < NG; g++) dsum[g] = floatx4{ci[2 * g].x, 0.0f, 2 * g + 1 < MROWS ? ci[2 * g + 1 < MROWS ? 2 * g + 1 : 0].x : 0.0f, 0.0f};
     if constexpr (FMT == MGN_FMT_Q4) {
+      // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks; with more than
+      // two activation rows a second group of four A rows (rows 2 and 3, hi and lo) follows
+      uint4 ax[NG][4];
+#pragma unroll
+      for (int g = 0; g < NG; g++)
+#pragma unroll
+        for (int ch = 0; ch < 4; ch++)
+          ax[g][ch] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + ch * plane * 16 + g * 64);
+      float2 ci[MROWS];  // {chain start value, factor that undoes the operand and block scales}
+#pragma unroll
+      for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_lane + so * (16 * MROWS * 8) + r * 8);
+      // the centring term rides in as the chain's start value (rows 2r and 2r+1 add up later)
+      floatx4 dsum[NG];
+#pragma unroll
+      for (int g = 0; g < NG; g++) dsum[g] = floatx4{ci[2 * g].x, 0.0f, 2 * g + 1 < MROWS ? ci[2 * g + 1 < MROWS ? 2 * g + 1 : 0].x : 0.0f, 0.0f};
       const uint32_t words[4] = {cur.q.x, cur.q.y, cur.q.z, cur.q.w};
 #pragma unroll
       for (int ch = 0; ch < 4; ch++) {
@@ -466,36 +548,57 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
           dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(as_half4(ax[g][ch].z, ax[g][ch].w), as_half4(o0, o1), dsum[g], 0, 0, 0);
         }
       }
+      const float dscale = half_bits_to_float(cur.meta & 0xFFFFu);
+      // (m + 8 d) * S with S = -ci * operand_scale / 8: fold the -1/8 into the block constant
+      const float mneg = __fmaf_rn(-0.125f, half_bits_to_float(cur.meta >> 16), -dscale);
+#pragma unroll
+      for (int r = 0; r < MROWS; r++) {
+        float v = dscale * (dsum[r / 2][2 * (r % 2)] + dsum[r / 2][2 * (r % 2) + 1]);
+        v = __fmaf_rn(mneg, ci[r].x, v);
+        acc[q][r] = __fmaf_rn(v, ci[r].y, acc[q][r]);
+      }
     } else {
-      const uint32_t words[8] = {cur.q0.x, cur.q0.y, cur.q0.z, cur.q0.w, cur.q1.x, cur.q1.y, cur.q1.z, cur.q1.w};
+      // two half blocks per step, each with its own chain of four MFMAs and its own scale
 #pragma unroll
-      for (int ch = 0; ch < 4; ch++) {
+      for (int hb = 0; hb < 2; hb++) {
+        const uint4 qw = hb == 0 ? cur.q0 : cur.q1;
+        uint4 ax[NG][2];
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const uint32_t u8 = words[2 * ch + h] ^ 0x80808080u;  // q + 128 in every byte
+        for (int g = 0; g < NG; g++)
+#pragma unroll
+          for (int c2 = 0; c2 < 2; c2++)
+            ax[g][c2] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + hb * (8 * NJ * 16) + c2 * plane * 16 + g * 64);
+        float2 ci[MROWS];
+#pragma unroll
+        for (int r = 0; r < MROWS; r++)
+          ci[r] = *(const float2*)(ci_lane + so * (16 * 2 * MROWS * 8) + hb * (8 * 2 * MROWS * 8) + r * 8);
+        floatx4 dsum[NG];
+#pragma unroll
+        for (int g = 0; g < NG; g++) dsum[g] = floatx4{ci[2 * g].x, 0.0f, 2 * g + 1 < MROWS ? ci[2 * g + 1 < MROWS ? 2 * g + 1 : 0].x : 0.0f, 0.0f};
+        const uint32_t words[4] = {qw.x, qw.y, qw.z, qw.w};
+#pragma unroll
+        for (int wi = 0; wi < 4; wi++) {
+          const uint32_t u8 = words[wi] ^ 0x80808080u;  // q + 128 in every byte
           const uint32_t lo2 = __builtin_amdgcn_perm(0u, u8, 0x0c010c00u);  // (b0, b1) as fp16 mantissas
           const uint32_t hi2 = __builtin_amdgcn_perm(0u, u8, 0x0c030c02u);  // (b2, b3)
 #pragma unroll
           for (int g = 0; g < NG; g++) {
-            const half4 aop = h == 0 ? as_half4(ax[g][ch].x, ax[g][ch].y) : as_half4(ax[g][ch].z, ax[g][ch].w);
+            const uint4 a8 = ax[g][wi >> 1];
+            const half4 aop = (wi & 1) == 0 ? as_half4(a8.x, a8.y) : as_half4(a8.z, a8.w);
             dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(aop, as_half4(lo2, hi2), dsum[g], 0, 0, 0);
           }
         }
-      }
-    }
-    const float dscale = half_bits_to_float(cur.meta & 0xFFFFu);
+        const float dscale = half_bits_to_float(hb == 0 ? cur.meta0 : cur.meta1);
 #pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      float v = dscale * (dsum[r / 2][2 * (r % 2)] + dsum[r / 2][2 * (r % 2) + 1]);
-      if constexpr (FMT == MGN_FMT_Q4) {
-        // (m + 8 d) * S with S = -ci * operand_scale / 8: fold the -1/8 into the block constant
-        const float mneg = __fmaf_rn(-0.125f, half_bits_to_float(cur.meta >> 16), -dscale);
-        v = __fmaf_rn(mneg, ci[r].x, v);
+        for (int r = 0; r < MROWS; r++) {
+          const float v = dscale * (dsum[r / 2][2 * (r % 2)] + dsum[r / 2][2 * (r % 2) + 1]);
+          acc[q][r] = __fmaf_rn(v, ci[r].y, acc[q][r]);
+        }
       }
-      acc[q][r] = __fmaf_rn(v, ci[r].y, acc[q][r]);
     }
     if (t == 0) MGN_STAMP(7);
     if (t == 3) MGN_STAMP(8);
+  }
   }
   MGN_STAMP(9);
   // ---- sum the 16 lanes of each column ----
@@ -549,6 +652,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 
 struct MfmaGemvPlan {
   uint32_t ksc, wnc, steps, qpw, tasks, grid;
+  bool exact;  // every step of every K split is a full one
   size_t lds;
 };
 
@@ -556,7 +660,7 @@ constexpr uint32_t kMaxSteps = 8;  // blocks a lane holds in flight: 8 x 20 B (Q
 
 // `nquads`: column quads over all weights of the launch; `one_quad_per_wave`: fused prologues
 // and batches of several weights come with QPW = 1 only.
-bool plan_mfma_gemv(uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bool one_quad_per_wave, MfmaGemvPlan* out) {
+bool plan_mfma_gemv(int fmt, uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bool one_quad_per_wave, MfmaGemvPlan* out) {
   const uint32_t bpc = k / 32, bpc_pad = (bpc + 15) & ~15u;
   const uint32_t steps_total = bpc_pad / 16;
   MfmaGemvPlan p{};
@@ -587,17 +691,19 @@ bool plan_mfma_gemv(uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bo
   if (p.wnc > max_wnc) return false;
   p.grid = (wave_quads + p.wnc - 1) / p.wnc;
   p.tasks = bpc_pad * 4 <= 64 * p.ksc * p.wnc ? 1 : 2;
-  const size_t nj = 2 * mrows;
-  p.lds = (size_t)4 * bpc_pad * nj * 16 + (size_t)bpc_pad * mrows * 8 + (size_t)p.wnc * p.ksc * mrows * 16 +
-          16 * mrows * 4 + 64;
+  p.exact = bpc % 16 == 0 && p.ksc * p.steps == steps_total;
+  const uint32_t nj = 2 * mrows;
+  const size_t plane = (size_t)bpc_pad * nj + (fmt == MGN_FMT_Q8 ? plane_pad<MGN_FMT_Q8>(nj) : 0u);
+  const size_t cpb = fmt == MGN_FMT_Q8 ? cinit_per_block<MGN_FMT_Q8>() : 1u;
+  p.lds = 4 * plane * 16 + (size_t)bpc_pad * cpb * mrows * 8 + (size_t)p.wnc * p.ksc * mrows * 16 + 16 * mrows * 4 + 64;
   if (p.lds > 150 * 1024) return false;
   *out = p;
   return true;
 }
 
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS>
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT>
 int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS>;
+  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS, EXACT>;
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
@@ -625,8 +731,11 @@ int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
 
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
 int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1>(s, x, p)
-                      : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2>(s, x, p);
+  if (p.exact)
+    return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, true>(s, x, p)
+                        : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, true>(s, x, p);
+  return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, false>(s, x, p)
+                      : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, false>(s, x, p);
 }
 
 template <int FMT, int MROWS, int STEPS, int QPW>
@@ -648,7 +757,7 @@ uint32_t total_quads(const LaunchArgs& x) {
 template <int FMT, int MROWS>
 int launch_t(ihipStream_t* s, const LaunchArgs& x) {
   MfmaGemvPlan p;
-  if (!plan_mfma_gemv(x.w.k, total_quads(x), MROWS, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p))
+  if (!plan_mfma_gemv(FMT, x.w.k, total_quads(x), MROWS, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p))
     return (int)hipErrorInvalidValue;
   switch (p.steps * 8 + p.qpw) {
     case 1 * 8 + 1: return launch_steps<FMT, MROWS, 1, 1>(s, x, p);

@@ -129,6 +129,8 @@ ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv_valu": capi.ROUTE_GEMV_VALU, "gem
 @pytest.mark.parametrize("m,k,n", [
     (1, 32, 1), (1, 64, 3), (1, 576, 192), (1, 576, 577), (1, 1536, 576), (1, 1024, 100),
     (2, 576, 65), (3, 2048, 130), (4, 4096, 257), (1, 14336, 64), (1, 3072, 1024),
+    # K a multiple of 512 (full steps only) with a ragged last quad, waves without a quad, several quads per wave
+    (2, 512, 2055), (1, 512, 32774),
 ])
 def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
     x = synth.normal(1000 + m + k + n, m * k).reshape(m, k)
