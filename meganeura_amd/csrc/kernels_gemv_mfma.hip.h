@@ -92,10 +92,10 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 template <int FMT>
 constexpr float operand_scale() { return FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f; }  // 2^20, 2^24
 constexpr int kMaxTasks = 2;  // activation chunks a thread prepares at most, per row
-#ifndef MGN_GEMV_DEPTH
-#define MGN_GEMV_DEPTH 3
-#endif
-constexpr int kDepth = MGN_GEMV_DEPTH;
+// weight blocks in flight per lane ahead of the one in use (measured: 3 for Q4's 20-byte
+// blocks, 2 for Q8's 34-byte blocks; one more or less costs 0.3-0.4 us on a 4096 x 14336 weight)
+template <int FMT>
+constexpr int prefetch_depth() { return FMT == MGN_FMT_Q8 ? 2 : 3; }
 
 __device__ __forceinline__ half4 as_half4(uint32_t lo, uint32_t hi) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -172,19 +172,17 @@ struct Raw<MGN_FMT_Q4> {
 template <>
 struct Raw<MGN_FMT_Q8> {
   uint4 q0, q1;
-  uint32_t meta0, meta1;
-  __device__ __forceinline__ void load(const WeightView& w, size_t b0, size_t b1, uint32_t half) {
+  uint32_t meta;  // scale of block kb0 + b: the scales of the two half blocks come from lanes b/2 and 8 + b/2
+  __device__ __forceinline__ void load(const WeightView& w, size_t b0, size_t b1, uint32_t half, size_t bm) {
     q0 = stream_load_u128((const uint4*)w.quants + b0 * 2 + half);
     q1 = stream_load_u128((const uint4*)w.quants + b1 * 2 + half);
-    meta0 = stream_load_u16((const uint16_t*)w.meta + b0);
-    meta1 = stream_load_u16((const uint16_t*)w.meta + b1);
+    meta = stream_load_u16((const uint16_t*)w.meta + bm);
   }
-  // pq, pm: this lane's half of block kb0 + b/2; the partner block is 8 blocks further on
+  // pq: this lane's half of block kb0 + b/2 (the partner block is 8 blocks further on); pm: scale of block kb0 + b
   __device__ __forceinline__ void load_at(const char* pq, const char* pm) {
     q0 = stream_load_u128(pq);
     q1 = stream_load_u128(pq + 8 * 32);
-    meta0 = stream_load_u16(pm);
-    meta1 = stream_load_u16(pm + 8 * 2);
+    meta = stream_load_u16(pm);
   }
 };
 
@@ -351,6 +349,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   // in the load queue (which drains at HBM speed) before it could prepare any activations.
   // load t = q * STEPS + s: K step s of the wave's quad q
   constexpr int TS = STEPS * QPW;
+  constexpr int kDepth = prefetch_depth<FMT>();
   Raw<FMT> blk[TS];
   const uint32_t wbase = (quad * 4 + i) * bpc + kb_first;
   // Q8: first block of this lane's pair, see Raw<MGN_FMT_Q8>
@@ -365,7 +364,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       const uint32_t col = min((quad + q) * 4 + i, w.n - 1);
       const uint32_t at = col * bpc + (FMT == MGN_FMT_Q8 ? kb8_first : kb_first);
       pq[q] = (const char*)w.quants + (size_t)at * QB + (FMT == MGN_FMT_Q8 ? (b & 1) * 16 : 0);
-      pm[q] = (const char*)w.meta + (size_t)at * MB;
+      pm[q] = (const char*)w.meta + (size_t)(col * bpc + kb_first) * MB;
     }
   }
   auto fetch = [&](int t) {
@@ -378,7 +377,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     if constexpr (FMT == MGN_FMT_Q8) {
       const bool ok0 = col_ok && kb8_first + s * 16 < bpc, ok1 = col_ok && kb8_first + s * 16 + 8 < bpc;
       const uint32_t at = wbase8 + q * 4 * bpc + s * 16;
-      blk[t].load(w, ok0 ? at : zero_block, ok1 ? at + 8 : zero_block, b & 1);
+      const bool okm = col_ok && kb_first + s * 16 < bpc;
+      blk[t].load(w, ok0 ? at : zero_block, ok1 ? at + 8 : zero_block, b & 1, okm ? wbase + q * 4 * bpc + s * 16 : zero_block);
     } else {
       const bool ok = col_ok && kb_first + s * 16 < bpc;
       blk[t].load(w, ok ? wbase + q * 4 * bpc + s * 16 : zero_block);
@@ -493,6 +493,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   // Lanes i >= NJ have no activation row of their own; they re-read row i % NJ (a broadcast
   // in LDS) and the D entries they produce are never looked at.
   const uint32_t jrow = NJ < 4 ? i % NJ : i;
+  const uint32_t scale_lane = (((b >> 1) << 2) | i) * 4;  // Q8: byte address of lane (b / 2, i) for ds_bpermute
   // Q4: K block kb_first + 16 s.  Q8: half (b & 1) of blocks kb8_first + 16 s and + 8, i.e. chunks
   // 2 (b & 1) and 2 (b & 1) + 1 of those blocks.
   const char* xa_lane = FMT == MGN_FMT_Q8
@@ -559,6 +560,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       }
     } else {
       // two half blocks per step, each with its own chain of four MFMAs and its own scale
+      const float dscale_own = half_bits_to_float(cur.meta);
 #pragma unroll
       for (int hb = 0; hb < 2; hb++) {
         const uint4 qw = hb == 0 ? cur.q0 : cur.q1;
@@ -588,7 +590,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
             dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(aop, as_half4(lo2, hi2), dsum[g], 0, 0, 0);
           }
         }
-        const float dscale = half_bits_to_float(hb == 0 ? cur.meta0 : cur.meta1);
+        // the half block's scale sits in lane (hb * 8 + b / 2, i)
+        const float dscale = __builtin_bit_cast(
+            float, __builtin_amdgcn_ds_bpermute((int)scale_lane + hb * (8 * 4 * 4), __builtin_bit_cast(int, dscale_own)));
 #pragma unroll
         for (int r = 0; r < MROWS; r++) {
           const float v = dscale * (dsum[r / 2][2 * (r % 2)] + dsum[r / 2][2 * (r % 2) + 1]);
