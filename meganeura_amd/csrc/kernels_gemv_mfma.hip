@@ -26,7 +26,7 @@ bool gemv_mfma_supported(const LaunchArgs& x) {
   for (int j = 0; j < x.n_more; j++)
     if (x.more[j].w.k != x.w.k || x.more[j].w.fmt != x.w.fmt) return false;
   if (x.n_more < 0 || x.n_more > kMaxBatch - 1) return false;
-  return plan_mfma_gemv(x.w.fmt, x.w.k, total_quads(x), x.m <= 2 ? x.m : 4, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p);
+  return plan_mfma_gemv(x, x.m <= 2 ? x.m : 4, &p);
 }
 
 int launch_matmul_gemv_mfma(ihipStream_t* s, const LaunchArgs& x) {

@@ -138,6 +138,13 @@ struct GemvBatch {
   float* c[kMaxBatch];
   uint32_t first_quad[kMaxBatch];  // [0] = 0; unused entries 0xFFFFFFFF
 };
+// K split over workgroups (KSPLIT): blockIdx.y is the K part; `kdim` is then one part's K.
+struct GemvSplit {
+  uint32_t k_full;     // the weight's K: column stride of its blocks, row stride of the activations
+  uint32_t kparts;
+  float* scratch;      // [kparts][MROWS][n] partial sums
+  uint32_t* counters;  // one arrival counter per blockIdx.x, zero between launches
+};
 template <typename T>
 __device__ __forceinline__ T pick3(uint32_t idx, T a0, T a1, T a2) {
   return idx == 0 ? a0 : idx == 1 ? a1 : a2;
@@ -253,7 +260,11 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 // live wave is a full one.  A lane's loads are then its base pointer plus a constant (no
 // address arithmetic or range checks per step), waves without a quad skip the walk, and only
 // the column index is clamped (for a last quad with fewer than four columns).
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT>
+// KSPLIT (with EXACT, one weight, no fused prologue, QPW = 1): the activations of all of K would
+// not fit in LDS (M = 4 with K > ~9000), so grid.y workgroups share a quad group, each with an
+// even part of K.  Their partial sums meet in a workspace; the last workgroup to arrive adds
+// them in part order (bit-identical from run to run) and writes C.
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // The leading scalar arguments are what a wave needs before it can issue its first loads;
     // they are declared first (and not inside a struct) so that the dispatcher can hand them
@@ -262,7 +273,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     const float* __restrict__ a, const void* __restrict__ meta0, const void* __restrict__ quants0, uint32_t m,
     uint32_t ksc, uint32_t wnc, uint32_t kdim, uint32_t n0, uint32_t first_quad1, uint32_t first_quad2,
     uint32_t ksc_recip,  // ceil(4096 / ksc): wave / ksc == (wave * ksc_recip) >> 12 for the 16 waves there can be
-    const float* __restrict__ norm_weight, float eps, GemvBatch bt MGN_TRACE_PARAM) {
+    const float* __restrict__ norm_weight, float eps, GemvBatch bt, GemvSplit sp MGN_TRACE_PARAM) {
   MGN_STAMP_INIT();
   const GemvPrologue pro{norm_weight, eps};
   constexpr int NJ = 2 * MROWS;       // A rows in LDS: hi and lo of every activation row
@@ -287,6 +298,10 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   w.fmt = FMT;
   const uint32_t quad_base = pick3(widx, 0u, first_quad1, first_quad2);  // first quad of that weight
   const uint32_t bpc = w.k / 32;
+  static_assert(!KSPLIT || (EXACT && PRO == kProNone && QPW == 1), "K parts come with full steps, one quad per wave and no prologue");
+  const uint32_t kpart = KSPLIT ? blockIdx.y : 0u;
+  const uint32_t bpc_full = KSPLIT ? sp.k_full / 32 : bpc;  // blocks per column of the weight
+  const uint32_t kb_part = kpart * bpc;                     // this workgroup's first K block
   const uint32_t bpc_pad = (bpc + 15) & ~15u;
   constexpr uint32_t CPB = cinit_per_block<FMT>();
   const uint32_t plane = bpc_pad * NJ + plane_pad<FMT>(NJ);
@@ -320,7 +335,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   float4 xraw[TASKS][MROWS][2];
   float4 xup[PRO == kProSwiglu ? TASKS : 1][MROWS][2];   // the "up" halves
   float4 gw[PRO == kProRmsNorm ? TASKS : 1][2];          // norm weights of the task's 8 columns
-  const uint32_t a_stride = PRO == kProSwiglu ? 2 * w.k : w.k;
+  const uint32_t a_stride = KSPLIT ? sp.k_full : PRO == kProSwiglu ? 2 * w.k : w.k;
 #pragma unroll
   for (int tt = 0; tt < TASKS; tt++) {
     const uint32_t t = tid + tt * nthreads, kb = t >> 2, ch = t & 3;
@@ -329,7 +344,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     for (int r = 0; r < MROWS; r++) {
       // always load (from element 0 when there is nothing to load) and zero afterwards
       const bool ok = live && (uint32_t)r < m;
-      const float4* src = (const float4*)(a + (ok ? (size_t)r * a_stride + (size_t)kb * 32 + ch * 8 : (size_t)0));
+      const float4* src = (const float4*)(a + (ok ? (size_t)r * a_stride + (size_t)(kb_part + kb) * 32 + ch * 8 : (size_t)0));
       xraw[tt][r][0] = src[0];
       xraw[tt][r][1] = src[1];
       if constexpr (PRO == kProSwiglu) {
@@ -362,9 +377,10 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 #pragma unroll
     for (int q = 0; q < QPW; q++) {
       const uint32_t col = min((quad + q) * 4 + i, w.n - 1);
-      const uint32_t at = col * bpc + (FMT == MGN_FMT_Q8 ? kb8_first : kb_first);
-      pq[q] = (const char*)w.quants + (size_t)at * QB + (FMT == MGN_FMT_Q8 ? (b & 1) * 16 : 0);
-      pm[q] = (const char*)w.meta + (size_t)(col * bpc + kb_first) * MB;
+      const uint32_t at0 = col * bpc_full + kb_part;
+      pq[q] = (const char*)w.quants + (size_t)(at0 + (FMT == MGN_FMT_Q8 ? kb8_first : kb_first)) * QB +
+              (FMT == MGN_FMT_Q8 ? (b & 1) * 16 : 0);
+      pm[q] = (const char*)w.meta + (size_t)(at0 + kb_first) * MB;
     }
   }
   auto fetch = [&](int t) {
@@ -606,7 +622,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   }
   MGN_STAMP(9);
   // ---- sum the 16 lanes of each column ----
-  if (QPW > 1 || ksc == 1) {
+  if (!KSPLIT && (QPW > 1 || ksc == 1)) {
     // no K split (always the case with QPW > 1): lanes 0..3 hold the four finished columns of a quad
 #pragma unroll
     for (int q = 0; q < QPW; q++) {
@@ -635,19 +651,47 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   lds_barrier();
   MGN_STAMP(11);
   // ---- combine the K splits, add the residual, store ----
-  for (uint32_t t = tid; t < wnc * MROWS * 4; t += nthreads) {
-    const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
-    // the quads of a workgroup may belong to different weights of the batch
-    const uint32_t gq = quad0 + ql;
-    const uint32_t wi = (gq >= first_quad1 ? 1u : 0u) + (gq >= first_quad2 ? 1u : 0u);
-    const uint32_t wn_cols = pick3(wi, n0, bt.w[1].n, bt.w[2].n);
-    const uint32_t n = (gq - pick3(wi, 0u, first_quad1, first_quad2)) * 4 + col;
-    if (r < m && n < wn_cols) {
-      float v = 0.0f;
-      for (uint32_t s = 0; s < ksc; s++) v += red[((ql * ksc + s) * MROWS + r) * 4 + col];
-      const size_t o = (size_t)r * wn_cols + n;
-      const float* const dd = pick3(wi, bt.d[0], bt.d[1], bt.d[2]);
-      pick3(wi, bt.c[0], bt.c[1], bt.c[2])[o] = dd ? v + dd[o] : v;
+  uint32_t* const last_flag = (uint32_t*)nrm;  // (KSPLIT comes without the prologue that uses nrm)
+  for (int pass = 0; pass < (KSPLIT ? 2 : 1); pass++) {
+    if (KSPLIT && pass == 1) {
+      // Each XCD has its own L2: the partial sums travel as device-scope relaxed atomics
+      // (write-through stores, L2-coherent loads) with one release fence per workgroup,
+      // ordered behind every wave's stores by the barrier.
+      __syncthreads();
+      if (tid == 0) {
+        uint32_t* const ctr = sp.counters + blockIdx.x;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = seen == sp.kparts - 1;
+        if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+        *last_flag = last ? 1u : 0u;
+      }
+      __syncthreads();
+      if (*last_flag == 0u) break;
+    }
+    for (uint32_t t = tid; t < wnc * MROWS * 4; t += nthreads) {
+      const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
+      // the quads of a workgroup may belong to different weights of the batch
+      const uint32_t gq = quad0 + ql;
+      const uint32_t wi = (gq >= first_quad1 ? 1u : 0u) + (gq >= first_quad2 ? 1u : 0u);
+      const uint32_t wn_cols = pick3(wi, n0, bt.w[1].n, bt.w[2].n);
+      const uint32_t n = (gq - pick3(wi, 0u, first_quad1, first_quad2)) * 4 + col;
+      if (r < m && n < wn_cols) {
+        float v = 0.0f;
+        if (!KSPLIT || pass == 0) {
+          for (uint32_t s = 0; s < ksc; s++) v += red[((ql * ksc + s) * MROWS + r) * 4 + col];
+        } else {  // the last workgroup: every part from memory, its own included, in part order
+          for (uint32_t p = 0; p < sp.kparts; p++)
+            v += __hip_atomic_load(sp.scratch + ((size_t)p * MROWS + r) * wn_cols + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (KSPLIT && pass == 0) {
+          __hip_atomic_store(sp.scratch + ((size_t)kpart * MROWS + r) * wn_cols + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          const size_t o = (size_t)r * wn_cols + n;
+          const float* const dd = pick3(wi, bt.d[0], bt.d[1], bt.d[2]);
+          pick3(wi, bt.c[0], bt.c[1], bt.c[2])[o] = dd ? v + dd[o] : v;
+        }
+      }
     }
   }
   MGN_STAMP(12);
@@ -656,6 +700,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 
 struct MfmaGemvPlan {
   uint32_t ksc, wnc, steps, qpw, tasks, grid;
+  uint32_t kparts;  // workgroups sharing a quad group, each with K / kparts (1: no split over workgroups)
   bool exact;  // every step of every K split is a full one
   size_t lds;
 };
@@ -664,10 +709,11 @@ constexpr uint32_t kMaxSteps = 8;  // blocks a lane holds in flight: 8 x 20 B (Q
 
 // `nquads`: column quads over all weights of the launch; `one_quad_per_wave`: fused prologues
 // and batches of several weights come with QPW = 1 only.
-bool plan_mfma_gemv(int fmt, uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bool one_quad_per_wave, MfmaGemvPlan* out) {
+bool plan_one_part(int fmt, uint32_t k, uint32_t nquads, uint32_t mrows, int num_cus, bool one_quad_per_wave, MfmaGemvPlan* out) {
   const uint32_t bpc = k / 32, bpc_pad = (bpc + 15) & ~15u;
   const uint32_t steps_total = bpc_pad / 16;
   MfmaGemvPlan p{};
+  p.kparts = 1;
   // K splits: at least enough that a wave's share fits in its registers; more when there
   // are too few column quads to give every CU a handful of waves
   uint32_t ksc = (steps_total + kMaxSteps - 1) / kMaxSteps;
@@ -705,9 +751,36 @@ bool plan_mfma_gemv(int fmt, uint32_t k, uint32_t nquads, uint32_t mrows, int nu
   return true;
 }
 
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT>
+uint32_t total_quads(const LaunchArgs& x) {
+  uint32_t q = (x.w.n + 3) / 4;
+  for (int j = 0; j < x.n_more; j++) q += (x.more[j].w.n + 3) / 4;
+  return q;
+}
+
+// The plan for a launch.  When the activations of all of K do not fit in LDS, K is cut into
+// even parts that different workgroups take (plain launches only: one weight, no prologue).
+bool plan_mfma_gemv(const LaunchArgs& x, uint32_t mrows, MfmaGemvPlan* out) {
+  const bool plain = x.pro_kind == kProNone && x.n_more == 0;
+  const uint32_t nquads = total_quads(x);
+  if (plan_one_part(x.w.fmt, x.w.k, nquads, mrows, x.num_cus, !plain, out)) return true;
+  if (!plain || !x.scratch || !x.counters) return false;
+  const uint32_t bpc = x.w.k / 32;
+  for (uint32_t kp = 2; kp <= 8; kp++) {
+    if (bpc % (16 * kp) != 0) continue;
+    if ((size_t)kp * mrows * x.w.n * sizeof(float) > x.scratch_bytes) return false;
+    MfmaGemvPlan p;
+    if (!plan_one_part(x.w.fmt, x.w.k / kp, nquads, mrows, std::max(1, x.num_cus / (int)kp), true, &p)) continue;
+    if (!p.exact || p.qpw != 1 || p.grid > x.n_counters) continue;
+    p.kparts = kp;
+    *out = p;
+    return true;
+  }
+  return false;
+}
+
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT>
 int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS, EXACT>;
+  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS, EXACT, KSPLIT>;
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
@@ -725,21 +798,27 @@ int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
       bt.first_quad[j] = 0xFFFFFFFFu;
     }
   }
-  hipLaunchKernelGGL(kern, dim3(p.grid), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants, x.m,
-                     p.ksc, p.wnc, x.w.k, x.w.n, bt.first_quad[1], bt.first_quad[2], (4096u + p.ksc - 1) / p.ksc, x.pro_weight,
-                     x.pro_eps,
-                     bt MGN_TRACE_ARG);
+  const GemvSplit sp{x.w.k, p.kparts, (float*)x.scratch, x.counters};
+  hipLaunchKernelGGL(kern, dim3(p.grid, p.kparts), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants,
+                     x.m, p.ksc, p.wnc, x.w.k / p.kparts, x.w.n, bt.first_quad[1], bt.first_quad[2],
+                     (4096u + p.ksc - 1) / p.ksc, x.pro_weight, x.pro_eps, bt, sp MGN_TRACE_ARG);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }
 
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
 int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
+  if (p.kparts > 1) {
+    if constexpr (PRO == kProNone && QPW == 1)
+      return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, true, true>(s, x, p)
+                          : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, true, true>(s, x, p);
+    return (int)hipErrorInvalidValue;
+  }
   if (p.exact)
-    return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, true>(s, x, p)
-                        : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, true>(s, x, p);
-  return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, false>(s, x, p)
-                      : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, false>(s, x, p);
+    return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, true, false>(s, x, p)
+                        : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, true, false>(s, x, p);
+  return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, false, false>(s, x, p)
+                      : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, false, false>(s, x, p);
 }
 
 template <int FMT, int MROWS, int STEPS, int QPW>
@@ -752,17 +831,10 @@ int launch_steps(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
   return launch_pro<FMT, MROWS, STEPS, QPW, kProNone>(s, x, p);
 }
 
-uint32_t total_quads(const LaunchArgs& x) {
-  uint32_t q = (x.w.n + 3) / 4;
-  for (int j = 0; j < x.n_more; j++) q += (x.more[j].w.n + 3) / 4;
-  return q;
-}
-
 template <int FMT, int MROWS>
 int launch_t(ihipStream_t* s, const LaunchArgs& x) {
   MfmaGemvPlan p;
-  if (!plan_mfma_gemv(FMT, x.w.k, total_quads(x), MROWS, x.num_cus, x.pro_kind != kProNone || x.n_more > 0, &p))
-    return (int)hipErrorInvalidValue;
+  if (!plan_mfma_gemv(x, MROWS, &p)) return (int)hipErrorInvalidValue;
   switch (p.steps * 8 + p.qpw) {
     case 1 * 8 + 1: return launch_steps<FMT, MROWS, 1, 1>(s, x, p);
     case 1 * 8 + 2: return launch_steps<FMT, MROWS, 1, 2>(s, x, p);

@@ -587,6 +587,10 @@ mgn_status mgn_matmul_q_batch(mgn_ctx* ctx, const mgn_buf* a, mgn_prologue prolo
   }
   x.n_more = (int)count - 1;
   x.device = ctx->device;
+  x.scratch = ctx->scratch;
+  x.scratch_bytes = ctx->scratch_bytes;
+  x.counters = ctx->counters;
+  x.n_counters = ctx->n_counters;
   x.pro_kind = (int)prologue;
   x.pro_weight = norm_weight ? (const float*)norm_weight->ptr : nullptr;
   x.pro_eps = eps;

@@ -131,6 +131,8 @@ ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv_valu": capi.ROUTE_GEMV_VALU, "gem
     (2, 576, 65), (3, 2048, 130), (4, 4096, 257), (1, 14336, 64), (1, 3072, 1024),
     # K a multiple of 512 (full steps only) with a ragged last quad, waves without a quad, several quads per wave
     (2, 512, 2055), (1, 512, 32774),
+    # four rows of a long K: the GEMV kernel cuts K into parts for different workgroups
+    (4, 14336, 518), (3, 12288, 64),
 ])
 def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
     x = synth.normal(1000 + m + k + n, m * k).reshape(m, k)
@@ -196,19 +198,20 @@ def test_linearity_and_zero_input(ctx):
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-def test_split_k_is_repeatable(ctx, orc, fmt):
+@pytest.mark.parametrize("m,k,n,route", [(16, 4096, 2048, "gemm_mfma"), (4, 14336, 1024, "gemv_mfma")])
+def test_split_k_is_repeatable(ctx, orc, fmt, m, k, n, route):
     """Few tiles and a long K: the tiled kernel splits K across workgroups and the last
-    one to arrive adds the partial tiles in part order.  Alternating two inputs makes a
+    one to arrive adds the partial tiles in part order (the GEMV kernel does the same when
+    four rows of a long K do not fit in LDS).  Alternating two inputs makes a
     partial tile left over from the previous call wrong for this one, so a stale read
     shows; the result must also be the same bits every time."""
-    m, k, n = 16, 4096, 2048
     w = synth.normal(91 + fmt, k * n, 0.02).reshape(k, n)
     wt = ctx.weight(fmt, w)
     packed = orc.quantize(fmt, w)
     xs = [synth.normal(92 + i, m * k, 1.0).reshape(m, k) for i in range(2)]
     bufs = [ctx.upload(x) for x in xs]
     c = ctx.buffer(m * n * 4)
-    ctx.set_route(capi.ROUTE_GEMM_MFMA)
+    ctx.set_route(ROUTES[route])
     try:
         first = []
         for i in range(2):
