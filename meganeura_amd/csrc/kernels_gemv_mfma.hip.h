@@ -161,10 +161,6 @@ template <>
 struct Raw<MGN_FMT_Q4> {
   uint4 q;
   uint32_t meta;
-  __device__ __forceinline__ void load(const WeightView& w, size_t b) {
-    q = stream_load_u128((const uint4*)w.quants + b);
-    meta = stream_load_u32((const uint32_t*)w.meta + b);
-  }
   __device__ __forceinline__ void load_at(const char* pq, const char* pm) {
     q = stream_load_u128(pq);
     meta = stream_load_u32(pm);
@@ -180,11 +176,6 @@ template <>
 struct Raw<MGN_FMT_Q8> {
   uint4 q0, q1;
   uint32_t meta;  // scale of block kb0 + b: the scales of the two half blocks come from lanes b/2 and 8 + b/2
-  __device__ __forceinline__ void load(const WeightView& w, size_t b0, size_t b1, uint32_t half, size_t bm) {
-    q0 = stream_load_u128((const uint4*)w.quants + b0 * 2 + half);
-    q1 = stream_load_u128((const uint4*)w.quants + b1 * 2 + half);
-    meta = stream_load_u16((const uint16_t*)w.meta + bm);
-  }
   // pq: this lane's half of block kb0 + b/2 (the partner block is 8 blocks further on); pm: scale of block kb0 + b
   __device__ __forceinline__ void load_at(const char* pq, const char* pm) {
     q0 = stream_load_u128(pq);
@@ -257,9 +248,7 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 // TASKS: activation chunks per thread (1 when the workgroup has a thread for every chunk; the
 // prologue in front of the first weight load is then half as long).
 // EXACT: K is a multiple of 512 and the K splits share the steps evenly, so every step of every
-// live wave is a full one.  A lane's loads are then its base pointer plus a constant (no
-// address arithmetic or range checks per step), waves without a quad skip the walk, and only
-// the column index is clamped (for a last quad with fewer than four columns).
+// wave is a full one and nothing needs masking.
 // KSPLIT (with EXACT, one weight, no fused prologue, QPW = 1): the activations of all of K would
 // not fit in LDS (M = 4 with K > ~9000), so grid.y workgroups share a quad group, each with an
 // even part of K.  Their partial sums meet in a workspace; the last workgroup to arrive adds
@@ -320,12 +309,16 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   const uint32_t nquads = (w.n + 3) / 4;
   const uint32_t quad = quad0 + wn * QPW - quad_base;  // first of this wave's QPW quads, within its weight
   const uint32_t steps_total = bpc_pad / 16;
-  const uint32_t step_begin = ks * STEPS;
-  // a wave past the last K step (or past the last quad) keeps running on the zero block:
-  // it contributes nothing and clamps its LDS reads to step 0
-  const bool wave_live = step_begin < steps_total && quad < nquads;
-  const uint32_t kb_first = (wave_live ? step_begin : 0u) * 16 + b;  // this lane's K block at step 0
-  const uint32_t zero_block = bpc * w.n;  // an all-zero block behind the last real one
+  // The wave's window of STEPS steps.  When the K splits do not share the steps evenly the
+  // last split's window is moved back to end with the last step; the steps it then has in
+  // common with its neighbour count for nothing (their scales are read as zero).
+  uint32_t step_begin = ks * STEPS, first_own = 0;
+  if (!EXACT && step_begin + STEPS > steps_total) {
+    first_own = step_begin + STEPS - steps_total;
+    step_begin = steps_total - STEPS;
+  }
+  const bool wave_live = quad < nquads;  // a wave without a quad only helps to prepare the activations
+  const uint32_t kb_first = step_begin * 16 + b;  // this lane's K block at step 0
 
   // Memory returns a wave's loads in issue order, so the (small, cache-resident)
   // activation loads go first and the weight loads right behind them: the activation
@@ -366,46 +359,34 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   constexpr int TS = STEPS * QPW;
   constexpr int kDepth = prefetch_depth<FMT>();
   Raw<FMT> blk[TS];
-  const uint32_t wbase = (quad * 4 + i) * bpc + kb_first;
   // Q8: first block of this lane's pair, see Raw<MGN_FMT_Q8>
-  const uint32_t kb8_first = (wave_live ? step_begin : 0u) * 16 + (b >> 1);
-  const uint32_t wbase8 = (quad * 4 + i) * bpc + kb8_first;
+  const uint32_t kb8_first = step_begin * 16 + (b >> 1);
+  // A lane's loads are its base pointer plus a constant: no address arithmetic or range
+  // checks per step.  The column index is clamped (a last quad with fewer than four columns,
+  // a wave without a quad); lanes of the last step that lie past the end of K read the
+  // blocks that follow in memory (the next column's, or the padding behind the last
+  // column) against all-zero activations, and their scales are read as zero.
   constexpr uint32_t QB = FMT == MGN_FMT_Q8 ? 32 : 16, MB = FMT == MGN_FMT_Q8 ? 2 : 4;  // bytes per block
   const char* pq[QPW];
   const char* pm[QPW];
-  if constexpr (EXACT) {
 #pragma unroll
-    for (int q = 0; q < QPW; q++) {
-      const uint32_t col = min((quad + q) * 4 + i, w.n - 1);
-      const uint32_t at0 = col * bpc_full + kb_part;
-      pq[q] = (const char*)w.quants + (size_t)(at0 + (FMT == MGN_FMT_Q8 ? kb8_first : kb_first)) * QB +
-              (FMT == MGN_FMT_Q8 ? (b & 1) * 16 : 0);
-      pm[q] = (const char*)w.meta + (size_t)(at0 + kb_first) * MB;
-    }
+  for (int q = 0; q < QPW; q++) {
+    const uint32_t col = min((quad + q) * 4 + i, w.n - 1);
+    const uint32_t at0 = col * bpc_full + kb_part;
+    pq[q] = (const char*)w.quants + (size_t)(at0 + (FMT == MGN_FMT_Q8 ? kb8_first : kb_first)) * QB +
+            (FMT == MGN_FMT_Q8 ? (b & 1) * 16 : 0);
+    pm[q] = (const char*)w.meta + (size_t)(at0 + kb_first) * MB;
   }
   auto fetch = [&](int t) {
     const int q = t / STEPS, s = t % STEPS;
-    if constexpr (EXACT) {
-      blk[t].load_at(pq[q] + s * (16 * QB), pm[q] + s * (16 * MB));
-      return;
-    }
-    const bool col_ok = wave_live && (quad + q) * 4 + i < w.n && step_begin + s < steps_total;
-    if constexpr (FMT == MGN_FMT_Q8) {
-      const bool ok0 = col_ok && kb8_first + s * 16 < bpc, ok1 = col_ok && kb8_first + s * 16 + 8 < bpc;
-      const uint32_t at = wbase8 + q * 4 * bpc + s * 16;
-      const bool okm = col_ok && kb_first + s * 16 < bpc;
-      blk[t].load(w, ok0 ? at : zero_block, ok1 ? at + 8 : zero_block, b & 1, okm ? wbase + q * 4 * bpc + s * 16 : zero_block);
-    } else {
-      const bool ok = col_ok && kb_first + s * 16 < bpc;
-      blk[t].load(w, ok ? wbase + q * 4 * bpc + s * 16 : zero_block);
-    }
+    blk[t].load_at(pq[q] + s * (16 * QB), pm[q] + s * (16 * MB));
   };
-  // (EXACT: a wave without a quad issues these too, from the last column's blocks, and skips
-  // the walk; a branch around the loads would make every wave wait for them at the join)
+  // (a wave without a quad issues these too, from the last column's blocks, and skips the
+  // walk; a branch around the loads would make every wave wait for them at the join)
 #pragma unroll
   for (int t = 0; t < TS && t < kDepth; t++) {
     fetch(t);
-    if constexpr (EXACT) __builtin_amdgcn_sched_barrier(0);  // in this order: step 0 waits for its own block only
+    __builtin_amdgcn_sched_barrier(0);  // in this order: step 0 waits for its own block only
   }
   for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += nthreads) red[t] = 0.0f;
   MGN_STAMP_EARLY();
@@ -522,20 +503,21 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   for (int q = 0; q < QPW; q++)
 #pragma unroll
     for (int r = 0; r < MROWS; r++) acc[q][r] = 0.0f;
-  if (!EXACT || wave_live) {
+  if (wave_live) {
 #pragma unroll
   for (int t = 0; t < TS; t++) {
     const int s = t % STEPS, q = t / STEPS;
-    // steps past the end of K multiply the zero block; keep their LDS reads in range
-    const uint32_t so = (EXACT || step_begin + s < steps_total) ? (uint32_t)s : 0u;
     if (t + kDepth < TS) {
       // keep the load where it is written: one step's loads per step, kDepth steps ahead (with
       // constant offsets the scheduler would otherwise gather the loads of several steps)
-      if constexpr (EXACT) __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_sched_barrier(0);
       fetch(t + kDepth);
-      if constexpr (EXACT) __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    const Raw<FMT>& cur = blk[t];
+    Raw<FMT> cur = blk[t];
+    // not every step is a full one: a block past the end of K or in a step that belongs to the
+    // neighbouring K split gets scale (and minimum) zero
+    if constexpr (!EXACT) cur.meta = ((uint32_t)s >= first_own && kb_first + s * 16 < bpc) ? cur.meta : 0u;
     if constexpr (FMT == MGN_FMT_Q4) {
       // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks; with more than
       // two activation rows a second group of four A rows (rows 2 and 3, hi and lo) follows
@@ -544,10 +526,10 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int ch = 0; ch < 4; ch++)
-          ax[g][ch] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + ch * plane * 16 + g * 64);
+          ax[g][ch] = *(const uint4*)(xa_lane + s * (16 * NJ * 16) + ch * plane * 16 + g * 64);
       float2 ci[MROWS];  // {chain start value, factor that undoes the operand and block scales}
 #pragma unroll
-      for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_lane + so * (16 * MROWS * 8) + r * 8);
+      for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_lane + s * (16 * MROWS * 8) + r * 8);
       // the centring term rides in as the chain's start value (rows 2r and 2r+1 add up later)
       floatx4 dsum[NG];
 #pragma unroll
@@ -585,11 +567,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         for (int g = 0; g < NG; g++)
 #pragma unroll
           for (int c2 = 0; c2 < 2; c2++)
-            ax[g][c2] = *(const uint4*)(xa_lane + so * (16 * NJ * 16) + hb * (8 * NJ * 16) + c2 * plane * 16 + g * 64);
+            ax[g][c2] = *(const uint4*)(xa_lane + s * (16 * NJ * 16) + hb * (8 * NJ * 16) + c2 * plane * 16 + g * 64);
         float2 ci[MROWS];
 #pragma unroll
         for (int r = 0; r < MROWS; r++)
-          ci[r] = *(const float2*)(ci_lane + so * (16 * 2 * MROWS * 8) + hb * (8 * 2 * MROWS * 8) + r * 8);
+          ci[r] = *(const float2*)(ci_lane + s * (16 * 2 * MROWS * 8) + hb * (8 * 2 * MROWS * 8) + r * 8);
         floatx4 dsum[NG];
 #pragma unroll
         for (int g = 0; g < NG; g++) dsum[g] = floatx4{ci[2 * g].x, 0.0f, 2 * g + 1 < MROWS ? ci[2 * g + 1 < MROWS ? 2 * g + 1 : 0].x : 0.0f, 0.0f};

@@ -58,18 +58,20 @@ mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn
   w->nb = (rows / 32) * cols;
   w->meta_bytes = w->nb * meta_elem(fmt);
   w->quant_bytes = w->nb * quant_elem(fmt);
-  // One extra all-zero block (index nb) follows the real ones in both arrays: lanes
-  // that have no block of their own load it and contribute exactly zero.
-  const size_t q_off = align_up(w->meta_bytes + 16, 256);
-  hipError_t e = hipMalloc(&w->base, q_off + w->quant_bytes + 256);
+  // Sixteen all-zero blocks follow the real ones in both arrays: lanes that have no block of
+  // their own load block nb and contribute exactly zero, and the GEMV kernels' last K step of
+  // the last column may read up to fifteen blocks past the end of K.
+  constexpr size_t kMetaPad = 64, kQuantPad = 512;
+  const size_t q_off = align_up(w->meta_bytes + kMetaPad, 256);
+  hipError_t e = hipMalloc(&w->base, q_off + w->quant_bytes + kQuantPad);
   if (e != hipSuccess) {
     delete w;
     return e == hipErrorOutOfMemory ? fail(ctx, MGN_ENOMEM, "out of device memory") : hip_fail(ctx, "hipMalloc", e);
   }
   w->meta = w->base;
   w->quants = (char*)w->base + q_off;
-  e = hipMemsetAsync((char*)w->meta + w->meta_bytes, 0, 16, ctx->stream);
-  if (e == hipSuccess) e = hipMemsetAsync((char*)w->quants + w->quant_bytes, 0, 256, ctx->stream);
+  e = hipMemsetAsync((char*)w->meta + w->meta_bytes, 0, kMetaPad, ctx->stream);
+  if (e == hipSuccess) e = hipMemsetAsync((char*)w->quants + w->quant_bytes, 0, kQuantPad, ctx->stream);
   if (e != hipSuccess) {
     (void)hipFree(w->base);
     delete w;

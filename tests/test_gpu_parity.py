@@ -133,6 +133,8 @@ ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv_valu": capi.ROUTE_GEMV_VALU, "gem
     (2, 512, 2055), (1, 512, 32774),
     # four rows of a long K: the GEMV kernel cuts K into parts for different workgroups
     (4, 14336, 518), (3, 12288, 64),
+    # K splits that do not share the 16-block steps evenly, with a partial last step
+    (1, 11008, 132), (2, 11040, 66),
 ])
 def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
     x = synth.normal(1000 + m + k + n, m * k).reshape(m, k)
@@ -378,6 +380,39 @@ def test_zero_rows_is_a_no_op(ctx):
     ctx.matmul_q_f16a(a, wt, c, 0)
     assert (c.download(np.float32, 8) == 7.0).all()
     a.free(); c.free(); wt.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m", [1, 4])
+def test_a_column_with_infinite_scales_stays_on_its_own(ctx, orc, fmt, m):
+    """K = 576 is 18 blocks: the GEMV kernel's second 16-block step reads past the end of a
+    column into the next one's blocks (against zero activations).  Scales of +inf in column 1
+    must make column 1 non-finite and leave every other column as it was."""
+    k, n = 576, 8
+    bpc = k // 32
+    w = synth.normal(990, k * n, 0.02).reshape(k, n)
+    x = synth.normal(991 + m, m * k, 1.0).reshape(m, k)
+    packed = orc.quantize(fmt, w).copy()
+    clean = orc.matmul_packed(fmt, x, packed, n)
+    for kb in range(bpc):
+        blk = 1 * bpc + kb
+        if fmt == Q4:
+            packed[blk * 4:blk * 4 + 2] = (0x00, 0x7C)  # d = +inf
+        else:
+            packed[blk * 36:blk * 36 + 2] = (0x00, 0x7C)
+    wt = ctx.weight_from_packed(fmt, packed, k, n)
+    a = ctx.upload(x)
+    c = ctx.buffer(m * n * 4)
+    ctx.set_route(capi.ROUTE_GEMV_MFMA)
+    try:
+        ctx.matmul_q(a, wt, c, m)
+        got = c.download(np.float32, m * n).reshape(m, n)
+    finally:
+        ctx.set_route(capi.ROUTE_AUTO)
+        a.free(); c.free(); wt.free()
+    assert not np.isfinite(got[:, 1]).any()
+    keep = [j for j in range(n) if j != 1]
+    orc.assert_close(got[:, keep], clean[:, keep], REL, ABS)
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
