@@ -637,12 +637,13 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   for (int pass = 0; pass < (KSPLIT ? 2 : 1); pass++) {
     if (KSPLIT && pass == 1) {
       // Each XCD has its own L2: the partial sums travel as device-scope relaxed atomics
-      // (write-through stores, L2-coherent loads) with one release fence per workgroup,
-      // ordered behind every wave's stores by the barrier.
+      // (write-through stores, L2-coherent loads).  Every wave waits until its stores have
+      // been acknowledged (they are in memory then), the barrier orders all of them before
+      // the count; a release fence instead would write back the XCD's whole L2 (4 us).
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0) {
         uint32_t* const ctr = sp.counters + blockIdx.x;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const bool last = seen == sp.kparts - 1;
         if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch

@@ -494,10 +494,10 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
 
   if (g.parts > 1) {
     // ---- K parts of other workgroups: the last one to arrive adds them up in part order ----
-    // Each XCD has its own L2, so partial tiles travel as device-scope relaxed atomics
-    // (write-through stores, L2-coherent loads), with a single release fence per
-    // workgroup; a fence in every wave plus an acquire on the reading side would write
-    // back and invalidate the whole L2 hundreds of times.
+    // Each XCD has its own L2, so partial tiles travel as device-scope relaxed atomics:
+    // write-through stores, complete (in memory) once acknowledged, and L2-coherent loads.
+    // No release fence: it would write back this XCD's whole L2 (4 us measured) for the
+    // sake of stores that have been written through already.
     const size_t plane = (size_t)tail.row_tiles * ROWS * w.n;  // floats per part
     float* const mine = g.scratch + (size_t)part * plane + (size_t)row0 * w.n + n;
     if (writer) {
@@ -507,16 +507,18 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
                            __HIP_MEMORY_SCOPE_AGENT);
     }
     MGN_GSTAMP(8);
+    // every wave waits until its write-through stores have been acknowledged, i.e. have
+    // reached memory; the barrier then orders all of them before the count
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     MGN_GSTAMP(9);
     uint32_t* const flag = (uint32_t*)lds4;
     if (tid == 0) {
       uint32_t* ctr = g.counters + blockIdx.z * g.colgroups + cg;
-      // one device-scope release per workgroup: the barrier above ordered every wave's
-      // stores before it, and it makes them visible to the other XCDs before the count
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+      MGN_GSTAMP(11);
       const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const bool last = seen == g.parts - 1;
+      if (seen != 0xFFFFFFFFu) MGN_GSTAMP(12);
       if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
       *flag = last ? 1u : 0u;
     }
