@@ -58,7 +58,9 @@ HEADLINE = "c5_q4_m1_4096x14336"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
 # same counters read for a 256 MiB device copy (one summary per workload under profiles/).
 MEASURED_TRAFFIC_BYTES = {
-    "c5_q4_m1_4096x14336": 37.02e6,
+    "c5_q4_m1_4096x14336": 37.01e6,
+    "c5_q8_m1_4096x14336": 63.52e6,
+    "c5_q4_m4_14336x4096": 39.3e6,
     "c5_q4_m16_4096x14336": 48.4e6,
     "c4_q4_prefill_up_512x1024x3072": 18.8e6,
 }
@@ -102,13 +104,20 @@ class Workload:
         self.i += 1
         self.fn(self.a, w, self.c, self.m, self.d)
 
+    def loop(self, steps):
+        """`steps` calls enqueued from C (no interpreter between the launches), weights in rotation."""
+        if steps <= 0:
+            return
+        n = len(self.weights)
+        order = [self.weights[(self.i + j) % n] for j in range(n)]
+        self.ctx.matmul_q_loop(self.a, order, self.c, self.m, steps, self.d, self.f16)
+        self.i += steps
+
     def run(self, steps, warmup):
-        for _ in range(warmup):
-            self.step()
+        self.loop(warmup)
         self.ctx.sync()
         self.ctx.timer_start()
-        for _ in range(steps):
-            self.step()
+        self.loop(steps)
         ms = self.ctx.timer_stop()  # waits for the stop event
         self.ctx.sync()
         return ms / steps

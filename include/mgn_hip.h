@@ -164,6 +164,13 @@ mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, con
 mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w,
                              const mgn_buf* d, mgn_buf* c, uint32_t m);
 
+/* `steps` such matmuls enqueued back to back, call i on weights[i % count]: the step loop of
+ * a compiled host (examples/matmul_throughput.rs:114-127) without an interpreter between the
+ * launches, for harnesses written in a scripting language.  Copies of one weight in rotation
+ * keep it out of the caches.  a_is_f16 != 0 selects the fp16-activation entry. */
+mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const mgn_weight* const* weights,
+                             size_t count, const mgn_buf* d, mgn_buf* c, uint32_t m, uint32_t steps);
+
 /* Two neighbours of the decode-time matmul folded into its activation staging, each
  * standing in for a dispatch pair of the reference's plan (M <= 4, f32 activations):
  *   RmsNorm then MatMul[Gemv][Add]   (src/shaders/rms_norm.wgsl:1-57; models/smollm2.rs:340-341,396):

@@ -615,6 +615,16 @@ mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weigh
   return matmul_impl(ctx, a_f16, true, w, d, c, m);
 }
 
+mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const mgn_weight* const* weights, size_t count,
+                             const mgn_buf* d, mgn_buf* c, uint32_t m, uint32_t steps) {
+  if (!ctx || !weights || count == 0) return fail(ctx, MGN_EINVAL, "null argument or no weights");
+  for (uint32_t i = 0; i < steps; i++) {
+    const mgn_status st = matmul_impl(ctx, a, a_is_f16 != 0, weights[i % count], d, c, m);
+    if (st != MGN_OK) return st;
+  }
+  return MGN_OK;
+}
+
 // ---- timing ----
 
 mgn_status mgn_timer_start(mgn_ctx* ctx) {

@@ -372,6 +372,27 @@ def test_weight_file_round_trip(ctx, orc, fmt, tmp_path):
         assert e.value.status == capi.EINVAL, name
 
 
+def test_matmul_loop_is_the_same_calls_in_a_row(ctx, orc):
+    """mgn_matmul_q_loop enqueues call i on weights[i % count]: after five steps over two
+    weights the output is what the first weight gives (bit for bit the single call's)."""
+    k, n, m = 576, 192, 1
+    ws = [synth.normal(960 + j, k * n, 0.02).reshape(k, n) for j in range(2)]
+    wts = [ctx.weight(Q4, w) for w in ws]
+    x = synth.normal(962, m * k).reshape(m, k)
+    a = ctx.upload(x)
+    c = ctx.buffer(m * n * 4)
+    ctx.matmul_q(a, wts[0], c, m)
+    single = c.download(np.float32, m * n)
+    ctx.matmul_q_loop(a, wts, c, m, 4)
+    assert (bits(c.download(np.float32, m * n)) != bits(single)).any()  # the fourth call ran on the other weight
+    ctx.matmul_q_loop(a, wts, c, m, 5)
+    assert (bits(c.download(np.float32, m * n)) == bits(single)).all()
+    orc.assert_close(single.reshape(m, n), orc.matmul_packed(Q4, x, orc.quantize(Q4, ws[0]), n), REL, ABS)
+    a.free(); c.free()
+    for w in wts:
+        w.free()
+
+
 def test_zero_rows_is_a_no_op(ctx):
     wt = ctx.weight(Q4, synth.normal(970, 64 * 8, 0.02).reshape(64, 8))
     a = ctx.buffer(4 * 64)
