@@ -134,13 +134,14 @@ class Workload:
             self.d.free()
 
 
-def decode_layer_times(steps, warmup):
-    """C2 as the reference runs it: one SmolLM2-135M decode layer's matmuls through the
+def decode_layer_times(steps, warmup, layers=8):
+    """C2 as the reference runs it: SmolLM2-135M decode layers' matmuls through the
     Graph/Session surface (models/smollm2.rs:340-414 without the attention core): rms_norm,
     q/k/v, o-projection + residual, rms_norm, gate||up as one fused matmul, SwiGLU, down +
-    residual -- 9 dispatches after the optimizer's fusions.  Returns microseconds per layer
-    step: every dispatch its own launch, norms and SwiGLU folded into the matmuls (the
-    default), and the folded step replayed as one captured graph."""
+    residual -- 9 dispatches per layer after the optimizer's fusions, `layers` of them chained
+    in one session so that the per-step cost of the host loop is spread as in a real model.
+    Returns microseconds per layer: every dispatch its own launch, norms and SwiGLU folded
+    into the matmuls (the default), and the folded step replayed as one captured graph."""
     from meganeura_amd import capi, synth
     from meganeura_amd.graph import Graph, build_inference_session
 
@@ -148,31 +149,36 @@ def decode_layer_times(steps, warmup):
     g = Graph()
     x = g.input("x", [1, hidden])
     attn = g.input("attn", [1, hidden])
-    n1 = g.rms_norm(x, g.parameter("norm1", [hidden]), 1e-5)
-    q = g.matmul(n1, g.parameter_q4("wq", [hidden, hidden]))
-    k = g.matmul(n1, g.parameter_q4("wk", [hidden, kv]))
-    v = g.matmul(n1, g.parameter_q4("wv", [hidden, kv]))
-    h = g.add(g.matmul(attn, g.parameter_q4("wo", [hidden, hidden])), x)
-    n2 = g.rms_norm(h, g.parameter("norm2", [hidden]), 1e-5)
-    gate = g.matmul(n2, g.parameter_q4("wg", [hidden, inter]))
-    up = g.matmul(n2, g.parameter_q4("wu", [hidden, inter]))
-    out = g.add(g.matmul(g.swiglu(gate, up), g.parameter_q4("wd", [inter, hidden])), h)
-    g.set_outputs([out, q, k, v])
+    outs, shapes = [], {}
+    for l in range(layers):
+        n1 = g.rms_norm(x, g.parameter(f"norm1.{l}", [hidden]), 1e-5)
+        q = g.matmul(n1, g.parameter_q4(f"wq.{l}", [hidden, hidden]))
+        k = g.matmul(n1, g.parameter_q4(f"wk.{l}", [hidden, kv]))
+        v = g.matmul(n1, g.parameter_q4(f"wv.{l}", [hidden, kv]))
+        h = g.add(g.matmul(attn, g.parameter_q4(f"wo.{l}", [hidden, hidden])), x)
+        n2 = g.rms_norm(h, g.parameter(f"norm2.{l}", [hidden]), 1e-5)
+        gate = g.matmul(n2, g.parameter_q4(f"wg.{l}", [hidden, inter]))
+        up = g.matmul(n2, g.parameter_q4(f"wu.{l}", [hidden, inter]))
+        x = g.add(g.matmul(g.swiglu(gate, up), g.parameter_q4(f"wd.{l}", [inter, hidden])), h)
+        outs += [q, k, v]
+        shapes.update({f"wq.{l}": (hidden, hidden), f"wk.{l}": (hidden, kv), f"wv.{l}": (hidden, kv),
+                       f"wo.{l}": (hidden, hidden), f"wg.{l}": (hidden, inter), f"wu.{l}": (hidden, inter),
+                       f"wd.{l}": (inter, hidden)})
+    g.set_outputs([x] + outs)
     sess = build_inference_session(g)
-    shapes = {"wq": (hidden, hidden), "wk": (hidden, kv), "wv": (hidden, kv), "wo": (hidden, hidden),
-              "wg": (hidden, inter), "wu": (hidden, inter), "wd": (inter, hidden)}
     for i, (name, (kk, nn)) in enumerate(shapes.items()):
-        sess.set_parameter(name, synth.weights(2, kk, nn, which=i))
-    sess.set_parameter("norm1", np.ones(hidden, np.float32))
-    sess.set_parameter("norm2", np.ones(hidden, np.float32))
+        sess.set_parameter(name, synth.weights(2, kk, nn, which=i % 7))
+    for l in range(layers):
+        sess.set_parameter(f"norm1.{l}", np.ones(hidden, np.float32))
+        sess.set_parameter(f"norm2.{l}", np.ones(hidden, np.float32))
     sess.set_input("x", synth.activations(2, 1, hidden, which=0))
     sess.set_input("attn", synth.activations(2, 1, hidden, which=1))
     ctx = sess.context()
-    res = {"dispatches": len(sess.plan())}
+    res = {"layers": layers, "dispatches_per_layer": len(sess.plan()) // layers}
     for label, fusion, replay in (("unfused", False, False), ("fused", True, False), ("fused_graph", True, True)):
         sess.set_fusion(fusion)
         sess.set_graph_replay(replay)
-        res[label + "_launches"] = sess.num_launches()
+        res[label + "_launches_per_layer"] = sess.num_launches() / layers
         for _ in range(warmup + 2):
             sess.step()
         ctx.sync()
@@ -181,7 +187,7 @@ def decode_layer_times(steps, warmup):
             sess.step()
         ms = ctx.timer_stop()
         ctx.sync()
-        res[label + "_us_per_layer"] = ms * 1e3 / steps
+        res[label + "_us_per_layer"] = ms * 1e3 / steps / layers
     sess.close()
     return res
 
