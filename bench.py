@@ -52,6 +52,9 @@ WORKLOADS = {
     "c2_q4_down_1536x576_add": (Q4, 1, 1536, 576, True, False, 2),
     "c4_q4_prefill_up_512x1024x3072": (Q4, 512, 1024, 3072, False, True, 4),
     "c4_q4_prefill_down_512x3072x1024": (Q4, 512, 3072, 1024, False, True, 4),
+    # not a BASELINE configuration: four times the headline weight, to separate the kernel's
+    # streaming rate from the fixed cost of a launch (sweep only)
+    "scale_q4_m1_8192x28672": (Q4, 1, 8192, 28672, False, False, 5),
 }
 HEADLINE = "c5_q4_m1_4096x14336"
 
