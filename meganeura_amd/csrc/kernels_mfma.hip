@@ -611,11 +611,14 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
         if (scratch > x.scratch_bytes || (parts > 1 && (uint64_t)grid_y * colgroups > x.n_counters)) break;
         if (wgs * 64 * ksc * wnc > (uint64_t)x.num_cus * 4096 && parts > 1) break;  // far more than enough already
         const double rounds = (double)((wgs + x.num_cus - 1) / x.num_cus);
+        // K parts: a workgroup writes its partial tiles, and the last one of a column group,
+        // which the launch ends with, reads all parts back behind a round trip for the count
+        const double tile_bytes = wnc * 32.0 * rows * 4;
         const double per_wg = nch * cb * (std::min(wnc, n_tiles) * wblock + ablock) + 32768.0 +
-                              (parts > 1 ? 2.0 * wnc * 32 * rows * 4 + 16384.0 : 0.0);
+                              (parts > 1 ? (1.0 + parts) * tile_bytes + 16384.0 : 0.0);
         // few waves hide little latency; a task count that does not divide over the threads
         // leaves part of the workgroup idle while the rest stages twice
-        const double cost = rounds * per_wg * (ksc * wnc < 8 ? 1.5 : 1.0) * (max_tasks % wnc ? 1.15 : 1.0) * (tpt > 2 ? 1.25 : 1.0);
+        const double cost = rounds * per_wg * (ksc * wnc < 8 ? 1.5 : 1.0) * (max_tasks % wnc ? 1.15 : 1.0) * (tpt > 2 ? 1.1 : 1.0);
         if (best == 0 || cost < best) {
           best = cost;
           bp.ksc = ksc, bp.wnc = wnc, bp.tpt = tpt <= 1 ? 1 : tpt <= 2 ? 2 : 4;
@@ -629,6 +632,8 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
   if (const char* dev = getenv("MGN_DEV_GEMM")) {
     unsigned a = 0, b = 0, c = 0;
     if (sscanf(dev, "%u,%u,%u", &a, &b, &c) == 3) {
+      // a forced plan has to pass every check the search applies, or the call is refused
+      if ((a != 1 && a != 2) || b < 1 || b > 8 / a || c < 1) return false;
       const uint32_t cb = 8 * a, chunks = (bpc + cb - 1) / cb;
       bp.ksc = a, bp.wnc = b, bp.parts = c;
       bp.nch = (chunks + c - 1) / c;
@@ -637,6 +642,10 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
       const uint32_t tpt = (max_tasks + b - 1) / b;
       bp.tpt = tpt <= 1 ? 1 : tpt <= 2 ? 2 : 4;
       bp.grid_y = grid_y;
+      bp.scratch_bytes = bp.parts > 1 ? (size_t)bp.parts * grid_y * rows * x.w.n * 4 : 0;
+      if (tpt > 4 || gemm_lds_bytes(x.w.fmt, a, b) > 160 * 1024 || bp.colgroups > 65535 || bp.scratch_bytes > x.scratch_bytes ||
+          (bp.parts > 1 && (uint64_t)grid_y * bp.colgroups > x.n_counters))
+        return false;
       best = 1;
     }
   }
