@@ -171,6 +171,27 @@ mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weigh
 mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const mgn_weight* const* weights,
                              size_t count, const mgn_buf* d, mgn_buf* c, uint32_t m, uint32_t steps);
 
+/* What mgn_matmul_q would launch for a shape, without a device: the kernel family the
+ * automatic choice takes (the analogue of reading compile.rs:1390 and runtime.rs:1634 for the
+ * reference) and the launch geometry.  For logs, and for checking the planner on the host.
+ * `num_cus` is the device's compute-unit count (256 on MI355X); the workspace is assumed to be
+ * the one every context owns.  MGN_EINVAL for shapes no weight can have. */
+typedef struct mgn_plan_info {
+  int route;              /* mgn_route (never MGN_ROUTE_AUTO) */
+  uint32_t grid[3];       /* workgroups */
+  uint32_t threads;       /* per workgroup */
+  uint32_t lds_bytes;     /* dynamic LDS per workgroup */
+  uint32_t waves_n;       /* column quads (GEMV) or 32-column tiles (tiled) per workgroup */
+  uint32_t k_splits;      /* waves that share a quad / tile inside a workgroup */
+  uint32_t k_parts;       /* workgroups that share a column group; > 1: partial sums through the workspace */
+  uint32_t steps;         /* GEMV: 16-block steps per wave; tiled: 8-block chunks per wave */
+  uint32_t quads_per_wave; /* GEMV only */
+  uint32_t full_steps;    /* GEMV only: 1 when no step needs masking */
+  uint64_t workspace_bytes; /* partial sums held in the context's workspace */
+} mgn_plan_info;
+mgn_status mgn_matmul_q_plan(mgn_fmt fmt, uint32_t m, uint64_t k, uint64_t n, int a_is_f16, int num_cus,
+                             mgn_plan_info* out);
+
 /* Two neighbours of the decode-time matmul folded into its activation staging, each
  * standing in for a dispatch pair of the reference's plan (M <= 4, f32 activations):
  *   RmsNorm then MatMul[Gemv][Add]   (src/shaders/rms_norm.wgsl:1-57; models/smollm2.rs:340-341,396):

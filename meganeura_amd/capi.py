@@ -22,7 +22,7 @@ HIP_SYMBOLS = [
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_weight_save", "mgn_weight_load", "mgn_matmul_q",
-    "mgn_matmul_q_f16a", "mgn_matmul_q_loop", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
+    "mgn_matmul_q_f16a", "mgn_matmul_q_loop", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
     "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [
@@ -103,6 +103,7 @@ def load():
         "mgn_weight_info": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(sz), C.POINTER(sz)]),
         "mgn_matmul_q": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_f16a": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
+        "mgn_matmul_q_plan": (C.c_int, [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.c_int, vp]),
         "mgn_matmul_q_loop": (C.c_int, [vp, vp, C.c_int, vp, C.c_size_t, vp, vp, C.c_uint32, C.c_uint32]),
         "mgn_matmul_q_rms_norm": (C.c_int, [vp, vp, vp, C.c_float, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_swiglu": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
@@ -159,6 +160,21 @@ def _ptr(arr):
 
 def packed_size(fmt, rows, cols):
     return int(load().mgn_packed_size(fmt, rows, cols))
+
+
+class PlanInfo(C.Structure):
+    _fields_ = [("route", C.c_int), ("grid", C.c_uint32 * 3), ("threads", C.c_uint32), ("lds_bytes", C.c_uint32),
+                ("waves_n", C.c_uint32), ("k_splits", C.c_uint32), ("k_parts", C.c_uint32), ("steps", C.c_uint32),
+                ("quads_per_wave", C.c_uint32), ("full_steps", C.c_uint32), ("workspace_bytes", C.c_uint64)]
+
+
+def matmul_plan(fmt, m, k, n, a_is_f16=False, num_cus=256):
+    """What mgn_matmul_q would launch for this shape (no device needed)."""
+    info = PlanInfo()
+    st = load().mgn_matmul_q_plan(fmt, m, k, n, 1 if a_is_f16 else 0, num_cus, C.byref(info))
+    if st != OK:
+        raise MgnError(st, "matmul_plan: no weight has this shape")
+    return info
 
 
 def quantize_ref(fmt, w):

@@ -29,6 +29,21 @@ bool gemv_mfma_supported(const LaunchArgs& x) {
   return plan_mfma_gemv(x, x.m <= 2 ? x.m : 4, &p);
 }
 
+bool describe_gemv_mfma(const LaunchArgs& x, mgn_plan_info* out) {
+  if (!gemv_mfma_supported(x)) return false;
+  const uint32_t mrows = x.m <= 2 ? x.m : 4;
+  MfmaGemvPlan p;
+  if (!plan_mfma_gemv(x, mrows, &p)) return false;
+  out->route = MGN_ROUTE_GEMV_MFMA;
+  out->grid[0] = p.grid, out->grid[1] = p.kparts, out->grid[2] = 1;
+  out->threads = 64 * p.ksc * p.wnc;
+  out->lds_bytes = (uint32_t)p.lds;
+  out->waves_n = p.wnc, out->k_splits = p.ksc, out->k_parts = p.kparts, out->steps = p.steps;
+  out->quads_per_wave = p.qpw, out->full_steps = p.exact ? 1 : 0;
+  out->workspace_bytes = p.kparts > 1 ? (uint64_t)p.kparts * mrows * x.w.n * sizeof(float) : 0;
+  return true;
+}
+
 int launch_matmul_gemv_mfma(ihipStream_t* s, const LaunchArgs& x) {
   if (x.w.fmt == MGN_FMT_Q4)
     return x.m == 1 ? launch_gemv_mfma_q4_m1(s, x) : x.m == 2 ? launch_gemv_mfma_q4_m2(s, x) : launch_gemv_mfma_q4_m4(s, x);

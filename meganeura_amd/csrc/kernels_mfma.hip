@@ -694,6 +694,19 @@ bool gemm_mfma_supported(const LaunchArgs& x) {
   return plan_gemm(x, &p);
 }
 
+bool describe_gemm_mfma(const LaunchArgs& x, mgn_plan_info* out) {
+  GemmPlan p;
+  if (!gemm_mfma_supported(x) || !plan_gemm(x, &p)) return false;
+  out->route = MGN_ROUTE_GEMM_MFMA;
+  out->grid[0] = p.parts, out->grid[1] = p.colgroups, out->grid[2] = p.grid_y;
+  out->threads = 64 * p.ksc * p.wnc;
+  out->lds_bytes = (uint32_t)p.lds;
+  out->waves_n = p.wnc, out->k_splits = p.ksc, out->k_parts = p.parts, out->steps = p.nch;
+  out->quads_per_wave = 0, out->full_steps = 0;
+  out->workspace_bytes = p.scratch_bytes;
+  return true;
+}
+
 int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& x) {
   if (x.w.fmt == MGN_FMT_Q4) return x.a_is_f16 ? launch_fa<MGN_FMT_Q4, false>(s, x) : launch_fa<MGN_FMT_Q4, true>(s, x);
   return x.a_is_f16 ? launch_fa<MGN_FMT_Q8, false>(s, x) : launch_fa<MGN_FMT_Q8, true>(s, x);

@@ -136,8 +136,8 @@ mgn_status mgn_ctx_create(int device_id, mgn_ctx** out) {
     return hip_fail(nullptr, "stream/event creation", e);
   }
   // workspace of the split-K matmul kernels: partial tiles, then 4096 arrival counters
-  constexpr size_t kScratchBytes = (size_t)16 << 20;
-  constexpr uint32_t kCounters = 4096;
+  constexpr size_t kScratchBytes = mgn::kWorkspaceBytes;
+  constexpr uint32_t kCounters = mgn::kWorkspaceCounters;
   // (+ two words the weight range scan reduces into)
   if ((e = hipMalloc(&ctx->scratch, kScratchBytes + (kCounters + 2) * sizeof(uint32_t))) != hipSuccess ||
       (e = hipMemsetAsync((char*)ctx->scratch + kScratchBytes, 0, (kCounters + 2) * sizeof(uint32_t), ctx->stream)) != hipSuccess) {
@@ -613,6 +613,27 @@ int mgn_matmul_q_can_fuse(mgn_ctx* ctx, const mgn_weight* w, uint32_t m) {
 mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
                              uint32_t m) {
   return matmul_impl(ctx, a_f16, true, w, d, c, m);
+}
+
+mgn_status mgn_matmul_q_plan(mgn_fmt fmt, uint32_t m, uint64_t k, uint64_t n, int a_is_f16, int num_cus, mgn_plan_info* out) {
+  if (!out || !valid_fmt(fmt) || m == 0 || k == 0 || n == 0 || k % 32 != 0 || num_cus <= 0) return MGN_EINVAL;
+  if (k > 0xFFFFFFE0ull || n > 0xFFFFFFFFull || (k / 32) * n >= 0x7FFFFFFFull) return MGN_EINVAL;
+  *out = mgn_plan_info{};
+  mgn::LaunchArgs x{};
+  x.w = mgn::WeightView{nullptr, nullptr, (uint32_t)k, (uint32_t)n, (int)fmt, true};
+  x.m = m;
+  x.a_is_f16 = a_is_f16 != 0;
+  x.num_cus = num_cus;
+  // the planners only look at whether a workspace exists, never through the pointers
+  static char workspace_stand_in;
+  x.scratch = &workspace_stand_in;
+  x.scratch_bytes = mgn::kWorkspaceBytes;
+  x.counters = (uint32_t*)&workspace_stand_in;
+  x.n_counters = mgn::kWorkspaceCounters;
+  if (mgn::describe_gemv_mfma(x, out)) return MGN_OK;
+  if (mgn::describe_gemm_mfma(x, out)) return MGN_OK;
+  out->route = mgn::gemv_supported(x) ? MGN_ROUTE_GEMV_VALU : MGN_ROUTE_GENERIC;
+  return MGN_OK;
 }
 
 mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const mgn_weight* const* weights, size_t count,

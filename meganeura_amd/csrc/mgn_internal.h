@@ -86,6 +86,12 @@ int launch_matmul_gemv(ihipStream_t* s, const LaunchArgs& a);
 bool gemv_mfma_supported(const LaunchArgs& a);
 int launch_matmul_gemv_mfma(ihipStream_t* s, const LaunchArgs& a);
 bool gemm_mfma_supported(const LaunchArgs& a);
+// launch geometry of the two MFMA routes (false: the route does not take the shape)
+bool describe_gemv_mfma(const LaunchArgs& a, mgn_plan_info* out);
+bool describe_gemm_mfma(const LaunchArgs& a, mgn_plan_info* out);
+// the workspace every context owns: partial sums of K parts, then arrival counters
+constexpr size_t kWorkspaceBytes = (size_t)16 << 20;
+constexpr uint32_t kWorkspaceCounters = 4096;
 int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& a);
 
 }  // namespace mgn

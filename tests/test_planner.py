@@ -1,0 +1,118 @@
+"""The launch planner on the host: mgn_matmul_q_plan tells what mgn_matmul_q would launch for a
+shape without touching a device.  Swept over decode and prefill shapes, the geometry must cover
+every column and every K block exactly once, stay inside the hardware limits (threads, LDS) and
+inside the context's workspace, and put the BASELINE configurations on the kernels built for them."""
+import itertools
+
+import pytest
+
+from meganeura_amd import capi
+
+Q4, Q8 = 0, 1
+GENERIC, GEMV_VALU, GEMV_MFMA, GEMM_MFMA = 1, 2, 3, 4
+WORKSPACE = 16 << 20
+COUNTERS = 4096
+
+KS = [32, 64, 96, 480, 512, 544, 576, 960, 1024, 1536, 2048, 3072, 4096, 5120, 8192, 11008, 11040, 12288, 14336,
+      16384, 28672, 32768, 65536]
+NS = [1, 3, 4, 64, 100, 192, 576, 1027, 3072, 4096, 14336, 49152, 151936]
+MS = [1, 2, 3, 4, 5, 8, 16, 17, 64, 512]
+
+
+def ceil_div(a, b):
+    return -(-a // b)
+
+
+def check_gemv(p, fmt, m, k, n):
+    mrows = m if m <= 2 else 4
+    bpc = k // 32
+    assert m <= 4
+    assert p.threads == 64 * p.k_splits * p.waves_n <= 1024
+    assert p.lds_bytes <= 150 * 1024
+    assert p.k_parts >= 1 and p.grid[1] == p.k_parts and p.grid[2] == 1
+    assert bpc % p.k_parts == 0
+    part_blocks = bpc // p.k_parts
+    if p.k_parts > 1:
+        assert part_blocks % 16 == 0 and p.full_steps == 1 and p.quads_per_wave == 1
+        assert p.workspace_bytes == p.k_parts * mrows * n * 4 <= WORKSPACE
+        assert p.grid[0] <= COUNTERS
+    else:
+        assert p.workspace_bytes == 0
+    steps_total = ceil_div(part_blocks, 16)
+    assert 1 <= p.steps <= 8
+    assert p.k_splits * p.steps >= steps_total          # all of K is walked
+    assert (p.k_splits - 1) * p.steps < steps_total      # no K split without a step of its own
+    assert p.full_steps == int(part_blocks % 16 == 0 and p.k_splits * p.steps == steps_total)
+    nquads = ceil_div(n, 4)
+    per_wg = p.waves_n * p.quads_per_wave
+    assert p.grid[0] * per_wg >= nquads                  # every column has a wave
+    assert (p.grid[0] - 1) * per_wg < nquads             # no workgroup without a column
+    if p.quads_per_wave > 1:
+        assert p.k_splits == 1 and p.steps * p.quads_per_wave <= 8
+
+
+def check_gemm(p, fmt, m, k, n, f16):
+    rows = 32 if f16 else 16
+    bpc = k // 32
+    assert p.grid[2] == ceil_div(m, rows)
+    assert p.threads == 64 * p.k_splits * p.waves_n <= 512
+    assert p.k_splits in (1, 2)
+    assert p.lds_bytes <= 160 * 1024
+    n_tiles = ceil_div(n, 32)
+    assert p.grid[1] * p.waves_n >= n_tiles and (p.grid[1] - 1) * p.waves_n < n_tiles
+    chunks = ceil_div(bpc, 8 * p.k_splits)
+    assert p.grid[0] == p.k_parts >= 1
+    assert p.k_parts * p.steps >= chunks and (p.k_parts - 1) * p.steps < chunks
+    if p.k_parts > 1:
+        assert p.workspace_bytes == p.k_parts * p.grid[2] * rows * n * 4 <= WORKSPACE
+        assert p.grid[1] * p.grid[2] <= COUNTERS
+    else:
+        assert p.workspace_bytes == 0
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+def test_plans_cover_the_problem_and_respect_the_limits(fmt):
+    routes = set()
+    for m, k, n in itertools.product(MS, KS, NS):
+        if (k // 32) * n >= 0x7FFFFFFF:
+            continue
+        for f16 in ((False, True) if m >= 5 else (False,)):
+            p = capi.matmul_plan(fmt, m, k, n, f16)
+            where = f"fmt={fmt} m={m} k={k} n={n} f16={f16} route={p.route}"
+            routes.add(p.route)
+            try:
+                assert p.route in (GENERIC, GEMV_VALU, GEMV_MFMA, GEMM_MFMA)
+                if m > 4 or f16:
+                    assert p.route in (GEMM_MFMA, GENERIC)
+                if p.route == GEMV_MFMA:
+                    check_gemv(p, fmt, m, k, n)
+                elif p.route == GEMM_MFMA:
+                    check_gemm(p, fmt, m, k, n, f16)
+            except AssertionError as e:
+                raise AssertionError(where) from e
+    assert {GEMV_MFMA, GEMM_MFMA} <= routes
+
+
+def test_baseline_configurations_take_the_kernels_built_for_them():
+    gemv = [(Q8, 1, 576, 1536), (Q4, 1, 576, 576), (Q4, 1, 576, 192), (Q4, 1, 576, 3072), (Q4, 1, 1536, 576),
+            (Q4, 1, 576, 49152)]
+    for fmt in (Q4, Q8):
+        for m in (1, 4):
+            gemv += [(fmt, m, 4096, 14336), (fmt, m, 14336, 4096)]
+    for fmt, m, k, n in gemv:
+        assert capi.matmul_plan(fmt, m, k, n).route == GEMV_MFMA, (fmt, m, k, n)
+    for fmt in (Q4, Q8):
+        for k, n in ((4096, 14336), (14336, 4096)):
+            assert capi.matmul_plan(fmt, 16, k, n).route == GEMM_MFMA
+    for k, n in ((1024, 3072), (3072, 1024)):
+        assert capi.matmul_plan(Q4, 512, k, n, True).route == GEMM_MFMA
+    head = capi.matmul_plan(Q4, 1, 4096, 14336)
+    assert (head.grid[0], head.threads, head.steps, head.k_splits, head.full_steps) == (256, 896, 8, 1, 1)
+    tall = capi.matmul_plan(Q4, 4, 14336, 4096)
+    assert tall.k_parts == 2 and tall.workspace_bytes == 2 * 4 * 4096 * 4
+
+
+def test_shapes_no_weight_can_have_are_refused():
+    for args in ((Q4, 1, 100, 8), (Q4, 0, 64, 8), (Q4, 1, 0, 8), (Q4, 1, 64, 0), (7, 1, 64, 8)):
+        with pytest.raises(capi.MgnError):
+            capi.matmul_plan(*args)
