@@ -249,9 +249,10 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 // prologue in front of the first weight load is then half as long).
 // EXACT: K is a multiple of 512 and the K splits share the steps evenly, so every step of every
 // wave is a full one and nothing needs masking.
-// KSPLIT (with EXACT, one weight, no fused prologue, QPW = 1): the activations of all of K would
-// not fit in LDS (M = 4 with K > ~9000), so grid.y workgroups share a quad group, each with an
-// even part of K.  Their partial sums meet in a workspace; the last workgroup to arrive adds
+// KSPLIT (one weight, no fused prologue, QPW = 1, steps masked as without EXACT): the activations
+// of all of K would not fit in LDS (M = 4 with K > ~9000) or need more threads to prepare than a
+// workgroup has (K > 16384), so grid.y workgroups share a quad group, each with a part of K
+// that is a whole number of steps (the last part may reach past the end of K).  Their partial sums meet in a workspace; the last workgroup to arrive adds
 // them in part order (bit-identical from run to run) and writes C.
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
@@ -287,10 +288,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   w.fmt = FMT;
   const uint32_t quad_base = pick3(widx, 0u, first_quad1, first_quad2);  // first quad of that weight
   const uint32_t bpc = w.k / 32;
-  static_assert(!KSPLIT || (EXACT && PRO == kProNone && QPW == 1), "K parts come with full steps, one quad per wave and no prologue");
+  static_assert(!KSPLIT || (!EXACT && PRO == kProNone && QPW == 1), "K parts come with masked steps, one quad per wave and no prologue");
   const uint32_t kpart = KSPLIT ? blockIdx.y : 0u;
   const uint32_t bpc_full = KSPLIT ? sp.k_full / 32 : bpc;  // blocks per column of the weight
   const uint32_t kb_part = kpart * bpc;                     // this workgroup's first K block
+  const uint32_t bpc_live = KSPLIT ? min(bpc, bpc_full - kb_part) : bpc;  // blocks of this part that exist
   const uint32_t bpc_pad = (bpc + 15) & ~15u;
   constexpr uint32_t CPB = cinit_per_block<FMT>();
   const uint32_t plane = bpc_pad * NJ + plane_pad<FMT>(NJ);
@@ -332,7 +334,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 #pragma unroll
   for (int tt = 0; tt < TASKS; tt++) {
     const uint32_t t = tid + tt * nthreads, kb = t >> 2, ch = t & 3;
-    const bool live = kb < bpc;
+    const bool live = kb < bpc_live;
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
       // always load (from element 0 when there is nothing to load) and zero afterwards
@@ -414,7 +416,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 #pragma unroll
       for (int tt = 0; tt < TASKS; tt++) {
         const uint32_t kb = (tid + tt * nthreads) >> 2;
-        if (kb < bpc && (uint32_t)r < m) {
+        if (kb < bpc_live && (uint32_t)r < m) {
 #pragma unroll
           for (int h = 0; h < 2; h++) {
             const float4 v = xraw[tt][r][h];
@@ -453,7 +455,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 #pragma unroll
       for (int r = 0; r < MROWS; r++) {
         float4 v0 = xraw[tt][r][0], v1 = xraw[tt][r][1];
-        if (!(kb < bpc && (uint32_t)r < m)) v0 = v1 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (!(kb < bpc_live && (uint32_t)r < m)) v0 = v1 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         // block maximum over the quad's 32 values; NaN never wins fmaxf, an infinity
         // does and switches scaling off
         float am = fmaxf(fmaxf(fmaxf(fabsf(v0.x), fabsf(v0.y)), fmaxf(fabsf(v0.z), fabsf(v0.w))),
@@ -517,7 +519,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     Raw<FMT> cur = blk[t];
     // not every step is a full one: a block past the end of K or in a step that belongs to the
     // neighbouring K split gets scale (and minimum) zero
-    if constexpr (!EXACT) cur.meta = ((uint32_t)s >= first_own && kb_first + s * 16 < bpc) ? cur.meta : 0u;
+    if constexpr (!EXACT) cur.meta = ((uint32_t)s >= first_own && kb_first + s * 16 < bpc_live) ? cur.meta : 0u;
     if constexpr (FMT == MGN_FMT_Q4) {
       // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks; with more than
       // two activation rows a second group of four A rows (rows 2 and 3, hi and lo) follows
@@ -683,7 +685,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 
 struct MfmaGemvPlan {
   uint32_t ksc, wnc, steps, qpw, tasks, grid;
-  uint32_t kparts;  // workgroups sharing a quad group, each with K / kparts (1: no split over workgroups)
+  uint32_t kparts;  // workgroups sharing a quad group (1: no split over workgroups)
+  uint32_t part_k;  // K of one part when kparts > 1: a whole number of 16-block steps
   bool exact;  // every step of every K split is a full one
   size_t lds;
 };
@@ -747,14 +750,18 @@ bool plan_mfma_gemv(const LaunchArgs& x, uint32_t mrows, MfmaGemvPlan* out) {
   const uint32_t nquads = total_quads(x);
   if (plan_one_part(x.w.fmt, x.w.k, nquads, mrows, x.num_cus, !plain, out)) return true;
   if (!plain || !x.scratch || !x.counters) return false;
-  const uint32_t bpc = x.w.k / 32;
+  const uint32_t steps_total = (x.w.k / 32 + 15) / 16;
   for (uint32_t kp = 2; kp <= 8; kp++) {
-    if (bpc % (16 * kp) != 0) continue;
+    // parts of a whole number of 16-block steps; the last one may be short, never empty
+    const uint32_t part_steps = (steps_total + kp - 1) / kp;
+    if ((kp - 1) * part_steps >= steps_total) continue;
     if ((size_t)kp * mrows * x.w.n * sizeof(float) > x.scratch_bytes) return false;
     MfmaGemvPlan p;
-    if (!plan_one_part(x.w.fmt, x.w.k / kp, nquads, mrows, std::max(1, x.num_cus / (int)kp), true, &p)) continue;
-    if (!p.exact || p.qpw != 1 || p.grid > x.n_counters) continue;
+    if (!plan_one_part(x.w.fmt, part_steps * 512, nquads, mrows, std::max(1, x.num_cus / (int)kp), true, &p)) continue;
+    if (p.qpw != 1 || p.grid > x.n_counters) continue;
     p.kparts = kp;
+    p.part_k = part_steps * 512;
+    p.exact = false;  // the K-part kernels always mask (the last part may reach past the end of K)
     *out = p;
     return true;
   }
@@ -783,7 +790,7 @@ int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
   }
   const GemvSplit sp{x.w.k, p.kparts, (float*)x.scratch, x.counters};
   hipLaunchKernelGGL(kern, dim3(p.grid, p.kparts), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants,
-                     x.m, p.ksc, p.wnc, x.w.k / p.kparts, x.w.n, bt.first_quad[1], bt.first_quad[2],
+                     x.m, p.ksc, p.wnc, p.kparts > 1 ? p.part_k : x.w.k, x.w.n, bt.first_quad[1], bt.first_quad[2],
                      (4096u + p.ksc - 1) / p.ksc, x.pro_weight, x.pro_eps, bt, sp MGN_TRACE_ARG);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
@@ -793,8 +800,8 @@ template <int FMT, int MROWS, int STEPS, int QPW, int PRO>
 int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
   if (p.kparts > 1) {
     if constexpr (PRO == kProNone && QPW == 1)
-      return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, true, true>(s, x, p)
-                          : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, true, true>(s, x, p);
+      return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, false, true>(s, x, p)
+                          : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, false, true>(s, x, p);
     return (int)hipErrorInvalidValue;
   }
   if (p.exact)

@@ -58,10 +58,11 @@ mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn
   w->nb = (rows / 32) * cols;
   w->meta_bytes = w->nb * meta_elem(fmt);
   w->quant_bytes = w->nb * quant_elem(fmt);
-  // Sixteen all-zero blocks follow the real ones in both arrays: lanes that have no block of
-  // their own load block nb and contribute exactly zero, and the GEMV kernels' last K step of
-  // the last column may read up to fifteen blocks past the end of K.
-  constexpr size_t kMetaPad = 64, kQuantPad = 512;
+  // 256 all-zero blocks follow the real ones in both arrays: lanes that have no block of
+  // their own load block nb and contribute exactly zero, and the GEMV kernels' last K steps of
+  // the last column may read past the end of K (up to 15 blocks; up to 8 x 16 + 15 when K is
+  // cut into parts of whole steps for different workgroups).
+  constexpr size_t kMetaPad = 1024, kQuantPad = 8192;
   const size_t q_off = align_up(w->meta_bytes + kMetaPad, 256);
   hipError_t e = hipMalloc(&w->base, q_off + w->quant_bytes + kQuantPad);
   if (e != hipSuccess) {

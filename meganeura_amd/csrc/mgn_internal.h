@@ -29,7 +29,7 @@ void dequantize_q8_host(const uint8_t* in, size_t rows, size_t cols, float* out)
 //   Q8: meta[b] = u16 scale_f16,             quants[b] = 32 int8
 //       -> the reference's 36-byte blocks with the pad dropped and scales
 //          gathered, so quants are 32-byte aligned for 128-bit loads.
-// Both arrays carry sixteen extra all-zero blocks from index nb = (K/32)*N on.
+// Both arrays carry 256 extra all-zero blocks from index nb = (K/32)*N on.
 struct WeightView {
   const void* meta;
   const void* quants;

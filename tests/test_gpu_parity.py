@@ -135,6 +135,8 @@ ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv_valu": capi.ROUTE_GEMV_VALU, "gem
     (4, 14336, 518), (3, 12288, 64),
     # K splits that do not share the 16-block steps evenly, with a partial last step
     (1, 11008, 132), (2, 11040, 66),
+    # K parts that are not even: 37 and 21.5 steps of 16 blocks
+    (1, 18944, 132), (4, 11008, 260), (3, 13824, 70),
 ])
 def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
     x = synth.normal(1000 + m + k + n, m * k).reshape(m, k)

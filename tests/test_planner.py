@@ -30,19 +30,21 @@ def check_gemv(p, fmt, m, k, n):
     assert p.threads == 64 * p.k_splits * p.waves_n <= 1024
     assert p.lds_bytes <= 150 * 1024
     assert p.k_parts >= 1 and p.grid[1] == p.k_parts and p.grid[2] == 1
-    assert bpc % p.k_parts == 0
-    part_blocks = bpc // p.k_parts
+    steps_all = ceil_div(bpc, 16)
     if p.k_parts > 1:
-        assert part_blocks % 16 == 0 and p.full_steps == 1 and p.quads_per_wave == 1
+        # parts of a whole number of 16-block steps, none of them empty; their kernels always mask
+        steps_total = ceil_div(steps_all, p.k_parts)
+        assert (p.k_parts - 1) * steps_total < steps_all
+        assert p.full_steps == 0 and p.quads_per_wave == 1
         assert p.workspace_bytes == p.k_parts * mrows * n * 4 <= WORKSPACE
         assert p.grid[0] <= COUNTERS
     else:
+        steps_total = steps_all
         assert p.workspace_bytes == 0
-    steps_total = ceil_div(part_blocks, 16)
+        assert p.full_steps == int(bpc % 16 == 0 and p.k_splits * p.steps == steps_total)
     assert 1 <= p.steps <= 8
     assert p.k_splits * p.steps >= steps_total          # all of K is walked
     assert (p.k_splits - 1) * p.steps < steps_total      # no K split without a step of its own
-    assert p.full_steps == int(part_blocks % 16 == 0 and p.k_splits * p.steps == steps_total)
     nquads = ceil_div(n, 4)
     per_wg = p.waves_n * p.quads_per_wave
     assert p.grid[0] * per_wg >= nquads                  # every column has a wave
@@ -110,6 +112,23 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
     assert (head.grid[0], head.threads, head.steps, head.k_splits, head.full_steps) == (256, 896, 8, 1, 1)
     tall = capi.matmul_plan(Q4, 4, 14336, 4096)
     assert tall.k_parts == 2 and tall.workspace_bytes == 2 * 4 * 4096 * 4
+    # K = 18944 is 37 steps of 16 blocks: more activation chunks than a workgroup has threads for
+    assert capi.matmul_plan(Q4, 1, 18944, 3584).route == GEMV_MFMA
+    assert capi.matmul_plan(Q4, 4, 11008, 4096).k_parts >= 2
+
+
+def test_edge_shapes_of_the_gpu_parity_tests_stay_on_the_gemv_kernel():
+    """tests/test_gpu_parity.py::test_small_m_routes skips a route that refuses a shape; these are
+    the shapes it lists for the sake of the MFMA GEMV's special cases, so that route must take them."""
+    for m, k, n in [(2, 512, 2055), (1, 512, 32774), (4, 14336, 518), (3, 12288, 64), (1, 11008, 132), (2, 11040, 66),
+                    (1, 18944, 132), (4, 11008, 260), (3, 13824, 70), (1, 576, 577), (4, 4096, 257), (1, 14336, 64)]:
+        for fmt in (Q4, Q8):
+            p = capi.matmul_plan(fmt, m, k, n)
+            assert p.route == GEMV_MFMA, (fmt, m, k, n)
+    assert capi.matmul_plan(Q4, 4, 14336, 518).k_parts > 1
+    assert capi.matmul_plan(Q4, 1, 18944, 132).k_parts > 1
+    assert capi.matmul_plan(Q4, 1, 11008, 132).full_steps == 0
+    assert capi.matmul_plan(Q4, 1, 512, 32774).quads_per_wave == 4
 
 
 def test_shapes_no_weight_can_have_are_refused():
