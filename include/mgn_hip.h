@@ -160,7 +160,8 @@ mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, con
 /* The same with fp16 activations A[M,K] (prefill): fp16 operands on MFMA with
  * f32 accumulation, the role matmul_coop.wgsl plays for unquantized weights
  * (src/codegen.rs:1168-1176; quantized weights are excluded from it in the
- * reference, src/runtime.rs:1634). */
+ * reference, src/runtime.rs:1634).  At M <= 4 the decode kernel takes it and
+ * widens the halves while it stages the activations. */
 mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w,
                              const mgn_buf* d, mgn_buf* c, uint32_t m);
 

@@ -21,7 +21,8 @@ int launch_gemv_mfma_q8_m2(ihipStream_t* s, const LaunchArgs& x);
 int launch_gemv_mfma_q8_m4(ihipStream_t* s, const LaunchArgs& x);
 
 bool gemv_mfma_supported(const LaunchArgs& x) {
-  if (x.a_is_f16 || x.m == 0 || x.m > 4) return false;
+  if (x.m == 0 || x.m > 4) return false;
+  if (x.a_is_f16 && x.pro_kind != kProNone) return false;  // fp16 activations: the plain matmul only
   MfmaGemvPlan p;
   for (int j = 0; j < x.n_more; j++)
     if (x.more[j].w.k != x.w.k || x.more[j].w.fmt != x.w.fmt) return false;

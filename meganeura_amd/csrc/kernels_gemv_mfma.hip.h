@@ -260,11 +260,14 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // they are declared first (and not inside a struct) so that the dispatcher can hand them
     // over in registers (kernel-argument preload) instead of the wave fetching them from memory.
     // (three pointers and eight 32-bit values: the 14 dwords that can be preloaded)
-    const float* __restrict__ a, const void* __restrict__ meta0, const void* __restrict__ quants0, uint32_t m,
+    const float* __restrict__ a, const void* __restrict__ meta0, const void* __restrict__ quants0,
+    uint32_t m_flags,  // rows in bits 0-7; bit 31: the activations are fp16 (kProNone only)
     uint32_t ksc, uint32_t wnc, uint32_t kdim, uint32_t n0, uint32_t first_quad1, uint32_t first_quad2,
     uint32_t ksc_recip,  // ceil(4096 / ksc): wave / ksc == (wave * ksc_recip) >> 12 for the 16 waves there can be
     const float* __restrict__ norm_weight, float eps, GemvBatch bt, GemvSplit sp MGN_TRACE_PARAM) {
   MGN_STAMP_INIT();
+  const uint32_t m = m_flags & 0xFFu;
+  const bool a_f16 = PRO == kProNone && (m_flags >> 31) != 0;
   const GemvPrologue pro{norm_weight, eps};
   constexpr int NJ = 2 * MROWS;       // A rows in LDS: hi and lo of every activation row
   constexpr int NG = (MROWS + 1) / 2;  // groups of four A rows = MFMA chains per weight chunk
@@ -339,9 +342,15 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     for (int r = 0; r < MROWS; r++) {
       // always load (from element 0 when there is nothing to load) and zero afterwards
       const bool ok = live && (uint32_t)r < m;
-      const float4* src = (const float4*)(a + (ok ? (size_t)r * a_stride + (size_t)(kb_part + kb) * 32 + ch * 8 : (size_t)0));
-      xraw[tt][r][0] = src[0];
-      xraw[tt][r][1] = src[1];
+      const size_t off = ok ? (size_t)r * a_stride + (size_t)(kb_part + kb) * 32 + ch * 8 : (size_t)0;
+      if (a_f16) {  // eight halves in one 16-byte load; widened once the weight loads are on their way
+        xraw[tt][r][0] = *(const float4*)((const _Float16*)(const void*)a + off);
+        xraw[tt][r][1] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      } else {
+        const float4* src = (const float4*)(a + off);
+        xraw[tt][r][0] = src[0];
+        xraw[tt][r][1] = src[1];
+      }
       if constexpr (PRO == kProSwiglu) {
         const float4* up = (const float4*)(a + (ok ? (size_t)r * a_stride + w.k + (size_t)kb * 32 + ch * 8 : (size_t)0));
         xup[tt][r][0] = up[0];
@@ -394,6 +403,18 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   MGN_STAMP_EARLY();
   MGN_STAMP_FLUSH();
 
+  if (a_f16) {
+#pragma unroll
+    for (int tt = 0; tt < TASKS; tt++)
+#pragma unroll
+      for (int r = 0; r < MROWS; r++) {
+        const float4 h = xraw[tt][r][0];
+        const uint32_t h0 = __builtin_bit_cast(uint32_t, h.x), h1 = __builtin_bit_cast(uint32_t, h.y);
+        const uint32_t h2 = __builtin_bit_cast(uint32_t, h.z), h3 = __builtin_bit_cast(uint32_t, h.w);
+        xraw[tt][r][0] = make_float4(half_lo(h0), half_hi(h0), half_lo(h1), half_hi(h1));
+        xraw[tt][r][1] = make_float4(half_lo(h2), half_hi(h2), half_lo(h3), half_hi(h3));
+      }
+  }
   // ---- fused prologue: turn the raw loads into the matmul's activations ----
   if constexpr (PRO == kProSwiglu) {
 #pragma unroll
@@ -802,7 +823,8 @@ int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
   }
   const GemvSplit sp{x.w.k, p.kparts, (float*)x.scratch, x.counters};
   hipLaunchKernelGGL(kern, dim3(p.grid, p.kparts), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants,
-                     x.m, p.ksc, p.wnc, p.kparts > 1 ? p.part_k : x.w.k, x.w.n, bt.first_quad[1], bt.first_quad[2],
+                     x.m | (x.a_is_f16 ? 0x80000000u : 0u), p.ksc, p.wnc, p.kparts > 1 ? p.part_k : x.w.k, x.w.n,
+                     bt.first_quad[1], bt.first_quad[2],
                      (4096u + p.ksc - 1) / p.ksc, x.pro_weight, x.pro_eps, bt, sp MGN_TRACE_ARG);
   MGN_HIP_LAUNCH_CHECK();
   return 0;

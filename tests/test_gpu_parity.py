@@ -155,6 +155,21 @@ def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m,k,n", [(1, 576, 192), (1, 4096, 257), (3, 1024, 100), (4, 14336, 70), (2, 11040, 66)])
+def test_small_m_fp16_activations(ctx, orc, fmt, m, k, n):
+    """mgn_matmul_q_f16a at decode sizes: the GEMV kernel widens the halves while it stages the
+    activations; the oracle multiplies the rounded values."""
+    x = synth.normal(21 + m + k + n, m * k).reshape(m, k)
+    w = synth.normal(22 + m + k + n, k * n, 0.02).reshape(k, n)
+    d = synth.normal(23 + n, m * n).reshape(m, n)
+    deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
+    x16 = x.astype(np.float16).astype(np.float32)
+    for route in ("generic", "gemv_mfma", "auto"):
+        got = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d, f16=True)
+        orc.assert_close(got, orc.matmul_f32(x16, deq, d), REL, ABS)
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
 @pytest.mark.parametrize("m,k,n", [(5, 64, 70), (6, 1024, 2048), (16, 576, 130), (17, 256, 64), (64, 128, 96), (130, 96, 67)])
 def test_larger_m(ctx, orc, fmt, m, k, n):
     x = synth.normal(11 + m + k + n, m * k).reshape(m, k)

@@ -78,14 +78,16 @@ def test_plans_cover_the_problem_and_respect_the_limits(fmt):
     for m, k, n in itertools.product(MS, KS, NS):
         if (k // 32) * n >= 0x7FFFFFFF:
             continue
-        for f16 in ((False, True) if m >= 5 else (False,)):
+        for f16 in (False, True):
             p = capi.matmul_plan(fmt, m, k, n, f16)
             where = f"fmt={fmt} m={m} k={k} n={n} f16={f16} route={p.route}"
             routes.add(p.route)
             try:
                 assert p.route in (GENERIC, GEMV_VALU, GEMV_MFMA, GEMM_MFMA)
-                if m > 4 or f16:
+                if m > 4:
                     assert p.route in (GEMM_MFMA, GENERIC)
+                if f16:
+                    assert p.route != GEMV_VALU  # the vector-ALU GEMV reads f32 activations only
                 if p.route == GEMV_MFMA:
                     check_gemv(p, fmt, m, k, n)
                 elif p.route == GEMM_MFMA:
