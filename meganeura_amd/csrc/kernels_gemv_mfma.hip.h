@@ -581,7 +581,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       }
     } else {
       // two half blocks per step, each with its own chain of four MFMAs and its own scale
-      const float dscale_own = half_bits_to_float(cur.meta);
+      // the half blocks' scales sit in lanes (b / 2, i) and (8 + b / 2, i); fetched first so that
+      // the answers are back when the chains end
+      const int dscale_own = __builtin_bit_cast(int, half_bits_to_float(cur.meta));
+      const float dscales[2] = {__builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((int)scale_lane, dscale_own)),
+                          __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((int)scale_lane + 8 * 4 * 4, dscale_own))};
 #pragma unroll
       for (int hb = 0; hb < 2; hb++) {
         const uint4 qw = hb == 0 ? cur.q0 : cur.q1;
@@ -611,9 +615,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
             dsum[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(aop, as_half4(lo2, hi2), dsum[g], 0, 0, 0);
           }
         }
-        // the half block's scale sits in lane (hb * 8 + b / 2, i)
-        const float dscale = __builtin_bit_cast(
-            float, __builtin_amdgcn_ds_bpermute((int)scale_lane + hb * (8 * 4 * 4), __builtin_bit_cast(int, dscale_own)));
+        const float dscale = dscales[hb];
 #pragma unroll
         for (int r = 0; r < MROWS; r++) {
           const float v = dscale * (dsum[r / 2][2 * (r % 2)] + dsum[r / 2][2 * (r % 2) + 1]);
