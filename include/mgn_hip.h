@@ -165,6 +165,22 @@ mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, con
 mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w,
                              const mgn_buf* d, mgn_buf* c, uint32_t m);
 
+/* The same followed by unary operations on every output element, first to last:
+ * C = f_n(... f_1(A x W + D)).  Stands in for a matmul dispatch that carries an epilogue
+ * (compile.rs:915-1035 fuse_epilogues folds a Relu / Sigmoid / Neg / Silu that is the only
+ * reader of a matmul's output into the matmul; formulas codegen.rs:62-100).  The reference
+ * builds that pipeline with the f32 weight format even when the weight is quantized
+ * (codegen.rs:617-642); here the epilogue rides on the quantized kernels.  n_ops <= 8. */
+typedef enum mgn_unary {
+  MGN_UNARY_NONE = 0,
+  MGN_UNARY_RELU = 1,    /* max(v, 0) */
+  MGN_UNARY_SIGMOID = 2, /* 1 / (1 + exp(-v)) */
+  MGN_UNARY_NEG = 3,     /* -v */
+  MGN_UNARY_SILU = 4     /* v / (1 + exp(-v)) */
+} mgn_unary;
+mgn_status mgn_matmul_q_epilogue(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d,
+                                 mgn_buf* c, uint32_t m, const mgn_unary* ops, size_t n_ops);
+
 /* `steps` such matmuls enqueued back to back, call i on weights[i % count]: the step loop of
  * a compiled host (examples/matmul_throughput.rs:114-127) without an interpreter between the
  * launches, for harnesses written in a scripting language.  Copies of one weight in rotation

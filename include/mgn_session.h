@@ -35,7 +35,11 @@ typedef enum mgn_shader {
   MGN_SHADER_SWIGLU_CONCAT = 6,
   MGN_SHADER_RMS_NORM = 7,
   MGN_SHADER_MATMUL_BT = 8,      /* ShaderEntry::MatMulBT:     C = A x B^T, B stored [N, K] */
-  MGN_SHADER_MATMUL_GEMV_BT = 9  /* ShaderEntry::MatMulGemvBT: its M = 1 form */
+  MGN_SHADER_MATMUL_GEMV_BT = 9, /* ShaderEntry::MatMulGemvBT: its M = 1 form */
+  MGN_SHADER_RELU = 10,          /* the unary entries fuse_epilogues can fold into a matmul */
+  MGN_SHADER_SIGMOID = 11,
+  MGN_SHADER_NEG = 12,
+  MGN_SHADER_SILU = 13
 } mgn_shader;
 
 /* compile::Dispatch (src/compile.rs:435-488), the fields this path uses.
@@ -43,8 +47,9 @@ typedef enum mgn_shader {
 typedef struct mgn_dispatch_info {
   int32_t shader;          /* mgn_shader */
   uint32_t workgroups[3];  /* the grid the reference would launch */
-  uint32_t params[4];      /* [m, k, n, 0] for matmuls, [m, n, k, 0] for the BT forms */
+  uint32_t params[4];      /* [m, k, n, 0] for matmuls, [m, n, k, 0] for the BT forms, [len, 0, 0, 0] for unary entries */
   int32_t weight_format;
+  uint32_t epilogue;       /* Dispatch::epilogue of a matmul: mgn_unary codes, four bits each, first in the low bits */
 } mgn_dispatch_info;
 
 /* Graph::new and the builders (src/graph.rs:714-795, 996-999).  Each builder
@@ -64,6 +69,10 @@ int32_t mgn_graph_matmul_bt(mgn_graph* g, int32_t a, int32_t b);
 int32_t mgn_graph_add(mgn_graph* g, int32_t a, int32_t b);
 int32_t mgn_graph_swiglu(mgn_graph* g, int32_t gate, int32_t up);
 int32_t mgn_graph_rms_norm(mgn_graph* g, int32_t x, int32_t weight, float eps);
+/* Graph::relu / sigmoid / neg / silu (src/graph.rs): kind is a mgn_unary.  A unary node that is
+ * the only reader of a tiled matmul's output becomes that matmul's epilogue when the graph is
+ * compiled (compile.rs:915-1035); otherwise it is a dispatch of its own. */
+int32_t mgn_graph_unary(mgn_graph* g, int32_t kind, int32_t x);
 mgn_status mgn_graph_set_outputs(mgn_graph* g, const int32_t* ids, size_t count);
 
 /* compile only (optimize + compile_with, src/train.rs:272-340 without the GPU

@@ -30,6 +30,23 @@ __device__ __forceinline__ uint16_t stream_load_u16(const void* p) {
   return __builtin_nontemporal_load((const uint16_t*)p);
 }
 
+// Unary operations applied to a finished output element, first to last, four bits each
+// (mgn_unary; 0 ends the chain): compile.rs:915-1035 fuse_epilogues with the formulas of
+// codegen.rs:62-100.  The chain is the same for every element, so the branches are uniform.
+__device__ __forceinline__ float apply_epilogue(float v, uint32_t ops) {
+  while (ops != 0) {
+    switch (ops & 15u) {
+      case MGN_UNARY_RELU: v = fmaxf(v, 0.0f); break;
+      case MGN_UNARY_SIGMOID: v = 1.0f / (1.0f + expf(-v)); break;
+      case MGN_UNARY_NEG: v = -v; break;
+      case MGN_UNARY_SILU: v = v / (1.0f + expf(-v)); break;
+      default: break;
+    }
+    ops >>= 4;
+  }
+  return v;
+}
+
 // Byte N of a word as float: the compiler selects v_cvt_f32_ubyteN for these.
 __device__ __forceinline__ float ubyte0(uint32_t v) { return (float)(v & 0xFFu); }
 __device__ __forceinline__ float ubyte1(uint32_t v) { return (float)((v >> 8) & 0xFFu); }

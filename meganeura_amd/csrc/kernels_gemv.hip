@@ -163,7 +163,7 @@ constexpr int max_waves() { return MR >= 4 ? 4 : 8; }
 
 template <int FMT, int KBW, int MR, int U>
 __global__ __launch_bounds__(64 * max_waves<MR>()) void gemv_kernel(WeightView w, const float* __restrict__ a, const float* __restrict__ d,
-                            float* __restrict__ c, uint32_t m, uint32_t steps, uint32_t kgc) {
+                            float* __restrict__ c, uint32_t m, uint32_t steps, uint32_t kgc, uint32_t epilogue) {
   extern __shared__ float lds[];
   const uint32_t x_floats = MR * (w.k / 32) * kXStride;
   float* xs = lds;               // [MR][bpc][36] staged activations
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(64 * max_waves<MR>()) void gemv_kernel(WeightView w
           if (kgc == 1) {
             if (n < w.n && (uint32_t)r < m) {
               const size_t idx = (size_t)r * w.n + n;
-              c[idx] = d ? v + d[idx] : v;
+              c[idx] = apply_epilogue(d ? v + d[idx] : v, epilogue);
             }
           } else {
             red[(kg * MR + r) * cols_per_wg + col0 + (step + u) * NW] = v;
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(64 * max_waves<MR>()) void gemv_kernel(WeightView w
         float v = 0.0f;
         for (uint32_t g = 0; g < kgc; g++) v += red[(g * MR + r) * cols_per_wg + col];
         const size_t o = (size_t)r * w.n + n;
-        c[o] = d ? v + d[o] : v;
+        c[o] = apply_epilogue(d ? v + d[o] : v, epilogue);
       }
     }
   }
@@ -288,7 +288,7 @@ int launch_gemv_t(ihipStream_t* s, const LaunchArgs& x) {
     static std::atomic<uint64_t> big_lds_done{0};                                                       \
     if (lds > 64 * 1024)                                                                                \
       if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;                               \
-    hipLaunchKernelGGL(kern, grid, block, lds, s, x.w, (const float*)x.a, x.d, x.c, x.m, p.steps, p.kgc); \
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x.w, (const float*)x.a, x.d, x.c, x.m, p.steps, p.kgc, x.epilogue); \
   } while (0)
   switch (p.kbw) {
     case 64: MGN_GEMV(64); break;

@@ -144,6 +144,7 @@ struct GemvSplit {
   uint32_t kparts;
   float* scratch;      // [kparts][MROWS][n] partial sums
   uint32_t* counters;  // one arrival counter per blockIdx.x, zero between launches
+  uint32_t epilogue;   // unary operations on the output (apply_epilogue); needed with or without K parts
 };
 template <typename T>
 __device__ __forceinline__ T pick3(uint32_t idx, T a0, T a1, T a2) {
@@ -641,7 +642,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
           const size_t o = (size_t)r * w.n + n;
           const float* const dres = pick3(widx, bt.d[0], bt.d[1], bt.d[2]);
           float* const c = pick3(widx, bt.c[0], bt.c[1], bt.c[2]);
-          c[o] = dres ? tot + dres[o] : tot;
+          c[o] = apply_epilogue(dres ? tot + dres[o] : tot, sp.epilogue);
         }
       }
     }
@@ -697,7 +698,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         } else {
           const size_t o = (size_t)r * wn_cols + n;
           const float* const dd = pick3(wi, bt.d[0], bt.d[1], bt.d[2]);
-          pick3(wi, bt.c[0], bt.c[1], bt.c[2])[o] = dd ? v + dd[o] : v;
+          pick3(wi, bt.c[0], bt.c[1], bt.c[2])[o] = apply_epilogue(dd ? v + dd[o] : v, sp.epilogue);
         }
       }
     }
@@ -823,7 +824,7 @@ int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
       bt.first_quad[j] = 0xFFFFFFFFu;
     }
   }
-  const GemvSplit sp{x.w.k, p.kparts, (float*)x.scratch, x.counters};
+  const GemvSplit sp{x.w.k, p.kparts, (float*)x.scratch, x.counters, x.epilogue};
   hipLaunchKernelGGL(kern, dim3(p.grid, p.kparts), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants,
                      x.m | (x.a_is_f16 ? 0x80000000u : 0u), p.ksc, p.wnc, p.kparts > 1 ? p.part_k : x.w.k, x.w.n,
                      bt.first_quad[1], bt.first_quad[2],

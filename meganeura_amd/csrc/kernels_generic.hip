@@ -43,7 +43,7 @@ __device__ __forceinline__ void load_block(const WeightView& w, size_t b, float 
 template <int FMT, typename AT>
 __global__ __launch_bounds__(256) void generic_kernel(WeightView w, const AT* __restrict__ a,
                                                       const float* __restrict__ d, float* __restrict__ c,
-                                                      uint32_t m) {
+                                                      uint32_t m, uint32_t epilogue) {
   __shared__ float red[4][TM][64];
   const uint32_t lane = threadIdx.x & 63, ks = threadIdx.x >> 6;
   const uint32_t n = blockIdx.x * 64 + lane;
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void generic_kernel(WeightView w, const AT* __
         float v = (red[0][r][lane] + red[1][r][lane]) + (red[2][r][lane] + red[3][r][lane]);
         const size_t idx = (size_t)(m0 + r) * w.n + n;
         if (d) v += d[idx];
-        c[idx] = v;
+        c[idx] = apply_epilogue(v, epilogue);
       }
     }
   }
@@ -88,7 +88,7 @@ int launch_matmul_generic(ihipStream_t* s, const LaunchArgs& x) {
   dim3 grid((x.w.n + 63) / 64, (x.m + TM - 1) / TM);
   dim3 block(256);
 #define MGN_GENERIC(FMT, AT) \
-  hipLaunchKernelGGL((generic_kernel<FMT, AT>), grid, block, 0, s, x.w, (const AT*)x.a, x.d, x.c, x.m)
+  hipLaunchKernelGGL((generic_kernel<FMT, AT>), grid, block, 0, s, x.w, (const AT*)x.a, x.d, x.c, x.m, x.epilogue)
   if (x.w.fmt == MGN_FMT_Q4) {
     if (x.a_is_f16) MGN_GENERIC(MGN_FMT_Q4, _Float16); else MGN_GENERIC(MGN_FMT_Q4, float);
   } else {

@@ -120,6 +120,7 @@ struct GemmTail {  // arguments first needed in the epilogue
   uint32_t* counters;  // one arrival counter per (row tile, column group), zero between launches
   uint32_t* range_flag;  // host-visible: set when an f32 activation does not fit the fp16 pair
   uint32_t row_tiles;
+  uint32_t epilogue;  // unary operations on the output (apply_epilogue)
 #ifdef MGN_TRACE
   unsigned long long* trace;
 #endif
@@ -561,7 +562,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
       const uint32_t row = row0 + 8 * (i >> 2) + 4 * gh + (i & 3);
       if (row < g.m) {
         const size_t o = (size_t)row * w.n + n;
-        g.c[o] = g.dres ? outv[i] + g.dres[o] : outv[i];
+        g.c[o] = apply_epilogue(g.dres ? outv[i] + g.dres[o] : outv[i], tail.epilogue);
       }
     }
   }
@@ -664,7 +665,7 @@ int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
   auto kern = gemm_mfma_kernel<FMT, F32A, TPT>;
   static std::atomic<uint64_t> big_lds_done{0};
   if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
-  GemmTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.range_flag, p.grid_y};
+  GemmTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.range_flag, p.grid_y, x.epilogue};
 #ifdef MGN_TRACE
   tail.trace = g_gemm_trace_host;
 #endif

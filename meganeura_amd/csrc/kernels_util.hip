@@ -207,8 +207,20 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
   for (uint32_t j = tid; j < cols; j += 256) dst[j] = src[j] * r * wt[j];
 }
 
+// relu / sigmoid / neg / silu as dispatches of their own (src/codegen.rs:85-96 for the formulas)
+__global__ __launch_bounds__(256) void unary_kernel(uint32_t kind, const float* __restrict__ in, float* __restrict__ out,
+                                                    size_t len) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < len) out[i] = apply_epilogue(in[i], kind);
+}
+
 }  // namespace
 
+int launch_unary(ihipStream_t* s, int kind, const float* in, float* out, size_t len) {
+  hipLaunchKernelGGL(unary_kernel, dim3((unsigned)((len + 255) / 256)), dim3(256), 0, s, (uint32_t)kind, in, out, len);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
 int launch_add(ihipStream_t* s, const float* a, const float* b, float* out, size_t len) {
   hipLaunchKernelGGL(add_kernel, dim3((unsigned)((len + 255) / 256)), dim3(256), 0, s, a, b, out, len);
   MGN_HIP_LAUNCH_CHECK();

@@ -492,7 +492,7 @@ mgn_status mgn_weight_load(mgn_ctx* ctx, const char* path, mgn_weight** out) {
 
 static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, const mgn_weight* w, const mgn_buf* d,
                               mgn_buf* c, uint32_t m, int pro_kind = mgn::kProNone, const mgn_buf* norm_weight = nullptr,
-                              float eps = 0.0f) {
+                              float eps = 0.0f, uint32_t epilogue = 0) {
   if (!ctx || !a || !w || !c) return fail(ctx, MGN_EINVAL, "null argument");
   if (m == 0) return MGN_OK;
   const size_t k = w->rows, n = w->cols;
@@ -514,6 +514,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   x.pro_kind = pro_kind;
   x.pro_weight = norm_weight ? (const float*)norm_weight->ptr : nullptr;
   x.pro_eps = eps;
+  x.epilogue = epilogue;
   mgn_route route = ctx->route;
   if (pro_kind != mgn::kProNone) {
     // only the MFMA GEMV stages its activations in a way a prologue can ride on
@@ -552,6 +553,17 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
 mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
                         uint32_t m) {
   return matmul_impl(ctx, a, false, w, d, c, m);
+}
+
+mgn_status mgn_matmul_q_epilogue(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
+                                 uint32_t m, const mgn_unary* ops, size_t n_ops) {
+  if (n_ops > 8 || (n_ops > 0 && !ops)) return fail(ctx, MGN_EINVAL, "an epilogue has at most 8 operations");
+  uint32_t packed = 0;
+  for (size_t i = 0; i < n_ops; i++) {
+    if (ops[i] < MGN_UNARY_RELU || ops[i] > MGN_UNARY_SILU) return fail(ctx, MGN_EINVAL, "unknown unary operation in the epilogue");
+    packed |= (uint32_t)ops[i] << (4 * i);
+  }
+  return matmul_impl(ctx, a, false, w, d, c, m, mgn::kProNone, nullptr, 0.0f, packed);
 }
 
 mgn_status mgn_matmul_q_rms_norm(mgn_ctx* ctx, const mgn_buf* x, const mgn_buf* norm_weight, float eps,

@@ -60,6 +60,7 @@ struct LaunchArgs {
   };
   More more[2] = {};
   int n_more = 0;
+  uint32_t epilogue = 0;  // unary operations on the output, four bits each, first in the low bits
   // fused prologue (GEMV-MFMA route only): what `a` goes through before the matmul
   int pro_kind = 0;                   // kProNone / kProRmsNorm / kProSwiglu
   const float* pro_weight = nullptr;  // norm weight [K]

@@ -85,6 +85,14 @@ NodeId Graph::rms_norm(NodeId x, NodeId weight, float eps) {
   return add_raw_node(Op::RmsNorm, {x, weight}, TensorType{xs, DType::F32}, {}, eps);
 }
 
+NodeId Graph::unary(mgn_unary kind, NodeId x) {
+  const Op op = kind == MGN_UNARY_RELU ? Op::Relu : kind == MGN_UNARY_SIGMOID ? Op::Sigmoid : kind == MGN_UNARY_NEG ? Op::Neg
+              : kind == MGN_UNARY_SILU ? Op::Silu : Op::Nop;
+  if (op == Op::Nop) throw GraphError("unknown unary operation");
+  if (node(x).ty.dtype != DType::F32) throw GraphError("unary operations take f32 tensors");
+  return add_raw_node(op, {x}, TensorType{node(x).ty.shape, DType::F32});
+}
+
 void Graph::set_outputs(std::vector<NodeId> ids) {
   for (NodeId id : ids) (void)node(id);
   outputs_ = std::move(ids);
@@ -214,6 +222,46 @@ static std::vector<NodeId> toposort(const Graph& g) {
   return order;
 }
 
+static mgn_unary unary_of(mgn_shader s) {
+  return s == MGN_SHADER_RELU ? MGN_UNARY_RELU : s == MGN_SHADER_SIGMOID ? MGN_UNARY_SIGMOID
+         : s == MGN_SHADER_NEG ? MGN_UNARY_NEG : s == MGN_SHADER_SILU ? MGN_UNARY_SILU : MGN_UNARY_NONE;
+}
+
+// fuse_epilogues (src/compile.rs:915-1035): a Relu / Sigmoid / Neg / Silu dispatch whose input
+// is written by a tiled matmul entry and read by nothing else is removed; the matmul takes its
+// output buffer and applies the operation to every element it stores.  Chains fold one by one.
+// The M = 1 entries (MatMulGemv*) are not candidates in the reference and are none here.
+// Differences: the reference builds the resulting pipeline with the f32 weight format whatever
+// the weight is (src/codegen.rs:617-642) -- here the quantized kernels apply the epilogue; and
+// it does not look at graph outputs, so a matmul result that is itself an output would never
+// be written -- here such a matmul keeps its buffer and the unary stays a dispatch.
+static void fuse_epilogues(ExecutionPlan& plan) {
+  auto& ds = plan.dispatches;
+  std::map<int, size_t> producer;
+  for (size_t i = 0; i < ds.size(); i++) producer[ds[i].output_buffer] = i;
+  std::map<int, size_t> read_count;
+  for (const Dispatch& d : ds)
+    for (int b : d.input_buffers) read_count[b]++;
+  std::vector<size_t> to_remove;
+  for (size_t i = 0; i < ds.size(); i++) {
+    const mgn_unary op = unary_of(ds[i].shader);
+    if (op == MGN_UNARY_NONE || ds[i].input_buffers.size() != 1) continue;
+    const int primary = ds[i].input_buffers[0];
+    auto pit = producer.find(primary);
+    if (pit == producer.end()) continue;
+    Dispatch& prod = ds[pit->second];
+    const bool tiled = prod.shader == MGN_SHADER_MATMUL || prod.shader == MGN_SHADER_FUSED_MATMUL_ADD ||
+                       prod.shader == MGN_SHADER_MATMUL_BT;
+    if (!tiled || read_count[primary] != 1 || prod.epilogue.size() >= 8) continue;
+    if (std::find(plan.output_buffers.begin(), plan.output_buffers.end(), primary) != plan.output_buffers.end()) continue;
+    prod.epilogue.push_back(op);
+    prod.output_buffer = ds[i].output_buffer;
+    producer[ds[i].output_buffer] = pit->second;
+    to_remove.push_back(i);
+  }
+  for (auto it = to_remove.rbegin(); it != to_remove.rend(); ++it) ds.erase(ds.begin() + (std::ptrdiff_t)*it);
+}
+
 ExecutionPlan compile(const Graph& g) {
   ExecutionPlan plan;
   std::map<NodeId, int> node_buf;
@@ -328,6 +376,19 @@ ExecutionPlan compile(const Graph& g) {
         d.params[0] = len, d.params[1] = (uint32_t)nd.ty.shape[1];
         break;
       }
+      case Op::Relu:
+      case Op::Sigmoid:
+      case Op::Neg:
+      case Op::Silu: {
+        // emit_unary (src/compile.rs:3433-3453): grid [ceil(len / 256), 1, 1], params [len, 0, 0, 0]
+        const uint32_t len = (uint32_t)nd.ty.num_elements();
+        d.shader = nd.op == Op::Relu ? MGN_SHADER_RELU : nd.op == Op::Sigmoid ? MGN_SHADER_SIGMOID
+                   : nd.op == Op::Neg ? MGN_SHADER_NEG : MGN_SHADER_SILU;
+        d.workgroups[0] = (len + 255) / 256, d.workgroups[1] = 1, d.workgroups[2] = 1;
+        d.input_buffers = {buf_of(nd.inputs[0])};
+        d.params[0] = len;
+        break;
+      }
       case Op::RmsNorm: {
         // src/compile.rs:1851-1872 (the hand-written entry: one workgroup per row)
         const auto& xs = g.node(nd.inputs[0]).ty.shape;
@@ -343,6 +404,7 @@ ExecutionPlan compile(const Graph& g) {
     plan.dispatches.push_back(std::move(d));
   }
   for (NodeId out : g.outputs()) plan.output_buffers.push_back(buf_of(out));
+  fuse_epilogues(plan);
   return plan;
 }
 
@@ -563,7 +625,7 @@ void Session::plan_launches() {
       const Dispatch& c = plan_.dispatches[ci];
       mgn_weight* w = is_matmul(c.shader) ? weights_[c.input_buffers[1]] : nullptr;
       ok = ok && (size_t)ci > pi && w && c.input_buffers[0] == out && is_matmul(c.shader) && matmul_k(c) == width &&
-           (c.input_buffers.size() < 3 || c.input_buffers[2] != out) && fused_[ci].kind == 0 &&
+           (c.input_buffers.size() < 3 || c.input_buffers[2] != out) && fused_[ci].kind == 0 && c.epilogue.empty() &&
            mgn_matmul_q_can_fuse(ctx_, w, c.params[0]) == 1;
     }
     if (!ok) continue;
@@ -580,7 +642,7 @@ void Session::plan_launches() {
   for (size_t i = 0; i < nd; i++) producer_of[plan_.dispatches[i].output_buffer] = (int)i;
   auto batchable = [&](size_t i) {
     const Dispatch& d = plan_.dispatches[i];
-    if (skipped_[i] || !is_matmul(d.shader)) return false;
+    if (skipped_[i] || !is_matmul(d.shader) || !d.epilogue.empty()) return false;
     mgn_weight* w = weights_[d.input_buffers[1]];
     return w && mgn_matmul_q_can_fuse(ctx_, w, d.params[0]) == 1;
   };
@@ -600,6 +662,26 @@ void Session::plan_launches() {
       fused_[i].more[found++] = (int)j;
       skipped_[j] = 1;
     }
+  }
+  // Unary dispatches behind a matmul that the compiler left alone (M = 1 entries): the matmul's
+  // launch applies them when nothing else reads the intermediate result.
+  for (size_t ui = 0; ui < nd; ui++) {
+    const Dispatch& u = plan_.dispatches[ui];
+    const mgn_unary op = unary_of(u.shader);
+    if (op == MGN_UNARY_NONE || skipped_[ui]) continue;
+    const int in = u.input_buffers[0];
+    const int pi = producer_of[in];
+    if (pi < 0 || (size_t)pi >= ui || skipped_[pi] || !is_matmul(plan_.dispatches[pi].shader)) continue;
+    Fused& f = fused_[pi];
+    if (f.kind != kProNone || f.more[0] >= 0 || is_output[in] || readers[in].size() != 1) continue;
+    if (!weights_[plan_.dispatches[pi].input_buffers[1]]) continue;
+    if (plan_.dispatches[pi].epilogue.size() + f.post.size() >= 8) continue;
+    // every dispatch between the two must leave the unary's output buffer alone (it is a buffer
+    // of its own in a compiled plan, so this always holds; checked because it is cheap)
+    f.post.push_back(op);
+    f.out_buffer = u.output_buffer;
+    producer_of[u.output_buffer] = pi;
+    skipped_[ui] = 1;
   }
 }
 
@@ -646,12 +728,24 @@ void Session::run_dispatches() {
           const Dispatch& p = plan_.dispatches[f.producer];
           check(mgn_matmul_q_swiglu(ctx_, buffers_[p.input_buffers[0]], w, addend, buffers_[d.output_buffer], d.params[0]),
                 "mgn_matmul_q_swiglu");
+        } else if (!d.epilogue.empty() || !f.post.empty()) {
+          std::vector<mgn_unary> ops = d.epilogue;
+          ops.insert(ops.end(), f.post.begin(), f.post.end());
+          mgn_buf* dst = buffers_[f.out_buffer >= 0 ? f.out_buffer : d.output_buffer];
+          check(mgn_matmul_q_epilogue(ctx_, buffers_[d.input_buffers[0]], w, addend, dst, d.params[0], ops.data(), ops.size()),
+                "mgn_matmul_q_epilogue");
         } else {
           check(mgn_matmul_q(ctx_, buffers_[d.input_buffers[0]], w, addend, buffers_[d.output_buffer], d.params[0]),
                 "mgn_matmul_q");
         }
         break;
       }
+      case MGN_SHADER_RELU:
+      case MGN_SHADER_SIGMOID:
+      case MGN_SHADER_NEG:
+      case MGN_SHADER_SILU:
+        rc = launch_unary(ctx_->stream, (int)unary_of(d.shader), fin(0), out, d.params[0]);
+        break;
       case MGN_SHADER_ADD:
         rc = launch_add(ctx_->stream, fin(0), fin(1), out, d.params[0]);
         break;
@@ -719,6 +813,8 @@ void fill_info(const mgn::Dispatch& d, mgn_dispatch_info* out) {
   for (int i = 0; i < 3; i++) out->workgroups[i] = d.workgroups[i];
   for (int i = 0; i < 4; i++) out->params[i] = d.params[i];
   out->weight_format = (int32_t)d.weight_format;
+  out->epilogue = 0;
+  for (size_t i = 0; i < d.epilogue.size() && i < 8; i++) out->epilogue |= (uint32_t)d.epilogue[i] << (4 * i);
 }
 
 template <class F>
@@ -779,6 +875,9 @@ int32_t mgn_graph_rms_norm(mgn_graph* g, int32_t x, int32_t weight, float eps) {
   return graph_node(g, [&] { return g->g.rms_norm((mgn::NodeId)x, (mgn::NodeId)weight, eps); });
 }
 
+int32_t mgn_graph_unary(mgn_graph* g, int32_t kind, int32_t x) {
+  return graph_node(g, [&] { return g->g.unary((mgn_unary)kind, (mgn::NodeId)x); });
+}
 mgn_status mgn_graph_set_outputs(mgn_graph* g, const int32_t* ids, size_t count) {
   if (!g || (!ids && count)) return MGN_EINVAL;
   try {

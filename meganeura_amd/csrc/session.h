@@ -45,7 +45,7 @@ struct TensorType {
   }
 };
 
-enum class Op { Input, Parameter, MatMul, Add, SwiGLU, RmsNorm, FusedMatMulAdd, SwiGLUConcat, Nop, MatMulBT };
+enum class Op { Input, Parameter, MatMul, Add, SwiGLU, RmsNorm, FusedMatMulAdd, SwiGLUConcat, Nop, MatMulBT, Relu, Sigmoid, Neg, Silu };
 
 struct Node {
   NodeId id;
@@ -78,6 +78,7 @@ class Graph {
   NodeId add(NodeId a, NodeId b);
   NodeId swiglu(NodeId gate, NodeId up);
   NodeId rms_norm(NodeId x, NodeId weight, float eps);
+  NodeId unary(mgn_unary kind, NodeId x);  // relu / sigmoid / neg / silu
   void set_outputs(std::vector<NodeId> ids);
 
   const Node& node(NodeId id) const;
@@ -106,6 +107,7 @@ struct Dispatch {
   uint32_t params[4];
   WeightFormat weight_format = WeightFormat::F32;
   float eps = 0.0f;
+  std::vector<mgn_unary> epilogue;  // compile::Dispatch::epilogue (src/compile.rs:466), matmuls only
 };
 
 // compile::ExecutionPlan (src/compile.rs:494-528), the fields this path uses.
@@ -148,8 +150,10 @@ class Session {
   // are a single graph launch.  Results are identical; only launch overhead changes --
   // less host work per step, but measured slower on the GPU side for chains of tiny kernels.
   void set_graph_replay(bool on);
-  // Fold RmsNorm / SwiGLUConcat dispatches into the decode matmuls that consume them and
-  // serve sibling decode matmuls (same activations, e.g. q/k/v) with one launch (default on).  The plan keeps the reference's dispatch list; only the launches differ.
+  // Fold RmsNorm / SwiGLUConcat dispatches into the decode matmuls that consume them, serve
+  // sibling decode matmuls (same activations, e.g. q/k/v) with one launch and let a matmul's
+  // launch apply the unary dispatches that follow it (the compiler folds those into tiled
+  // matmul entries only, not into the M = 1 ones) (default on).  The plan keeps the reference's dispatch list; only the launches differ.
   void set_fusion(bool on);
   size_t num_launches();  // kernel launches one step makes with the current settings
   bool graph_active() const { return exec_ != nullptr; }
@@ -169,6 +173,8 @@ class Session {
     int kind = 0;          // kProNone / kProRmsNorm / kProSwiglu
     int producer = -1;     // the folded-in dispatch
     int more[2] = {-1, -1};  // sibling matmuls (same activations) served by this dispatch's launch
+    std::vector<mgn_unary> post;  // unary dispatches behind an M = 1 matmul, applied by its launch
+    int out_buffer = -1;          // ... whose last output buffer the launch then writes
   };
   std::vector<Fused> fused_;     // per dispatch (matmuls only)
   std::vector<char> skipped_;    // per dispatch: folded into its consumers
@@ -194,5 +200,6 @@ int launch_swiglu(ihipStream_t* s, const float* gate, const float* up, float* ou
 int launch_swiglu_concat(ihipStream_t* s, const float* in, float* out, size_t len, uint32_t half_n);
 int launch_rms_norm(ihipStream_t* s, const float* x, const float* weight, float* out, uint32_t rows, uint32_t cols,
                     float eps);
+int launch_unary(ihipStream_t* s, int kind, const float* in, float* out, size_t len);
 
 }  // namespace mgn

@@ -29,6 +29,18 @@ class ShaderEntry(IntEnum):
     RmsNorm = 7
     MatMulBT = 8
     MatMulGemvBT = 9
+    Relu = 10
+    Sigmoid = 11
+    Neg = 12
+    Silu = 13
+
+
+class EpilogueOp(IntEnum):
+    """compile::EpilogueOp (src/compile.rs:382-391), the unary ones."""
+    Relu = 1
+    Sigmoid = 2
+    Neg = 3
+    Silu = 4
 
 
 class WeightFormat(IntEnum):
@@ -43,9 +55,15 @@ class Dispatch:
         self.workgroups = list(info.workgroups)
         self.params = list(info.params)
         self.weight_format = WeightFormat(info.weight_format)
+        self.epilogue = []
+        e = info.epilogue
+        while e:
+            self.epilogue.append(EpilogueOp(e & 15))
+            e >>= 4
 
     def __repr__(self):
-        return f"Dispatch({self.shader.name}, wg={self.workgroups}, params={self.params}, {self.weight_format.name})"
+        return (f"Dispatch({self.shader.name}, wg={self.workgroups}, params={self.params}, {self.weight_format.name}, "
+                f"epilogue={[o.name for o in self.epilogue]})")
 
 
 def _shape2(shape):
@@ -99,6 +117,18 @@ class Graph:
 
     def rms_norm(self, x, weight, eps):
         return self._node(self.lib.mgn_graph_rms_norm(self.h, x, weight, eps))
+
+    def relu(self, x):
+        return self._node(self.lib.mgn_graph_unary(self.h, int(EpilogueOp.Relu), x))
+
+    def sigmoid(self, x):
+        return self._node(self.lib.mgn_graph_unary(self.h, int(EpilogueOp.Sigmoid), x))
+
+    def neg(self, x):
+        return self._node(self.lib.mgn_graph_unary(self.h, int(EpilogueOp.Neg), x))
+
+    def silu(self, x):
+        return self._node(self.lib.mgn_graph_unary(self.h, int(EpilogueOp.Silu), x))
 
     def set_outputs(self, ids):
         arr = (C.c_int32 * len(ids))(*ids)

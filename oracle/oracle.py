@@ -142,6 +142,24 @@ def matmul_packed(fmt, a, packed, n, d=None, tiled=False):
     return c
 
 
+def unary(kind, v):
+    """The reference's unary epilogue operations in f32 (src/codegen.rs:85-96):
+    relu max(v, 0); sigmoid 1 / (1 + exp(-v)); neg -v; silu v / (1 + exp(-v))."""
+    v = np.asarray(v, dtype=np.float32)
+    one = np.float32(1.0)
+    if kind == "relu":
+        return np.maximum(v, np.float32(0.0))
+    if kind == "neg":
+        return -v
+    with np.errstate(over="ignore"):
+        e = np.exp(-v).astype(np.float32)
+    if kind == "sigmoid":
+        return (one / (one + e)).astype(np.float32)
+    if kind == "silu":
+        return (v / (one + e)).astype(np.float32)
+    raise ValueError(kind)
+
+
 def num_threads():
     return int(lib().orc_num_threads())
 

@@ -389,6 +389,59 @@ def test_weight_file_round_trip(ctx, orc, fmt, tmp_path):
         assert e.value.status == capi.EINVAL, name
 
 
+UNARY = {"relu": capi.UNARY_RELU, "sigmoid": capi.UNARY_SIGMOID, "neg": capi.UNARY_NEG, "silu": capi.UNARY_SILU}
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("route", ["generic", "gemv_valu", "gemv_mfma", "gemm_mfma", "auto"])
+@pytest.mark.parametrize("m,k,n", [(1, 576, 192), (4, 14336, 70), (6, 1024, 300), (16, 4096, 2048)])
+def test_unary_epilogues(ctx, orc, fmt, route, m, k, n):
+    """C = f(A x W + D) in the matmul's own launch: every operation the reference folds into a
+    matmul (Relu, Sigmoid, Neg, Silu; compile.rs:915-1035), a chain of two, with and without the
+    residual, on every kernel family (K parts and split-K shapes included)."""
+    x = synth.normal(31 + m + k + n, m * k).reshape(m, k)
+    w = synth.normal(32 + m + k + n, k * n, 0.02).reshape(k, n)
+    d = synth.normal(33 + n, m * n).reshape(m, n)
+    deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
+    plain = orc.matmul_f32(x, deq)
+    plain_d = orc.matmul_f32(x, deq, d)
+    wt = ctx.weight(fmt, w)
+    a = ctx.upload(x)
+    db = ctx.upload(d)
+    c = ctx.buffer(m * n * 4)
+    ctx.set_route(ROUTES[route])
+    try:
+        for chain, with_d in ((("relu",), False), (("sigmoid",), True), (("neg",), False), (("silu",), True),
+                              (("relu", "neg"), True), ((), False)):
+            try:
+                ctx.matmul_q_epilogue(a, wt, c, m, [UNARY[o] for o in chain], db if with_d else None)
+            except capi.MgnError as e:
+                if route != "generic" and "does not support" in str(e):
+                    pytest.skip("shape outside this kernel's range")
+                raise
+            got = c.download(np.float32, m * n).reshape(m, n)
+            want = plain_d if with_d else plain
+            for o in chain:
+                want = orc.unary(o, want)
+            orc.assert_close(got, want, REL, ABS)
+    finally:
+        ctx.set_route(capi.ROUTE_AUTO)
+        a.free(); db.free(); c.free(); wt.free()
+
+
+def test_epilogue_arguments_are_checked(ctx):
+    wt = ctx.weight(Q4, synth.normal(970, 64 * 8, 0.02).reshape(64, 8))
+    a = ctx.buffer(4 * 64)
+    c = ctx.buffer(4 * 8)
+    with pytest.raises(capi.MgnError) as e:
+        ctx.matmul_q_epilogue(a, wt, c, 1, [capi.UNARY_RELU] * 9)
+    assert e.value.status == capi.EINVAL
+    with pytest.raises(capi.MgnError) as e:
+        ctx.matmul_q_epilogue(a, wt, c, 1, [7])
+    assert e.value.status == capi.EINVAL
+    a.free(); c.free(); wt.free()
+
+
 def test_matmul_loop_is_the_same_calls_in_a_row(ctx, orc):
     """mgn_matmul_q_loop enqueues call i on weights[i % count]: after five steps over two
     weights the output is what the first weight gives (bit for bit the single call's)."""

@@ -269,6 +269,47 @@ def test_decode_layer_fuses_norm_and_swiglu_into_the_matmuls(orc):
     sess.close()
 
 
+@pytest.mark.parametrize("quant", ["q4", "q8"])
+@pytest.mark.parametrize("m,k,n", [(6, 1024, 300), (1, 576, 192), (1, 576, 49152), (2, 1536, 64)])
+def test_unary_ops_behind_a_quantized_matmul(orc, quant, m, k, n):
+    """relu(x W + r) then -silu(.): for M > 1 the compiler folds both into the matmul dispatch
+    (compile.rs:915-1035); for M = 1 they stay dispatches of their own in the plan and the
+    matmul's launch applies them.  One launch either way, same numbers as launched one by one."""
+    fmt = Q4 if quant == "q4" else Q8
+    g = Graph()
+    x = g.input("x", [m, k])
+    r = g.input("r", [m, n])
+    w = (g.parameter_q4 if fmt == Q4 else g.parameter_q8)("w", [k, n])
+    h = g.neg(g.silu(g.relu(g.add(g.matmul(x, w), r))))
+    g.set_outputs([h])
+    sess = build_inference_session(g)
+    xv = synth.normal(700 + m + k, m * k).reshape(m, k)
+    rv = synth.normal(701 + n, m * n).reshape(m, n)
+    wv = synth.normal(702 + k + n, k * n, 0.02).reshape(k, n)
+    sess.set_input("x", xv)
+    sess.set_input("r", rv)
+    sess.set_parameter("w", wv)
+    plan = sess.plan()
+    if m == 1 and n % 4 == 0:
+        assert [d.shader for d in plan] == [ShaderEntry.MatMulGemvAdd, ShaderEntry.Relu, ShaderEntry.Silu, ShaderEntry.Neg]
+    else:
+        assert [d.shader for d in plan] == [ShaderEntry.FusedMatMulAdd] and len(plan[0].epilogue) == 3
+    assert sess.num_launches() == 1
+    sess.step()
+    sess.wait()
+    got = sess.read_output(m * n)
+    want = orc.matmul_f32(xv, orc.dequantize(fmt, orc.quantize(fmt, wv), k, n), rv)
+    for op in ("relu", "silu", "neg"):
+        want = orc.unary(op, want)
+    orc.assert_close(got, want.reshape(-1), 1e-3, 1e-4)
+    sess.set_fusion(False)
+    assert sess.num_launches() == len(plan)
+    sess.step()
+    sess.wait()
+    orc.assert_close(sess.read_output(m * n), want.reshape(-1), 1e-3, 1e-4)
+    sess.close()
+
+
 def test_norm_with_another_reader_is_not_folded():
     # the normed activations are also an output: the RmsNorm dispatch must run on its own
     hidden = 576

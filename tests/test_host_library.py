@@ -143,6 +143,58 @@ def test_matmul_that_is_an_output_is_not_fused():
     assert shaders == [ShaderEntry.MatMulGemv, ShaderEntry.Add]
 
 
+def test_unary_after_a_tiled_matmul_becomes_its_epilogue():
+    # src/compile.rs:3498-3512 (test_compile_fused), with the weight quantized: one MatMul dispatch
+    # that carries the Relu; a chain folds one by one; the M = 1 entries are left alone
+    # (compile.rs:971-983 lists the tiled entries only)
+    from meganeura_amd.graph import EpilogueOp
+    g = Graph()
+    x = g.input("x", [4, 800])
+    h = g.relu(g.matmul(x, g.parameter_q4("w", [800, 128])))
+    g.set_outputs([h])
+    (d,) = g.compile()
+    assert d.shader == ShaderEntry.MatMul and d.weight_format == WeightFormat.Q4 and d.epilogue == [EpilogueOp.Relu]
+
+    g = Graph()
+    x = g.input("x", [4, 800])
+    mm = g.add(g.matmul(x, g.parameter_q8("w", [800, 128])), g.input("r", [4, 128]))
+    g.set_outputs([g.neg(g.silu(mm))])
+    (d,) = g.compile()
+    assert d.shader == ShaderEntry.FusedMatMulAdd and d.epilogue == [EpilogueOp.Silu, EpilogueOp.Neg]
+
+    g = Graph()
+    x = g.input("x", [1, 800])
+    g.set_outputs([g.sigmoid(g.matmul(x, g.parameter_q4("w", [800, 128])))])
+    plan = g.compile()
+    assert [d.shader for d in plan] == [ShaderEntry.MatMulGemv, ShaderEntry.Sigmoid] and plan[0].epilogue == []
+    assert plan[1].workgroups == [1, 1, 1] and plan[1].params == [128, 0, 0, 0]
+
+
+def test_unary_is_not_folded_when_the_matmul_result_is_needed():
+    # a second reader, or the result being a graph output (the reference does not look at outputs
+    # there and would leave such an output unwritten)
+    for keep in ("reader", "output"):
+        g = Graph()
+        x = g.input("x", [4, 800])
+        mm = g.matmul(x, g.parameter_q4("w", [800, 128]))
+        r = g.relu(mm)
+        outs = [r, g.add(mm, g.input("r", [4, 128]))] if keep == "reader" else [r, mm]
+        g.set_outputs(outs)
+        plan = g.compile()
+        assert plan[0].shader == ShaderEntry.MatMul and plan[0].epilogue == []
+        assert ShaderEntry.Relu in [d.shader for d in plan]
+
+
+def test_all_unary_entries():
+    # src/compile.rs:3515-3531 (test_compile_all_unary_ops)
+    g = Graph()
+    x = g.input("x", [4, 8])
+    g.set_outputs([g.relu(x), g.sigmoid(x), g.neg(x), g.silu(x)])
+    plan = g.compile()
+    assert [d.shader for d in plan] == [ShaderEntry.Relu, ShaderEntry.Sigmoid, ShaderEntry.Neg, ShaderEntry.Silu]
+    assert all(d.params == [32, 0, 0, 0] and d.workgroups == [1, 1, 1] for d in plan)
+
+
 def test_swiglu_of_two_matmuls_becomes_one_wide_matmul():
     # src/optimize.rs:776-879; the concatenated weight keeps the Q4 dtype (848-854)
     g = Graph()
