@@ -236,10 +236,11 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 
 // blockDim.x = 64 * ksc * wnc.  Wave w: K split ks = w % ksc, quad slot wn = w / ksc.
 // The workgroup owns quads [blockIdx.x * wnc, +wnc); wave (ks, wn) takes quad wn and the
-// K steps [ks * STEPS, (ks+1) * STEPS) of 16 blocks each.  Every wave issues all of its
-// STEPS block loads up front and then runs straight-line code: with no branch around a
-// load the compiler's wait counts are exact, so step s starts as soon as its own block
-// has arrived while the later ones are still in flight.
+// K steps [ks * STEPS, (ks+1) * STEPS) of 16 blocks each (the last split's window is moved back
+// when the steps do not divide evenly).  A wave keeps two or three block loads ahead of the
+// step it works on and runs straight-line code: with no branch around a load the compiler's
+// wait counts are exact, so step s starts as soon as its own block has arrived while the
+// later ones are still in flight.
 // QPW > 1 (short K, many columns): a wave takes QPW consecutive quads, so that it still has
 // QPW * STEPS block loads to keep in flight and the workgroup count stays near the CU count.
 // PRO: what the activations go through on their way into LDS, in place of a kernel of its own:
@@ -253,8 +254,9 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 // KSPLIT (one weight, no fused prologue, QPW = 1, steps masked as without EXACT): the activations
 // of all of K would not fit in LDS (M = 4 with K > ~9000) or need more threads to prepare than a
 // workgroup has (K > 16384), so grid.y workgroups share a quad group, each with a part of K
-// that is a whole number of steps (the last part may reach past the end of K).  Their partial sums meet in a workspace; the last workgroup to arrive adds
-// them in part order (bit-identical from run to run) and writes C.
+// that is a whole number of steps (the last part may reach past the end of K).  Their partial
+// sums meet in a workspace; the last workgroup to arrive adds them in part order (bit-identical
+// from run to run) and writes C.
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // The leading scalar arguments are what a wave needs before it can issue its first loads;
