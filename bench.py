@@ -13,7 +13,7 @@ kernels run on, with a device synchronisation on both sides.
 
 Prints ONE JSON line on stdout.  `--sweep` additionally measures every
 BASELINE configuration (cache-cold and cache-warm) and writes the table to
-stderr and, if the directory exists, to gpurun_out/bench_sweep.json.
+stderr and, with `--sweep-out FILE`, as JSON to that file.
 """
 import argparse
 import json
@@ -255,6 +255,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
     ap.add_argument("--sweep", action="store_true", help="also measure every configuration (stderr)")
+    ap.add_argument("--sweep-out", default=None, help="with --sweep: also write the table to this JSON file")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--profile", action="store_true",
                     help="for rocprofv3 runs: only the timed cache-cold workload plus one 256 MiB device copy "
@@ -359,9 +360,8 @@ def main():
             row = quantizer_times(ctx, fmt)
             rows.append(row)
             print(json.dumps(row), file=sys.stderr, flush=True)
-        out_dir = os.path.join(ROOT, "gpurun_out")
-        if os.path.isdir(out_dir):
-            with open(os.path.join(out_dir, "bench_sweep.json"), "w") as f:
+        if args.sweep_out:
+            with open(args.sweep_out, "w") as f:
                 json.dump(rows, f, indent=1)
 
     ctx.close()
