@@ -144,7 +144,12 @@ __device__ __forceinline__ uint4 f16_operand(uint4 v) {
 // TPT = staging tasks per thread per chunk (one task = 8 consecutive k of one row).
 // The leading scalar arguments are the ones a wave needs before its first loads; as plain
 // scalars (not struct members) they can be handed over in registers at wave launch.
-template <int FMT, bool F32A, int TPT>
+// AM: how the activations arrive and sit in the tile.  0: fp16, 32 rows per tile.  1: f32 split
+// hi + lo into two fp16 rows of the tile (rows r and r + 16): 16 real rows per tile, one MFMA
+// pair per block -- the form for M <= 16.  2: f32 split hi + lo into two A operands that are
+// multiplied into the same accumulator: 32 real rows per tile at twice the MFMAs per block but
+// the same vector-ALU work, which is what the kernel is bound by -- the form for M > 16.
+template <int FMT, int AM, int TPT>
 __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__ a_arg, const void* __restrict__ meta_arg,
                                                         const void* __restrict__ quants_arg, uint32_t m_arg, uint32_t ksc_arg,
                                                         uint32_t wnc_arg, uint32_t nch_arg, uint32_t k_arg, uint32_t n_arg,
@@ -169,14 +174,17 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
 #ifdef MGN_TRACE
   g.trace = tail.trace;
 #endif
-  constexpr int ROWS = F32A ? 16 : 32;  // real rows per tile
-  constexpr int NI = F32A ? 8 : 16;     // result registers per lane
+  constexpr bool F32A = AM != 0;
+  constexpr bool CHAIN = AM == 2;
+  constexpr int ROWS = AM == 1 ? 16 : 32;  // real rows per tile
+  constexpr int NI = AM == 1 ? 8 : 16;     // result registers per lane
+  constexpr int HL = CHAIN ? 2 : 1;        // A operands per (block, k half): hi and lo
   constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;
   extern __shared__ uint4 lds4[];
   const WeightView& w = g.w;
   const uint32_t ksc = g.ksc, wnc = g.wnc;
   const uint32_t cb = 8 * ksc;                  // blocks per chunk
-  const uint32_t a_stride = cb * 2 * 64;        // uint4 per aimg buffer
+  const uint32_t a_stride = cb * 2 * HL * 64;   // uint4 per aimg buffer
   const uint32_t s_stride = (cb / 2) * 64;      // uint4 per simg buffer
   uint4* const aimg = lds4;
   uint4* const simg = lds4 + 2 * a_stride;
@@ -213,7 +221,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
     t_live[tt] = lb < cb;
     t_rowok[tt] = t_live[tt] && row0 + r < g.m;
     t_off[tt] = t_rowok[tt] ? (size_t)(row0 + r) * w.k + (size_t)lb * 32 + sub * 8 : (size_t)0;
-    t_slot[tt] = (lb * 2 + (sub >> 1)) * 64 + 32 * (sub & 1) + r;
+    t_slot[tt] = (lb * 2 + (sub >> 1)) * HL * 64 + 32 * (sub & 1) + r;
   }
   uint4 raw[TPT][F32A ? 2 : 1];
   auto load_a = [&](uint32_t chunk) {  // unconditional loads; dead tasks re-read element 0
@@ -289,13 +297,13 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
       }
       if (t_live[tt]) {
         ab[t_slot[tt]] = op_hi;
-        if constexpr (F32A) ab[t_slot[tt] + 16] = op_lo;
+        if constexpr (F32A) ab[t_slot[tt] + (CHAIN ? 64 : 16)] = op_lo;  // lo: an operand of its own, or rows 16-31
         if ((tid & 3) == 0) {
           uint32_t* sdst = sb + (lb >> 1) * 256 + (lb & 1);
-          const float mean = s_hi * 0.03125f;
+          const float mean = (CHAIN ? s_hi + s_lo : s_hi) * 0.03125f;
           const uint32_t mh = pack_rtz(mean, 0.0f);
           sdst[r * 4] = (mh & 0xFFFFu) | (pack_rtz(mean - half_lo(mh), 0.0f) << 16);
-          if constexpr (F32A) {
+          if constexpr (AM == 1) {
             const float mean_l = s_lo * 0.03125f;
             const uint32_t ml = pack_rtz(mean_l, 0.0f);
             sdst[(16 + r) * 4] = (ml & 0xFFFFu) | (pack_rtz(mean_l - half_lo(ml), 0.0f) << 16);
@@ -432,12 +440,16 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
         add0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add0) * kb);
         add1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add1) * kb);
       }
-      uint4 aop[2][2];
+      uint4 aop[2][2], lop[2][2];  // [block][k half]; lop: the low halves' operands (CHAIN)
 #pragma unroll
       for (int t = 0; t < 2; t++) {
-        const uint4* ap = ab + ((lb0 + t) * 2) * 64 + lane;
+        const uint4* ap = ab + ((lb0 + t) * 2) * HL * 64 + lane;
         aop[t][0] = ap[0];
-        aop[t][1] = ap[64];
+        aop[t][1] = ap[HL * 64];
+        if constexpr (CHAIN) {
+          lop[t][0] = ap[64];
+          lop[t][1] = ap[HL * 64 + 64];
+        }
       }
       const uint4 sop = sb[(lb0 >> 1) * 64 + lane];
       __builtin_amdgcn_sched_barrier(0);
@@ -447,6 +459,10 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
 #pragma unroll
         for (int i = 0; i < 16; i++) z[i] = 0.0f;
         z = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(aop[t][0]), bop[t][0], z, 0, 0, 0);
+        if constexpr (CHAIN) {
+          z = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(lop[t][0]), bop[t][0], z, 0, 0, 0);
+          z = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(lop[t][1]), bop[t][1], z, 0, 0, 0);
+        }
         dsum[s & 1][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(aop[t][1]), bop[t][1], z, 0, 0, 0);
       }
       acc2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as_half8(sop), as_half8(add0, add1, add0, add1), acc2, 0, 0, 0);
@@ -476,10 +492,10 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
 
   // ---- combine the two K halves of the workgroup ----
   // D layout: lane -> column lane%32; register i -> tile row 8*(i/4) + 4*(lane/32) + i%4.
-  // With f32 activations rows r and r+16 (registers i and i+8) are the hi and lo parts.
+  // In the 16-row f32 form rows r and r+16 (registers i and i+8) are the hi and lo parts.
   float outv[NI];
 #pragma unroll
-  for (int i = 0; i < NI; i++) outv[i] = F32A ? (acc[i] + acc2[i]) + (acc[i + 8] + acc2[i + 8]) : acc[i] + acc2[i];
+  for (int i = 0; i < NI; i++) outv[i] = AM == 1 ? (acc[i] + acc2[i]) + (acc[i + 8] + acc2[i + 8]) : acc[i] + acc2[i];
   if (ksc == 2) {
     if (ks == 1) {
 #pragma unroll
@@ -533,7 +549,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
       float sum[NI];
 #pragma unroll
       for (int i = 0; i < NI; i++) sum[i] = 0.0f;
-      constexpr int PB = F32A ? 4 : 2;  // parts in flight together
+      constexpr int PB = AM == 1 ? 4 : 2;  // parts in flight together
       for (uint32_t p0 = 0; p0 < g.parts; p0 += PB) {
         float tmp[PB][NI];
 #pragma unroll
@@ -569,13 +585,14 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
   MGN_GSTAMP(7);
 }
 
-size_t gemm_lds_bytes(int fmt, uint32_t ksc, uint32_t wnc) {
-  const uint32_t cb = 8 * ksc;
-  return std::max<size_t>((size_t)2 * (cb * 2 * 64 + (cb / 2) * 64) * 16 + (size_t)ksc * wnc * 32 * slice_stride(fmt),
+size_t gemm_lds_bytes(int fmt, uint32_t ksc, uint32_t wnc, bool chain) {
+  const uint32_t cb = 8 * ksc, hl = chain ? 2 : 1;
+  return std::max<size_t>((size_t)2 * (cb * 2 * hl * 64 + (cb / 2) * 64) * 16 + (size_t)ksc * wnc * 32 * slice_stride(fmt),
                           (size_t)wnc * 16 * 64 * 4);
 }
 
 struct GemmPlan {
+  uint32_t am;  // the kernel's AM: 0 fp16 activations, 1 f32 in 16-row tiles (M <= 16), 2 f32 in 32-row tiles
   uint32_t ksc, wnc, tpt, nch, parts, colgroups, grid_y;
   size_t lds, scratch_bytes;
 };
@@ -585,13 +602,14 @@ struct GemmPlan {
 // model is: rounds of workgroups over the CUs x bytes per workgroup.
 bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
   const bool f32a = !x.a_is_f16;
-  const uint32_t rows = f32a ? 16 : 32;
+  const uint32_t am = !f32a ? 0 : x.m > 16 ? 2 : 1;
+  const uint32_t rows = am == 1 ? 16 : 32;
   const uint32_t bpc = x.w.k / 32, n_tiles = (x.w.n + 31) / 32;
   const uint32_t grid_y = (x.m + rows - 1) / rows;
   if (x.m == 0 || bpc == 0 || grid_y > 65535) return false;
   const double wblock = x.w.fmt == MGN_FMT_Q4 ? 20.0 * 32 : 34.0 * 32;  // bytes per K block of a column tile
   const double ablock = rows * 32.0 * (f32a ? 4 : 2);
-  const uint32_t max_tasks = f32a ? 8 : 16;  // staging tasks per chunk per ksc, in units of 64 threads
+  const uint32_t max_tasks = am == 1 ? 8 : 16;  // staging tasks per chunk per ksc, in units of 64 threads
   double best = 0;
   GemmPlan bp{};
   for (uint32_t ksc = 1; ksc <= 2; ksc++) {
@@ -600,7 +618,7 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
     for (uint32_t wnc = 8 / ksc; wnc >= 1; wnc--) {
       const uint32_t tpt = (max_tasks + wnc - 1) / wnc;
       if (tpt > 4) break;
-      if (gemm_lds_bytes(x.w.fmt, ksc, wnc) > 160 * 1024) continue;
+      if (gemm_lds_bytes(x.w.fmt, ksc, wnc, am == 2) > 160 * 1024) continue;
       if (wnc > n_tiles && wnc * ksc > 8 && wnc > 4) continue;  // idle waves only help staging up to a point
       const uint32_t colgroups = (n_tiles + wnc - 1) / wnc;
       if (colgroups > 65535) continue;  // grid.y
@@ -644,7 +662,7 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
       bp.tpt = tpt <= 1 ? 1 : tpt <= 2 ? 2 : 4;
       bp.grid_y = grid_y;
       bp.scratch_bytes = bp.parts > 1 ? (size_t)bp.parts * grid_y * rows * x.w.n * 4 : 0;
-      if (tpt > 4 || gemm_lds_bytes(x.w.fmt, a, b) > 160 * 1024 || bp.colgroups > 65535 || bp.scratch_bytes > x.scratch_bytes ||
+      if (tpt > 4 || gemm_lds_bytes(x.w.fmt, a, b, am == 2) > 160 * 1024 || bp.colgroups > 65535 || bp.scratch_bytes > x.scratch_bytes ||
           (bp.parts > 1 && (uint64_t)grid_y * bp.colgroups > x.n_counters))
         return false;
       best = 1;
@@ -655,14 +673,15 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
             bp.parts, bp.nch, bp.tpt, bp.colgroups * bp.parts * bp.grid_y);
 #endif
   if (best == 0 || (uint64_t)bp.colgroups * bp.parts > 0x7fffffffu) return false;
-  bp.lds = gemm_lds_bytes(x.w.fmt, bp.ksc, bp.wnc);
+  bp.lds = gemm_lds_bytes(x.w.fmt, bp.ksc, bp.wnc, am == 2);
+  bp.am = am;
   *out = bp;
   return true;
 }
 
-template <int FMT, bool F32A, int TPT>
+template <int FMT, int AM, int TPT>
 int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
-  auto kern = gemm_mfma_kernel<FMT, F32A, TPT>;
+  auto kern = gemm_mfma_kernel<FMT, AM, TPT>;
   static std::atomic<uint64_t> big_lds_done{0};
   if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
   GemmTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.range_flag, p.grid_y, x.epilogue};
@@ -676,15 +695,20 @@ int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
   return 0;
 }
 
-template <int FMT, bool F32A>
-int launch_fa(ihipStream_t* s, const LaunchArgs& x) {
+template <int FMT, int AM>
+int launch_am(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
+  switch (p.tpt) {
+    case 1: return launch_tpt<FMT, AM, 1>(s, x, p);
+    case 2: return launch_tpt<FMT, AM, 2>(s, x, p);
+    default: return launch_tpt<FMT, AM, 4>(s, x, p);
+  }
+}
+
+template <int FMT>
+int launch_fmt(ihipStream_t* s, const LaunchArgs& x) {
   GemmPlan p;
   if (!plan_gemm(x, &p)) return (int)hipErrorInvalidValue;
-  switch (p.tpt) {
-    case 1: return launch_tpt<FMT, F32A, 1>(s, x, p);
-    case 2: return launch_tpt<FMT, F32A, 2>(s, x, p);
-    default: return launch_tpt<FMT, F32A, 4>(s, x, p);
-  }
+  return p.am == 0 ? launch_am<FMT, 0>(s, x, p) : p.am == 1 ? launch_am<FMT, 1>(s, x, p) : launch_am<FMT, 2>(s, x, p);
 }
 
 }  // namespace
@@ -709,8 +733,7 @@ bool describe_gemm_mfma(const LaunchArgs& x, mgn_plan_info* out) {
 }
 
 int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& x) {
-  if (x.w.fmt == MGN_FMT_Q4) return x.a_is_f16 ? launch_fa<MGN_FMT_Q4, false>(s, x) : launch_fa<MGN_FMT_Q4, true>(s, x);
-  return x.a_is_f16 ? launch_fa<MGN_FMT_Q8, false>(s, x) : launch_fa<MGN_FMT_Q8, true>(s, x);
+  return x.w.fmt == MGN_FMT_Q4 ? launch_fmt<MGN_FMT_Q4>(s, x) : launch_fmt<MGN_FMT_Q8>(s, x);
 }
 
 }  // namespace mgn

@@ -54,7 +54,7 @@ def check_gemv(p, fmt, m, k, n):
 
 
 def check_gemm(p, fmt, m, k, n, f16):
-    rows = 32 if f16 else 16
+    rows = 32 if f16 or m > 16 else 16  # f32 rows travel as fp16 pairs: 16 per tile up to M = 16, 32 beyond
     bpc = k // 32
     assert p.grid[2] == ceil_div(m, rows)
     assert p.threads == 64 * p.k_splits * p.waves_n <= 512
