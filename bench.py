@@ -52,6 +52,9 @@ WORKLOADS = {
     "c2_q4_down_1536x576_add": (Q4, 1, 1536, 576, True, False, 2),
     "c4_q4_prefill_up_512x1024x3072": (Q4, 512, 1024, 3072, False, True, 4),
     "c4_q4_prefill_down_512x3072x1024": (Q4, 512, 3072, 1024, False, True, 4),
+    # C4 with the f32 activations the reference's Session hands to a matmul (BASELINE names fp16)
+    "c4_f32a_q4_prefill_up_512x1024x3072": (Q4, 512, 1024, 3072, False, False, 4),
+    "c4_f32a_q4_prefill_down_512x3072x1024": (Q4, 512, 3072, 1024, False, False, 4),
     # not a BASELINE configuration: four times the headline weight, to separate the kernel's
     # streaming rate from the fixed cost of a launch (sweep only)
     "scale_q4_m1_8192x28672": (Q4, 1, 8192, 28672, False, False, 5),
@@ -61,11 +64,11 @@ HEADLINE = "c5_q4_m1_4096x14336"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
 # same counters read for a 256 MiB device copy (one summary per workload under profiles/).
 MEASURED_TRAFFIC_BYTES = {
-    "c5_q4_m1_4096x14336": 37.01e6,
+    "c5_q4_m1_4096x14336": 37.02e6,
     "c5_q8_m1_4096x14336": 63.52e6,
     "c5_q4_m4_14336x4096": 39.3e6,
-    "c5_q4_m16_4096x14336": 48.4e6,
-    "c4_q4_prefill_up_512x1024x3072": 18.8e6,
+    "c5_q4_m16_4096x14336": 48.3e6,
+    "c4_q4_prefill_up_512x1024x3072": 18.9e6,
 }
 
 
