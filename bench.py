@@ -65,7 +65,7 @@ HEADLINE = "c5_q4_m1_4096x14336"
 # same counters read for a 256 MiB device copy (one summary per workload under profiles/).
 MEASURED_TRAFFIC_BYTES = {
     "c5_q4_m1_4096x14336": 37.02e6,
-    "c5_q8_m1_4096x14336": 63.52e6,
+    "c5_q8_m1_4096x14336": 63.59e6,
     "c5_q4_m4_14336x4096": 39.3e6,
     "c5_q4_m16_4096x14336": 48.3e6,
     "c4_q4_prefill_up_512x1024x3072": 18.9e6,
