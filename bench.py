@@ -223,7 +223,7 @@ def quantizer_times(ctx, fmt=Q4, k=4096, n=14336):
             "device_GBs_f32_in": w.nbytes / (dev_ms * 1e-3) / 1e9, "device_bytes_equal_host": same}
 
 
-def cpu_baseline(wl, budget_s=20.0):
+def cpu_baseline(wl, cpu_seconds=20.0):
     """The reference's tiled dequant-on-load algorithm restated for the CPU
     (oracle/mgn_oracle.c: orc_matmul_q_tiled), one OpenMP task per workgroup, on
     this box's host cores.  Checker infrastructure used as the timing baseline
@@ -235,7 +235,8 @@ def cpu_baseline(wl, budget_s=20.0):
     t0 = time.perf_counter()
     out = oracle.matmul_packed(wl.fmt, x, packed_ref, wl.n, wl.d_host, tiled=True)
     first = time.perf_counter() - t0
-    reps = int(max(1, min(10, budget_s / max(first, 1e-3) - 1)))
+    # sample size: about `cpu_seconds` of CPU work (threads x wall clock), never fewer than 2 calls
+    reps = int(max(1, min(500, cpu_seconds / oracle.num_threads() / max(first, 1e-4) - 1)))
     t0 = time.perf_counter()
     for _ in range(reps):
         oracle.matmul_packed(wl.fmt, x, packed_ref, wl.n, wl.d_host, tiled=True)
@@ -246,8 +247,8 @@ def cpu_baseline(wl, budget_s=20.0):
         "cores": oracle.num_threads(),
         "kind": "port",
         "ms_per_call": per * 1e3,
-        "sample": f"{reps + 1} full calls of {wl.name} (64x64x32-tiled per-element dequant, "
-                  "the reference shader's algorithm, OpenMP over workgroups)",
+        "sample": f"{reps + 1} full calls of {wl.name}, about {(reps + 1) * per * oracle.num_threads():.0f} s of CPU work "
+                  "(64x64x32-tiled per-element dequant, the reference shader's algorithm, OpenMP over workgroups)",
     }
 
 
