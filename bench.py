@@ -223,6 +223,23 @@ def quantizer_times(ctx, fmt=Q4, k=4096, n=14336):
             "device_GBs_f32_in": w.nbytes / (dev_ms * 1e-3) / 1e9, "device_bytes_equal_host": same}
 
 
+def copy_ceiling(ctx, nbytes=256 << 20, reps=20):
+    """What a plain device-to-device copy moves on this box (bytes read + bytes written per
+    second): an achievable figure to set beside the published HBM peak."""
+    src, dst = ctx.buffer(nbytes), ctx.buffer(nbytes)
+    for _ in range(3):
+        ctx.copy(dst, src, nbytes)
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(reps):
+        ctx.copy(dst, src, nbytes)
+    ms = ctx.timer_stop() / reps
+    ctx.sync()
+    src.free()
+    dst.free()
+    return 2.0 * nbytes / (ms * 1e-3) / 1e9
+
+
 def cpu_baseline(wl, cpu_seconds=20.0):
     """The reference's tiled dequant-on-load algorithm restated for the CPU
     (oracle/mgn_oracle.c: orc_matmul_q_tiled), one OpenMP task per workgroup, on
@@ -301,11 +318,12 @@ def main():
         oracle.assert_close(cpu_out, want, 1e-3, 1e-4)
 
     # cache-warm figure for the same shape (one weight, reused every step)
-    warm_ms = None
+    warm_ms = copy_gbs = None
     if not args.profile:
         warm = Workload(ctx, args.workload, 0)
         warm_ms = warm.run(args.steps, args.warmup)
         warm.free()
+        copy_gbs = copy_ceiling(ctx)
 
     if is_gemm:
         roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -339,6 +357,9 @@ def main():
         "cache_warm": None if warm_ms is None else
         {"us_per_call": warm_ms * 1e3, "GB/s": wl.bytes / (warm_ms * 1e-3) / 1e9},
         "pct_of_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
+        "copy_ceiling": None if copy_gbs is None else
+        {"GB/s": copy_gbs, "what": "256 MiB device-to-device copy, bytes read + written per second",
+         "pct_of_it": 100.0 * gbs / copy_gbs},
     }
     wl.free()
 
