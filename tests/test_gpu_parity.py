@@ -185,6 +185,42 @@ def test_larger_m(ctx, orc, fmt, m, k, n):
         orc.assert_close(got, orc.matmul_f32(x16, deq), REL, ABS)
 
 
+def _random_shapes(count, seed=0x4D474E51):
+    """Seeded shapes across every route's territory: M from the GEMV sizes to several row tiles,
+    K any multiple of 32 up to past the K-part thresholds, N ragged more often than not."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        m = int(rng.choice([1, 1, 1, 2, 2, 3, 4, 4, 5, 8, 15, 16, 17, 31, 33, 70]))
+        k = 32 * int(rng.choice([rng.integers(1, 20), rng.integers(20, 160), rng.integers(160, 640)]))
+        budget = 60_000_000 // (m * k)  # keeps the oracle's triple loop short
+        n = int(min(rng.choice([rng.integers(1, 40), rng.integers(40, 700), rng.integers(700, 9000)]), max(1, budget)))
+        out.append((m, k, n))
+    return out
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m,k,n", _random_shapes(40))
+def test_random_shapes_on_the_automatic_route(ctx, orc, fmt, m, k, n):
+    """What a caller gets without choosing a kernel, on shapes nobody picked by hand; the
+    generic kernel on the same inputs is the second opinion.  With and without a residual,
+    and from fp16 activations."""
+    x = synth.normal(31 + m + k + n, m * k).reshape(m, k)
+    w = synth.normal(32 + m + k + n, k * n, 0.02).reshape(k, n)
+    d = synth.normal(33 + n, m * n).reshape(m, n)
+    deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
+    weight = ctx.weight(fmt, w)
+    try:
+        want = orc.matmul_f32(x, deq)
+        orc.assert_close(run_matmul(ctx, fmt, x, weight), want, REL, ABS)
+        orc.assert_close(run_matmul(ctx, fmt, x, weight, ROUTES["generic"]), want, REL, ABS)
+        orc.assert_close(run_matmul(ctx, fmt, x, weight, d=d), orc.matmul_f32(x, deq, d), REL, ABS)
+        x16 = x.astype(np.float16).astype(np.float32)
+        orc.assert_close(run_matmul(ctx, fmt, x, weight, f16=True), orc.matmul_f32(x16, deq), REL, ABS)
+    finally:
+        weight.free()
+
+
 def test_reference_q4_matmul_correctness_inputs(ctx, orc):
     # tests/gpu_smoke.rs:2681-2771 (m=6, k=1024, n=2048; the reference's own bar is abs 0.1)
     a, b = ref_test_inputs_q4_matmul()
