@@ -180,6 +180,13 @@ typedef enum mgn_unary {
 } mgn_unary;
 mgn_status mgn_matmul_q_epilogue(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d,
                                  mgn_buf* c, uint32_t m, const mgn_unary* ops, size_t n_ops);
+/* C[M,N] = A^T x W (+ D): the MatMulAT / FusedMatMulATAdd dispatches with a quantized B
+ * (src/compile.rs:1423-1445, 1526-1549; codegen.rs gen_matmul_at).  a_t holds A as [K, M]
+ * row-major, M = m.  The activations are transposed into a staging area of the context
+ * (allocated or grown on the first call that needs it, kept afterwards) and the call then
+ * is mgn_matmul_q_epilogue's: ops / n_ops as there, NULL / 0 for none.  c must not alias a_t. */
+mgn_status mgn_matmul_q_at(mgn_ctx* ctx, const mgn_buf* a_t, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
+                           uint32_t m, const mgn_unary* ops, size_t n_ops);
 
 /* `steps` such matmuls enqueued back to back, call i on weights[i % count]: the step loop of
  * a compiled host (examples/matmul_throughput.rs:114-127) without an interpreter between the

@@ -39,7 +39,10 @@ typedef enum mgn_shader {
   MGN_SHADER_RELU = 10,          /* the unary entries fuse_epilogues can fold into a matmul */
   MGN_SHADER_SIGMOID = 11,
   MGN_SHADER_NEG = 12,
-  MGN_SHADER_SILU = 13
+  MGN_SHADER_SILU = 13,
+  MGN_SHADER_MATMUL_AT = 14,           /* ShaderEntry::MatMulAT: C = A^T x B, A stored [K, M] (src/compile.rs:1423-1445) */
+  MGN_SHADER_FUSED_MATMUL_AT_ADD = 15, /* ShaderEntry::FusedMatMulATAdd: A^T x B + D (src/compile.rs:1526-1549) */
+  MGN_SHADER_FUSED_MATMUL_BT_ADD = 16  /* ShaderEntry::FusedMatMulBTAdd: A x B^T + D (src/compile.rs:1551-1574) */
 } mgn_shader;
 
 /* compile::Dispatch (src/compile.rs:435-488), the fields this path uses.
@@ -47,7 +50,7 @@ typedef enum mgn_shader {
 typedef struct mgn_dispatch_info {
   int32_t shader;          /* mgn_shader */
   uint32_t workgroups[3];  /* the grid the reference would launch */
-  uint32_t params[4];      /* [m, k, n, 0] for matmuls, [m, n, k, 0] for the BT forms, [len, 0, 0, 0] for unary entries */
+  uint32_t params[4];      /* [m, k, n, 0] for matmuls, [m, n, k, 0] for the AT and BT forms, [len, 0, 0, 0] for unary entries */
   int32_t weight_format;
   uint32_t epilogue;       /* Dispatch::epilogue of a matmul: mgn_unary codes, four bits each, first in the low bits */
 } mgn_dispatch_info;
@@ -66,6 +69,9 @@ int32_t mgn_graph_matmul(mgn_graph* g, int32_t a, int32_t b);
 /* Graph::matmul_bt (src/graph.rs:809-817): a[M,K], b[N,K] -> [M,N].  With a quantized b the
  * parameter is blocked along K (see mgn_weight_create_nk). */
 int32_t mgn_graph_matmul_bt(mgn_graph* g, int32_t a, int32_t b);
+/* Graph::matmul_at (src/graph.rs:798-806): a[K,M], b[K,N] -> [M,N] = a^T x b; what the ONNX / NNEF
+ * loaders emit for a Gemm with a transposed first operand (src/load/onnx.rs:607). */
+int32_t mgn_graph_matmul_at(mgn_graph* g, int32_t a, int32_t b);
 int32_t mgn_graph_add(mgn_graph* g, int32_t a, int32_t b);
 int32_t mgn_graph_swiglu(mgn_graph* g, int32_t gate, int32_t up);
 int32_t mgn_graph_rms_norm(mgn_graph* g, int32_t x, int32_t weight, float eps);

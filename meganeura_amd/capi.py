@@ -22,12 +22,12 @@ HIP_SYMBOLS = [
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_weight_save", "mgn_weight_load", "mgn_matmul_q",
-    "mgn_matmul_q_f16a", "mgn_matmul_q_epilogue", "mgn_matmul_q_loop", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
+    "mgn_matmul_q_f16a", "mgn_matmul_q_epilogue", "mgn_matmul_q_at", "mgn_matmul_q_loop", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
     "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [
     "mgn_graph_new", "mgn_graph_free", "mgn_graph_last_error", "mgn_graph_input", "mgn_graph_parameter",
-    "mgn_graph_parameter_q4", "mgn_graph_parameter_q8", "mgn_graph_matmul", "mgn_graph_matmul_bt", "mgn_graph_add",
+    "mgn_graph_parameter_q4", "mgn_graph_parameter_q8", "mgn_graph_matmul", "mgn_graph_matmul_bt", "mgn_graph_matmul_at", "mgn_graph_add",
     "mgn_graph_swiglu", "mgn_graph_rms_norm", "mgn_graph_unary", "mgn_graph_set_outputs", "mgn_graph_compile",
     "mgn_build_inference_session", "mgn_session_free", "mgn_session_last_error",
     "mgn_session_num_dispatches", "mgn_session_dispatch_info", "mgn_session_set_parameter",
@@ -105,6 +105,7 @@ def load():
         "mgn_matmul_q": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_f16a": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_epilogue": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32, vp, C.c_size_t]),
+        "mgn_matmul_q_at": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32, vp, C.c_size_t]),
         "mgn_matmul_q_plan": (C.c_int, [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.c_int, vp]),
         "mgn_matmul_q_loop": (C.c_int, [vp, vp, C.c_int, vp, C.c_size_t, vp, vp, C.c_uint32, C.c_uint32]),
         "mgn_matmul_q_rms_norm": (C.c_int, [vp, vp, vp, C.c_float, vp, vp, vp, C.c_uint32]),
@@ -124,6 +125,7 @@ def load():
         "mgn_graph_parameter_q8": (C.c_int32, [vp, C.c_char_p, sz, sz]),
         "mgn_graph_matmul": (C.c_int32, [vp, C.c_int32, C.c_int32]),
         "mgn_graph_matmul_bt": (C.c_int32, [vp, C.c_int32, C.c_int32]),
+        "mgn_graph_matmul_at": (C.c_int32, [vp, C.c_int32, C.c_int32]),
         "mgn_graph_add": (C.c_int32, [vp, C.c_int32, C.c_int32]),
         "mgn_graph_swiglu": (C.c_int32, [vp, C.c_int32, C.c_int32]),
         "mgn_graph_rms_norm": (C.c_int32, [vp, C.c_int32, C.c_int32, C.c_float]),
@@ -318,6 +320,12 @@ class Context:
         """C = f_n(...f_1(A x W + D)) with ops a sequence of UNARY_* codes."""
         arr = (C.c_int * max(1, len(ops)))(*ops)
         self.check(self.lib.mgn_matmul_q_epilogue(self.h, a.h, w.h, d.h if d is not None else None, c.h, m, arr, len(ops)))
+
+    def matmul_q_at(self, a_t, w, c, m, d=None, ops=()):
+        """C = f(A^T x W + D) with A stored [K, M]; ops as in matmul_q_epilogue."""
+        arr = (C.c_int * max(1, len(ops)))(*ops)
+        self.check(self.lib.mgn_matmul_q_at(self.h, a_t.h, w.h, d.h if d is not None else None, c.h, m,
+                                            arr if len(ops) else None, len(ops)))
 
     def matmul_q_loop(self, a, weights, c, m, steps, d=None, a_is_f16=False):
         """`steps` matmuls enqueued back to back from C, call i on weights[i % len(weights)]."""

@@ -208,6 +208,24 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__
 }
 
 // relu / sigmoid / neg / silu as dispatches of their own (src/codegen.rs:85-96 for the formulas)
+// in[rows][cols] -> out[cols][rows], 32 x 32 tiles through LDS so that both sides move whole
+// 128-byte rows.  Used for the A^T forms of the matmul (rows = K, cols = M).
+__global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict__ in, float* __restrict__ out, uint32_t rows,
+                                                        uint32_t cols) {
+  __shared__ float tile[32][33];
+  const uint32_t tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const uint32_t r0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+  for (uint32_t j = ty; j < 32; j += 8) {
+    const uint32_t r = r0 + j, c = c0 + tx;
+    if (r < rows && c < cols) tile[j][tx] = in[(size_t)r * cols + c];
+  }
+  __syncthreads();
+  for (uint32_t j = ty; j < 32; j += 8) {
+    const uint32_t c = c0 + j, r = r0 + tx;
+    if (r < rows && c < cols) out[(size_t)c * rows + r] = tile[tx][j];
+  }
+}
+
 __global__ __launch_bounds__(256) void unary_kernel(uint32_t kind, const float* __restrict__ in, float* __restrict__ out,
                                                     size_t len) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -216,6 +234,13 @@ __global__ __launch_bounds__(256) void unary_kernel(uint32_t kind, const float* 
 
 }  // namespace
 
+int launch_transpose(ihipStream_t* s, const float* in, float* out, uint32_t rows, uint32_t cols) {
+  if (rows == 0 || cols == 0) return 0;
+  if ((cols + 31) / 32 > 65535) return (int)hipErrorInvalidValue;  // grid.y
+  hipLaunchKernelGGL(transpose_kernel, dim3((rows + 31) / 32, (cols + 31) / 32), dim3(256), 0, s, in, out, rows, cols);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
 int launch_unary(ihipStream_t* s, int kind, const float* in, float* out, size_t len) {
   hipLaunchKernelGGL(unary_kernel, dim3((unsigned)((len + 255) / 256)), dim3(256), 0, s, (uint32_t)kind, in, out, len);
   MGN_HIP_LAUNCH_CHECK();

@@ -167,6 +167,7 @@ void mgn_ctx_destroy(mgn_ctx* ctx) {
     (void)hipStreamDestroy(ctx->stream);
   }
   if (ctx->scratch) (void)hipFree(ctx->scratch);
+  if (ctx->at_stage) (void)hipFree(ctx->at_stage);
   if (ctx->range_flag_host) (void)hipHostFree(ctx->range_flag_host);
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
   if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
@@ -621,6 +622,40 @@ int mgn_matmul_q_can_fuse(mgn_ctx* ctx, const mgn_weight* w, uint32_t m) {
   mgn::LaunchArgs x{view_of(w), nullptr, nullptr, nullptr, m, false, ctx->num_cus};
   x.pro_kind = mgn::kProRmsNorm;
   return (ctx->route == MGN_ROUTE_AUTO || ctx->route == MGN_ROUTE_GEMV_MFMA) && mgn::gemv_mfma_supported(x) ? 1 : 0;
+}
+
+mgn_status mgn_matmul_q_at(mgn_ctx* ctx, const mgn_buf* a_t, const mgn_weight* w, const mgn_buf* d, mgn_buf* c, uint32_t m,
+                           const mgn_unary* ops, size_t n_ops) {
+  if (!ctx || !a_t || !w || !c) return fail(ctx, MGN_EINVAL, "null argument");
+  if (n_ops > 8 || (n_ops > 0 && !ops)) return fail(ctx, MGN_EINVAL, "an epilogue has at most 8 operations");
+  uint32_t packed = 0;
+  for (size_t i = 0; i < n_ops; i++) {
+    if (ops[i] < MGN_UNARY_RELU || ops[i] > MGN_UNARY_SILU) return fail(ctx, MGN_EINVAL, "unknown unary operation in the epilogue");
+    packed |= (uint32_t)ops[i] << (4 * i);
+  }
+  if (m == 0) return MGN_OK;
+  const size_t k = w->rows, need = (size_t)m * k * sizeof(float);
+  if (a_t->bytes < need) return fail(ctx, MGN_EINVAL, "A^T is smaller than K rows of m floats");
+  if (c->ptr == a_t->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
+  if (((size_t)m + 31) / 32 > 65535) return fail(ctx, MGN_EINVAL, "m is too large for the transposed form");
+  if (ctx->at_stage_bytes < need) {
+    // earlier launches may still read the old area
+    MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->at_stage) (void)hipFree(ctx->at_stage);
+    ctx->at_stage = nullptr;
+    ctx->at_stage_bytes = 0;
+    const size_t grown = align_up(need, (size_t)1 << 20);
+    hipError_t e = hipMalloc(&ctx->at_stage, grown);
+    if (e != hipSuccess) {
+      ctx->at_stage = nullptr;
+      return e == hipErrorOutOfMemory ? fail(ctx, MGN_ENOMEM, "out of device memory") : hip_fail(ctx, "hipMalloc", e);
+    }
+    ctx->at_stage_bytes = grown;
+  }
+  const int rc = mgn::launch_transpose(ctx->stream, (const float*)a_t->ptr, (float*)ctx->at_stage, (uint32_t)k, m);
+  if (rc != 0) return hip_fail(ctx, "transpose launch", (hipError_t)rc);
+  const mgn_buf staged{ctx->at_stage, need};
+  return matmul_impl(ctx, &staged, false, w, d, c, m, mgn::kProNone, nullptr, 0.0f, packed);
 }
 
 mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,

@@ -81,6 +81,8 @@ int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* m
 int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev);  // out: max |scale|, max |min| bits
 int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, uint32_t n, void* meta,
                     void* quants);
+// in[rows][cols] -> out[cols][rows] (f32); cols at most 65535 * 32
+int launch_transpose(ihipStream_t* s, const float* in, float* out, uint32_t rows, uint32_t cols);
 int launch_matmul_generic(ihipStream_t* s, const LaunchArgs& a);
 bool gemv_supported(const LaunchArgs& a);
 int launch_matmul_gemv(ihipStream_t* s, const LaunchArgs& a);
@@ -110,6 +112,8 @@ struct mgn_ctx {
   uint32_t n_counters = 0;
   uint32_t* range_flag_host = nullptr;  // pinned, mapped: written by kernels, read at sync points
   uint32_t* range_flag_dev = nullptr;   // the same word as the device sees it
+  void* at_stage = nullptr;             // transposed activations of the A^T matmul forms, grown on demand
+  size_t at_stage_bytes = 0;
   std::string err;
 };
 

@@ -63,6 +63,15 @@ NodeId Graph::matmul_bt(NodeId a, NodeId b) {
   return add_raw_node(Op::MatMulBT, {a, b}, TensorType{{as[0], bs[0]}, DType::F32});
 }
 
+// src/graph.rs:798-806
+NodeId Graph::matmul_at(NodeId a, NodeId b) {
+  const auto& as = node(a).ty.shape;
+  const auto& bs = node(b).ty.shape;
+  if (as.size() != 2 || bs.size() != 2) throw GraphError("matmul_at requires 2D tensors");
+  if (as[0] != bs[0]) throw GraphError("MatMulAT: K dimensions must match");
+  return add_raw_node(Op::MatMulAT, {a, b}, TensorType{{as[1], bs[1]}, DType::F32});
+}
+
 // src/graph.rs:821-827
 NodeId Graph::add(NodeId a, NodeId b) {
   if (node(a).ty.shape != node(b).ty.shape) throw GraphError("add requires matching shapes");
@@ -108,19 +117,20 @@ static size_t use_count(const Graph& g, NodeId id) {
 }
 
 // src/optimize.rs:724-767: Add(MatMul(a,b), d) -> FusedMatMulAdd(a,b,d) when the
-// matmul feeds only this Add and is not itself a graph output.
+// matmul feeds only this Add and is not itself a graph output; the same for the AT and BT forms.
 static bool apply_matmul_add_fusions(Graph& g) {
   bool changed = false;
   const size_t count = g.nodes().size();
+  auto plain_matmul = [](Op op) { return op == Op::MatMul || op == Op::MatMulAT || op == Op::MatMulBT; };
   for (size_t id = 0; id < count; id++) {
     const Node& nd = g.nodes()[id];
     if (nd.op != Op::Add) continue;
     const NodeId lhs = nd.inputs[0], rhs = nd.inputs[1];
     NodeId mm, addend;
-    if (g.node(lhs).op == Op::MatMul) {
+    if (plain_matmul(g.node(lhs).op)) {
       mm = lhs;
       addend = rhs;
-    } else if (g.node(rhs).op == Op::MatMul) {
+    } else if (plain_matmul(g.node(rhs).op)) {
       mm = rhs;
       addend = lhs;
     } else {
@@ -128,7 +138,8 @@ static bool apply_matmul_add_fusions(Graph& g) {
     }
     if (use_count(g, mm) != 1 || g.is_output(mm)) continue;
     const NodeId a = g.node(mm).inputs[0], b = g.node(mm).inputs[1];
-    g.nodes_mut()[id].op = Op::FusedMatMulAdd;
+    const Op mm_op = g.node(mm).op;
+    g.nodes_mut()[id].op = mm_op == Op::MatMul ? Op::FusedMatMulAdd : mm_op == Op::MatMulAT ? Op::FusedMatMulATAdd : Op::FusedMatMulBTAdd;
     g.nodes_mut()[id].inputs = {a, b, addend};
     g.nodes_mut()[mm].op = Op::Nop;
     changed = true;
@@ -251,7 +262,8 @@ static void fuse_epilogues(ExecutionPlan& plan) {
     if (pit == producer.end()) continue;
     Dispatch& prod = ds[pit->second];
     const bool tiled = prod.shader == MGN_SHADER_MATMUL || prod.shader == MGN_SHADER_FUSED_MATMUL_ADD ||
-                       prod.shader == MGN_SHADER_MATMUL_BT;
+                       prod.shader == MGN_SHADER_MATMUL_BT || prod.shader == MGN_SHADER_MATMUL_AT ||
+                       prod.shader == MGN_SHADER_FUSED_MATMUL_AT_ADD || prod.shader == MGN_SHADER_FUSED_MATMUL_BT_ADD;
     if (!tiled || read_count[primary] != 1 || prod.epilogue.size() >= 8) continue;
     if (std::find(plan.output_buffers.begin(), plan.output_buffers.end(), primary) != plan.output_buffers.end()) continue;
     prod.epilogue.push_back(op);
@@ -285,15 +297,15 @@ ExecutionPlan compile(const Graph& g) {
   }
   // a quantized parameter read by matmul_bt is blocked along its second dimension
   for (const Node& nd : g.nodes()) {
-    if (nd.op != Op::MatMul && nd.op != Op::MatMulBT && nd.op != Op::FusedMatMulAdd) continue;
+    if (nd.op != Op::MatMulBT && nd.op != Op::FusedMatMulBTAdd) continue;
     auto it = node_buf.find(nd.inputs[1]);
     if (it == node_buf.end()) continue;
     auto wb = plan.weight_buffers.find(it->second);
     if (wb == plan.weight_buffers.end()) continue;
-    if (nd.op == Op::MatMulBT) wb->second.nk = true;
+    wb->second.nk = true;
   }
   for (const Node& nd : g.nodes()) {
-    if (nd.op != Op::MatMul && nd.op != Op::FusedMatMulAdd) continue;
+    if (nd.op != Op::MatMul && nd.op != Op::FusedMatMulAdd && nd.op != Op::MatMulAT && nd.op != Op::FusedMatMulATAdd) continue;
     auto it = node_buf.find(nd.inputs[1]);
     if (it == node_buf.end()) continue;
     auto wb = plan.weight_buffers.find(it->second);
@@ -337,6 +349,34 @@ ExecutionPlan compile(const Graph& g) {
         d.input_buffers = {buf_of(nd.inputs[0]), buf_of(nd.inputs[1])};
         if (fused) d.input_buffers.push_back(buf_of(nd.inputs[2]));
         d.params[0] = m, d.params[1] = k, d.params[2] = n, d.params[3] = 0;
+        d.weight_format = weight_format_from(bn.ty.dtype);
+        break;
+      }
+      case Op::MatMulAT:
+      case Op::FusedMatMulATAdd: {
+        // src/compile.rs:1423-1445, 1526-1549: A is [K, M]; always the 64x64 tiled entry;
+        // parameter order [m, n, k, 0]
+        const auto& as = g.node(nd.inputs[0]).ty.shape;
+        const Node& bn = g.node(nd.inputs[1]);
+        const uint32_t k = (uint32_t)as[0], m = (uint32_t)as[1], n = (uint32_t)bn.ty.shape[1];
+        const bool fused = nd.op == Op::FusedMatMulATAdd;
+        d.shader = fused ? MGN_SHADER_FUSED_MATMUL_AT_ADD : MGN_SHADER_MATMUL_AT;
+        d.workgroups[0] = (n + 63) / 64, d.workgroups[1] = (m + 63) / 64, d.workgroups[2] = 1;
+        d.input_buffers = {buf_of(nd.inputs[0]), buf_of(nd.inputs[1])};
+        if (fused) d.input_buffers.push_back(buf_of(nd.inputs[2]));
+        d.params[0] = m, d.params[1] = n, d.params[2] = k, d.params[3] = 0;
+        d.weight_format = weight_format_from(bn.ty.dtype);
+        break;
+      }
+      case Op::FusedMatMulBTAdd: {
+        // src/compile.rs:1551-1574: always the tiled entry, [m, n, k, 0]
+        const auto& as = g.node(nd.inputs[0]).ty.shape;
+        const Node& bn = g.node(nd.inputs[1]);
+        const uint32_t m = (uint32_t)as[0], k = (uint32_t)as[1], n = (uint32_t)bn.ty.shape[0];
+        d.shader = MGN_SHADER_FUSED_MATMUL_BT_ADD;
+        d.workgroups[0] = (n + 63) / 64, d.workgroups[1] = (m + 63) / 64, d.workgroups[2] = 1;
+        d.input_buffers = {buf_of(nd.inputs[0]), buf_of(nd.inputs[1]), buf_of(nd.inputs[2])};
+        d.params[0] = m, d.params[1] = n, d.params[2] = k, d.params[3] = 0;
         d.weight_format = weight_format_from(bn.ty.dtype);
         break;
       }
@@ -414,10 +454,14 @@ void Session::check(mgn_status st, const char* what) {
   if (st != MGN_OK) throw std::runtime_error(std::string(what) + ": " + mgn_last_error(ctx_));
 }
 
-static bool is_bt(mgn_shader s) { return s == MGN_SHADER_MATMUL_BT || s == MGN_SHADER_MATMUL_GEMV_BT; }
-static bool is_matmul(mgn_shader s) { return s <= MGN_SHADER_MATMUL_GEMV_ADD || is_bt(s); }
-// K of a matmul dispatch: params are [m, k, n, 0], or [m, n, k, 0] for the BT forms
-static uint32_t matmul_k(const Dispatch& d) { return is_bt(d.shader) ? d.params[2] : d.params[1]; }
+static bool is_bt(mgn_shader s) {
+  return s == MGN_SHADER_MATMUL_BT || s == MGN_SHADER_MATMUL_GEMV_BT || s == MGN_SHADER_FUSED_MATMUL_BT_ADD;
+}
+// the forms whose activations arrive transposed ([K, M])
+static bool is_at(mgn_shader s) { return s == MGN_SHADER_MATMUL_AT || s == MGN_SHADER_FUSED_MATMUL_AT_ADD; }
+static bool is_matmul(mgn_shader s) { return s <= MGN_SHADER_MATMUL_GEMV_ADD || is_bt(s) || is_at(s); }
+// K of a matmul dispatch: params are [m, k, n, 0], or [m, n, k, 0] for the AT and BT forms
+static uint32_t matmul_k(const Dispatch& d) { return is_bt(d.shader) || is_at(d.shader) ? d.params[2] : d.params[1]; }
 
 Session::Session(ExecutionPlan plan, int device_id) : plan_(std::move(plan)) {
   // This backend serves matmuls whose weight is quantized; a plain f32 weight
@@ -624,7 +668,7 @@ void Session::plan_launches() {
     for (int ci : readers[out]) {
       const Dispatch& c = plan_.dispatches[ci];
       mgn_weight* w = is_matmul(c.shader) ? weights_[c.input_buffers[1]] : nullptr;
-      ok = ok && (size_t)ci > pi && w && c.input_buffers[0] == out && is_matmul(c.shader) && matmul_k(c) == width &&
+      ok = ok && (size_t)ci > pi && w && c.input_buffers[0] == out && is_matmul(c.shader) && !is_at(c.shader) && matmul_k(c) == width &&
            (c.input_buffers.size() < 3 || c.input_buffers[2] != out) && fused_[ci].kind == 0 && c.epilogue.empty() &&
            mgn_matmul_q_can_fuse(ctx_, w, c.params[0]) == 1;
     }
@@ -642,7 +686,7 @@ void Session::plan_launches() {
   for (size_t i = 0; i < nd; i++) producer_of[plan_.dispatches[i].output_buffer] = (int)i;
   auto batchable = [&](size_t i) {
     const Dispatch& d = plan_.dispatches[i];
-    if (skipped_[i] || !is_matmul(d.shader) || !d.epilogue.empty()) return false;
+    if (skipped_[i] || !is_matmul(d.shader) || is_at(d.shader) || !d.epilogue.empty()) return false;
     mgn_weight* w = weights_[d.input_buffers[1]];
     return w && mgn_matmul_q_can_fuse(ctx_, w, d.params[0]) == 1;
   };
@@ -699,12 +743,21 @@ void Session::run_dispatches() {
       case MGN_SHADER_FUSED_MATMUL_ADD:
       case MGN_SHADER_MATMUL_GEMV_ADD:
       case MGN_SHADER_MATMUL_BT:
-      case MGN_SHADER_MATMUL_GEMV_BT: {
+      case MGN_SHADER_MATMUL_GEMV_BT:
+      case MGN_SHADER_FUSED_MATMUL_BT_ADD:
+      case MGN_SHADER_MATMUL_AT:
+      case MGN_SHADER_FUSED_MATMUL_AT_ADD: {
         mgn_weight* w = weights_[d.input_buffers[1]];
         if (!w) throw std::runtime_error("quantized parameter was never set");
         const mgn_buf* addend = d.input_buffers.size() > 2 ? buffers_[d.input_buffers[2]] : nullptr;
         const Fused& f = fused_[di];
-        if (f.more[0] >= 0) {
+        if (is_at(d.shader)) {
+          std::vector<mgn_unary> ops = d.epilogue;
+          ops.insert(ops.end(), f.post.begin(), f.post.end());
+          mgn_buf* dst = buffers_[f.out_buffer >= 0 ? f.out_buffer : d.output_buffer];
+          check(mgn_matmul_q_at(ctx_, buffers_[d.input_buffers[0]], w, addend, dst, d.params[0], ops.data(), ops.size()),
+                "mgn_matmul_q_at");
+        } else if (f.more[0] >= 0) {
           mgn_matmul_item items[3] = {{w, addend, buffers_[d.output_buffer]}, {}, {}};
           size_t count = 1;
           for (int sib : f.more) {
@@ -864,6 +917,9 @@ int32_t mgn_graph_matmul(mgn_graph* g, int32_t a, int32_t b) {
 }
 int32_t mgn_graph_matmul_bt(mgn_graph* g, int32_t a, int32_t b) {
   return graph_node(g, [&] { return g->g.matmul_bt((mgn::NodeId)a, (mgn::NodeId)b); });
+}
+int32_t mgn_graph_matmul_at(mgn_graph* g, int32_t a, int32_t b) {
+  return graph_node(g, [&] { return g->g.matmul_at((mgn::NodeId)a, (mgn::NodeId)b); });
 }
 int32_t mgn_graph_add(mgn_graph* g, int32_t a, int32_t b) {
   return graph_node(g, [&] { return g->g.add((mgn::NodeId)a, (mgn::NodeId)b); });

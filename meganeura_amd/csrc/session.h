@@ -45,7 +45,10 @@ struct TensorType {
   }
 };
 
-enum class Op { Input, Parameter, MatMul, Add, SwiGLU, RmsNorm, FusedMatMulAdd, SwiGLUConcat, Nop, MatMulBT, Relu, Sigmoid, Neg, Silu };
+enum class Op {
+  Input, Parameter, MatMul, Add, SwiGLU, RmsNorm, FusedMatMulAdd, SwiGLUConcat, Nop, MatMulBT, Relu, Sigmoid, Neg, Silu,
+  MatMulAT, FusedMatMulATAdd, FusedMatMulBTAdd
+};
 
 struct Node {
   NodeId id;
@@ -75,6 +78,7 @@ class Graph {
   NodeId parameter_q8(const std::string& name, std::vector<size_t> shape);
   NodeId matmul(NodeId a, NodeId b);
   NodeId matmul_bt(NodeId a, NodeId b);
+  NodeId matmul_at(NodeId a, NodeId b);
   NodeId add(NodeId a, NodeId b);
   NodeId swiglu(NodeId gate, NodeId up);
   NodeId rms_norm(NodeId x, NodeId weight, float eps);

@@ -33,6 +33,9 @@ class ShaderEntry(IntEnum):
     Sigmoid = 11
     Neg = 12
     Silu = 13
+    MatMulAT = 14
+    FusedMatMulATAdd = 15
+    FusedMatMulBTAdd = 16
 
 
 class EpilogueOp(IntEnum):
@@ -108,6 +111,10 @@ class Graph:
     def matmul_bt(self, a, b):
         """a[M,K] x b[N,K]^T (src/graph.rs:809-817)."""
         return self._node(self.lib.mgn_graph_matmul_bt(self.h, a, b))
+
+    def matmul_at(self, a, b):
+        """a[K,M]^T x b[K,N] (src/graph.rs:798-806)."""
+        return self._node(self.lib.mgn_graph_matmul_at(self.h, a, b))
 
     def add(self, a, b):
         return self._node(self.lib.mgn_graph_add(self.h, a, b))

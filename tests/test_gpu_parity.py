@@ -465,6 +465,42 @@ def test_unary_epilogues(ctx, orc, fmt, route, m, k, n):
         a.free(); db.free(); c.free(); wt.free()
 
 
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m,k,n", [(1, 576, 192), (3, 4096, 257), (6, 1024, 300), (33, 96, 67), (70, 2048, 40)])
+def test_transposed_activations(ctx, orc, fmt, m, k, n):
+    """mgn_matmul_q_at: A arrives as [K, M] (the MatMulAT / FusedMatMulATAdd dispatches); the result
+    is the plain matmul on A^T, with the residual and an epilogue, and a second call with a larger
+    M (the staging area grows) leaves the first result's inputs alone."""
+    x = synth.normal(41 + m + k + n, m * k).reshape(m, k)
+    w = synth.normal(42 + m + k + n, k * n, 0.02).reshape(k, n)
+    d = synth.normal(43 + n, m * n).reshape(m, n)
+    deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
+    weight = ctx.weight(fmt, w)
+    a_t = ctx.upload(np.ascontiguousarray(x.T))
+    dbuf = ctx.upload(d)
+    c = ctx.buffer(m * n * 4)
+    try:
+        ctx.matmul_q_at(a_t, weight, c, m)
+        orc.assert_close(c.download(np.float32, m * n).reshape(m, n), orc.matmul_f32(x, deq), REL, ABS)
+        ctx.matmul_q_at(a_t, weight, c, m, d=dbuf, ops=[capi.UNARY_NEG, capi.UNARY_RELU])
+        want = orc.unary("relu", orc.unary("neg", orc.matmul_f32(x, deq, d)))
+        orc.assert_close(c.download(np.float32, m * n).reshape(m, n), want, REL, ABS)
+        # a taller A^T right behind it: the staging area is replaced while nothing reads it
+        m2 = m + 40
+        x2 = synth.normal(44 + m + k + n, m2 * k).reshape(m2, k)
+        a2 = ctx.upload(np.ascontiguousarray(x2.T))
+        c2 = ctx.buffer(m2 * n * 4)
+        ctx.matmul_q_at(a2, weight, c2, m2)
+        ctx.matmul_q_at(a_t, weight, c, m)
+        orc.assert_close(c2.download(np.float32, m2 * n).reshape(m2, n), orc.matmul_f32(x2, deq), REL, ABS)
+        orc.assert_close(c.download(np.float32, m * n).reshape(m, n), orc.matmul_f32(x, deq), REL, ABS)
+        a2.free(); c2.free()
+        with pytest.raises(capi.MgnError):  # A^T shorter than K x m
+            ctx.matmul_q_at(a_t, weight, c, m + 1)
+    finally:
+        a_t.free(); dbuf.free(); c.free(); weight.free()
+
+
 def test_epilogue_arguments_are_checked(ctx):
     wt = ctx.weight(Q4, synth.normal(970, 64 * 8, 0.02).reshape(64, 8))
     a = ctx.buffer(4 * 64)

@@ -356,3 +356,46 @@ def test_matmul_bt_with_quantized_table(orc, quant, m, k, n):
     want = orc.matmul_packed(fmt, xv, orc.quantize(fmt, np.ascontiguousarray(embed.T)), n)
     orc.assert_close(got, want, 1e-3, 1e-4)
     sess.close()
+
+
+@pytest.mark.parametrize("quant", ["q4", "q8"])
+@pytest.mark.parametrize("m,k,n", [(1, 64, 66), (6, 128, 200), (40, 576, 96)])
+def test_matmul_at_and_fused_add_forms(orc, quant, m, k, n):
+    """matmul_at (a stored [K, M]) alone, with a residual and a relu folded in, and matmul_bt
+    with a residual: each is one dispatch of the plan, as in the reference
+    (src/optimize.rs:724-767, src/compile.rs:1423-1445, 1526-1574), and equals the plain
+    quantized matmul on the transposed operand."""
+    fmt = Q4 if quant == "q4" else Q8
+    param = "parameter_q4" if quant == "q4" else "parameter_q8"
+    g = Graph()
+    xt = g.input("xt", [k, m])
+    x = g.input("x", [m, k])
+    r = g.input("r", [m, n])
+    w = getattr(g, param)("w", [k, n])
+    e = getattr(g, param)("e", [n, k])
+    g.set_outputs([g.matmul_at(xt, w), g.relu(g.add(g.matmul_at(xt, w), r)), g.add(r, g.matmul_bt(x, e))])
+    sess = build_inference_session(g)
+    assert [d.shader for d in sess.plan()] == [ShaderEntry.MatMulAT, ShaderEntry.FusedMatMulATAdd, ShaderEntry.FusedMatMulBTAdd]
+    wv = synth.normal(910 + n, k * n, 0.02).reshape(k, n)
+    ev = synth.normal(911 + n, n * k, 0.02).reshape(n, k)
+    xv = synth.normal(912 + k, m * k, 1.0).reshape(m, k)
+    rv = synth.normal(913 + k, m * n, 1.0).reshape(m, n)
+    sess.set_parameter("w", wv)
+    sess.set_parameter("e", ev)
+    sess.set_input("xt", np.ascontiguousarray(xv.T))
+    sess.set_input("x", xv)
+    sess.set_input("r", rv)
+    plain = orc.matmul_packed(fmt, xv, orc.quantize(fmt, wv), n)
+    fused = np.maximum(orc.matmul_packed(fmt, xv, orc.quantize(fmt, wv), n, rv), 0.0)
+    bt = orc.matmul_packed(fmt, xv, orc.quantize(fmt, np.ascontiguousarray(ev.T)), n, rv)
+    # plain launches (the second step finds the staging area in place), then the step captured
+    # as a graph and replayed
+    for step in range(5):
+        if step == 2:
+            sess.set_graph_replay(True)
+        sess.step()
+        sess.wait()
+        orc.assert_close(sess.read_output_by_index(0, m * n).reshape(m, n), plain, 1e-3, 1e-4)
+        orc.assert_close(sess.read_output_by_index(1, m * n).reshape(m, n), fused, 1e-3, 1e-4)
+        orc.assert_close(sess.read_output_by_index(2, m * n).reshape(m, n), bt, 1e-3, 1e-4)
+    sess.close()

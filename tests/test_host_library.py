@@ -268,6 +268,47 @@ def test_matmul_bt_lowering_and_mixed_use():
         g3.compile()
 
 
+def test_matmul_at_and_fused_add_forms_lowering():
+    # src/compile.rs:1423-1445, 1526-1574: A stored [K, M]; always the tiled entry; params
+    # [m, n, k, 0]; Add(MatMulAT) and Add(MatMulBT) fuse like Add(MatMul) (src/optimize.rs:724-767)
+    from meganeura_amd.graph import EpilogueOp, Graph, ShaderEntry, WeightFormat
+    g = Graph()
+    xt = g.input("xt", [64, 1])
+    w = g.parameter_q8("w", [64, 132])
+    g.set_outputs([g.matmul_at(xt, w)])
+    (d,) = g.compile()
+    assert d.shader == ShaderEntry.MatMulAT and d.workgroups == [3, 1, 1]
+    assert d.params == [1, 132, 64, 0] and d.weight_format == WeightFormat.Q8
+    g = Graph()
+    xt = g.input("xt", [96, 70])
+    r = g.input("r", [70, 40])
+    w = g.parameter_q4("w", [96, 40])
+    g.set_outputs([g.relu(g.add(r, g.matmul_at(xt, w)))])
+    (d,) = g.compile()
+    assert d.shader == ShaderEntry.FusedMatMulATAdd and d.workgroups == [1, 2, 1] and d.params == [70, 40, 96, 0]
+    assert d.epilogue == [EpilogueOp.Relu]
+    g = Graph()
+    x = g.input("x", [1, 64])
+    r = g.input("r", [1, 48])
+    e = g.parameter_q4("e", [48, 64])
+    g.set_outputs([g.add(g.matmul_bt(x, e), r)])
+    (d,) = g.compile()  # no GEMV form of the fused BT entry in the reference
+    assert d.shader == ShaderEntry.FusedMatMulBTAdd and d.workgroups == [1, 1, 1] and d.params == [1, 48, 64, 0]
+    with pytest.raises(ValueError, match="K dimensions must match"):
+        g2 = Graph()
+        g2.matmul_at(g2.input("x", [32, 4]), g2.parameter_q4("w", [64, 8]))
+    # matmul and matmul_at read a parameter the same way; matmul_at and matmul_bt do not
+    g3 = Graph()
+    w = g3.parameter_q4("w", [64, 64])
+    g3.set_outputs([g3.matmul(g3.input("x", [2, 64]), w), g3.matmul_at(g3.input("xt", [64, 2]), w)])
+    assert [d.shader for d in g3.compile()] == [ShaderEntry.MatMul, ShaderEntry.MatMulAT]
+    g4 = Graph()
+    w = g4.parameter_q4("w", [64, 64])
+    g4.set_outputs([g4.matmul_at(g4.input("xt", [64, 2]), w), g4.matmul_bt(g4.input("x", [2, 64]), w)])
+    with pytest.raises(ValueError, match="both matmul and matmul_bt"):
+        g4.compile()
+
+
 def test_host_quantizer_matches_golden_vectors():
     from helpers import check_golden_packed, golden_vectors
     vectors, _ = golden_vectors()
