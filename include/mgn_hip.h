@@ -211,6 +211,8 @@ typedef struct mgn_plan_info {
   uint32_t steps;         /* GEMV: 16-block steps per wave; tiled: 8-block chunks per wave */
   uint32_t quads_per_wave; /* GEMV only */
   uint32_t full_steps;    /* GEMV only: 1 when no step needs masking */
+  uint32_t tail_blocks;   /* GEMV only: 0, or the K blocks per column beyond `steps` full steps that the wave's
+                           * quads share one more step for (K = 32 * (16 * steps + tail_blocks)) */
   uint64_t workspace_bytes; /* partial sums held in the context's workspace */
 } mgn_plan_info;
 mgn_status mgn_matmul_q_plan(mgn_fmt fmt, uint32_t m, uint64_t k, uint64_t n, int a_is_f16, int num_cus,

@@ -173,7 +173,8 @@ UNARY_RELU, UNARY_SIGMOID, UNARY_NEG, UNARY_SILU = 1, 2, 3, 4
 class PlanInfo(C.Structure):
     _fields_ = [("route", C.c_int), ("grid", C.c_uint32 * 3), ("threads", C.c_uint32), ("lds_bytes", C.c_uint32),
                 ("waves_n", C.c_uint32), ("k_splits", C.c_uint32), ("k_parts", C.c_uint32), ("steps", C.c_uint32),
-                ("quads_per_wave", C.c_uint32), ("full_steps", C.c_uint32), ("workspace_bytes", C.c_uint64)]
+                ("quads_per_wave", C.c_uint32), ("full_steps", C.c_uint32), ("tail_blocks", C.c_uint32),
+                ("workspace_bytes", C.c_uint64)]
 
 
 def matmul_plan(fmt, m, k, n, a_is_f16=False, num_cus=256):

@@ -257,7 +257,7 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 // that is a whole number of steps (the last part may reach past the end of K).  Their partial
 // sums meet in a workspace; the last workgroup to arrive adds them in part order (bit-identical
 // from run to run) and writes C.
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT>
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT, bool TAIL = false>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // The leading scalar arguments are what a wave needs before it can issue its first loads;
     // they are declared first (and not inside a struct) so that the dispatcher can hand them
@@ -295,6 +295,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   const uint32_t quad_base = pick3(widx, 0u, first_quad1, first_quad2);  // first quad of that weight
   const uint32_t bpc = w.k / 32;
   static_assert(!KSPLIT || (!EXACT && PRO == kProNone && QPW == 1), "K parts come with masked steps, one quad per wave and no prologue");
+  static_assert(!TAIL || (FMT == MGN_FMT_Q4 && QPW > 1 && EXACT && !KSPLIT && PRO == kProNone),
+                "the shared tail step: Q4, several quads per wave, full regular steps, one K part, no prologue");
   const uint32_t kpart = KSPLIT ? blockIdx.y : 0u;
   const uint32_t bpc_full = KSPLIT ? sp.k_full / 32 : bpc;  // blocks per column of the weight
   const uint32_t kb_part = kpart * bpc;                     // this workgroup's first K block
@@ -372,7 +374,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   // load t = q * STEPS + s: K step s of the wave's quad q
   constexpr int TS = STEPS * QPW;
   constexpr int kDepth = prefetch_depth<FMT>();
-  Raw<FMT> blk[TS];
+  // TAIL: K is STEPS full steps plus 1, 2 or 4 leftover blocks per column.  Instead of a second,
+  // nearly empty step for every quad, one more step takes the leftovers of all QPW quads at once:
+  // the MFMA's 16 blocks are independent, so slot b serves quad b / T, K block 16 * STEPS + b % T.
+  constexpr int TS_ALL = TS + (TAIL ? 1 : 0);
+  Raw<FMT> blk[TS_ALL];
   // Q8: first block of this lane's pair, see Raw<MGN_FMT_Q8>
   const uint32_t kb8_first = step_begin * 16 + (b >> 1);
   // A lane's loads are its base pointer plus a constant: no address arithmetic or range
@@ -391,14 +397,30 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
             (FMT == MGN_FMT_Q8 ? (b & 1) * 16 : 0);
     pm[q] = (const char*)w.meta + (size_t)(at0 + kb_first) * MB;
   }
+  uint32_t tail_q = 0, tail_kb = 0;  // this lane's quad (within the wave) and K block in the tail step
+  const char* pq_tail = nullptr;
+  const char* pm_tail = nullptr;
+  if constexpr (TAIL) {
+    const uint32_t tcount = bpc - 16 * STEPS;  // 1, 2 or 4, and QPW * tcount <= 16 (the planner sees to both)
+    const uint32_t tshift = (uint32_t)__builtin_ctz(tcount);
+    tail_q = b >> tshift;  // slots with tail_q >= QPW serve nobody: their results are never selected
+    tail_kb = 16 * STEPS + (b & (tcount - 1));
+    const uint32_t col = min((quad + min(tail_q, (uint32_t)QPW - 1)) * 4 + i, w.n - 1);
+    pq_tail = (const char*)w.quants + ((size_t)col * bpc_full + tail_kb) * QB;
+    pm_tail = (const char*)w.meta + ((size_t)col * bpc_full + tail_kb) * MB;
+  }
   auto fetch = [&](int t) {
+    if (TAIL && t == TS) {
+      blk[t].load_at(pq_tail, pm_tail);
+      return;
+    }
     const int q = t / STEPS, s = t % STEPS;
     blk[t].load_at(pq[q] + s * (16 * QB), pm[q] + s * (16 * MB));
   };
   // (a wave without a quad issues these too, from the last column's blocks, and skips the
   // walk; a branch around the loads would make every wave wait for them at the join)
 #pragma unroll
-  for (int t = 0; t < TS && t < kDepth; t++) {
+  for (int t = 0; t < TS_ALL && t < kDepth; t++) {
     fetch(t);
     __builtin_amdgcn_sched_barrier(0);  // in this order: step 0 waits for its own block only
   }
@@ -531,9 +553,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     for (int r = 0; r < MROWS; r++) acc[q][r] = 0.0f;
   if (wave_live) {
 #pragma unroll
-  for (int t = 0; t < TS; t++) {
+  for (int t = 0; t < TS_ALL; t++) {
     const int s = t % STEPS, q = t / STEPS;
-    if (t + kDepth < TS) {
+    if (t + kDepth < TS_ALL) {
       // keep the load where it is written: one step's loads per step, kDepth steps ahead (with
       // constant offsets the scheduler would otherwise gather the loads of several steps)
       __builtin_amdgcn_sched_barrier(0);
@@ -545,6 +567,10 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // neighbouring K split gets scale (and minimum) zero
     if constexpr (!EXACT) cur.meta = ((uint32_t)s >= first_own && kb_first + s * 16 < bpc_live) ? cur.meta : 0u;
     if constexpr (FMT == MGN_FMT_Q4) {
+      const bool tail_step = TAIL && t == TS;
+      // the step's activations and block constants: K block kb_first + 16 s, or the lane's tail block
+      const char* const xa_step = tail_step ? (const char*)xa + ((size_t)tail_kb * NJ + jrow) * 16 : xa_lane + s * (16 * NJ * 16);
+      const char* const ci_step = tail_step ? (const char*)cinit + (size_t)tail_kb * MROWS * 8 : ci_lane + s * (16 * MROWS * 8);
       // A operands: 4 chunks of 16 bytes, consecutive lanes -> consecutive chunks; with more than
       // two activation rows a second group of four A rows (rows 2 and 3, hi and lo) follows
       uint4 ax[NG][4];
@@ -552,10 +578,10 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int ch = 0; ch < 4; ch++)
-          ax[g][ch] = *(const uint4*)(xa_lane + s * (16 * NJ * 16) + ch * plane * 16 + g * 64);
+          ax[g][ch] = *(const uint4*)(xa_step + ch * plane * 16 + g * 64);
       float2 ci[MROWS];  // {chain start value, factor that undoes the operand and block scales}
 #pragma unroll
-      for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_lane + s * (16 * MROWS * 8) + r * 8);
+      for (int r = 0; r < MROWS; r++) ci[r] = *(const float2*)(ci_step + r * 8);
       // the centring term rides in as the chain's start value (rows 2r and 2r+1 add up later)
       floatx4 dsum[NG];
 #pragma unroll
@@ -580,7 +606,18 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       for (int r = 0; r < MROWS; r++) {
         float v = dscale * (dsum[r / 2][2 * (r % 2)] + dsum[r / 2][2 * (r % 2) + 1]);
         v = __fmaf_rn(mneg, ci[r].x, v);
-        acc[q][r] = __fmaf_rn(v, ci[r].y, acc[q][r]);
+        if (tail_step) {
+          // the slot's quad differs from lane to lane: every accumulator takes what is its own
+#pragma unroll
+          for (int qq = 0; qq < QPW; qq++) {
+            const float sum = __fmaf_rn(v, ci[r].y, acc[qq][r]);
+            acc[qq][r] = tail_q == (uint32_t)qq ? sum : acc[qq][r];
+          }
+        } else {
+          constexpr int QMAX = QPW - 1;
+          const int qa = q < QPW ? q : QMAX;  // (q == QPW only in the tail step, which does not come here)
+          acc[qa][r] = __fmaf_rn(v, ci[r].y, acc[qa][r]);
+        }
       }
     } else {
       // two half blocks per step, each with its own chain of four MFMAs and its own scale
@@ -714,6 +751,7 @@ struct MfmaGemvPlan {
   uint32_t kparts;  // workgroups sharing a quad group (1: no split over workgroups)
   uint32_t part_k;  // K of one part when kparts > 1: a whole number of 16-block steps
   bool exact;  // every step of every K split is a full one
+  uint32_t tail;  // 0, or the leftover blocks per column (1, 2, 4) that all quads of a wave share one more step for
   size_t lds;
 };
 
@@ -766,6 +804,17 @@ bool plan_one_part(int fmt, uint32_t k, uint32_t nquads, uint32_t mrows, int num
   p.grid = (wave_quads + p.wnc - 1) / p.wnc;
   p.tasks = bpc_pad * 4 <= 64 * p.ksc * p.wnc ? 1 : 2;
   p.exact = bpc % 16 == 0 && p.ksc * p.steps == steps_total;
+  // A short K with a few blocks beyond its full steps (576 = 16 + 2 blocks), four quads per wave:
+  // the quads share one more step for their leftovers instead of a nearly empty step each.
+  p.tail = 0;
+  if (fmt == MGN_FMT_Q4 && p.ksc == 1 && p.qpw == 4 && p.steps == 2 && p.tasks == 1) {
+    const uint32_t left = bpc - 16;
+    if (left == 1 || left == 2 || left == 4) {
+      p.tail = left;
+      p.steps = 1;
+      p.exact = true;
+    }
+  }
   const uint32_t nj = 2 * mrows;
   const size_t plane = (size_t)bpc_pad * nj + (fmt == MGN_FMT_Q8 ? plane_pad<MGN_FMT_Q8>(nj) : 0u);
   const size_t cpb = fmt == MGN_FMT_Q8 ? cinit_per_block<MGN_FMT_Q8>() : 1u;
@@ -806,9 +855,9 @@ bool plan_mfma_gemv(const LaunchArgs& x, uint32_t mrows, MfmaGemvPlan* out) {
   return false;
 }
 
-template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT>
+template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT, bool TAIL = false>
 int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
-  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS, EXACT, KSPLIT>;
+  auto kern = gemv_mfma_kernel<FMT, MROWS, STEPS, QPW, PRO, TASKS, EXACT, KSPLIT, TAIL>;
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
@@ -841,6 +890,11 @@ int launch_pro(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
     if constexpr (PRO == kProNone && QPW == 1)
       return p.tasks == 1 ? launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, false, true>(s, x, p)
                           : launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 2, false, true>(s, x, p);
+    return (int)hipErrorInvalidValue;
+  }
+  if (p.tail != 0) {
+    if constexpr (FMT == MGN_FMT_Q4 && STEPS == 1 && QPW == 4 && PRO == kProNone)
+      return launch_tasks<FMT, MROWS, STEPS, QPW, PRO, 1, true, false, true>(s, x, p);
     return (int)hipErrorInvalidValue;
   }
   if (p.exact)

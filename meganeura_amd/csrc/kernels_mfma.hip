@@ -727,7 +727,7 @@ bool describe_gemm_mfma(const LaunchArgs& x, mgn_plan_info* out) {
   out->threads = 64 * p.ksc * p.wnc;
   out->lds_bytes = (uint32_t)p.lds;
   out->waves_n = p.wnc, out->k_splits = p.ksc, out->k_parts = p.parts, out->steps = p.nch;
-  out->quads_per_wave = 0, out->full_steps = 0;
+  out->quads_per_wave = 0, out->full_steps = 0, out->tail_blocks = 0;
   out->workspace_bytes = p.scratch_bytes;
   return true;
 }

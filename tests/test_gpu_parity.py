@@ -137,6 +137,9 @@ ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv_valu": capi.ROUTE_GEMV_VALU, "gem
     (1, 11008, 132), (2, 11040, 66),
     # K parts that are not even: 37 and 21.5 steps of 16 blocks
     (1, 18944, 132), (4, 11008, 260), (3, 13824, 70),
+    # one full step plus 2, 1, 4 leftover blocks and very many columns: the quads of a wave share a
+    # step for the leftovers (Q4); ragged last quad, last wave with fewer than four quads
+    (1, 576, 40000), (2, 544, 33001), (4, 640, 36002), (3, 576, 49153),
 ])
 def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
     x = synth.normal(1000 + m + k + n, m * k).reshape(m, k)

@@ -38,6 +38,12 @@ def check_gemv(p, fmt, m, k, n):
         assert p.full_steps == 0 and p.quads_per_wave == 1
         assert p.workspace_bytes == p.k_parts * mrows * n * 4 <= WORKSPACE
         assert p.grid[0] <= COUNTERS
+    elif p.tail_blocks:
+        # full steps plus a few leftover blocks that the wave's quads share one more step for
+        assert fmt == Q4 and p.k_splits == 1 and p.full_steps == 1 and p.workspace_bytes == 0
+        assert bpc == 16 * p.steps + p.tail_blocks and p.tail_blocks in (1, 2, 4)
+        assert p.quads_per_wave * p.tail_blocks <= 16
+        steps_total = p.steps
     else:
         steps_total = steps_all
         assert p.workspace_bytes == 0
@@ -50,7 +56,7 @@ def check_gemv(p, fmt, m, k, n):
     assert p.grid[0] * per_wg >= nquads                  # every column has a wave
     assert (p.grid[0] - 1) * per_wg < nquads             # no workgroup without a column
     if p.quads_per_wave > 1:
-        assert p.k_splits == 1 and p.steps * p.quads_per_wave <= 8
+        assert p.k_splits == 1 and p.steps * p.quads_per_wave + (1 if p.tail_blocks else 0) <= 8
 
 
 def check_gemm(p, fmt, m, k, n, f16):
@@ -131,6 +137,11 @@ def test_edge_shapes_of_the_gpu_parity_tests_stay_on_the_gemv_kernel():
     assert capi.matmul_plan(Q4, 1, 18944, 132).k_parts > 1
     assert capi.matmul_plan(Q4, 1, 11008, 132).full_steps == 0
     assert capi.matmul_plan(Q4, 1, 512, 32774).quads_per_wave == 4
+    # lm_head of SmolLM2-135M: 18 blocks = one full step + 2 leftover blocks shared by the wave's four quads
+    lm = capi.matmul_plan(Q4, 1, 576, 49152)
+    assert (lm.steps, lm.quads_per_wave, lm.tail_blocks, lm.full_steps) == (1, 4, 2, 1)
+    assert capi.matmul_plan(Q8, 1, 576, 49152).tail_blocks == 0  # Q8 keeps its two steps
+    assert capi.matmul_plan(Q4, 1, 608, 49152).tail_blocks == 0  # 3 leftover blocks do not divide the slots
 
 
 def test_shapes_no_weight_can_have_are_refused():
