@@ -69,6 +69,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c5_q4_m4_14336x4096": 39.3e6,
     "c5_q4_m16_4096x14336": 48.3e6,
     "c4_q4_prefill_up_512x1024x3072": 18.9e6,
+    "c3_q4_lm_head_576x49152": 18.03e6,
 }
 
 
