@@ -318,3 +318,53 @@ def test_host_quantizer_matches_golden_vectors():
         deq = capi.dequantize_ref(fmt, packed, *w.shape).reshape(-1)
         for idx, bits_ in entry.get("dequant_f32_bits", {}).items():
             assert int(deq[int(idx)].view(np.uint32)) == bits_, name
+
+
+def test_a_c_program_links_against_the_library(tmp_path):
+    """The boundary is C: a C99 translation unit includes both headers, links the shared library
+    and calls the entries that need no device (sizes, host quantizer, planner, graph lowering)."""
+    import os
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler here")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    libdir = os.path.join(root, "meganeura_amd")
+    src = tmp_path / "consumer.c"
+    src.write_text(r"""
+#include <stdio.h>
+#include <string.h>
+#include "mgn_hip.h"
+#include "mgn_session.h"
+int main(void) {
+  float w[32];
+  unsigned char packed[20];
+  float back[32];
+  int i;
+  mgn_plan_info plan;
+  mgn_graph* g;
+  int x, p, y;
+  for (i = 0; i < 32; i++) w[i] = (float)(i - 16) * 0.1f;           /* src/runtime.rs:2223-2226 */
+  if (mgn_packed_size(MGN_FMT_Q4, 32, 1) != 20 || mgn_packed_size(MGN_FMT_Q8, 64, 3) != 216) return 1;
+  if (mgn_quantize_ref(MGN_FMT_Q4, w, 32, 1, packed) != MGN_OK) return 2;
+  if (packed[0] != 0x9D || packed[1] != 0x32 || packed[2] != 0x66 || packed[3] != 0xBE) return 3;
+  if (mgn_dequantize_ref(MGN_FMT_Q4, packed, 32, 1, back) != MGN_OK) return 4;
+  for (i = 0; i < 32; i++) if (back[i] - w[i] > 0.3f || w[i] - back[i] > 0.3f) return 5;
+  if (mgn_matmul_q_plan(MGN_FMT_Q4, 1, 4096, 14336, 0, 256, &plan) != MGN_OK) return 6;
+  if (plan.route != MGN_ROUTE_GEMV_MFMA || plan.grid[0] != 256) return 7;
+  g = mgn_graph_new();
+  x = mgn_graph_input(g, "x", 1, 64);
+  p = mgn_graph_parameter_q4(g, "w", 64, 8);
+  y = mgn_graph_matmul(g, x, p);
+  if (x < 0 || p < 0 || y < 0) return 8;
+  if (mgn_graph_matmul(g, x, x) >= 0 || strlen(mgn_graph_last_error(g)) == 0) return 9;  /* 64 != 1 */
+  mgn_graph_free(g);
+  puts("ok");
+  return 0;
+}
+""")
+    exe = tmp_path / "consumer"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(root, "include"), str(src), "-o", str(exe),
+                    "-L", libdir, "-lmgn_hip", "-Wl,-rpath," + libdir], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0 and out.stdout.strip() == "ok", (out.returncode, out.stdout, out.stderr)
