@@ -129,6 +129,17 @@ class Workload:
         self.ctx.sync()
         return ms / steps
 
+    def read_floor(self, steps, warmup):
+        """ms per launch of a kernel that reads the same weight copies in the same rotation and
+        computes nothing: one launch plus one pass over the packed bytes, on this box."""
+        self.ctx.weight_read_loop(self.weights, warmup)
+        self.ctx.sync()
+        self.ctx.timer_start()
+        self.ctx.weight_read_loop(self.weights, steps)
+        ms = self.ctx.timer_stop()
+        self.ctx.sync()
+        return ms / steps
+
     def output(self):
         return self.c.download(np.float32, self.m * self.n).reshape(self.m, self.n)
 
@@ -295,6 +306,8 @@ def main():
     ms = wl.run(args.steps, args.warmup)
     got = wl.output()
 
+    floor_ms = None if args.profile else wl.read_floor(args.steps, args.warmup)
+
     is_gemm = wl.m > 16
     gbs = wl.bytes / (ms * 1e-3) / 1e9
     tflops = wl.flops / (ms * 1e-3) / 1e12
@@ -361,6 +374,11 @@ def main():
         "copy_ceiling": None if copy_gbs is None else
         {"GB/s": copy_gbs, "what": "256 MiB device-to-device copy, bytes read + written per second",
          "pct_of_it": 100.0 * gbs / copy_gbs},
+        "read_floor": None if floor_ms is None else
+        {"us_per_launch": floor_ms * 1e3, "GB/s": wl.bytes / (floor_ms * 1e-3) / 1e9,
+         "what": "a kernel that only reads the same rotating weight copies (quants and scales), timed the same way: "
+                 "one launch plus one pass over the packed bytes on this box",
+         "pct_of_it": 100.0 * floor_ms / ms},
     }
     wl.free()
 

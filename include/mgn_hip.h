@@ -195,6 +195,13 @@ mgn_status mgn_matmul_q_at(mgn_ctx* ctx, const mgn_buf* a_t, const mgn_weight* w
 mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const mgn_weight* const* weights,
                              size_t count, const mgn_buf* d, mgn_buf* c, uint32_t m, uint32_t steps);
 
+/* Measurement aid with no counterpart in the reference: `steps` launches, back to back like
+ * mgn_matmul_q_loop's, of a kernel that reads the packed bytes of weights[i % count] (quants and
+ * scales) once and computes nothing.  Timed like a matmul it gives the time the device needs
+ * for one launch plus one pass over a weight's bytes, the floor a bandwidth-bound matmul on
+ * that weight can be held against. */
+mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, size_t count, uint32_t steps);
+
 /* What mgn_matmul_q would launch for a shape, without a device: the kernel family the
  * automatic choice takes (the analogue of reading compile.rs:1390 and runtime.rs:1634 for the
  * reference) and the launch geometry.  For logs, and for checking the planner on the host.

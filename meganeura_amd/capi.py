@@ -22,7 +22,7 @@ HIP_SYMBOLS = [
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_weight_save", "mgn_weight_load", "mgn_matmul_q",
-    "mgn_matmul_q_f16a", "mgn_matmul_q_epilogue", "mgn_matmul_q_at", "mgn_matmul_q_loop", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
+    "mgn_matmul_q_f16a", "mgn_matmul_q_epilogue", "mgn_matmul_q_at", "mgn_matmul_q_loop", "mgn_weight_read_loop", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
     "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [
@@ -108,6 +108,7 @@ def load():
         "mgn_matmul_q_at": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32, vp, C.c_size_t]),
         "mgn_matmul_q_plan": (C.c_int, [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.c_int, vp]),
         "mgn_matmul_q_loop": (C.c_int, [vp, vp, C.c_int, vp, C.c_size_t, vp, vp, C.c_uint32, C.c_uint32]),
+        "mgn_weight_read_loop": (C.c_int, [vp, vp, C.c_size_t, C.c_uint32]),
         "mgn_matmul_q_rms_norm": (C.c_int, [vp, vp, vp, C.c_float, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_swiglu": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_can_fuse": (C.c_int, [vp, vp, C.c_uint32]),
@@ -333,6 +334,11 @@ class Context:
         arr = (C.c_void_p * len(weights))(*[w.h for w in weights])
         self.check(self.lib.mgn_matmul_q_loop(self.h, a.h, 1 if a_is_f16 else 0, arr, len(weights),
                                               d.h if d is not None else None, c.h, m, steps))
+
+    def weight_read_loop(self, weights, steps):
+        """`steps` launches of a kernel that only reads the packed bytes of weights[i % len(weights)]."""
+        arr = (C.c_void_p * len(weights))(*[w.h for w in weights])
+        self.check(self.lib.mgn_weight_read_loop(self.h, arr, len(weights), steps))
 
     def matmul_q_rms_norm(self, x, norm_weight, eps, w, c, m, d=None):
         """C = rms_norm(x; norm_weight, eps) x W (+ D) in one launch."""

@@ -268,6 +268,41 @@ int launch_rms_norm(ihipStream_t* s, const float* x, const float* weight, float*
   return 0;
 }
 
+// Measurement aid: reads a weight's packed bytes (scales and quants) once and computes
+// nothing, so that a harness can time what the memory system alone allows for one pass over a
+// weight.  Every workgroup takes a contiguous share, a wave reads 1 KiB per
+// instruction with eight loads in flight.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4_t read_share(const u32x4_t* __restrict__ p, size_t n16) {
+  const size_t per_wg = (n16 + gridDim.x - 1) / gridDim.x;
+  const size_t beg = (size_t)blockIdx.x * per_wg, end = beg + per_wg < n16 ? beg + per_wg : n16;
+  u32x4_t acc = {0, 0, 0, 0};
+  size_t i = beg + threadIdx.x;
+  for (; i + (size_t)7 * blockDim.x < end; i += (size_t)8 * blockDim.x) {
+    u32x4_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) v[u] = __builtin_nontemporal_load(p + i + (size_t)u * blockDim.x);
+#pragma unroll
+    for (int u = 0; u < 8; u++) acc ^= v[u];
+  }
+  // what is left of the share: up to eight more loads, issued together (no serial tail)
+  u32x4_t v[8];
+#pragma unroll
+  for (int u = 0; u < 8; u++) {
+    const size_t j = i + (size_t)u * blockDim.x;
+    v[u] = u32x4_t{0, 0, 0, 0};
+    if (j < end) v[u] = __builtin_nontemporal_load(p + j);
+  }
+#pragma unroll
+  for (int u = 0; u < 8; u++) acc ^= v[u];
+  return acc;
+}
+__global__ __launch_bounds__(512) void read_probe_kernel(const u32x4_t* __restrict__ p, size_t n16, uint32_t* __restrict__ sink) {
+  const u32x4_t a = read_share(p, n16);
+  // keeps the loads alive; the stored value is never looked at
+  if ((a.x ^ a.y ^ a.z ^ a.w) == 0x9E3779B9u) sink[0] = 1u;
+}
+
 int launch_dequantize(ihipStream_t* s, const WeightView& w, float* out_dev) {
   dim3 grid((w.n + 255) / 256, w.k / 32);
   hipLaunchKernelGGL(dequantize_kernel, grid, dim3(256), 0, s, w, out_dev);
@@ -302,6 +337,17 @@ int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, ui
                     void* quants) {
   dim3 grid((n + 255) / 256, k / 32);
   hipLaunchKernelGGL(quantize_kernel, grid, dim3(256), 0, s, fmt, w_dev, k, n, meta, quants);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_read_probe(ihipStream_t* s, const WeightView& w, int num_cus, uint32_t* sink) {
+  // A weight's scales and quants share one allocation, scales first, about 1 KiB of padding
+  // between them: one span from the first scale to the last quant covers both.
+  const size_t nb = (size_t)(w.k / 32) * w.n;
+  const char* const end = (const char*)w.quants + nb * (w.fmt == MGN_FMT_Q8 ? 32 : 16);
+  const size_t n16 = (size_t)(end - (const char*)w.meta) / 16;
+  hipLaunchKernelGGL(read_probe_kernel, dim3((unsigned)num_cus), dim3(512), 0, s, (const u32x4_t*)w.meta, n16, sink);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

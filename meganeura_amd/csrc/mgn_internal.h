@@ -83,6 +83,8 @@ int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, ui
                     void* quants);
 // in[rows][cols] -> out[cols][rows] (f32); cols at most 65535 * 32
 int launch_transpose(ihipStream_t* s, const float* in, float* out, uint32_t rows, uint32_t cols);
+// measurement aid: one pass of plain reads over the weight's quants and scales
+int launch_read_probe(ihipStream_t* s, const WeightView& w, int num_cus, uint32_t* sink);
 int launch_matmul_generic(ihipStream_t* s, const LaunchArgs& a);
 bool gemv_supported(const LaunchArgs& a);
 int launch_matmul_gemv(ihipStream_t* s, const LaunchArgs& a);

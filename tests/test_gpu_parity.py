@@ -538,6 +538,30 @@ def test_matmul_loop_is_the_same_calls_in_a_row(ctx, orc):
         w.free()
 
 
+def test_weight_read_loop_leaves_results_alone(ctx, orc):
+    """mgn_weight_read_loop (a timing aid: plain reads of the packed bytes) runs on weights of
+    both formats, the smallest included, and a K-part matmul enqueued right behind it, whose
+    partial sums use the workspace the probe's sink lives in, still gives the oracle's result."""
+    with pytest.raises(capi.MgnError):
+        ctx.weight_read_loop([], 3)
+    tiny = ctx.weight(Q8, synth.normal(975, 32, 0.02).reshape(32, 1))
+    ctx.weight_read_loop([tiny], 3)
+    m, k, n = 4, 14336, 70
+    for fmt in (Q4, Q8):
+        w = synth.normal(976 + fmt, k * n, 0.02).reshape(k, n)
+        x = synth.normal(978, m * k).reshape(m, k)
+        wt = ctx.weight(fmt, w)
+        a = ctx.upload(x)
+        c = ctx.buffer(m * n * 4)
+        ctx.weight_read_loop([wt, tiny], 7)
+        ctx.matmul_q(a, wt, c, m)
+        ctx.weight_read_loop([wt], 2)
+        got = c.download(np.float32, m * n).reshape(m, n)
+        orc.assert_close(got, orc.matmul_packed(fmt, x, orc.quantize(fmt, w), n), REL, ABS)
+        a.free(); c.free(); wt.free()
+    tiny.free()
+
+
 def test_zero_rows_is_a_no_op(ctx):
     wt = ctx.weight(Q4, synth.normal(970, 64 * 8, 0.02).reshape(64, 8))
     a = ctx.buffer(4 * 64)
