@@ -70,6 +70,13 @@ MEASURED_TRAFFIC_BYTES = {
     "c5_q4_m16_4096x14336": 48.3e6,
     "c4_q4_prefill_up_512x1024x3072": 18.9e6,
     "c3_q4_lm_head_576x49152": 18.03e6,
+    "c1_q8_up_576x1536": 1.17e6,
+    "c2_q4_gate_up_576x3072": 1.32e6,
+    "c2_q4_down_1536x576_add": 0.72e6,
+    "c4_q4_prefill_down_512x3072x1024": 25.5e6,
+    "c5_q4_m1_14336x4096": 37.4e6,
+    "c5_q4_m4_4096x14336": 37.8e6,
+    "c5_q8_m16_4096x14336": 80.9e6,
 }
 
 
