@@ -400,6 +400,8 @@ def main():
                 row[label + "_GBs"] = w.bytes / (t * 1e-3) / 1e9
                 row[label + "_TFLOPs"] = w.flops / (t * 1e-3) / 1e12
                 row["bytes"] = w.bytes
+                if rot:  # the read-only pass over the same rotating copies, see read_floor above
+                    row["read_floor_us"] = w.read_floor(max(50, args.steps // 2), args.warmup) * 1e3
                 w.free()
             row["cold_pct_hbm"] = 100.0 * row["cold_GBs"] / HBM_PEAK_GBS
             rows.append(row)
