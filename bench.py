@@ -66,7 +66,7 @@ HEADLINE = "c5_q4_m1_4096x14336"
 MEASURED_TRAFFIC_BYTES = {
     "c5_q4_m1_4096x14336": 37.02e6,
     "c5_q8_m1_4096x14336": 63.59e6,
-    "c5_q4_m4_14336x4096": 39.3e6,
+    "c5_q4_m4_14336x4096": 39.6e6,
     "c5_q4_m16_4096x14336": 48.3e6,
     "c4_q4_prefill_up_512x1024x3072": 18.9e6,
     "c3_q4_lm_head_576x49152": 18.03e6,

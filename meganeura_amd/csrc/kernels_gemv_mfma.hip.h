@@ -838,11 +838,16 @@ bool plan_mfma_gemv(const LaunchArgs& x, uint32_t mrows, MfmaGemvPlan* out) {
   if (plan_one_part(x.w.fmt, x.w.k, nquads, mrows, x.num_cus, !plain, out)) return true;
   if (!plain || !x.scratch || !x.counters) return false;
   const uint32_t steps_total = (x.w.k / 32 + 15) / 16;
-  for (uint32_t kp = 2; kp <= 8; kp++) {
+  // Four parts first: a workgroup then prepares a quarter of the activations and mostly needs no
+  // K split of its own, which outweighs the two further partial sums per output (measured on
+  // twelve shapes with K from 9728 to 32768: 2 to 25 % faster than two parts on ten, 3 % slower
+  // on K = 11008).  Three, six and seven parts leave a ragged last round of workgroups.
+  static const uint32_t kPartOrder[] = {4, 2, 3, 5, 6, 7, 8};
+  for (const uint32_t kp : kPartOrder) {
     // parts of a whole number of 16-block steps; the last one may be short, never empty
     const uint32_t part_steps = (steps_total + kp - 1) / kp;
     if ((kp - 1) * part_steps >= steps_total) continue;
-    if ((size_t)kp * mrows * x.w.n * sizeof(float) > x.scratch_bytes) return false;
+    if ((size_t)kp * mrows * x.w.n * sizeof(float) > x.scratch_bytes) continue;
     MfmaGemvPlan p;
     if (!plan_one_part(x.w.fmt, part_steps * 512, nquads, mrows, std::max(1, x.num_cus / (int)kp), true, &p)) continue;
     if (p.qpw != 1 || p.grid > x.n_counters) continue;

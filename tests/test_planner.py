@@ -119,7 +119,7 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
     head = capi.matmul_plan(Q4, 1, 4096, 14336)
     assert (head.grid[0], head.threads, head.steps, head.k_splits, head.full_steps) == (256, 896, 8, 1, 1)
     tall = capi.matmul_plan(Q4, 4, 14336, 4096)
-    assert tall.k_parts == 2 and tall.workspace_bytes == 2 * 4 * 4096 * 4
+    assert tall.k_parts == 4 and tall.workspace_bytes == 4 * 4 * 4096 * 4
     # K = 18944 is 37 steps of 16 blocks: more activation chunks than a workgroup has threads for
     assert capi.matmul_plan(Q4, 1, 18944, 3584).route == GEMV_MFMA
     assert capi.matmul_plan(Q4, 4, 11008, 4096).k_parts >= 2
