@@ -785,13 +785,14 @@ bool plan_one_part(int fmt, uint32_t k, uint32_t nquads, uint32_t mrows, int num
   if (per_cu > max_wnc) {
     // Several rounds of workgroups.  With the largest workgroups the last round may be nearly
     // empty (296 workgroups of 16 waves: 216 CUs idle while 40 work through a second one);
-    // when that wastes more than a fifth of the time, as many workgroups go to every CU, each
+    // when that wastes more than an eighth of the time, as many workgroups go to every CU, each
     // as small as that allows.  (Smaller workgroups prepare the activations more often, so a
-    // better filled last round is left alone: 8192 x 28672 lost 13 % to this.)
+    // better filled last round is left alone: 8192 x 28672, an eighth exactly, lost 10-13 % to
+    // this, while 5120 x 13824, 80 CUs idle in the second of two rounds, gains 3 %.)
     const uint32_t grid_max = (wave_quads + max_wnc - 1) / max_wnc;
     const uint32_t rounds = (grid_max + num_cus - 1) / num_cus;
     const uint32_t last = grid_max - (rounds - 1) * num_cus;  // workgroups in the last round
-    if ((num_cus - last) * 5 > (uint32_t)num_cus * rounds) per_cu = (wave_quads + num_cus * rounds - 1) / (num_cus * rounds);
+    if ((num_cus - last) * 8 > (uint32_t)num_cus * rounds) per_cu = (wave_quads + num_cus * rounds - 1) / (num_cus * rounds);
   }
   p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, per_cu));
 #ifdef MGN_TRACE  // development build only: force the waves per workgroup
