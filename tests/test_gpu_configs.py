@@ -16,14 +16,26 @@ def ctx():
     c.close()
 
 
+def assert_dequant_bits(orc, wt, fmt, packed, k, n):
+    """The device's dequantized weight against the oracle's, bit for bit, at the weight's full size
+    (the kernel's block indexing depends on the size: every element is compared, none sampled)."""
+    got = bits(wt.dequantize())
+    want = bits(orc.dequantize(fmt, packed, k, n))
+    assert got.shape == want.shape == (k, n)
+    if not np.array_equal(got, want):
+        bad = np.argwhere(got != want)
+        r, c = bad[0]
+        raise AssertionError(f"{len(bad)} of {k * n} dequantized elements differ; first at [{r}, {c}]: "
+                             f"{got[r, c]:#010x} != {want[r, c]:#010x}")
+
+
 def check(ctx, orc, fmt, x, w, d=None, f16=False, routes=("auto",), check_weight=True):
     k, n = w.shape
     packed = orc.quantize(fmt, w)
     wt = ctx.weight(fmt, w)
     if check_weight:
         assert (wt.export_ref() == packed).all()
-        if k * n <= 1 << 24:
-            assert (bits(wt.dequantize()) == bits(orc.dequantize(fmt, packed, k, n))).all()
+        assert_dequant_bits(orc, wt, fmt, packed, k, n)
     xo = x.astype(np.float16).astype(np.float32) if f16 else x
     want = orc.matmul_packed(fmt, xo, packed, n, d)
     for route in routes:
@@ -67,6 +79,7 @@ def test_c5_llama_ffn(ctx, orc, fmt, k, n):
     wt = ctx.weight(fmt, w)
     assert (wt.export_ref() == packed).all()
     del w
+    assert_dequant_bits(orc, wt, fmt, packed, k, n)
     for m in (1, 4, 16):
         x = synth.activations(5, m, k, which=m)
         want = orc.matmul_packed(fmt, x, packed, n)
