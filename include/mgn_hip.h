@@ -165,6 +165,22 @@ mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, con
 mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weight* w,
                              const mgn_buf* d, mgn_buf* c, uint32_t m);
 
+/* mgn_matmul_q for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Shapes whose K is cut into parts for different workgroups keep their partial sums and arrival
+ * counters in a workspace; mgn_matmul_q uses one the context allocated, this entry uses an
+ * array inside the library's own device image (MGN_STATIC_WORKSPACE_BYTES = 4 MiB of partial
+ * sums plus 4096 counters, held on every device the library runs on until the process ends)
+ * and calls no hipMalloc / hipFree or any other allocating routine.  Same plan, same kernels
+ * and bit-identical results as mgn_matmul_q; MGN_EUNSUPPORTED, with the byte counts in
+ * mgn_last_error, when the shape's partial sums do not fit the static array.  All contexts
+ * of a device share the array: calls that overlap on one device (two contexts, two threads)
+ * race; calls on one context are ordered by its stream.  The arrival counters are cleared by a
+ * small fill kernel in front of every launch that uses them. */
+#define MGN_STATIC_WORKSPACE_BYTES ((size_t)4 << 20)
+mgn_status mgn_matmul_q_static(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d,
+                               mgn_buf* c, uint32_t m);
+
 /* The same followed by unary operations on every output element, first to last:
  * C = f_n(... f_1(A x W + D)).  Stands in for a matmul dispatch that carries an epilogue
  * (compile.rs:915-1035 fuse_epilogues folds a Relu / Sigmoid / Neg / Silu that is the only

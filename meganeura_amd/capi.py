@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_DIR, "libmgn_hip.so")
 
 OK, EINVAL, ENOMEM, EHIP, ENOTFOUND, ENODEVICE, EUNSUPPORTED, ERANGE = range(8)
 FMT_Q4, FMT_Q8 = 0, 1
+STATIC_WORKSPACE_BYTES = 4 << 20  # MGN_STATIC_WORKSPACE_BYTES
 ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA = range(5)
 
 # every symbol include/mgn_hip.h and include/mgn_session.h declare
@@ -22,7 +23,7 @@ HIP_SYMBOLS = [
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_weight_save", "mgn_weight_load", "mgn_matmul_q",
-    "mgn_matmul_q_f16a", "mgn_matmul_q_epilogue", "mgn_matmul_q_at", "mgn_matmul_q_loop", "mgn_weight_read_loop", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
+    "mgn_matmul_q_f16a", "mgn_matmul_q_static", "mgn_matmul_q_epilogue", "mgn_matmul_q_at", "mgn_matmul_q_loop", "mgn_weight_read_loop", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
     "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [
@@ -104,6 +105,7 @@ def load():
         "mgn_weight_info": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(sz), C.POINTER(sz)]),
         "mgn_matmul_q": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_f16a": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
+        "mgn_matmul_q_static": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_epilogue": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32, vp, C.c_size_t]),
         "mgn_matmul_q_at": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32, vp, C.c_size_t]),
         "mgn_matmul_q_plan": (C.c_int, [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.c_int, vp]),
@@ -314,6 +316,10 @@ class Context:
 
     def matmul_q(self, a, w, c, m, d=None):
         self.check(self.lib.mgn_matmul_q(self.h, a.h, w.h, d.h if d is not None else None, c.h, m))
+
+    def matmul_q_static(self, a, w, c, m, d=None):
+        """mgn_matmul_q on the library's static workspace: no device allocation in the call."""
+        self.check(self.lib.mgn_matmul_q_static(self.h, a.h, w.h, d.h if d is not None else None, c.h, m))
 
     def matmul_q_f16a(self, a, w, c, m, d=None):
         self.check(self.lib.mgn_matmul_q_f16a(self.h, a.h, w.h, d.h if d is not None else None, c.h, m))

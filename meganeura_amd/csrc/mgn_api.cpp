@@ -5,13 +5,46 @@
 #include <cstdlib>
 #include <cmath>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
 
 #include "mgn_internal.h"
 
+// ---- split-K workspace in the library's own image, for callers that cannot allocate ----
+// mgn_matmul_q_static hands this array to the kernels in place of the context's workspace.
+// The name below is a host-side stand-in: the device address comes from hipGetSymbolAddress,
+// once per device (every device holds its own copy), and only that pointer is passed on.
+constexpr size_t kStaticPartialBytes = MGN_STATIC_WORKSPACE_BYTES;  // partial sums of K parts
+constexpr uint32_t kStaticCounters = mgn::kWorkspaceCounters;      // arrival counters behind them
+static __device__ __align__(256) unsigned char scratch[kStaticPartialBytes + kStaticCounters * sizeof(uint32_t)];
+
+__global__ void clear_words_kernel(uint32_t* p, uint32_t n) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+void* g_static_scratch[kMaxDevices] = {};  // device address of `scratch`, per device ordinal
+
+// With `device` current: the address of this device's copy of `scratch` (looked up once).
+hipError_t static_scratch_for(int device, void** out) {
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (!g_static_scratch[device]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_static_scratch[device] = p;
+  }
+  *out = g_static_scratch[device];
+  return hipSuccess;
+}
 
 thread_local std::string g_create_error;
 
@@ -131,6 +164,10 @@ mgn_status mgn_ctx_create(int device_id, mgn_ctx** out) {
   if (!ctx) return fail(nullptr, MGN_ENOMEM, "out of host memory");
   ctx->device = device_id;
   ctx->num_cus = prop.multiProcessorCount;
+  if ((e = static_scratch_for(device_id, &ctx->static_scratch)) != hipSuccess) {
+    delete ctx;
+    return hip_fail(nullptr, "hipGetSymbolAddress(static workspace)", e);
+  }
   if ((e = hipStreamCreate(&ctx->stream)) != hipSuccess || (e = hipEventCreate(&ctx->ev_start)) != hipSuccess ||
       (e = hipEventCreate(&ctx->ev_stop)) != hipSuccess) {
     mgn_ctx_destroy(ctx);
@@ -493,7 +530,7 @@ mgn_status mgn_weight_load(mgn_ctx* ctx, const char* path, mgn_weight** out) {
 
 static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, const mgn_weight* w, const mgn_buf* d,
                               mgn_buf* c, uint32_t m, int pro_kind = mgn::kProNone, const mgn_buf* norm_weight = nullptr,
-                              float eps = 0.0f, uint32_t epilogue = 0) {
+                              float eps = 0.0f, uint32_t epilogue = 0, bool static_workspace = false) {
   if (!ctx || !a || !w || !c) return fail(ctx, MGN_EINVAL, "null argument");
   if (m == 0) return MGN_OK;
   const size_t k = w->rows, n = w->cols;
@@ -529,6 +566,30 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
     else if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV_VALU;
     else route = MGN_ROUTE_GENERIC;
   }
+  if (static_workspace) {
+    // Same plan as the allocating entry point (the planners see the same workspace limits), run
+    // on the library's static array if the plan's partial sums fit it; refused otherwise.
+    mgn_plan_info plan{};
+    const bool parts = route == MGN_ROUTE_GEMV_MFMA   ? mgn::describe_gemv_mfma(x, &plan)
+                       : route == MGN_ROUTE_GEMM_MFMA ? mgn::describe_gemm_mfma(x, &plan)
+                                                      : false;
+    const uint64_t need = parts ? plan.workspace_bytes : 0;
+    if (need > kStaticPartialBytes)
+      return fail(ctx, MGN_EUNSUPPORTED,
+                  "mgn_matmul_q_static: this shape's K parts need " + std::to_string(need) +
+                      " bytes of workspace, the static one holds " + std::to_string(kStaticPartialBytes) +
+                      "; use mgn_matmul_q");
+    x.scratch = ctx->static_scratch;
+    x.counters = (uint32_t*)((char*)ctx->static_scratch + kStaticPartialBytes);
+    if (need > 0) {
+      // every call on this device shares the array: the arrival counters must start at zero
+      // whatever an earlier call left (a fill kernel, not a memset node: safe under graph capture)
+      hipLaunchKernelGGL(clear_words_kernel, dim3((kStaticCounters + 255) / 256), dim3(256), 0, ctx->stream, x.counters,
+                         kStaticCounters);
+      const hipError_t le = hipGetLastError();
+      if (le != hipSuccess) return hip_fail(ctx, "counter clear launch", le);
+    }
+  }
   int rc;
   switch (route) {
     case MGN_ROUTE_GEMV_VALU:
@@ -554,6 +615,11 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
 mgn_status mgn_matmul_q(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
                         uint32_t m) {
   return matmul_impl(ctx, a, false, w, d, c, m);
+}
+
+mgn_status mgn_matmul_q_static(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
+                               uint32_t m) {
+  return matmul_impl(ctx, a, false, w, d, c, m, mgn::kProNone, nullptr, 0.0f, 0, true);
 }
 
 mgn_status mgn_matmul_q_epilogue(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,

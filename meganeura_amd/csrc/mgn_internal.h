@@ -114,6 +114,7 @@ struct mgn_ctx {
   uint32_t n_counters = 0;
   uint32_t* range_flag_host = nullptr;  // pinned, mapped: written by kernels, read at sync points
   uint32_t* range_flag_dev = nullptr;   // the same word as the device sees it
+  void* static_scratch = nullptr;       // this device's copy of the library's static workspace (mgn_matmul_q_static)
   void* at_stage = nullptr;             // transposed activations of the A^T matmul forms, grown on demand
   size_t at_stage_bytes = 0;
   std::string err;
