@@ -11,9 +11,17 @@ cache: the figure is an HBM figure.  Inputs are resident in HBM before the
 timed region; the region is bracketed by HIP events recorded on the stream the
 kernels run on, with a device synchronisation on both sides.
 
-Prints ONE JSON line on stdout.  `--sweep` additionally measures every
-BASELINE configuration (cache-cold and cache-warm) and writes the table to
-stderr and, with `--sweep-out FILE`, as JSON to that file.
+Timing method (examples/matmul_throughput.rs:114-127 is the model): the weight
+copies are created and touched, the device is pre-heated with at least 100 ms
+of launches, `--warmup` further untimed steps follow, then `--steps` launches
+are timed `--repeats` times (at least 5); `ms_per_step` is the median repeat,
+the fastest and slowest are reported beside it.  The same line carries, under
+`configs`, every BASELINE workload timed the same way (200 launches per
+repeat, median of 5).
+
+Prints ONE JSON line on stdout.  `--sweep` additionally measures the cache-warm
+figures and the quantizers and writes the table to stderr and, with
+`--sweep-out FILE`, as JSON to that file.
 """
 import argparse
 import json
@@ -43,6 +51,8 @@ WORKLOADS = {
     "c5_q8_m16_4096x14336": (Q8, 16, 4096, 14336, False, False, 5),
     "c5_q4_m4_14336x4096": (Q4, 4, 14336, 4096, False, False, 5),
     "c5_q4_m16_14336x4096": (Q4, 16, 14336, 4096, False, False, 5),
+    "c5_q8_m4_14336x4096": (Q8, 4, 14336, 4096, False, False, 5),
+    "c5_q8_m16_14336x4096": (Q8, 16, 14336, 4096, False, False, 5),
     "c3_q4_lm_head_576x49152": (Q4, 1, 576, 49152, False, False, 3),
     "c1_q8_up_576x1536": (Q8, 1, 576, 1536, False, False, 1),
     "c2_q4_q_576x576": (Q4, 1, 576, 576, False, False, 2),
@@ -89,20 +99,58 @@ def algorithmic_bytes(fmt, m, k, n, resid, f16):
     return wbytes + (2 if f16 else 4) * m * k + 4 * m * n * (2 if resid else 1)
 
 
+class WeightSets:
+    """Host weights, packed bytes and rotating device copies, shared by the workloads that use
+    the same (format, K, N): the three M values of a C5 weight need one set, not three."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+        self.host = {}
+        self.sets = {}
+
+    def host_weight(self, cfg, k, n):
+        from meganeura_amd import synth
+
+        key = (cfg, k * n)
+        if key not in self.host:
+            self.host[key] = synth.weights(cfg, 1, k * n).reshape(-1)
+        return self.host[key].reshape(k, n)  # [K,N] and [N,K] shapes of one size share the draws
+
+    def get(self, fmt, cfg, k, n, min_rotate_bytes):
+        from meganeura_amd import capi
+
+        dev_bytes = (k // 32) * n * (20 if fmt == Q4 else 34)
+        copies = max(2, -(-min_rotate_bytes // dev_bytes)) if min_rotate_bytes else 1
+        key = (fmt, cfg, k, n)
+        if key not in self.sets:
+            w = self.host_weight(cfg, k, n)
+            self.sets[key] = (w, capi.quantize_ref(fmt, w), [])
+        w, packed, devs = self.sets[key]
+        while len(devs) < copies:
+            devs.append(self.ctx.weight_from_packed(fmt, packed, k, n))
+        return w, packed, devs[:copies]
+
+    def drop(self, fmt, cfg, k, n):
+        for wt in self.sets.pop((fmt, cfg, k, n), (None, None, []))[2]:
+            wt.free()
+
+    def free(self):
+        for key in list(self.sets):
+            self.drop(*key)
+
+
 class Workload:
-    def __init__(self, ctx, name, min_rotate_bytes):
-        from meganeura_amd import capi, synth
+    def __init__(self, ctx, name, min_rotate_bytes, sets=None):
+        from meganeura_amd import synth
 
         self.name = name
         fmt, m, k, n, resid, f16, cfg = WORKLOADS[name]
         self.fmt, self.m, self.k, self.n, self.resid, self.f16 = fmt, m, k, n, resid, f16
         self.ctx = ctx
-        self.w_host = synth.weights(cfg, k, n)
+        self.own_sets = sets is None
+        self.sets = sets if sets is not None else WeightSets(ctx)
+        self.w_host, self.packed, self.weights = self.sets.get(fmt, cfg, k, n, min_rotate_bytes)
         self.x_host = synth.activations(cfg, m, k)
-        self.packed = capi.quantize_ref(fmt, self.w_host)
-        dev_bytes = (k // 32) * n * (20 if fmt == Q4 else 34)
-        copies = max(2, -(-min_rotate_bytes // dev_bytes)) if min_rotate_bytes else 1
-        self.weights = [ctx.weight_from_packed(fmt, self.packed, k, n) for _ in range(copies)]
         xs = self.x_host.astype(np.float16) if f16 else self.x_host
         self.a = ctx.upload(xs)
         self.c = ctx.buffer(m * n * 4)
@@ -110,53 +158,114 @@ class Workload:
         self.d = ctx.upload(self.d_host) if resid else None
         self.bytes = algorithmic_bytes(fmt, m, k, n, resid, f16)
         self.flops = 2.0 * m * n * k
-        self.fn = ctx.matmul_q_f16a if f16 else ctx.matmul_q
+        self.is_gemm = m > 16
+        self.rot = ctx.rotation(self.weights)  # built once: nothing is prepared on the host inside a timed region
         self.i = 0
-
-    def step(self):
-        w = self.weights[self.i % len(self.weights)]
-        self.i += 1
-        self.fn(self.a, w, self.c, self.m, self.d)
 
     def loop(self, steps):
         """`steps` calls enqueued from C (no interpreter between the launches), weights in rotation."""
         if steps <= 0:
             return
-        n = len(self.weights)
-        order = [self.weights[(self.i + j) % n] for j in range(n)]
-        self.ctx.matmul_q_loop(self.a, order, self.c, self.m, steps, self.d, self.f16)
+        self.ctx.matmul_q_loop(self.a, self.rot, self.c, self.m, steps, self.d, self.f16, first=self.i)
         self.i += steps
 
-    def run(self, steps, warmup):
-        self.loop(warmup)
+    def preheat(self, min_ms, loop=None):
+        """Launches until `min_ms` of wall clock have passed and every weight copy has been read at
+        least twice: clocks are up and no copy is first touched inside a timed region."""
+        loop = loop or self.loop
+        t0 = time.perf_counter()
+        batch = max(2 * len(self.weights), 64)
+        while True:
+            loop(batch)
+            self.ctx.sync()
+            if (time.perf_counter() - t0) * 1e3 >= min_ms:
+                break
+
+    def timed(self, steps, loop=None):
+        loop = loop or self.loop
         self.ctx.sync()
         self.ctx.timer_start()
-        self.loop(steps)
+        loop(steps)
         ms = self.ctx.timer_stop()  # waits for the stop event
-        self.ctx.sync()
         return ms / steps
 
-    def read_floor(self, steps, warmup):
-        """ms per launch of a kernel that reads the same weight copies in the same rotation and
-        computes nothing: one launch plus one pass over the packed bytes, on this box."""
-        self.ctx.weight_read_loop(self.weights, warmup)
-        self.ctx.sync()
-        self.ctx.timer_start()
-        self.ctx.weight_read_loop(self.weights, steps)
-        ms = self.ctx.timer_stop()
-        self.ctx.sync()
-        return ms / steps
+    def measure(self, steps, warmup, repeats, preheat_ms=100.0, loop=None):
+        """Median, fastest and slowest of `repeats` timed regions of `steps` launches, in ms per step."""
+        self.preheat(preheat_ms, loop)
+        (loop or self.loop)(warmup)
+        t = sorted(self.timed(steps, loop) for _ in range(repeats))
+        return {"median": t[len(t) // 2] if len(t) % 2 else 0.5 * (t[len(t) // 2 - 1] + t[len(t) // 2]),
+                "min": t[0], "max": t[-1], "repeats": repeats}
+
+    def read_loop(self, steps):
+        if steps > 0:
+            self.ctx.weight_read_loop(self.rot, steps, first=self.i)
+            self.i += steps
 
     def output(self):
         return self.c.download(np.float32, self.m * self.n).reshape(self.m, self.n)
 
+    def check(self):
+        """The last launch's result against the oracle, within the matmul bar."""
+        import oracle
+
+        x = self.x_host.astype(np.float16).astype(np.float32) if self.f16 else self.x_host
+        want = oracle.matmul_packed(self.fmt, x, oracle.quantize(self.fmt, self.w_host), self.n, self.d_host)
+        oracle.assert_close(self.output(), want, 1e-3, 1e-4)
+        return want
+
+    def roofline(self, ms):
+        gbs = self.bytes / (ms * 1e-3) / 1e9
+        tflops = self.flops / (ms * 1e-3) / 1e12
+        if self.is_gemm:
+            return {"bound": "mfma", "achieved": tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": tflops / MFMA_F16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(self.name)}
+        return {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(self.name)}
+
     def free(self):
-        for w in self.weights:
-            w.free()
         self.a.free()
         self.c.free()
         if self.d is not None:
             self.d.free()
+        if self.own_sets:
+            self.sets.free()
+
+
+# every BASELINE workload, in the order of BASELINE.json's configs (the sweep-only entries are left out)
+CONFIG_LINE = [
+    "c1_q8_up_576x1536",
+    "c2_q4_q_576x576", "c2_q4_kv_576x192", "c2_q4_o_576x576_add", "c2_q4_gate_up_576x3072", "c2_q4_down_1536x576_add",
+    "c3_q4_lm_head_576x49152",
+    "c4_q4_prefill_up_512x1024x3072", "c4_q4_prefill_down_512x3072x1024",
+    "c5_q4_m1_4096x14336", "c5_q4_m4_4096x14336", "c5_q4_m16_4096x14336",
+    "c5_q4_m1_14336x4096", "c5_q4_m4_14336x4096", "c5_q4_m16_14336x4096",
+    "c5_q8_m1_4096x14336", "c5_q8_m4_4096x14336", "c5_q8_m16_4096x14336",
+    "c5_q8_m1_14336x4096", "c5_q8_m4_14336x4096", "c5_q8_m16_14336x4096",
+]
+
+
+def config_table(ctx, sets, steps=200, repeats=5, preheat_ms=20.0):
+    """Cache-cold time and roofline fraction of every BASELINE workload: `steps` launches per timed
+    region after a pre-heat, median of `repeats`, each result checked against the oracle."""
+    table = {}
+    last_key = None
+    for name in CONFIG_LINE:
+        fmt, m, k, n, resid, f16, cfg = WORKLOADS[name]
+        if last_key is not None and last_key != (fmt, cfg, k, n):
+            sets.drop(*last_key)  # the rotating copies of the previous weight are no longer needed
+        last_key = (fmt, cfg, k, n)
+        wl = Workload(ctx, name, 512 << 20, sets)
+        r = wl.measure(steps, 20, repeats, preheat_ms)
+        wl.check()
+        roof = wl.roofline(r["median"])
+        table[name] = {"us": r["median"] * 1e3, "us_min": r["min"] * 1e3, "us_max": r["max"] * 1e3,
+                       "bound": roof["bound"], "achieved": roof["achieved"], "unit": roof["unit"], "frac": roof["frac"],
+                       "algorithmic_bytes": wl.bytes}
+        wl.free()
+    if last_key is not None:
+        sets.drop(*last_key)
+    return table
 
 
 def decode_layer_times(steps, warmup, layers=8):
@@ -293,10 +402,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--repeats", type=int, default=0,
+                    help="timed regions of --steps launches each (median reported); default: at least 5, "
+                         "more when --steps is small, so that about 2000 launches are timed in all")
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
-    ap.add_argument("--sweep", action="store_true", help="also measure every configuration (stderr)")
+    ap.add_argument("--sweep", action="store_true", help="also measure cache-warm figures and the quantizers (stderr)")
     ap.add_argument("--sweep-out", default=None, help="with --sweep: also write the table to this JSON file")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration table of the JSON line")
     ap.add_argument("--profile", action="store_true",
                     help="for rocprofv3 runs: only the timed cache-cold workload plus one 256 MiB device copy "
                          "(a known size to calibrate FETCH_SIZE / WRITE_SIZE against); no CPU leg, no warm leg")
@@ -304,28 +417,27 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (column-parallel "
                  "sharding needs no exchange); run with --gpus 1")
+    if args.steps <= 0:
+        sys.exit("--steps must be positive")
+    repeats = args.repeats if args.repeats > 0 else max(5, min(100, -(-2000 // args.steps)))
 
     from meganeura_amd import capi
     import oracle
 
     ctx = capi.Context(0)
-    wl = Workload(ctx, args.workload, 512 << 20)
-    ms = wl.run(args.steps, args.warmup)
-    got = wl.output()
+    sets = WeightSets(ctx)
+    wl = Workload(ctx, args.workload, 512 << 20, sets)
+    timing = wl.measure(args.steps, args.warmup, repeats, preheat_ms=20.0 if args.profile else 100.0)
+    ms = timing["median"]
+    want = wl.check()  # the timed kernel's result against the oracle, before anything is reported
 
-    floor_ms = None if args.profile else wl.read_floor(args.steps, args.warmup)
+    floor = None if args.profile else wl.measure(args.steps, args.warmup, repeats, preheat_ms=20.0, loop=wl.read_loop)
 
-    is_gemm = wl.m > 16
     gbs = wl.bytes / (ms * 1e-3) / 1e9
     tflops = wl.flops / (ms * 1e-3) / 1e12
 
-    # the timed kernel's result is checked against the oracle before it is reported
-    x = wl.x_host.astype(np.float16).astype(np.float32) if wl.f16 else wl.x_host
-    want = oracle.matmul_packed(wl.fmt, x, oracle.quantize(wl.fmt, wl.w_host), wl.n, wl.d_host)
-    oracle.assert_close(got, want, 1e-3, 1e-4)
-
     if args.profile:
-        args.no_cpu = True
+        args.no_cpu = args.no_configs = True
         cal = 256 << 20
         src, dst = ctx.buffer(cal), ctx.buffer(cal)
         ctx.copy(dst, src, cal)
@@ -339,28 +451,25 @@ def main():
         oracle.assert_close(cpu_out, want, 1e-3, 1e-4)
 
     # cache-warm figure for the same shape (one weight, reused every step)
-    warm_ms = copy_gbs = None
+    warm = copy_gbs = None
     if not args.profile:
-        warm = Workload(ctx, args.workload, 0)
-        warm_ms = warm.run(args.steps, args.warmup)
-        warm.free()
+        ww = Workload(ctx, args.workload, 0, sets)
+        warm = ww.measure(args.steps, args.warmup, repeats, preheat_ms=20.0)
+        ww.free()
         copy_gbs = copy_ceiling(ctx)
 
-    if is_gemm:
-        roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": tflops / MFMA_F16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
-    else:
-        roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)}
     line = {
         "metric": "Q4/Q8 GEMV HBM GB/s (% of peak) + us/call; prefill dequant-GEMM TFLOP/s",
-        "value": tflops if is_gemm else gbs,
-        "unit": "TFLOP/s" if is_gemm else "GB/s",
+        "value": tflops if wl.is_gemm else gbs,
+        "unit": "TFLOP/s" if wl.is_gemm else "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms,
         "us_per_call": ms * 1e3,
+        "repeats": repeats,
+        "us_per_call_min": timing["min"] * 1e3,
+        "us_per_call_max": timing["max"] * 1e3,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -372,41 +481,54 @@ def main():
             "m": wl.m, "k": wl.k, "n": wl.n,
             "algorithmic_bytes": wl.bytes,
             "cache": f"cold: rotating {len(wl.weights)} weight copies",
+            "timing": f"median of {repeats} timed regions of {args.steps} back-to-back launches, after a pre-heat of "
+                      ">= 100 ms of launches over every copy and the warm-up steps",
         },
-        "roofline": roof,
+        "roofline": wl.roofline(ms),
         "cpu_baseline": cpu,
-        "cache_warm": None if warm_ms is None else
-        {"us_per_call": warm_ms * 1e3, "GB/s": wl.bytes / (warm_ms * 1e-3) / 1e9},
+        "cache_warm": None if warm is None else
+        {"us_per_call": warm["median"] * 1e3, "GB/s": wl.bytes / (warm["median"] * 1e-3) / 1e9},
         "pct_of_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
         "copy_ceiling": None if copy_gbs is None else
         {"GB/s": copy_gbs, "what": "256 MiB device-to-device copy, bytes read + written per second",
          "pct_of_it": 100.0 * gbs / copy_gbs},
-        "read_floor": None if floor_ms is None else
-        {"us_per_launch": floor_ms * 1e3, "GB/s": wl.bytes / (floor_ms * 1e-3) / 1e9,
+        "read_floor": None if floor is None else
+        {"us_per_launch": floor["median"] * 1e3, "GB/s": wl.bytes / (floor["median"] * 1e-3) / 1e9,
          "what": "a kernel that only reads the same rotating weight copies (quants and scales), timed the same way: "
                  "one launch plus one pass over the packed bytes on this box",
-         "pct_of_it": 100.0 * floor_ms / ms},
+         "pct_of_it": 100.0 * floor["median"] / ms},
     }
     wl.free()
+
+    if not args.no_configs:
+        line["configs"] = config_table(ctx, sets)
+        layer = decode_layer_times(200, 20)
+        line["configs"]["c2_q4_decode_layer_session"] = {
+            "us": layer["fused_us_per_layer"], "unfused_us": layer["unfused_us_per_layer"],
+            "launches": layer["fused_launches_per_layer"], "dispatches": layer["dispatches_per_layer"],
+            "what": "one SmolLM2-135M decode layer's matmuls, norms and SwiGLU through the Graph/Session surface, per layer"}
 
     if args.sweep:
         rows = []
         for name in WORKLOADS:
             row = {"workload": name}
             for label, rot in (("cold", 512 << 20), ("warm", 0)):
-                w = Workload(ctx, name, rot)
-                t = w.run(max(50, args.steps // 2), args.warmup)
+                w = Workload(ctx, name, rot, sets)
+                r = w.measure(200, 20, 5, preheat_ms=20.0)
+                t = r["median"]
                 row[label + "_us"] = t * 1e3
                 row[label + "_GBs"] = w.bytes / (t * 1e-3) / 1e9
                 row[label + "_TFLOPs"] = w.flops / (t * 1e-3) / 1e12
                 row["bytes"] = w.bytes
                 if rot:  # the read-only pass over the same rotating copies, see read_floor above
-                    row["read_floor_us"] = w.read_floor(max(50, args.steps // 2), args.warmup) * 1e3
+                    row["read_floor_us"] = w.measure(200, 20, 5, preheat_ms=5.0, loop=w.read_loop)["median"] * 1e3
                 w.free()
+            fmt, m, k, n, resid, f16, cfg = WORKLOADS[name]
+            sets.drop(fmt, cfg, k, n)
             row["cold_pct_hbm"] = 100.0 * row["cold_GBs"] / HBM_PEAK_GBS
             rows.append(row)
             print(json.dumps(row), file=sys.stderr, flush=True)
-        layer = {"workload": "c2_q4_decode_layer_session", **decode_layer_times(max(50, args.steps // 2), args.warmup)}
+        layer = {"workload": "c2_q4_decode_layer_session", **decode_layer_times(200, 20)}
         rows.append(layer)
         print(json.dumps(layer), file=sys.stderr, flush=True)
         for fmt in (Q4, Q8):
@@ -417,6 +539,7 @@ def main():
             with open(args.sweep_out, "w") as f:
                 json.dump(rows, f, indent=1)
 
+    sets.free()
     ctx.close()
     print(json.dumps(line), flush=True)
 

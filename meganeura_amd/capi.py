@@ -335,16 +335,26 @@ class Context:
         self.check(self.lib.mgn_matmul_q_at(self.h, a_t.h, w.h, d.h if d is not None else None, c.h, m,
                                             arr if len(ops) else None, len(ops)))
 
-    def matmul_q_loop(self, a, weights, c, m, steps, d=None, a_is_f16=False):
-        """`steps` matmuls enqueued back to back from C, call i on weights[i % len(weights)]."""
-        arr = (C.c_void_p * len(weights))(*[w.h for w in weights])
-        self.check(self.lib.mgn_matmul_q_loop(self.h, a.h, 1 if a_is_f16 else 0, arr, len(weights),
+    @staticmethod
+    def rotation(weights):
+        """The handles of `weights`, twice over, as a C array: a rotation that starts at copy `first`
+        is the `len(weights)` entries from there, with nothing to build when a timed loop starts."""
+        n = len(weights)
+        return (C.c_void_p * (2 * n))(*([w.h for w in weights] * 2)), n
+
+    def matmul_q_loop(self, a, weights, c, m, steps, d=None, a_is_f16=False, first=0):
+        """`steps` matmuls enqueued back to back from C, call i on weights[(first + i) % len(weights)];
+        `weights` is a list of weights or what rotation() made of one."""
+        arr, n = weights if isinstance(weights, tuple) else self.rotation(weights)
+        start = C.cast(C.byref(arr, (first % n) * C.sizeof(C.c_void_p)), C.c_void_p) if n else None
+        self.check(self.lib.mgn_matmul_q_loop(self.h, a.h, 1 if a_is_f16 else 0, start, n,
                                               d.h if d is not None else None, c.h, m, steps))
 
-    def weight_read_loop(self, weights, steps):
-        """`steps` launches of a kernel that only reads the packed bytes of weights[i % len(weights)]."""
-        arr = (C.c_void_p * len(weights))(*[w.h for w in weights])
-        self.check(self.lib.mgn_weight_read_loop(self.h, arr, len(weights), steps))
+    def weight_read_loop(self, weights, steps, first=0):
+        """`steps` launches of a kernel that only reads the packed bytes of weights[(first + i) % len(weights)]."""
+        arr, n = weights if isinstance(weights, tuple) else self.rotation(weights)
+        start = C.cast(C.byref(arr, (first % n) * C.sizeof(C.c_void_p)), C.c_void_p) if n else None
+        self.check(self.lib.mgn_weight_read_loop(self.h, start, n, steps))
 
     def matmul_q_rms_norm(self, x, norm_weight, eps, w, c, m, d=None):
         """C = rms_norm(x; norm_weight, eps) x W (+ D) in one launch."""
