@@ -1,0 +1,38 @@
+/*
+ * mgn_bench.h -- entry points of libmgn_hip that only test and benchmark harnesses use.
+ *
+ * None of them stands in for anything in the reference, and a host runtime that binds
+ * mgn_hip.h does not need them: forcing a kernel family so that tests can drive every kernel
+ * at every shape, and launch loops written in C for harnesses written in a scripting
+ * language (an interpreter between launches would be what gets measured).
+ */
+#ifndef MGN_BENCH_H
+#define MGN_BENCH_H
+
+#include "mgn_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Force a kernel family for the context's matmuls (default MGN_ROUTE_AUTO).  A family that
+ * does not serve a shape makes the matmul return MGN_EINVAL ("... does not support this shape"). */
+mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route);
+
+/* `steps` matmuls (mgn_matmul_q, or mgn_matmul_q_f16a when a_is_f16 != 0) enqueued back to back,
+ * call i on weights[i % count]: the step loop of a compiled host
+ * (examples/matmul_throughput.rs:114-127).  Copies of one weight in rotation keep it out of
+ * the caches. */
+mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const mgn_weight* const* weights,
+                             size_t count, const mgn_buf* d, mgn_buf* c, uint32_t m, uint32_t steps);
+
+/* `steps` launches, back to back like mgn_matmul_q_loop's, of a kernel that reads the packed
+ * bytes of weights[i % count] (quants and scales) once and computes nothing.  Timed like a
+ * matmul it gives the time the device needs for one launch plus one pass over a weight's
+ * bytes: the floor a bandwidth-bound matmul on that weight can be held against. */
+mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, size_t count, uint32_t steps);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MGN_BENCH_H */

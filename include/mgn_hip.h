@@ -72,9 +72,6 @@ void mgn_ctx_destroy(mgn_ctx* ctx);
 const char* mgn_last_error(const mgn_ctx* ctx);
 /* Session::wait (src/runtime.rs:2835-2841). */
 mgn_status mgn_sync(mgn_ctx* ctx);
-/* Test hook: force a kernel family (default MGN_ROUTE_AUTO). */
-mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route);
-
 /* ---- plain device buffers: the reference allocates every plan buffer
  *      zero-filled (src/runtime.rs:1737-1755) and moves data with memcpy
  *      through mapped memory (upload_buffer 2552-2558, read_buffer 2623-2629). */
@@ -203,20 +200,6 @@ mgn_status mgn_matmul_q_epilogue(mgn_ctx* ctx, const mgn_buf* a, const mgn_weigh
  * is mgn_matmul_q_epilogue's: ops / n_ops as there, NULL / 0 for none.  c must not alias a_t. */
 mgn_status mgn_matmul_q_at(mgn_ctx* ctx, const mgn_buf* a_t, const mgn_weight* w, const mgn_buf* d, mgn_buf* c,
                            uint32_t m, const mgn_unary* ops, size_t n_ops);
-
-/* `steps` such matmuls enqueued back to back, call i on weights[i % count]: the step loop of
- * a compiled host (examples/matmul_throughput.rs:114-127) without an interpreter between the
- * launches, for harnesses written in a scripting language.  Copies of one weight in rotation
- * keep it out of the caches.  a_is_f16 != 0 selects the fp16-activation entry. */
-mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const mgn_weight* const* weights,
-                             size_t count, const mgn_buf* d, mgn_buf* c, uint32_t m, uint32_t steps);
-
-/* Measurement aid with no counterpart in the reference: `steps` launches, back to back like
- * mgn_matmul_q_loop's, of a kernel that reads the packed bytes of weights[i % count] (quants and
- * scales) once and computes nothing.  Timed like a matmul it gives the time the device needs
- * for one launch plus one pass over a weight's bytes, the floor a bandwidth-bound matmul on
- * that weight can be held against. */
-mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, size_t count, uint32_t steps);
 
 /* What mgn_matmul_q would launch for a shape, without a device: the kernel family the
  * automatic choice takes (the analogue of reading compile.rs:1390 and runtime.rs:1634 for the

@@ -16,14 +16,15 @@ FMT_Q4, FMT_Q8 = 0, 1
 STATIC_WORKSPACE_BYTES = 4 << 20  # MGN_STATIC_WORKSPACE_BYTES
 ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA = range(5)
 
-# every symbol include/mgn_hip.h and include/mgn_session.h declare
+# every symbol include/mgn_hip.h, include/mgn_bench.h and include/mgn_session.h declare
+BENCH_SYMBOLS = ["mgn_ctx_set_route", "mgn_matmul_q_loop", "mgn_weight_read_loop"]
 HIP_SYMBOLS = [
-    "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync", "mgn_ctx_set_route",
+    "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync",
     "mgn_buf_alloc", "mgn_buf_free", "mgn_buf_size", "mgn_buf_device_ptr", "mgn_buf_upload",
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_weight_save", "mgn_weight_load", "mgn_matmul_q",
-    "mgn_matmul_q_f16a", "mgn_matmul_q_static", "mgn_matmul_q_epilogue", "mgn_matmul_q_at", "mgn_matmul_q_loop", "mgn_weight_read_loop", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
+    "mgn_matmul_q_f16a", "mgn_matmul_q_static", "mgn_matmul_q_epilogue", "mgn_matmul_q_at", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
     "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [

@@ -5,6 +5,7 @@
 #include <string>
 
 #include "../../include/mgn_hip.h"
+#include "../../include/mgn_bench.h"
 
 struct ihipStream_t;
 struct ihipEvent_t;

@@ -18,11 +18,13 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(capi.LIB_PATH)
     declared = set()
-    for header in ("mgn_hip.h", "mgn_session.h"):
+    for header, listed in (("mgn_hip.h", capi.HIP_SYMBOLS), ("mgn_bench.h", capi.BENCH_SYMBOLS),
+                           ("mgn_session.h", capi.SESSION_SYMBOLS)):
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        declared |= set(re.findall(r"\b(mgn_[a-z0-9_]+)\s*\(", text))
-    assert declared == set(capi.HIP_SYMBOLS) | set(capi.SESSION_SYMBOLS)
+        here = set(re.findall(r"\b(mgn_[a-z0-9_]+)\s*\(", text))
+        assert here == set(listed), header
+        declared |= here
     for name in sorted(declared):
         assert hasattr(lib, name), name
     assert capi.load().mgn_built_for() == b"gfx950"
