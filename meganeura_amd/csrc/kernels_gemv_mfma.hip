@@ -3,14 +3,6 @@
 // instantiates it for one weight format and one row count so that they compile in parallel.
 #include "kernels_gemv_mfma.hip.h"
 
-#ifdef MGN_TRACE
-unsigned long long* g_gemv_trace_host = nullptr;
-extern "C" int mgn_debug_set_trace(void* p) {
-  g_gemv_trace_host = (unsigned long long*)p;
-  return 0;
-}
-#endif
-
 namespace mgn {
 
 int launch_gemv_mfma_q4_m1(ihipStream_t* s, const LaunchArgs& x);

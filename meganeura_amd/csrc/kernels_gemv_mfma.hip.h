@@ -41,45 +41,7 @@
 // are prepared once per workgroup in LDS, laid out so that consecutive lanes
 // read consecutive 16-byte chunks.
 #pragma once
-#include <cstdlib>
-
 #include "kernels_common.hip.h"
-
-#ifdef MGN_TRACE
-// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.  The
-// buffer travels as a kernel argument, so a stamp is one clock read and one store.
-extern unsigned long long* g_gemv_trace_host;  // defined next to the route's dispatcher
-#define MGN_TRACE_PARAM , unsigned long long* trace_arg
-#define MGN_TRACE_ARG , g_gemv_trace_host
-// The first two stamps are taken into registers and written once the buffer pointer (an
-// argument that lives in memory) is first needed, so that tracing does not itself make the
-// wave wait for an argument fetch before its first loads.
-#define MGN_STAMP_INIT()                                              \
-  const unsigned long long trace_t0 = __builtin_readcyclecounter();   \
-  const unsigned long long trace_w0 = wall_clock64();                 \
-  unsigned long long trace_t1 = 0
-#define MGN_STAMP_EARLY() trace_t1 = __builtin_readcyclecounter()
-#define MGN_STAMP_FLUSH()                                                                                     \
-  unsigned long long* const trace_base =                                                                      \
-      trace_arg ? trace_arg + ((size_t)blockIdx.x * 16 + (threadIdx.x >> 6)) * 16 : nullptr;                  \
-  if (trace_base && (threadIdx.x & 63) == 0) trace_base[0] = trace_t0, trace_base[1] = trace_t1, trace_base[13] = trace_w0
-#define MGN_STAMP(slot)                                                                          \
-  do {                                                                                           \
-    if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = __builtin_readcyclecounter();   \
-  } while (0)
-#define MGN_STAMP_WALL(slot)                                                        \
-  do {                                                                             \
-    if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = wall_clock64();  \
-  } while (0)
-#else
-#define MGN_STAMP_WALL(slot) do {} while (0)
-#define MGN_TRACE_PARAM
-#define MGN_TRACE_ARG
-#define MGN_STAMP_INIT() do {} while (0)
-#define MGN_STAMP_EARLY() do {} while (0)
-#define MGN_STAMP_FLUSH() do {} while (0)
-#define MGN_STAMP(slot) do {} while (0)
-#endif
 
 namespace mgn {
 namespace {
@@ -267,8 +229,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     uint32_t m_flags,  // rows in bits 0-7; bit 31: the activations are fp16 (kProNone only)
     uint32_t ksc, uint32_t wnc, uint32_t kdim, uint32_t n0, uint32_t first_quad1, uint32_t first_quad2,
     uint32_t ksc_recip,  // ceil(4096 / ksc): wave / ksc == (wave * ksc_recip) >> 12 for the 16 waves there can be
-    const float* __restrict__ norm_weight, float eps, GemvBatch bt, GemvSplit sp MGN_TRACE_PARAM) {
-  MGN_STAMP_INIT();
+    const float* __restrict__ norm_weight, float eps, GemvBatch bt, GemvSplit sp) {
   const uint32_t m = m_flags & 0xFFu;
   const bool a_f16 = PRO == kProNone && (m_flags >> 31) != 0;
   const GemvPrologue pro{norm_weight, eps};
@@ -425,8 +386,6 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     __builtin_amdgcn_sched_barrier(0);  // in this order: step 0 waits for its own block only
   }
   for (uint32_t t = tid; t < wnc * ksc * MROWS * 4; t += nthreads) red[t] = 0.0f;
-  MGN_STAMP_EARLY();
-  MGN_STAMP_FLUSH();
 
   if (a_f16) {
 #pragma unroll
@@ -530,9 +489,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       }
     }
   }
-  MGN_STAMP(5);
   lds_barrier();
-  MGN_STAMP(6);
 
   // ---- the K walk: STEPS blocks per lane, straight-line ----
   // Lanes i >= NJ have no activation row of their own; they re-read row i % NJ (a broadcast
@@ -663,11 +620,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         }
       }
     }
-    if (t == 0) MGN_STAMP(7);
-    if (t == 3) MGN_STAMP(8);
   }
   }
-  MGN_STAMP(9);
   // ---- sum the 16 lanes of each column ----
   if (!KSPLIT && (QPW > 1 || ksc == 1)) {
     // no K split (always the case with QPW > 1): lanes 0..3 hold the four finished columns of a quad
@@ -685,8 +639,6 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         }
       }
     }
-    MGN_STAMP(12);
-    MGN_STAMP_WALL(14);
     return;
   }
 #pragma unroll
@@ -694,9 +646,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     const float tot = sum_over_blocks(acc[0][r]);
     if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot;
   }
-  MGN_STAMP(10);
   lds_barrier();
-  MGN_STAMP(11);
   // ---- combine the K splits, add the residual, store ----
   uint32_t* const last_flag = (uint32_t*)nrm;  // (KSPLIT comes without the prologue that uses nrm)
   for (int pass = 0; pass < (KSPLIT ? 2 : 1); pass++) {
@@ -742,8 +692,6 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       }
     }
   }
-  MGN_STAMP(12);
-  MGN_STAMP_WALL(14);
 }
 
 struct MfmaGemvPlan {
@@ -795,9 +743,6 @@ bool plan_one_part(int fmt, uint32_t k, uint32_t nquads, uint32_t mrows, int num
     if ((num_cus - last) * 8 > (uint32_t)num_cus * rounds) per_cu = (wave_quads + num_cus * rounds - 1) / (num_cus * rounds);
   }
   p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, per_cu));
-#ifdef MGN_TRACE  // development build only: force the waves per workgroup
-  if (const char* e = getenv("MGN_DEV_WNC")) p.wnc = std::max<uint32_t>(1, std::min<uint32_t>(max_wnc, (uint32_t)atoi(e)));
-#endif
   // enough threads to prepare the activations (waves without a quad only help there)
   const uint32_t prep_waves = (bpc_pad * 4 + kMaxTasks * 64 - 1) / (kMaxTasks * 64);
   p.wnc = std::max<uint32_t>(p.wnc, (prep_waves + p.ksc - 1) / p.ksc);
@@ -885,7 +830,7 @@ int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
   hipLaunchKernelGGL(kern, dim3(p.grid, p.kparts), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants,
                      x.m | (x.a_is_f16 ? 0x80000000u : 0u), p.ksc, p.wnc, p.kparts > 1 ? p.part_k : x.w.k, x.w.n,
                      bt.first_quad[1], bt.first_quad[2],
-                     (4096u + p.ksc - 1) / p.ksc, x.pro_weight, x.pro_eps, bt, sp MGN_TRACE_ARG);
+                     (4096u + p.ksc - 1) / p.ksc, x.pro_weight, x.pro_eps, bt, sp);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

@@ -36,30 +36,8 @@
 // different workgroups whose partial tiles the last one to finish adds up in part
 // order (deterministic).
 #include <algorithm>
-#include <cstdio>
-#include <cstdlib>
 
 #include "kernels_common.hip.h"
-
-#ifdef MGN_TRACE
-// Development aid: per-wave shader-clock timestamps at fixed points of the kernel.  The
-// buffer travels as a kernel argument, so a stamp is one clock read and one store.
-static unsigned long long* g_gemm_trace_host = nullptr;
-extern "C" int mgn_debug_set_trace_gemm(void* p) {
-  g_gemm_trace_host = (unsigned long long*)p;
-  return 0;
-}
-#define MGN_GSTAMP_INIT()                                                                                  \
-  unsigned long long* const trace_base =                                                                   \
-      g.trace ? g.trace + ((((size_t)blockIdx.z * g.colgroups + blockIdx.y) * g.parts + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 16 : nullptr
-#define MGN_GSTAMP(slot)                                                                  \
-  do {                                                                                    \
-    if (trace_base && (threadIdx.x & 63) == 0) trace_base[slot] = __builtin_readcyclecounter(); \
-  } while (0)
-#else
-#define MGN_GSTAMP_INIT() do {} while (0)
-#define MGN_GSTAMP(slot) do {} while (0)
-#endif
 
 namespace mgn {
 namespace {
@@ -121,9 +99,6 @@ struct GemmTail {  // arguments first needed in the epilogue
   uint32_t* range_flag;  // host-visible: set when an f32 activation does not fit the fp16 pair
   uint32_t row_tiles;
   uint32_t epilogue;  // unary operations on the output (apply_epilogue)
-#ifdef MGN_TRACE
-  unsigned long long* trace;
-#endif
 };
 
 template <int FMT>
@@ -163,17 +138,11 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
     float* scratch;
     uint32_t* counters;
     uint32_t m, ksc, wnc, nch, parts, colgroups;
-#ifdef MGN_TRACE
-    unsigned long long* trace;
-#endif
   } g;
   g.w.meta = meta_arg, g.w.quants = quants_arg, g.w.k = k_arg, g.w.n = n_arg, g.w.fmt = FMT;
   g.a = a_arg, g.m = m_arg, g.ksc = ksc_arg, g.wnc = wnc_arg, g.nch = nch_arg;
   g.parts = parts_arg, g.colgroups = colgroups_arg;
   g.dres = tail.dres, g.c = tail.c, g.scratch = tail.scratch, g.counters = tail.counters;
-#ifdef MGN_TRACE
-  g.trace = tail.trace;
-#endif
   constexpr bool F32A = AM != 0;
   constexpr bool CHAIN = AM == 2;
   constexpr int ROWS = AM == 1 ? 16 : 32;  // real rows per tile
@@ -204,9 +173,6 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
   const uint32_t row0 = blockIdx.z * ROWS;
   const uint32_t zero_block = bpc * w.n;
   const uint32_t chunk0 = part * g.nch;  // first chunk of this workgroup
-
-  MGN_GSTAMP_INIT();
-  MGN_GSTAMP(0);
 
   // ---- per-thread staging tasks: task t = (lb * ROWS + r) * 4 + sub, sub = 2h + g ----
   uint32_t t_lb[TPT], t_slot[TPT], t_r[TPT];
@@ -371,14 +337,11 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
 
   load_a(chunk0);
   fetch_slice(chunk0, true);
-  MGN_GSTAMP(1);
   // the additive operands' unused slots must read as zero for the whole kernel
   for (uint32_t t = tid; t < 2 * s_stride; t += nthreads) simg[t] = make_uint4(0, 0, 0, 0);
   lds_barrier();
   stage(chunk0, 0);
-  MGN_GSTAMP(2);
   lds_barrier();
-  MGN_GSTAMP(3);
 
   floatx16 acc, acc2;  // scaled quant sums (vector ALU), additive parts (MFMA)
 #pragma unroll
@@ -483,12 +446,9 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
       scale_step(s);
       asm volatile("" : "+v"(acc));  // the scaling stays here, between the two MFMA groups
     }
-    if (c == 0) MGN_GSTAMP(4);
     if (more) stage(chunk + 1, buf ^ 1);  // the other buffer was last read before the previous barrier
     lds_barrier();
-    if (c == 0) MGN_GSTAMP(5);
   }
-  MGN_GSTAMP(6);
 
   // ---- combine the two K halves of the workgroup ----
   // D layout: lane -> column lane%32; register i -> tile row 8*(i/4) + 4*(lane/32) + i%4.
@@ -523,24 +483,19 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
         __hip_atomic_store(mine + (size_t)(8 * (i >> 2) + 4 * gh + (i & 3)) * w.n, outv[i], __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     }
-    MGN_GSTAMP(8);
     // every wave waits until its write-through stores have been acknowledged, i.e. have
     // reached memory; the barrier then orders all of them before the count
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    MGN_GSTAMP(9);
     uint32_t* const flag = (uint32_t*)lds4;
     if (tid == 0) {
       uint32_t* ctr = g.counters + blockIdx.z * g.colgroups + cg;
-      MGN_GSTAMP(11);
       const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const bool last = seen == g.parts - 1;
-      if (seen != 0xFFFFFFFFu) MGN_GSTAMP(12);
       if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
       *flag = last ? 1u : 0u;
     }
     __syncthreads();
-    MGN_GSTAMP(10);
     if (*flag == 0u) return;
     if (writer) {
       // every part comes from memory, this workgroup's own included: NI loads of a part in
@@ -582,7 +537,6 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
       }
     }
   }
-  MGN_GSTAMP(7);
 }
 
 size_t gemm_lds_bytes(int fmt, uint32_t ksc, uint32_t wnc, bool chain) {
@@ -647,31 +601,6 @@ bool plan_gemm(const LaunchArgs& x, GemmPlan* out) {
       }
     }
   }
-#ifdef MGN_TRACE  // development build only: force a plan, print the chosen one
-  if (const char* dev = getenv("MGN_DEV_GEMM")) {
-    unsigned a = 0, b = 0, c = 0;
-    if (sscanf(dev, "%u,%u,%u", &a, &b, &c) == 3) {
-      // a forced plan has to pass every check the search applies, or the call is refused
-      if ((a != 1 && a != 2) || b < 1 || b > 8 / a || c < 1) return false;
-      const uint32_t cb = 8 * a, chunks = (bpc + cb - 1) / cb;
-      bp.ksc = a, bp.wnc = b, bp.parts = c;
-      bp.nch = (chunks + c - 1) / c;
-      bp.parts = (chunks + bp.nch - 1) / bp.nch;
-      bp.colgroups = (n_tiles + b - 1) / b;
-      const uint32_t tpt = (max_tasks + b - 1) / b;
-      bp.tpt = tpt <= 1 ? 1 : tpt <= 2 ? 2 : 4;
-      bp.grid_y = grid_y;
-      bp.scratch_bytes = bp.parts > 1 ? (size_t)bp.parts * grid_y * rows * x.w.n * 4 : 0;
-      if (tpt > 4 || gemm_lds_bytes(x.w.fmt, a, b, am == 2) > 160 * 1024 || bp.colgroups > 65535 || bp.scratch_bytes > x.scratch_bytes ||
-          (bp.parts > 1 && (uint64_t)grid_y * bp.colgroups > x.n_counters))
-        return false;
-      best = 1;
-    }
-  }
-  if (getenv("MGN_DEV_PLAN"))
-    fprintf(stderr, "gemm plan m=%u k=%u n=%u: ksc=%u wnc=%u parts=%u nch=%u tpt=%u wgs=%u\n", x.m, x.w.k, x.w.n, bp.ksc, bp.wnc,
-            bp.parts, bp.nch, bp.tpt, bp.colgroups * bp.parts * bp.grid_y);
-#endif
   if (best == 0 || (uint64_t)bp.colgroups * bp.parts > 0x7fffffffu) return false;
   bp.lds = gemm_lds_bytes(x.w.fmt, bp.ksc, bp.wnc, am == 2);
   bp.am = am;
@@ -685,9 +614,6 @@ int launch_tpt(ihipStream_t* s, const LaunchArgs& x, const GemmPlan& p) {
   static std::atomic<uint64_t> big_lds_done{0};
   if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
   GemmTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.range_flag, p.grid_y, x.epilogue};
-#ifdef MGN_TRACE
-  tail.trace = g_gemm_trace_host;
-#endif
   if (p.colgroups > 65535 || p.grid_y > 65535) return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups, p.grid_y), dim3(64 * p.ksc * p.wnc), p.lds, s, x.a, x.w.meta, x.w.quants,
                      x.m, p.ksc, p.wnc, p.nch, x.w.k, x.w.n, p.parts, p.colgroups, tail);
