@@ -40,7 +40,8 @@ typedef enum mgn_status {
   MGN_ENODEVICE = 5, /* no usable gfx950 device */
   MGN_EUNSUPPORTED = 6, /* a fused entry point asked for a shape its kernel does not serve */
   MGN_ERANGE = 7 /* reported by the next synchronising call: an f32 activation too large for the kernel
-                    that ran (|x| >= 65504 on the tiled MFMA route, M >= 5); outputs of that call are wrong */
+                    that ran (|x| >= 65504 on MGN_ROUTE_GEMM_MFMA, M >= 5); outputs of that call are wrong;
+                    MGN_ROUTE_TILE_MFMA takes such data */
 } mgn_status;
 
 /* compile::WeightFormat::{Q4,Q8} (src/compile.rs:8-29), graph::DType::{Q4_0,Q8_0}
@@ -55,7 +56,11 @@ typedef enum mgn_route {
   MGN_ROUTE_GENERIC = 1,   /* scalar f32 fallback, any M */
   MGN_ROUTE_GEMV_VALU = 2, /* streaming dequant-GEMV on the vector ALU, M <= 4 */
   MGN_ROUTE_GEMV_MFMA = 3, /* streaming dequant-GEMV, raw quants x split-fp16 activations on MFMA, M <= 4 */
-  MGN_ROUTE_GEMM_MFMA = 4  /* tiled dequant-GEMM on MFMA, larger M */
+  MGN_ROUTE_GEMM_MFMA = 4, /* tiled dequant-GEMM on MFMA (32x32x16 tiles), larger M: the fast form, for weights whose
+                              block minima stay below 2047 (Q8: scales below 15.99) and f32 activations below 65504 */
+  MGN_ROUTE_TILE_MFMA = 5  /* tiled dequant-GEMM on MFMA (16x16x32 tiles, activations rescaled per row and 256-element
+                              K slice): any finite weight and activation magnitude, larger M; the automatic choice
+                              for weights outside the range of the form above */
 } mgn_route;
 
 typedef struct mgn_ctx mgn_ctx;

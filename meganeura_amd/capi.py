@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_DIR, "libmgn_hip.so")
 OK, EINVAL, ENOMEM, EHIP, ENOTFOUND, ENODEVICE, EUNSUPPORTED, ERANGE = range(8)
 FMT_Q4, FMT_Q8 = 0, 1
 STATIC_WORKSPACE_BYTES = 4 << 20  # MGN_STATIC_WORKSPACE_BYTES
-ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA = range(5)
+ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA, ROUTE_TILE_MFMA = range(6)
 
 # every symbol include/mgn_hip.h, include/mgn_bench.h and include/mgn_session.h declare
 BENCH_SYMBOLS = ["mgn_ctx_set_route", "mgn_matmul_q_loop", "mgn_weight_read_loop"]

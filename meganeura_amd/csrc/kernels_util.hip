@@ -70,23 +70,34 @@ __global__ __launch_bounds__(256) void import_q8_kernel(const uint32_t* __restri
 // out[0], out[1] must be zero before the launch.
 __global__ __launch_bounds__(256) void scale_range_kernel(int fmt, const void* __restrict__ meta, size_t nb,
                                                           uint32_t* __restrict__ out) {
+  __shared__ uint32_t part[2][4];
   uint32_t smax = 0, mmax = 0;
-  for (size_t b = (size_t)blockIdx.x * 256 + threadIdx.x; b < nb; b += (size_t)gridDim.x * 256) {
-    if (fmt == MGN_FMT_Q4) {
-      const uint32_t dm = ((const uint32_t*)meta)[b];
-      smax = max(smax, __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(dm & 0xFFFFu))));
-      mmax = max(mmax, __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(dm >> 16))));
-    } else {
-      smax = max(smax, __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(((const uint16_t*)meta)[b]))));
+  // four scale words (Q8: eight scales) per load; the tail past a multiple of four reads the
+  // all-zero blocks that follow the real ones
+  const size_t n16 = fmt == MGN_FMT_Q4 ? (nb + 3) / 4 : (nb + 7) / 8;
+  for (size_t v = (size_t)blockIdx.x * 256 + threadIdx.x; v < n16; v += (size_t)gridDim.x * 256) {
+    const uint4 q = ((const uint4*)meta)[v];
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const uint32_t lo = __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(w[e] & 0xFFFFu)));
+      const uint32_t hi = __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(w[e] >> 16)));
+      smax = max(smax, lo);
+      if (fmt == MGN_FMT_Q4) mmax = max(mmax, hi);
+      else smax = max(smax, hi);
     }
   }
-  // one atomic per wave, not per thread: a million atomics on one address take 0.4 ms
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     smax = max(smax, (uint32_t)__shfl_xor((int)smax, off, 64));
     mmax = max(mmax, (uint32_t)__shfl_xor((int)mmax, off, 64));
   }
-  if ((threadIdx.x & 63) == 0) {
+  // one atomic pair per workgroup: thousands of atomics on one address would take longer than the scan
+  if ((threadIdx.x & 63) == 0) part[0][threadIdx.x >> 6] = smax, part[1][threadIdx.x >> 6] = mmax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    smax = max(max(part[0][0], part[0][1]), max(part[0][2], part[0][3]));
+    mmax = max(max(part[1][0], part[1][1]), max(part[1][2], part[1][3]));
     if (smax) atomicMax(out, smax);
     if (mmax) atomicMax(out + 1, mmax);
   }
@@ -320,7 +331,7 @@ int launch_export_q8(ihipStream_t* s, const WeightView& w, uint8_t* out_dev) {
 
 int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev) {
   const size_t nb = (size_t)(w.k / 32) * w.n;
-  hipLaunchKernelGGL(scale_range_kernel, dim3((unsigned)std::min<size_t>((nb + 255) / 256, 1024)), dim3(256), 0, s, w.fmt,
+  hipLaunchKernelGGL(scale_range_kernel, dim3((unsigned)std::min<size_t>((nb / 4 + 255) / 256 + 1, 256)), dim3(256), 0, s, w.fmt,
                      w.meta, nb, out2_dev);
   MGN_HIP_LAUNCH_CHECK();
   return 0;

@@ -121,7 +121,7 @@ mgn_status check_range_flag(mgn_ctx* ctx) {
   *(volatile uint32_t*)ctx->range_flag_host = 0;
   return fail(ctx, MGN_ERANGE,
               "an f32 activation of magnitude >= 65504 reached the tiled MFMA kernel (M >= 5), which splits activations "
-              "into fp16 pairs: the affected outputs are wrong; select MGN_ROUTE_GENERIC for such data");
+              "into fp16 pairs: the affected outputs are wrong; select MGN_ROUTE_TILE_MFMA for such data");
 }
 
 // Looks at every block's scale (and minimum) once, right after a weight's blocks are on the
@@ -142,6 +142,25 @@ mgn_status scan_weight_range(mgn_ctx* ctx, mgn_weight* w) {
 }
 
 }  // namespace
+
+namespace mgn {
+// Would one launch serve these weights together (mgn_matmul_q_batch's own check)?  The plan
+// depends on the column count of the whole batch, so a weight that plans alone need not plan
+// next to its siblings.
+bool batch_plans(const mgn_ctx* ctx, const mgn_weight* const* ws, size_t count, uint32_t m, int pro_kind) {
+  if (!ctx || !ws || count == 0 || count > 3 || m == 0) return false;
+  if (ctx->route != MGN_ROUTE_AUTO && ctx->route != MGN_ROUTE_GEMV_MFMA) return false;
+  LaunchArgs x{view_of(ws[0]), nullptr, nullptr, nullptr, m, false, ctx->num_cus};
+  for (size_t j = 1; j < count; j++) x.more[j - 1] = {view_of(ws[j]), nullptr, nullptr};
+  x.n_more = (int)count - 1;
+  x.scratch = ctx->scratch;
+  x.scratch_bytes = ctx->scratch_bytes;
+  x.counters = ctx->counters;
+  x.n_counters = ctx->n_counters;
+  x.pro_kind = pro_kind;
+  return gemv_mfma_supported(x);
+}
+}  // namespace mgn
 
 extern "C" {
 
@@ -221,7 +240,7 @@ mgn_status mgn_sync(mgn_ctx* ctx) {
 
 mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route) {
   if (!ctx) return MGN_EINVAL;
-  if (route < MGN_ROUTE_AUTO || route > MGN_ROUTE_GEMM_MFMA) return fail(ctx, MGN_EINVAL, "unknown route");
+  if (route < MGN_ROUTE_AUTO || route > MGN_ROUTE_TILE_MFMA) return fail(ctx, MGN_EINVAL, "unknown route");
   ctx->route = route;
   return MGN_OK;
 }
@@ -563,6 +582,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   if (route == MGN_ROUTE_AUTO) {
     if (mgn::gemv_mfma_supported(x)) route = MGN_ROUTE_GEMV_MFMA;
     else if (mgn::gemm_mfma_supported(x)) route = MGN_ROUTE_GEMM_MFMA;
+    else if (mgn::tile_mfma_supported(x)) route = MGN_ROUTE_TILE_MFMA;  // e.g. a weight whose block minima the kernel above cannot hold
     else if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV_VALU;
     else route = MGN_ROUTE_GENERIC;
   }
@@ -572,6 +592,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
     mgn_plan_info plan{};
     const bool parts = route == MGN_ROUTE_GEMV_MFMA   ? mgn::describe_gemv_mfma(x, &plan)
                        : route == MGN_ROUTE_GEMM_MFMA ? mgn::describe_gemm_mfma(x, &plan)
+                       : route == MGN_ROUTE_TILE_MFMA ? mgn::describe_tile_mfma(x, &plan)
                                                       : false;
     const uint64_t need = parts ? plan.workspace_bytes : 0;
     if (need > kStaticPartialBytes)
@@ -599,6 +620,10 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
     case MGN_ROUTE_GEMV_MFMA:
       if (!mgn::gemv_mfma_supported(x)) return fail(ctx, MGN_EINVAL, "GEMV_MFMA route does not support this shape");
       rc = mgn::launch_matmul_gemv_mfma(ctx->stream, x);
+      break;
+    case MGN_ROUTE_TILE_MFMA:
+      if (!mgn::tile_mfma_supported(x)) return fail(ctx, MGN_EINVAL, "TILE_MFMA route does not support this shape");
+      rc = mgn::launch_matmul_tile_mfma(ctx->stream, x);
       break;
     case MGN_ROUTE_GEMM_MFMA:
       if (!mgn::gemm_mfma_supported(x)) return fail(ctx, MGN_EINVAL, "GEMM_MFMA route does not support this shape");
@@ -746,6 +771,7 @@ mgn_status mgn_matmul_q_plan(mgn_fmt fmt, uint32_t m, uint64_t k, uint64_t n, in
   x.n_counters = mgn::kWorkspaceCounters;
   if (mgn::describe_gemv_mfma(x, out)) return MGN_OK;
   if (mgn::describe_gemm_mfma(x, out)) return MGN_OK;
+  if (mgn::describe_tile_mfma(x, out)) return MGN_OK;
   out->route = mgn::gemv_supported(x) ? MGN_ROUTE_GEMV_VALU : MGN_ROUTE_GENERIC;
   return MGN_OK;
 }

@@ -99,6 +99,10 @@ bool describe_gemm_mfma(const LaunchArgs& a, mgn_plan_info* out);
 constexpr size_t kWorkspaceBytes = (size_t)16 << 20;
 constexpr uint32_t kWorkspaceCounters = 4096;
 int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& a);
+// kernels_tile.hip: the 16x16x32 tiled kernel (activation image + weight streaming)
+bool tile_mfma_supported(const LaunchArgs& a);
+bool describe_tile_mfma(const LaunchArgs& a, mgn_plan_info* out);
+int launch_matmul_tile_mfma(ihipStream_t* s, const LaunchArgs& a);
 
 }  // namespace mgn
 
@@ -120,6 +124,11 @@ struct mgn_ctx {
   size_t at_stage_bytes = 0;
   std::string err;
 };
+
+namespace mgn {
+// whether mgn_matmul_q_batch would take these weights in one launch (same K and format assumed checked)
+bool batch_plans(const mgn_ctx* ctx, const mgn_weight* const* ws, size_t count, uint32_t m, int pro_kind);
+}  // namespace mgn
 
 struct mgn_buf {
   void* ptr = nullptr;

@@ -703,6 +703,12 @@ void Session::plan_launches() {
                               dj.weight_format == di.weight_format;
       const bool addend_ready = dj.input_buffers.size() < 3 || producer_of[dj.input_buffers[2]] < (int)i;
       if (!same_src || !same_shape || !addend_ready) continue;
+      // the launch is planned for the columns of the whole batch: a sibling joins only if the
+      // batch with it still has a plan (each weight planning alone does not settle that)
+      const mgn_weight* group[3] = {weights_[di.input_buffers[1]], nullptr, nullptr};
+      for (int f = 0; f < found; f++) group[1 + f] = weights_[plan_.dispatches[fused_[i].more[f]].input_buffers[1]];
+      group[1 + found] = weights_[dj.input_buffers[1]];
+      if (!batch_plans(ctx_, group, (size_t)found + 2, di.params[0], fused_[i].kind)) continue;
       fused_[i].more[found++] = (int)j;
       skipped_[j] = 1;
     }
@@ -770,8 +776,16 @@ void Session::run_dispatches() {
           const Dispatch* p = f.kind != kProNone ? &plan_.dispatches[f.producer] : nullptr;
           const mgn_buf* act = p ? buffers_[p->input_buffers[0]] : buffers_[d.input_buffers[0]];
           const mgn_buf* nw = f.kind == kProRmsNorm ? buffers_[p->input_buffers[1]] : nullptr;
-          check(mgn_matmul_q_batch(ctx_, act, (mgn_prologue)f.kind, nw, p ? p->eps : 0.0f, items, count, d.params[0]),
-                "mgn_matmul_q_batch");
+          mgn_status st = mgn_matmul_q_batch(ctx_, act, (mgn_prologue)f.kind, nw, p ? p->eps : 0.0f, items, count, d.params[0]);
+          if (st == MGN_EUNSUPPORTED) {
+            // planned as one launch, refused now (the route was changed since): one launch per weight
+            st = MGN_OK;
+            for (size_t j = 0; j < count && st == MGN_OK; j++)
+              st = f.kind == kProRmsNorm  ? mgn_matmul_q_rms_norm(ctx_, act, nw, p->eps, items[j].w, items[j].d, items[j].c, d.params[0])
+                   : f.kind == kProSwiglu ? mgn_matmul_q_swiglu(ctx_, act, items[j].w, items[j].d, items[j].c, d.params[0])
+                                          : mgn_matmul_q(ctx_, act, items[j].w, items[j].d, items[j].c, d.params[0]);
+          }
+          check(st, "mgn_matmul_q_batch");
         } else if (f.kind == kProRmsNorm) {
           const Dispatch& p = plan_.dispatches[f.producer];
           check(mgn_matmul_q_rms_norm(ctx_, buffers_[p.input_buffers[0]], buffers_[p.input_buffers[1]], p.eps, w, addend,

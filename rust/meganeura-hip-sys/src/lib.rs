@@ -46,6 +46,7 @@ pub const MGN_ROUTE_GENERIC: mgn_route = 1;
 pub const MGN_ROUTE_GEMV_VALU: mgn_route = 2;
 pub const MGN_ROUTE_GEMV_MFMA: mgn_route = 3;
 pub const MGN_ROUTE_GEMM_MFMA: mgn_route = 4;
+pub const MGN_ROUTE_TILE_MFMA: mgn_route = 5;
 
 /// `mgn_unary`: the operations `fuse_epilogues` folds into a matmul (src/compile.rs:915-1035).
 pub type mgn_unary = c_int;

@@ -120,12 +120,22 @@ def test_weight_errors(ctx):
 
 # ---- matmul: every route at small and ragged shapes ----------------------------------------
 
+# (route, m, k, n) combinations of the tests below that a forced kernel family refuses, each with
+# the reason; every other combination must run and match the oracle (the automatic route never refuses)
+REFUSED = {
+    # the vector-ALU GEMV keeps all K groups of a column in one workgroup and the staged activations in LDS
+    ("gemv_valu", 4, 14336, 518), ("gemv_valu", 3, 12288, 64), ("gemv_valu", 1, 18944, 132),
+    ("gemv_valu", 4, 11008, 260), ("gemv_valu", 3, 13824, 70), ("gemv_valu", 4, 14336, 70),
+    # both GEMV kernels serve at most four activation rows
+    ("gemv_valu", 6, 1024, 300), ("gemv_mfma", 6, 1024, 300), ("gemv_valu", 16, 4096, 2048), ("gemv_mfma", 16, 4096, 2048),
+}
+
 ROUTES = {"generic": capi.ROUTE_GENERIC, "gemv_valu": capi.ROUTE_GEMV_VALU, "gemv_mfma": capi.ROUTE_GEMV_MFMA,
-          "gemm_mfma": capi.ROUTE_GEMM_MFMA, "auto": capi.ROUTE_AUTO}
+          "gemm_mfma": capi.ROUTE_GEMM_MFMA, "tile_mfma": capi.ROUTE_TILE_MFMA, "auto": capi.ROUTE_AUTO}
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-@pytest.mark.parametrize("route", ["generic", "gemv_valu", "gemv_mfma", "gemm_mfma", "auto"])
+@pytest.mark.parametrize("route", ["generic", "gemv_valu", "gemv_mfma", "gemm_mfma", "tile_mfma", "auto"])
 @pytest.mark.parametrize("m,k,n", [
     (1, 32, 1), (1, 64, 3), (1, 576, 192), (1, 576, 577), (1, 1536, 576), (1, 1024, 100),
     (2, 576, 65), (3, 2048, 130), (4, 4096, 257), (1, 14336, 64), (1, 3072, 1024),
@@ -145,14 +155,13 @@ def test_small_m_routes(ctx, orc, fmt, route, m, k, n):
     x = synth.normal(1000 + m + k + n, m * k).reshape(m, k)
     w = synth.normal(2000 + m + k + n, k * n, 0.02).reshape(k, n)
     d = synth.normal(3000 + n, m * n).reshape(m, n)
+    if (route, m, k, n) in REFUSED:
+        with pytest.raises(capi.MgnError, match="does not support"):
+            run_matmul(ctx, fmt, x, w, ROUTES[route])
+        return
     deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
-    try:
-        got = run_matmul(ctx, fmt, x, w, ROUTES[route])
-        got_d = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d)
-    except capi.MgnError as e:
-        if route != "generic" and "does not support" in str(e):
-            pytest.skip("shape outside this GEMV kernel's range")
-        raise
+    got = run_matmul(ctx, fmt, x, w, ROUTES[route])
+    got_d = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d)
     orc.assert_close(got, orc.matmul_f32(x, deq), REL, ABS)
     orc.assert_close(got_d, orc.matmul_f32(x, deq, d), REL, ABS)
 
@@ -179,7 +188,7 @@ def test_larger_m(ctx, orc, fmt, m, k, n):
     w = synth.normal(12 + m + k + n, k * n, 0.02).reshape(k, n)
     d = synth.normal(13 + n, m * n).reshape(m, n)
     deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
-    for route in ("generic", "gemm_mfma", "auto"):
+    for route in ("generic", "gemm_mfma", "tile_mfma", "auto"):
         got = run_matmul(ctx, fmt, x, w, ROUTES[route], d=d)
         orc.assert_close(got, orc.matmul_f32(x, deq, d), REL, ABS)
         # fp16 activations: the oracle multiplies the rounded values
@@ -256,7 +265,7 @@ def test_linearity_and_zero_input(ctx):
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-@pytest.mark.parametrize("m,k,n,route", [(16, 4096, 2048, "gemm_mfma"), (4, 14336, 1024, "gemv_mfma")])
+@pytest.mark.parametrize("m,k,n,route", [(16, 4096, 2048, "gemm_mfma"), (4, 14336, 1024, "gemv_mfma"), (16, 14336, 1024, "tile_mfma")])
 def test_split_k_is_repeatable(ctx, orc, fmt, m, k, n, route):
     """Few tiles and a long K: the tiled kernel splits K across workgroups and the last
     one to arrive adds the partial tiles in part order (the GEMV kernel does the same when
@@ -432,7 +441,7 @@ UNARY = {"relu": capi.UNARY_RELU, "sigmoid": capi.UNARY_SIGMOID, "neg": capi.UNA
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-@pytest.mark.parametrize("route", ["generic", "gemv_valu", "gemv_mfma", "gemm_mfma", "auto"])
+@pytest.mark.parametrize("route", ["generic", "gemv_valu", "gemv_mfma", "gemm_mfma", "tile_mfma", "auto"])
 @pytest.mark.parametrize("m,k,n", [(1, 576, 192), (4, 14336, 70), (6, 1024, 300), (16, 4096, 2048)])
 def test_unary_epilogues(ctx, orc, fmt, route, m, k, n):
     """C = f(A x W + D) in the matmul's own launch: every operation the reference folds into a
@@ -452,12 +461,11 @@ def test_unary_epilogues(ctx, orc, fmt, route, m, k, n):
     try:
         for chain, with_d in ((("relu",), False), (("sigmoid",), True), (("neg",), False), (("silu",), True),
                               (("relu", "neg"), True), ((), False)):
-            try:
-                ctx.matmul_q_epilogue(a, wt, c, m, [UNARY[o] for o in chain], db if with_d else None)
-            except capi.MgnError as e:
-                if route != "generic" and "does not support" in str(e):
-                    pytest.skip("shape outside this kernel's range")
-                raise
+            if (route, m, k, n) in REFUSED:
+                with pytest.raises(capi.MgnError, match="does not support"):
+                    ctx.matmul_q_epilogue(a, wt, c, m, [UNARY[o] for o in chain], db if with_d else None)
+                continue
+            ctx.matmul_q_epilogue(a, wt, c, m, [UNARY[o] for o in chain], db if with_d else None)
             got = c.download(np.float32, m * n).reshape(m, n)
             want = plain_d if with_d else plain
             for o in chain:
@@ -606,7 +614,7 @@ def test_a_column_with_infinite_scales_stays_on_its_own(ctx, orc, fmt, m):
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-@pytest.mark.parametrize("m,route", [(1, "gemv_mfma"), (4, "gemv_mfma"), (16, "gemm_mfma")])
+@pytest.mark.parametrize("m,route", [(1, "gemv_mfma"), (4, "gemv_mfma"), (16, "gemm_mfma"), (16, "tile_mfma"), (40, "tile_mfma")])
 def test_activations_and_weights_with_a_large_mean(ctx, orc, fmt, m, route):
     """All-positive activations against weights whose blocks sit far from zero: the format's
     additive part (block minimum x sum of activations) and the scaled quant sums are then both
@@ -622,52 +630,79 @@ def test_activations_and_weights_with_a_large_mean(ctx, orc, fmt, m, route):
     orc.assert_close(got, want, REL, ABS)
 
 
+def assert_close_rowwise(got, want, x):
+    """The matmul bar with its absolute part scaled by each row's activation magnitude: the
+    reference's 1e-4 is meant for activations of order one, and a row scaled by s has outputs and
+    errors scaled by s."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    rms = np.sqrt((np.asarray(x, np.float64) ** 2).mean(axis=1, keepdims=True))
+    err = np.abs(got - want)
+    ok = (err <= REL * np.abs(want)) | (err <= ABS * rms)
+    assert np.isfinite(got).all()
+    assert ok.all(), f"{(~ok).sum()} of {ok.size} outside the bar; worst {err.max():.3e} at row {np.unravel_index(err.argmax(), err.shape)[0]}"
+
+
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-def test_weights_outside_the_tiled_kernels_range_take_another_route(ctx, orc, fmt):
-    """The tiled MFMA kernel hands 32 x block-minimum (Q4) or 4096 x scale (Q8) to the matrix
-    cores as fp16.  A weight with a block beyond that is recognised when it is created: the
-    automatic route then avoids that kernel and the result is still the oracle's."""
+def test_weights_with_huge_minima_and_scales_stay_on_the_matrix_cores(ctx, orc, fmt):
+    """Blocks whose minimum (Q4) or scale (Q8) is far beyond anything a model holds.  The 16x16x32
+    tiled kernel multiplies the block's m (or scale) as the fp16 value it is stored as, against
+    block means that stay below 2^12, so no weight is out of its range; the automatic route
+    takes it for weights the faster 32x32x16 kernel cannot hold -- however the weight was created."""
     m, k, n = 16, 256, 96
     w = synth.normal(990 + fmt, k * n, 0.02).reshape(k, n)
     w[32:64, 5] = np.linspace(-5000.0, -4990.0, 32, dtype=np.float32)   # block minimum -5000
     w[64:96, 7] = np.linspace(-3000.0, 3000.0, 32, dtype=np.float32)    # Q8 scale 23.6
+    w[96:128, 9] = np.linspace(-60000.0, 60000.0, 32, dtype=np.float32)  # near the largest half
     x = synth.normal(991, m * k, 1.0).reshape(m, k)
-    wt = ctx.weight(fmt, w)
-    want = orc.matmul_packed(fmt, x, orc.quantize(fmt, w), n)
-    got = run_matmul(ctx, fmt, x, wt)
-    assert np.isfinite(got).all()
-    orc.assert_close(got, want, REL, ABS)
-    with pytest.raises(capi.MgnError, match="does not support"):
-        run_matmul(ctx, fmt, x, wt, ROUTES["gemm_mfma"])
-    # batch-1 stays on the MFMA GEMV, which has no such limit
-    got1 = run_matmul(ctx, fmt, x[:1], wt, ROUTES["gemv_mfma"])
-    orc.assert_close(got1, want[:1], REL, ABS)
-    wt.free()
-    # same weight through the device quantizer and from packed bytes
+    packed = orc.quantize(fmt, w)
+    want = orc.matmul_f64(x, orc.dequantize(fmt, packed, k, n))
     src = ctx.upload(w)
-    for other in (ctx.weight_from_device(fmt, src, k, n), ctx.weight_from_packed(fmt, orc.quantize(fmt, w), k, n)):
+    for wt in (ctx.weight(fmt, w), ctx.weight_from_device(fmt, src, k, n), ctx.weight_from_packed(fmt, packed, k, n)):
+        for route in ("auto", "tile_mfma"):
+            got = run_matmul(ctx, fmt, x, wt, ROUTES[route])
+            assert np.isfinite(got).all()
+            # the huge columns' outputs are of order 1e5: relative bar there, absolute elsewhere
+            orc.assert_close(got, want, REL, ABS)
+        # the 32x32x16 kernel feeds 32 x m (Q8: 4096 x scale) to the matrix cores as fp16 and refuses the weight
         with pytest.raises(capi.MgnError, match="does not support"):
-            run_matmul(ctx, fmt, x, other, ROUTES["gemm_mfma"])
-        other.free()
+            run_matmul(ctx, fmt, x, wt, ROUTES["gemm_mfma"])
+        got1 = run_matmul(ctx, fmt, x[:1], wt, ROUTES["gemv_mfma"])
+        orc.assert_close(got1, want[:1], REL, ABS)
+        wt.free()
     src.free()
 
 
-def test_activations_beyond_the_fp16_pair_are_reported(ctx, orc):
-    """An f32 activation >= 65504 cannot be split into an fp16 pair: the tiled kernel flags it
-    and the next synchronising call fails loudly instead of handing back wrong numbers.  The
-    generic route computes such data; batch-1..4 (MFMA GEMV) rescales per block and has no limit."""
-    m, k, n = 16, 256, 96
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m", [5, 16, 40])
+def test_activations_of_any_magnitude_on_the_rescaling_tiled_kernel(ctx, orc, fmt, m):
+    """f32 activations are scaled per (row, 256-element slice) by a power of two before they are
+    split into fp16 pairs: rows of magnitude 1e-20, 1e-4, 1 and 1e6 side by side, an outlier of
+    2e5 in an ordinary row and a value near the largest float all come out within the bar of the
+    f64 product (absolute part scaled by the row's magnitude).  The reference computes in f32."""
+    k, n = 1280, 208
     w = synth.normal(995, k * n, 0.02).reshape(k, n)
-    x = synth.normal(996, m * k, 1.0).reshape(m, k)
-    x[3, 17] = np.float32(2.0e5)
-    wt = ctx.weight(Q4, w)
-    want = orc.matmul_packed(Q4, x, orc.quantize(Q4, w), n)
+    x = synth.normal(996 + m, m * k, 1.0).reshape(m, k)
+    mags = np.array([1e-20, 1e-4, 1.0, 1e6, 3e-3, 1e12, 1e-9], np.float32)
+    for r in range(m):
+        x[r] *= mags[r % len(mags)]
+    x[2, 17] = np.float32(2.0e5)      # outlier in a row of order one
+    x[m - 1, 300] = np.float32(1e30)  # dominates its row and its slice
+    packed = orc.quantize(fmt, w)
+    want = orc.matmul_f64(x, orc.dequantize(fmt, packed, k, n))
+    wt = ctx.weight(fmt, w)
+    for route in ("tile_mfma", "generic"):
+        assert_close_rowwise(run_matmul(ctx, fmt, x, wt, ROUTES[route]), want, x)
+    # the 32x32x16 kernel splits activations into fp16 pairs without rescaling: it flags such data
+    # and the next synchronising call fails loudly instead of handing back wrong numbers
     with pytest.raises(capi.MgnError) as e:
-        run_matmul(ctx, Q4, x, wt, ROUTES["gemm_mfma"])
+        run_matmul(ctx, fmt, x, wt, ROUTES["gemm_mfma"])
     assert e.value.status == capi.ERANGE
     ctx.sync()  # reported once; the context keeps working
-    orc.assert_close(run_matmul(ctx, Q4, x, wt, ROUTES["generic"]), want, REL, ABS)
-    orc.assert_close(run_matmul(ctx, Q4, x[:4], wt, ROUTES["gemv_mfma"]), want[:4], REL, ABS)
-    x[3, 17] = np.float32(60000.0)  # inside the range
-    orc.assert_close(run_matmul(ctx, Q4, x, wt, ROUTES["gemm_mfma"]), orc.matmul_packed(Q4, x, orc.quantize(Q4, w), n), REL, ABS)
+    # non-finite activations give non-finite outputs in their own rows only
+    x[1, 5] = np.float32(np.inf)
+    x[3, 700] = np.float32(np.nan)
+    got = run_matmul(ctx, fmt, x, wt, ROUTES["tile_mfma"])
+    assert not np.isfinite(got[1]).any() and not np.isfinite(got[3]).any()
+    rest = [r for r in range(m) if r not in (1, 3)]
+    assert_close_rowwise(got[rest], want[rest], x[rest])
     wt.free()

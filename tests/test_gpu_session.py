@@ -399,3 +399,33 @@ def test_matmul_at_and_fused_add_forms(orc, quant, m, k, n):
         orc.assert_close(sess.read_output_by_index(1, m * n).reshape(m, n), fused, 1e-3, 1e-4)
         orc.assert_close(sess.read_output_by_index(2, m * n).reshape(m, n), bt, 1e-3, 1e-4)
     sess.close()
+
+
+@pytest.mark.parametrize("k", [15392, 16000, 16384])
+def test_siblings_that_plan_alone_but_not_together_run_as_separate_launches(orc, k):
+    """q, k, v with a long K and few columns: each weight alone has a one-launch plan with a
+    fused norm, three of them in one launch have none (the launch is planned for the columns of
+    the whole batch).  The step must fall back to fewer weights per launch, not fail."""
+    n = 544
+    g = Graph()
+    x = g.input("x", [1, k])
+    h = g.rms_norm(x, g.parameter("norm", [k]), 1e-5)
+    outs = [g.matmul(h, g.parameter_q4(name, [k, n])) for name in ("wq", "wk", "wv")]
+    g.set_outputs(outs)
+    sess = build_inference_session(g)
+    ws = {name: synth.normal(700 + i + k, k * n, 0.02).reshape(k, n) for i, name in enumerate(("wq", "wk", "wv"))}
+    for name, w in ws.items():
+        sess.set_parameter(name, w)
+    gamma = (1.0 + 0.1 * synth.normal(710, k, 1.0)).astype(np.float32)
+    xs = synth.normal(711 + k, k, 1.0)
+    sess.set_parameter("norm", gamma)
+    sess.set_input("x", xs)
+    sess.step()
+    sess.wait()
+    x64 = xs.astype(np.float64)
+    normed = (x64 / np.sqrt((x64 * x64).mean() + 1e-5) * gamma).astype(np.float32).reshape(1, k)
+    for i, name in enumerate(("wq", "wk", "wv")):
+        got = sess.read_output_by_index(i, n)
+        want = orc.matmul_f32(normed, orc.dequantize(Q4, orc.quantize(Q4, ws[name]), k, n))
+        orc.assert_close(got.reshape(1, n), want, 1e-3, 1e-4)
+    sess.close()
