@@ -182,6 +182,43 @@ __device__ __forceinline__ void make_chunks(const float (&x)[8], uint4& hi, uint
   lo = make_uint4(l[0], l[1], l[2], l[3]);
 }
 
+// ---- one activation row: integer digits on the int8 matrix instruction ----
+// With a single activation row the four A rows of v_mfma_i32_4x4x4_16B_i8 hold the base-128
+// digits of the activations instead of fp16 halves: x, scaled per 32-element block by a power of
+// two to |x| < 2^20 and rounded to an integer, is d0 + 128 d1 + 16384 d2 with d0, d1 in
+// [0, 127] and d2 in [-64, 64] -- three int8 rows (the fourth is not used).  The B operand is
+// then the nibbles as bytes (two mask operations per four weights instead of seven for eight) or,
+// for Q8, the weight bytes as they are; the products are exact integers and the three digit sums
+// are put together with two shift-adds.  The vector ALU work per block drops by a third, which
+// is what bounds the Q4 kernel when the engine clock is low.
+// A block's image is 128 bytes: Q4 [plane i][MFMA 0..7] dwords (MFMA 2c holds elements 8c + 0, 2,
+// 4, 6 and MFMA 2c + 1 elements 8c + 1, 3, 5, 7, as the two nibble masks deliver them); Q8
+// [half][plane i][MFMA 0..3] dwords in natural order.
+
+// eight scaled activations -> their three digit planes, four bytes per dword: lo[i], hi[i] hold
+// plane i of elements (e0, e1, e2, e3) and (e4, e5, e6, e7) of the given order
+__device__ __forceinline__ void make_digits(const float (&x)[8], const int (&order)[8], uint32_t (&lo)[3], uint32_t (&hi)[3], int* sum) {
+  int v[8];
+  int s = 0;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    v[e] = (int)__builtin_rintf(x[e]);
+    s += v[e];
+  }
+  *sum = s;
+#pragma unroll
+  for (int i = 0; i < 3; i++) {
+    uint32_t d[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const int val = v[order[e]];
+      d[e] = i == 0 ? (uint32_t)val & 127u : i == 1 ? ((uint32_t)val >> 7) & 127u : (uint32_t)(val >> 14) & 255u;
+    }
+    lo[i] = d[0] | (d[1] << 8) | (d[2] << 16) | (d[3] << 24);
+    hi[i] = d[4] | (d[5] << 8) | (d[6] << 16) | (d[7] << 24);
+  }
+}
+
 // Power of two that brings a block's largest magnitude below 2^12 (1 if the block
 // is all zero, tiny or not finite).  *inv gets the reciprocal.
 __device__ __forceinline__ float block_scale(float amax, float* inv) {
@@ -233,6 +270,10 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   const uint32_t m = m_flags & 0xFFu;
   const bool a_f16 = PRO == kProNone && (m_flags >> 31) != 0;
   const GemvPrologue pro{norm_weight, eps};
+  // one activation row of a Q4 weight: integer digits, int8 matrix instruction (see above).  (Q8 has the
+  // code path too but measured 3 % slower with it, 12.35 against 12.0 us on 4096 x 14336: its bytes
+  // need no unpacking in either form, so there is little vector-ALU work to save.)
+  constexpr bool I8 = MROWS == 1 && FMT == MGN_FMT_Q4;
   constexpr int NJ = 2 * MROWS;       // A rows in LDS: hi and lo of every activation row
   constexpr int NG = (MROWS + 1) / 2;  // groups of four A rows = MFMA chains per weight chunk
   extern __shared__ uint4 lds4[];
@@ -465,10 +506,45 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         // does and switches scaling off
         float am = fmaxf(fmaxf(fmaxf(fabsf(v0.x), fabsf(v0.y)), fmaxf(fabsf(v0.z), fabsf(v0.w))),
                          fmaxf(fmaxf(fabsf(v1.x), fabsf(v1.y)), fmaxf(fabsf(v1.z), fabsf(v1.w))));
+        if constexpr (I8) {
+          // integers cannot carry a NaN along: a block that holds one (or an infinity, or values
+          // beyond 2^100, which are not rescaled) is given a NaN factor, so its column sums come
+          // out non-finite as the reference's would
+          const bool has_nan = __builtin_isunordered(v0.x, v0.y) || __builtin_isunordered(v0.z, v0.w) ||
+                               __builtin_isunordered(v1.x, v1.y) || __builtin_isunordered(v1.z, v1.w);
+          am = has_nan ? __builtin_inff() : am;
+        }
         am = fmaxf(am, dpp_move<kDppQuadXor1>(am));
         am = fmaxf(am, dpp_move<kDppQuadXor2>(am));
         float inv;
-        const float scale = block_scale(am, &inv);
+        float scale = block_scale(am, &inv);
+        if constexpr (I8) {
+          // |x| * scale < 2^20 (block_scale leaves 2^12), so that rounding cannot reach 2^21 and the top
+          // digit stays within int8
+          if (scale != 1.0f || inv != 1.0f) scale *= 256.0f, inv *= 0.00390625f;
+          if (!(am < 1.0e30f)) inv = __builtin_nanf("");
+          const float x[8] = {v0.x * scale, v0.y * scale, v0.z * scale, v0.w * scale,
+                              v1.x * scale, v1.y * scale, v1.z * scale, v1.w * scale};
+          uint32_t dlo[3], dhi[3];
+          int isum;
+          uint32_t* const xw = (uint32_t*)xa;
+          if constexpr (FMT == MGN_FMT_Q4) {
+            const int order[8] = {0, 2, 4, 6, 1, 3, 5, 7};
+            make_digits(x, order, dlo, dhi, &isum);
+#pragma unroll
+            for (int pl = 0; pl < 3; pl++) *(uint2*)(xw + kb * 32 + pl * 8 + 2 * ch) = make_uint2(dlo[pl], dhi[pl]);
+            isum += __builtin_amdgcn_update_dpp(0, isum, kDppQuadXor1, 0xF, 0xF, true);
+            isum += __builtin_amdgcn_update_dpp(0, isum, kDppQuadXor2, 0xF, 0xF, true);
+            if (ch == 0) cinit[kb * MROWS + r] = make_float2(-8.0f * (float)isum, inv);
+          } else {
+            const int order[8] = {0, 1, 2, 3, 4, 5, 6, 7};
+            make_digits(x, order, dlo, dhi, &isum);
+            // half ch / 2 of the block, MFMAs 2 (ch % 2) and 2 (ch % 2) + 1 of that half
+#pragma unroll
+            for (int pl = 0; pl < 3; pl++) *(uint2*)(xw + kb * 32 + (ch >> 1) * 16 + pl * 4 + 2 * (ch & 1)) = make_uint2(dlo[pl], dhi[pl]);
+            if ((ch & 1) == 0) cinit[(kb * 2 + (ch >> 1)) * MROWS + r] = make_float2(0.0f, inv);
+          }
+        } else {
         const float x[8] = {v0.x * scale, v0.y * scale, v0.z * scale, v0.w * scale,
                             v1.x * scale, v1.y * scale, v1.z * scale, v1.w * scale};
         uint4 hi, lo;
@@ -486,6 +562,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
           s += dpp_move<kDppQuadXor2>(s);
           if (ch == 0) cinit[kb * MROWS + r] = make_float2(s * (-bias / operand_scale<FMT>()), inv * operand_scale<FMT>());
         }
+        }
       }
     }
   }
@@ -498,7 +575,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   const uint32_t scale_lane = (((b >> 1) << 2) | i) * 4;  // Q8: byte address of lane (b / 2, i) for ds_bpermute
   // Q4: K block kb_first + 16 s.  Q8: half (b & 1) of blocks kb8_first + 16 s and + 8, i.e. chunks
   // 2 (b & 1) and 2 (b & 1) + 1 of those blocks.
-  const char* xa_lane = FMT == MGN_FMT_Q8
+  const char* xa_lane = I8 ? (FMT == MGN_FMT_Q8 ? (const char*)xa + (size_t)kb8_first * 128 + (b & 1) * 64 + i * 16
+                                                : (const char*)xa + (size_t)kb_first * 128 + i * 32)
+                        : FMT == MGN_FMT_Q8
                             ? (const char*)xa + ((size_t)kb8_first * NJ + jrow + (size_t)2 * (b & 1) * plane) * 16
                             : (const char*)xa + ((size_t)kb_first * NJ + jrow) * 16;
   const char* ci_lane = FMT == MGN_FMT_Q8 ? (const char*)cinit + (size_t)(kb8_first * 2 + (b & 1)) * MROWS * 8
@@ -523,7 +602,59 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // not every step is a full one: a block past the end of K or in a step that belongs to the
     // neighbouring K split gets scale (and minimum) zero
     if constexpr (!EXACT) cur.meta = ((uint32_t)s >= first_own && kb_first + s * 16 < bpc_live) ? cur.meta : 0u;
-    if constexpr (FMT == MGN_FMT_Q4) {
+    if constexpr (I8 && FMT == MGN_FMT_Q4) {
+      typedef int intx4 __attribute__((ext_vector_type(4)));
+      const bool tail_step = TAIL && t == TS;
+      const char* const xa_step = tail_step ? (const char*)xa + (size_t)tail_kb * 128 + i * 32 : xa_lane + s * (16 * 128);
+      const char* const ci_step = tail_step ? (const char*)cinit + (size_t)tail_kb * MROWS * 8 : ci_lane + s * (16 * MROWS * 8);
+      const uint4 a0 = *(const uint4*)xa_step, a1 = *(const uint4*)(xa_step + 16);  // this lane's digit plane, 8 MFMAs
+      const float2 ci0 = *(const float2*)ci_step;  // {-8 * sum of the block's integers, factor that undoes the block scale}
+      const uint32_t aw[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+      const uint32_t words[4] = {cur.q.x, cur.q.y, cur.q.z, cur.q.w};
+      intx4 dsum = {0, 0, 0, 0};
+#pragma unroll
+      for (int ch = 0; ch < 4; ch++) {
+        const uint32_t wd = words[ch];
+        const uint32_t even = wd & 0x0F0F0F0Fu, odd = (wd >> 4) & 0x0F0F0F0Fu;  // (n0,n2,n4,n6), (n1,n3,n5,n7)
+        dsum = __builtin_amdgcn_mfma_i32_4x4x4i8((int)aw[2 * ch], (int)even, dsum, 0, 0, 0);
+        dsum = __builtin_amdgcn_mfma_i32_4x4x4i8((int)aw[2 * ch + 1], (int)odd, dsum, 0, 0, 0);
+      }
+      const int tot = (((dsum[2] << 7) + dsum[1]) << 7) + dsum[0];  // digits back together: sum n * x
+      const float dscale = half_bits_to_float(cur.meta & 0xFFFFu);
+      const float mneg = __fmaf_rn(-0.125f, half_bits_to_float(cur.meta >> 16), -dscale);  // (m + 8 d) S = mneg * (-8 S)
+      float v = dscale * ((float)tot + ci0.x);
+      v = __fmaf_rn(mneg, ci0.x, v);
+      if (tail_step) {
+#pragma unroll
+        for (int qq = 0; qq < QPW; qq++) {
+          const float sum = __fmaf_rn(v, ci0.y, acc[qq][0]);
+          acc[qq][0] = tail_q == (uint32_t)qq ? sum : acc[qq][0];
+        }
+      } else {
+        constexpr int QMAX = QPW - 1;
+        const int qa = q < QPW ? q : QMAX;
+        acc[qa][0] = __fmaf_rn(v, ci0.y, acc[qa][0]);
+      }
+    } else if constexpr (I8) {
+      typedef int intx4 __attribute__((ext_vector_type(4)));
+      // Q8: two half blocks per step; the weight bytes are the B operand as they are
+      const int dscale_own = __builtin_bit_cast(int, half_bits_to_float(cur.meta));
+      const float dscales[2] = {__builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((int)scale_lane, dscale_own)),
+                                __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((int)scale_lane + 8 * 4 * 4, dscale_own))};
+#pragma unroll
+      for (int hb = 0; hb < 2; hb++) {
+        const uint4 qw = hb == 0 ? cur.q0 : cur.q1;
+        const uint4 a4 = *(const uint4*)(xa_lane + s * (16 * 128) + hb * (8 * 128));
+        const float2 ci0 = *(const float2*)(ci_lane + s * (16 * 2 * MROWS * 8) + hb * (8 * 2 * MROWS * 8));
+        intx4 dsum = {0, 0, 0, 0};
+        dsum = __builtin_amdgcn_mfma_i32_4x4x4i8((int)a4.x, (int)qw.x, dsum, 0, 0, 0);
+        dsum = __builtin_amdgcn_mfma_i32_4x4x4i8((int)a4.y, (int)qw.y, dsum, 0, 0, 0);
+        dsum = __builtin_amdgcn_mfma_i32_4x4x4i8((int)a4.z, (int)qw.z, dsum, 0, 0, 0);
+        dsum = __builtin_amdgcn_mfma_i32_4x4x4i8((int)a4.w, (int)qw.w, dsum, 0, 0, 0);
+        const int tot = (((dsum[2] << 7) + dsum[1]) << 7) + dsum[0];
+        acc[q][0] = __fmaf_rn(dscales[hb] * (float)tot, ci0.y, acc[q][0]);
+      }
+    } else if constexpr (FMT == MGN_FMT_Q4) {
       const bool tail_step = TAIL && t == TS;
       // the step's activations and block constants: K block kb_first + 16 s, or the lane's tail block
       const char* const xa_step = tail_step ? (const char*)xa + ((size_t)tail_kb * NJ + jrow) * 16 : xa_lane + s * (16 * NJ * 16);
