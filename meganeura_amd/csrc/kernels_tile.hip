@@ -10,16 +10,15 @@
 //   v_mfma_f32_16x16x32_f16: one instruction contracts one 32-element quant block of 16
 //   columns against 16 activation rows.  Lane (c, g), c = lane % 16, g = lane / 16, supplies
 //   k = 8g..8g+7 of column c (B) or of row c (A) and receives rows 4g..4g+3 of column c (D).
-//   B operand: dword g of the block's nibbles, masked to fp16 bits 4-7 (n * 2^-20, exact;
-//     Q8: the block's bytes 8g..8g+7 as (q + 128) * 2^-24 in bits 0-7).  The quants travel from
-//     memory as whole 128/256-byte runs of a column's blocks, are parked in a wave-private LDS
-//     slice and read back one dword (Q8: two) per lane and block.
-//   A operand: the activations, converted ONCE per call by a small kernel into an "image" in
-//     the instruction's own lane order (image_kernel below), which every workgroup then only
-//     copies into LDS, slice by slice, double-buffered.  f32 activations are scaled per (row,
-//     256-element K slice) by a power of two and split hi + lo into two fp16 operands that are
-//     multiplied into the same accumulator, so products are exact, any finite magnitude is
-//     representable and only f32 accumulation rounds; fp16 activations are used as they are.
+//   B operand: dword g of the block's nibbles, masked into the mantissa bits of fp16 subnormals
+//     (n * 2^-20, exact; with f32 activations the even nibbles stay at n * 2^-24 and their
+//     activations are stored times 16: two shifts fewer per dword; Q8: the block's bytes
+//     8g..8g+7 as (q + 128) * 2^-24 in bits 0-7).
+//   A operand: the activations, converted into an "image" in the instruction's own lane order.
+//     f32 activations are scaled per (row, 256-element K slice) by a power of two and split
+//     hi + lo into two fp16 operands that are multiplied into the same accumulator, so products
+//     are exact, any finite magnitude is representable and only f32 accumulation rounds; fp16
+//     activations are used as they are.
 //   Per block: D = sum n x on the matrix cores, then P += d * D on the vector ALU (4 FMAs per
 //     lane).  The format's additive part (m * sum(x) for Q4, -128 * scale * sum(x) for Q8's byte
 //     bias) is one more MFMA per slice of 8 blocks: its A operand holds the blocks' mean
@@ -27,12 +26,20 @@
 //     A slice's P is multiplied by the rows' inverse power-of-two scales and added to the
 //     accumulators.
 //
-// Work split: grid = (K parts, column groups, row groups).  A workgroup owns wnc column tiles of
-// 16 columns, R row tiles of 16 rows and a range of K slices; ksc waves share a column tile and
-// take the slices of a phase side by side (their sums meet in LDS, in a fixed order); with too
-// few tiles to fill the chip K is also cut into parts for different workgroups, whose partial
-// tiles the last one to finish adds in part order (deterministic).
+// Two kernels share this arithmetic.
+//   tile_mfma_kernel (any M): image_kernel converts the activations ONCE per call into images
+//     in the workspace, which every workgroup copies into LDS slice by slice, double-buffered.
+//     The quants travel from memory as whole 128/256-byte runs of a column's blocks, are parked
+//     in a wave-private LDS slice and read back one dword (Q8: two) per lane and block.
+//     grid = (K parts, column groups, row groups): a workgroup owns wnc column tiles of 16
+//     columns, R row tiles of 16 rows and a range of K slices; ksc waves share a column tile and
+//     take the slices of a phase side by side (their sums meet in LDS, in a fixed order).
+//   tile_resident_kernel (M <= 32): every workgroup converts its own K part and keeps the
+//     images in LDS; no second launch, no image traffic (see there).
+// With too few tiles to fill the chip K is also cut into parts for different workgroups, whose
+// partial tiles the last one to finish adds in part order (deterministic).
 #include <algorithm>
+#include <type_traits>
 
 #include "kernels_common.hip.h"
 
@@ -55,8 +62,15 @@ __device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
 __device__ __forceinline__ float half_lo(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[0]; }
 __device__ __forceinline__ float half_hi(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[1]; }
 
-// one dword of nibbles -> B operand (8 fp16): (n0,n4),(n1,n5),(n2,n6),(n3,n7), each n * 2^-20
+// one dword of nibbles -> B operand (8 fp16): (n0,n4),(n1,n5),(n2,n6),(n3,n7), each n * 2^-20.
+// SPLIT: the even nibbles stay in bits 0-3 of their halves, n * 2^-24 (two shifts fewer); the
+// activations they meet are stored times 16 in the image.
+template <bool SPLIT>
 __device__ __forceinline__ half8 nibbles_to_operand(uint32_t wd) {
+  if constexpr (SPLIT) {
+    const uint32_t hi = wd >> 8;
+    return as_half8(wd & 0x000F000Fu, wd & 0x00F000F0u, hi & 0x000F000Fu, hi & 0x00F000F0u);
+  }
   return as_half8((wd << 4) & 0x00F000F0u, wd & 0x00F000F0u, (wd >> 4) & 0x00F000F0u, (wd >> 8) & 0x00F000F0u);
 }
 // two dwords of int8 -> B operand: (b0,b1),(b2,b3),(b4,b5),(b6,b7), each (q + 128) * 2^-24
@@ -76,8 +90,9 @@ __device__ __forceinline__ float group_max32(float v) {
   return v;
 }
 
-// Power of two that brings a row slice's largest magnitude into [2^11, 2^12) (1 if the slice
-// is all zero, tiny, huge or not finite).  *inv gets the reciprocal.
+// Power of two that brings a row slice's largest magnitude into [2^TOP, 2^(TOP+1)) (1 if the
+// slice is all zero, tiny, huge or not finite).  *inv gets the reciprocal.
+template <int TOP>
 __device__ __forceinline__ float slice_scale(float amax, float* inv) {
   const uint32_t bits = __builtin_bit_cast(uint32_t, amax);
   const int e = (int)(bits >> 23) - 127;  // floor(log2(amax)) for normal values
@@ -85,55 +100,52 @@ __device__ __forceinline__ float slice_scale(float amax, float* inv) {
     *inv = 1.0f;
     return 1.0f;
   }
-  const int sh = 11 - e;
+  const int sh = TOP - e;
   *inv = __builtin_bit_cast(float, (uint32_t)(127 - sh) << 23);
   return __builtin_bit_cast(float, (uint32_t)(127 + sh) << 23);
 }
 
 // ---- the activation image ----
 // One image per (row tile of 16 rows, K slice of 8 blocks = 256 elements), in uint4 units:
-//   [(kb * HL + h) * 64 + lane]  A operand of block kb, h = 0 high halves, h = 1 low halves (f32
-//                                activations only: HL = 2), for A lane = row + 16 * g
+//   [(kb * HL + h) * 64 + image_slot(row, g, kb)]
+//                                A operand of block kb, h = 0 high halves, h = 1 low halves (f32
+//                                activations only: HL = 2), for A lane = row + 16 * g.  The slot is
+//                                the lane with its row rotated by 2 g + 8 (kb % 2): the eight lanes
+//                                that write together during the conversion (one row, two blocks, four
+//                                g) then fall into different LDS banks, and so do the readers'.
 //   [8 * HL * 64 + lane]         A operand of the slice's additive MFMA: lanes (row, g' < 2) hold
 //                                (mean_hi | mean_lo << 16) of blocks 4g'..4g'+3, the rest is zero
 //   [8 * HL * 64 + 64 + 0..15]   (as float) the rows' inverse scales times the quants' operand scale
 //                                (2^20 for Q4, 2^24 for Q8; f32 activations only)
 // The element order inside an operand follows the B side: Q4 pairs k with k + 4, Q8 is natural.
+// Q4 with f32 activations: the even elements are stored times 16 (see nibbles_to_operand) and the
+// slice scale aims at 2^7 instead of 2^11 to leave room for that.
 constexpr uint32_t kSliceBlocks = 8;
+__device__ __forceinline__ uint32_t image_slot(uint32_t row, uint32_t g, uint32_t kb_parity) {
+  return ((row + 2 * g + 8 * kb_parity) & 15u) + 16 * g;
+}
 constexpr uint32_t image_units(bool f32a) { return kSliceBlocks * (f32a ? 2u : 1u) * 64u + 64u + 16u; }
 
-// grid.x = row tiles * slices; 512 threads: half-wave r (0..15) converts row r of the tile,
-// lane l = kb * 4 + g of it the 8 elements k = 32 kb + 8 g .. + 7 of the slice.
+// One task of the conversion: half-wave lane l = kb * 4 + g turns the 8 activations k0 .. k0 + 7
+// (k0 = 256 slice + 32 kb + 8 g) of row `row` into its piece of the image `img` of that (row tile,
+// slice); r = row % 16.  All 32 lanes of the half-wave (one row of one slice) must call it together.
 template <int FMT, bool F32A>
-__global__ __launch_bounds__(512) void image_kernel(const void* __restrict__ a, uint4* __restrict__ image, uint32_t m,
-                                                    uint32_t k, uint32_t nslices, uint32_t a_stride) {
+__device__ __forceinline__ void convert_task(const float (&xin)[8], bool ok, uint4* __restrict__ img, uint32_t r, uint32_t l) {
   constexpr uint32_t HL = F32A ? 2 : 1;
-  constexpr uint32_t UNITS = image_units(F32A);
-  const uint32_t rt = blockIdx.x / nslices, sl = blockIdx.x - rt * nslices;
-  const uint32_t r = threadIdx.x >> 5, l = threadIdx.x & 31, kb = l >> 2, g = l & 3;
-  const uint32_t row = rt * 16 + r, k0 = sl * 256 + kb * 32 + g * 8;
-  const bool ok = row < m && k0 < k;  // K is a multiple of 32: a task lies inside or outside as a whole
+  const uint32_t kb = l >> 2, g = l & 3;
   float x[8];
-  if constexpr (F32A) {
-    const float4* src = (const float4*)((const float*)a + (ok ? (size_t)row * a_stride + k0 : (size_t)0));
-    const float4 v0 = src[0], v1 = src[1];
-    x[0] = v0.x, x[1] = v0.y, x[2] = v0.z, x[3] = v0.w, x[4] = v1.x, x[5] = v1.y, x[6] = v1.z, x[7] = v1.w;
-  } else {
-    const uint4 v = *(const uint4*)((const _Float16*)a + (ok ? (size_t)row * a_stride + k0 : (size_t)0));
-    x[0] = half_lo(v.x), x[1] = half_hi(v.x), x[2] = half_lo(v.y), x[3] = half_hi(v.y);
-    x[4] = half_lo(v.z), x[5] = half_hi(v.z), x[6] = half_lo(v.w), x[7] = half_hi(v.w);
-  }
 #pragma unroll
-  for (int e = 0; e < 8; e++) x[e] = ok ? x[e] : 0.0f;
+  for (int e = 0; e < 8; e++) x[e] = ok ? xin[e] : 0.0f;
   float inv = 1.0f;
   if constexpr (F32A) {
     // NaN never wins fmaxf; an infinity does and switches scaling off
     float am = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))),
                      fmaxf(fmaxf(fabsf(x[4]), fabsf(x[5])), fmaxf(fabsf(x[6]), fabsf(x[7]))));
     am = group_max32(am);
-    const float scale = slice_scale(am, &inv);
+    constexpr bool kSplit = FMT == MGN_FMT_Q4;
+    const float scale = slice_scale<kSplit ? 7 : 11>(am, &inv);
 #pragma unroll
-    for (int e = 0; e < 8; e++) x[e] *= scale;
+    for (int e = 0; e < 8; e++) x[e] *= (kSplit && e % 2 == 0) ? scale * 16.0f : scale;
   }
   float p[8];
   if constexpr (FMT == MGN_FMT_Q4) {
@@ -142,11 +154,9 @@ __global__ __launch_bounds__(512) void image_kernel(const void* __restrict__ a, 
 #pragma unroll
     for (int e = 0; e < 8; e++) p[e] = x[e];
   }
-  uint4* const img = image + ((size_t)rt * nslices + sl) * UNITS;
-  const uint32_t alane = r + 16 * g;
+  const uint32_t alane = image_slot(r, g, kb & 1);
   const uint32_t hp[4] = {pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7])};
   img[(kb * HL) * 64 + alane] = make_uint4(hp[0], hp[1], hp[2], hp[3]);  // fp16 inputs convert back exactly
-  float s = 0.0f;
   if constexpr (F32A) {
     float res[8];
 #pragma unroll
@@ -157,7 +167,9 @@ __global__ __launch_bounds__(512) void image_kernel(const void* __restrict__ a, 
     img[(kb * HL + 1) * 64 + alane] =
         make_uint4(pack_rtz(res[0], res[1]), pack_rtz(res[2], res[3]), pack_rtz(res[4], res[5]), pack_rtz(res[6], res[7]));
   }
-  s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+  float s;
+  if constexpr (F32A && FMT == MGN_FMT_Q4) s = ((x[0] + x[2]) + (x[4] + x[6])) * 0.0625f + ((x[1] + x[3]) + (x[5] + x[7]));
+  else s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
   s += dpp_move<kDppQuadXor1>(s);
   s += dpp_move<kDppQuadXor2>(s);
   uint32_t* const extra = (uint32_t*)(img + kSliceBlocks * HL * 64);
@@ -166,10 +178,134 @@ __global__ __launch_bounds__(512) void image_kernel(const void* __restrict__ a, 
     const uint32_t mh = pack_rtz(mean, 0.0f);
     extra[(r + 16 * (kb >> 2)) * 4 + (kb & 3)] = (mh & 0xFFFFu) | (pack_rtz(mean - half_lo(mh), 0.0f) << 16);
   }
-  // lanes (row, g' >= 2) of the additive operand stay zero; the rows' inverse scales follow
-  if (threadIdx.x < 32 * 4) extra[32 * 4 + threadIdx.x] = 0u;
+  // lanes (row, g' >= 2) of the additive operand stay zero (8 dwords per half-wave lane... 16 rows x 32
+  // lanes cover the 128 dwords); the rows' inverse scales follow
+  if (l < 8) extra[32 * 4 + r * 8 + l] = 0u;
   if (l == 0) ((float*)extra)[64 * 4 + r] = inv * (FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f);
 }
+
+// eight consecutive activations of a row, as float
+template <bool F32A>
+__device__ __forceinline__ void load_task(const void* __restrict__ a, size_t elem, float (&x)[8]) {
+  if constexpr (F32A) {
+    const float4* src = (const float4*)((const float*)a + elem);
+    const float4 v0 = src[0], v1 = src[1];
+    x[0] = v0.x, x[1] = v0.y, x[2] = v0.z, x[3] = v0.w, x[4] = v1.x, x[5] = v1.y, x[6] = v1.z, x[7] = v1.w;
+  } else {
+    const uint4 v = *(const uint4*)((const _Float16*)a + elem);
+    x[0] = half_lo(v.x), x[1] = half_hi(v.x), x[2] = half_lo(v.y), x[3] = half_hi(v.y);
+    x[4] = half_lo(v.z), x[5] = half_hi(v.z), x[6] = half_lo(v.w), x[7] = half_hi(v.w);
+  }
+}
+
+// grid.x = row tiles * slices; 512 threads: half-wave r (0..15) converts row r of the tile,
+// lane l = kb * 4 + g of it the 8 elements k = 32 kb + 8 g .. + 7 of the slice.
+template <int FMT, bool F32A>
+__global__ __launch_bounds__(512) void image_kernel(const void* __restrict__ a, uint4* __restrict__ image, uint32_t m,
+                                                    uint32_t k, uint32_t nslices, uint32_t a_stride) {
+  constexpr uint32_t UNITS = image_units(F32A);
+  const uint32_t rt = blockIdx.x / nslices, sl = blockIdx.x - rt * nslices;
+  const uint32_t r = threadIdx.x >> 5, l = threadIdx.x & 31;
+  const uint32_t row = rt * 16 + r, k0 = sl * 256 + l * 8;
+  const bool ok = row < m && k0 < k;  // K is a multiple of 32: a task lies inside or outside as a whole
+  float x[8];
+  load_task<F32A>(a, ok ? (size_t)row * a_stride + k0 : (size_t)0, x);
+  convert_task<FMT, F32A>(x, ok, image + ((size_t)rt * nslices + sl) * UNITS, r, l);
+}
+
+// One slice (8 K blocks) of one 16-column tile against R row tiles: the wave's parked quants at
+// park_rd (this lane's piece of block 0 of its column), the slice's image at ib (row tile 0, row
+// tiles rstride bytes apart), the column's 8 scale words in mw.
+template <int FMT, bool F32A, int R>
+__device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t* ib, uint32_t rstride, const uint32_t (&mw)[8],
+                                          uint32_t g, uint32_t lane, floatx4 (&acc)[R]) {
+  constexpr uint32_t HL = F32A ? 2 : 1;
+  constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;  // 2^20, 2^24
+    // Software pipeline over the 8 blocks: LDS reads two blocks ahead, unpack and MFMAs one
+    // block ahead of the scaling FMAs that consume the previous block's products.
+    const uint32_t slot_off[2] = {image_slot(lane & 15, g, 0) * 16, image_slot(lane & 15, g, 1) * 16};
+    uint32_t bq[8][FMT == MGN_FMT_Q4 ? 1 : 2];
+    u32x4_t aop[8][R][HL];
+    floatx4 dsum[2][R];
+    floatx4 P[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) P[r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    auto lds_reads = [&](int s) {
+      if constexpr (FMT == MGN_FMT_Q4) {
+        bq[s][0] = *(const uint32_t*)(park_rd + s * 16);
+      } else {
+        const uint2 q = *(const uint2*)(park_rd + s * 32);
+        bq[s][0] = q.x, bq[s][1] = q.y;
+      }
+#pragma unroll
+      for (int r = 0; r < R; r++)
+#pragma unroll
+        for (uint32_t h = 0; h < HL; h++) aop[s][r][h] = *(const u32x4_t*)(ib + slot_off[s & 1] + r * rstride + (s * HL + h) * 64 * 16);
+    };
+    auto mfmas = [&](int s) {
+      half8 bop;
+      if constexpr (FMT == MGN_FMT_Q4) bop = nibbles_to_operand<F32A>(bq[s][0]);
+      else bop = bytes_to_operand(bq[s][0], bq[s][1]);
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aop[s][r][0]), bop,
+                                                           floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        if constexpr (F32A) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aop[s][r][HL - 1]), bop, d, 0, 0, 0);
+        dsum[s & 1][r] = d;
+      }
+    };
+    auto scale = [&](int s) {
+      const float dq = half_bits_to_float(mw[s] & 0xFFFFu);
+#pragma unroll
+      for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) P[r][i] = __fmaf_rn(dq, dsum[s & 1][r][i], P[r][i]);
+    };
+    lds_reads(0);
+    lds_reads(1);
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+      if (s + 2 < 8) lds_reads(s + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 1 < 8) mfmas(s + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      scale(s);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // additive part of the slice's 8 blocks: mean(x) * m (Q4) or mean(x) * scale (Q8), times 32
+    // (the means) and, for Q8, times -128 (the byte bias); 2^-20 (2^-24) like the quant sums
+    uint32_t bw[4];
+    const uint32_t upper = 0u - (g & 1u);  // all ones in the lanes that take blocks 4..7
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      // (bit arithmetic, not a select between array elements: that would be turned into an
+      // indexed load from a stack copy of the array)
+      const uint32_t w = mw[j] ^ ((mw[j] ^ mw[4 + j]) & upper);
+      bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
+    }
+    const half8 bm = as_half8(bw[0], bw[1], bw[2], bw[3]);
+    constexpr float kAdd = (FMT == MGN_FMT_Q4 ? 32.0f : -4096.0f) / kOpScale;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const uint8_t* const ir = ib + lane * 16 + r * rstride + 8 * HL * 64 * 16;
+      const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, *(const u32x4_t*)ir), bm,
+                                                               floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+      if constexpr (F32A) {
+        // the rows' inverse slice scales (times 2^20 or 2^24: the operand scale of the quants)
+        const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
+        acc[r][0] = __fmaf_rn(__fmaf_rn(kAdd, d[0], P[r][0]), inv.x, acc[r][0]);
+        acc[r][1] = __fmaf_rn(__fmaf_rn(kAdd, d[1], P[r][1]), inv.y, acc[r][1]);
+        acc[r][2] = __fmaf_rn(__fmaf_rn(kAdd, d[2], P[r][2]), inv.z, acc[r][2]);
+        acc[r][3] = __fmaf_rn(__fmaf_rn(kAdd, d[3], P[r][3]), inv.w, acc[r][3]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[r][i] += __fmaf_rn(kAdd, d[i], P[r][i]);
+      }
+    }
+  }
 
 struct TileTail {  // arguments first needed in the epilogue
   const float* dres;
@@ -198,7 +334,6 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
                                                          const void* __restrict__ quants_arg, uint32_t m, uint32_t kdim,
                                                          uint32_t n, uint32_t wnc, uint32_t ksc, uint32_t nph, uint32_t parts,
                                                          uint32_t nslices, TileTail tail) {
-  constexpr uint32_t HL = F32A ? 2 : 1;
   constexpr uint32_t UNITS = image_units(F32A);
   constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;  // 2^20, 2^24
   constexpr int QB = FMT == MGN_FMT_Q4 ? 16 : 32;  // quant bytes per block
@@ -329,92 +464,10 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
 #pragma unroll
             for (int s = 0; s < 8; s++) mw[s] = kb0 + s < bpc ? mw[s] : 0u;
           }
-          const uint8_t* const ib = (const uint8_t*)(imgbuf + (p & 1) * buf_units + ks * UNITS + lane);
+          const uint8_t* const ib = (const uint8_t*)(imgbuf + (p & 1) * buf_units + ks * UNITS);
           constexpr uint32_t kRowTile = 16;  // bytes per uint4 unit
           const uint32_t rstride = ksc * UNITS * kRowTile;  // bytes between the row tiles of a buffer
-          // Software pipeline over the 8 blocks: LDS reads two blocks ahead, unpack and MFMAs one
-          // block ahead of the scaling FMAs that consume the previous block's products.
-          uint32_t bq[8][FMT == MGN_FMT_Q4 ? 1 : 2];
-          u32x4_t aop[8][R][HL];
-          floatx4 dsum[2][R];
-          floatx4 P[R];
-#pragma unroll
-          for (int r = 0; r < R; r++) P[r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-          auto lds_reads = [&](int s) {
-            if constexpr (FMT == MGN_FMT_Q4) {
-              bq[s][0] = *(const uint32_t*)(park_rd + s * 16);
-            } else {
-              const uint2 q = *(const uint2*)(park_rd + s * 32);
-              bq[s][0] = q.x, bq[s][1] = q.y;
-            }
-#pragma unroll
-            for (int r = 0; r < R; r++)
-#pragma unroll
-              for (uint32_t h = 0; h < HL; h++) aop[s][r][h] = *(const u32x4_t*)(ib + r * rstride + (s * HL + h) * 64 * 16);
-          };
-          auto mfmas = [&](int s) {
-            half8 bop;
-            if constexpr (FMT == MGN_FMT_Q4) bop = nibbles_to_operand(bq[s][0]);
-            else bop = bytes_to_operand(bq[s][0], bq[s][1]);
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-              floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aop[s][r][0]), bop,
-                                                                 floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-              if constexpr (F32A) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aop[s][r][HL - 1]), bop, d, 0, 0, 0);
-              dsum[s & 1][r] = d;
-            }
-          };
-          auto scale = [&](int s) {
-            const float dq = half_bits_to_float(mw[s] & 0xFFFFu);
-#pragma unroll
-            for (int r = 0; r < R; r++)
-#pragma unroll
-              for (int i = 0; i < 4; i++) P[r][i] = __fmaf_rn(dq, dsum[s & 1][r][i], P[r][i]);
-          };
-          lds_reads(0);
-          lds_reads(1);
-          __builtin_amdgcn_sched_barrier(0);
-          mfmas(0);
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int s = 0; s < 8; s++) {
-            if (s + 2 < 8) lds_reads(s + 2);
-            __builtin_amdgcn_sched_barrier(0);
-            if (s + 1 < 8) mfmas(s + 1);
-            __builtin_amdgcn_sched_barrier(0);
-            scale(s);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-          // additive part of the slice's 8 blocks: mean(x) * m (Q4) or mean(x) * scale (Q8), times 32
-          // (the means) and, for Q8, times -128 (the byte bias); 2^-20 (2^-24) like the quant sums
-          uint32_t bw[4];
-          const uint32_t upper = 0u - (g & 1u);  // all ones in the lanes that take blocks 4..7
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            // (bit arithmetic, not a select between array elements: that would be turned into an
-            // indexed load from a stack copy of the array)
-            const uint32_t w = mw[j] ^ ((mw[j] ^ mw[4 + j]) & upper);
-            bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
-          }
-          const half8 bm = as_half8(bw[0], bw[1], bw[2], bw[3]);
-          constexpr float kAdd = (FMT == MGN_FMT_Q4 ? 32.0f : -4096.0f) / kOpScale;
-#pragma unroll
-          for (int r = 0; r < R; r++) {
-            const uint8_t* const ir = ib + r * rstride + 8 * HL * 64 * 16;
-            const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, *(const u32x4_t*)ir), bm,
-                                                                     floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-            if constexpr (F32A) {
-              // the rows' inverse slice scales (times 2^20 or 2^24: the operand scale of the quants)
-              const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
-              acc[r][0] = __fmaf_rn(__fmaf_rn(kAdd, d[0], P[r][0]), inv.x, acc[r][0]);
-              acc[r][1] = __fmaf_rn(__fmaf_rn(kAdd, d[1], P[r][1]), inv.y, acc[r][1]);
-              acc[r][2] = __fmaf_rn(__fmaf_rn(kAdd, d[2], P[r][2]), inv.z, acc[r][2]);
-              acc[r][3] = __fmaf_rn(__fmaf_rn(kAdd, d[3], P[r][3]), inv.w, acc[r][3]);
-            } else {
-#pragma unroll
-              for (int i = 0; i < 4; i++) acc[r][i] += __fmaf_rn(kAdd, d[i], P[r][i]);
-            }
-          }
+          slice_mac<FMT, F32A, R>(park_rd, ib, rstride, mw, g, lane, acc);
         }
         copy_store((ph + 1) & 1, (p + 1) & 1);  // that LDS buffer was last read before the previous barrier
         lds_barrier();
@@ -504,6 +557,476 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
         }
       }
   }
+}
+
+// ---- few activation rows (M <= 32): the images stay in LDS ----
+// grid = (K parts, column groups); 512 threads.  A workgroup converts the activations of its K
+// part (all M rows, NSL slices of 256 elements) into images in LDS itself, once; after one barrier
+// every wave walks its own Q pairs of column tiles down the part's slices, pair after pair, with
+// whole slices of both tiles in flight in registers and no further synchronisation.  The two
+// tiles of a pair are multiplied side by side, so every A operand read from LDS serves both (LDS
+// bandwidth is what limits a wave that reads each operand for one tile only).
+//
+// The quants reach the B operand's lane order without LDS: lane (c, g) loads 16 bytes of
+// column c, and the four lanes of a column exchange dwords with the row swap instructions
+// (v_permlane32_swap, v_permlane16_swap: rows of 16 lanes).
+//   Q4: lane (c, g) loads block g (then 4 + g) of the slice; a 4x4 transpose over (row, dword)
+//       leaves dword g of blocks 0..3 (4..7): the block's elements 8g..8g+7.
+//   Q8: load j, lane (c, g): half g / 2 of block 2j + g % 2; swapping (x, z) and (y, w) between
+//       the odd and even rows leaves dwords 2g, 2g+1 of block 2j in (x, y), of 2j+1 in (z, w).
+// The scale words are wanted by all four lanes of a column; loading them per lane would ask the
+// memory pipeline for every word four times.  Each wave instead loads the words of all its
+// columns and slices once, in whole cache lines, parks them in its own LDS strip and reads a
+// step's eight words per tile from there.
+//
+// What a call costs outside the multiplication is what these choices are about: a CU's vector
+// memory pipeline takes about three cycles per cache line a load instruction touches, so the
+// loads of the prologue (activations, scale words, the first slices) hold the waves for
+// thousands of cycles before the first multiplication; only DEPTH slices are requested ahead, the
+// rest step by step.  The walk is written out step by step (NSL and Q are compile-time) with
+// scheduling fences between its stages: left to itself the compiler moves the loads of later
+// steps behind the multiplications and the call takes a third longer.
+// K is cut into parts of NSL slices; the parts' partial tiles meet as in the kernel above.
+constexpr int kSide = 2;            // column tiles a wave multiplies side by side
+
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+// component j of lane (c, g) <- component g of lane (c, j)
+__device__ __forceinline__ void transpose_rows(u32x4_t& v) {
+  u32x2_t s = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);
+  v.x = s.x, v.z = s.y;
+  s = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
+  v.y = s.x, v.w = s.y;
+  s = __builtin_amdgcn_permlane16_swap(v.x, v.y, false, false);
+  v.x = s.x, v.y = s.y;
+  s = __builtin_amdgcn_permlane16_swap(v.z, v.w, false, false);
+  v.z = s.x, v.w = s.y;
+}
+// odd rows of (x, y) <-> even rows of (z, w)
+__device__ __forceinline__ void swap_row_pairs(u32x4_t& v) {
+  u32x2_t s = __builtin_amdgcn_permlane16_swap(v.x, v.z, false, false);
+  v.x = s.x, v.z = s.y;
+  s = __builtin_amdgcn_permlane16_swap(v.y, v.w, false, false);
+  v.y = s.x, v.w = s.y;
+}
+
+// One slice (8 K blocks) of kSide column tiles against R row tiles: the tiles' quants in B operand
+// order (q, see above), their 8 scale words (mw), the slice's image at ib (row tile 0, row tiles
+// rstride bytes apart).
+template <int FMT, bool F32A, int R>
+__device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == MGN_FMT_Q4 ? 2 : 4], const uint32_t (&mw)[kSide][8],
+                                               const uint8_t* ib, uint32_t rstride, uint32_t g, uint32_t lane,
+                                               floatx4 (&acc)[kSide][R]) {
+  constexpr uint32_t HL = F32A ? 2 : 1;
+  constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;  // 2^20, 2^24
+  const uint32_t slot_off[2] = {image_slot(lane & 15, g, 0) * 16, image_slot(lane & 15, g, 1) * 16};
+  u32x4_t aop[3][R][HL];
+  floatx4 dsum[2][kSide][R];
+  floatx4 P[kSide][R];
+#pragma unroll
+  for (int u = 0; u < kSide; u++)
+#pragma unroll
+    for (int r = 0; r < R; r++) P[u][r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+  auto lds_reads = [&](int s) {
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+      for (uint32_t h = 0; h < HL; h++) aop[s % 3][r][h] = *(const u32x4_t*)(ib + slot_off[s & 1] + r * rstride + (s * HL + h) * 64 * 16);
+  };
+  auto mfmas = [&](int s) {
+#pragma unroll
+    for (int u = 0; u < kSide; u++) {
+      half8 bop;
+      if constexpr (FMT == MGN_FMT_Q4) {
+        bop = nibbles_to_operand<F32A>(q[u][s >> 2][s & 3]);
+      } else {
+        bop = (s & 1) ? bytes_to_operand(q[u][s >> 1].z, q[u][s >> 1].w) : bytes_to_operand(q[u][s >> 1].x, q[u][s >> 1].y);
+      }
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aop[s % 3][r][0]), bop,
+                                                           floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        if constexpr (F32A) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, aop[s % 3][r][HL - 1]), bop, d, 0, 0, 0);
+        dsum[s & 1][u][r] = d;
+      }
+    }
+  };
+  auto scale = [&](int s) {
+#pragma unroll
+    for (int u = 0; u < kSide; u++) {
+      const float dq = half_bits_to_float(mw[u][s] & 0xFFFFu);
+#pragma unroll
+      for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) P[u][r][i] = __fmaf_rn(dq, dsum[s & 1][u][r][i], P[u][r][i]);
+    }
+  };
+  lds_reads(0);
+  lds_reads(1);
+  __builtin_amdgcn_sched_barrier(0);
+  mfmas(0);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < 8; s++) {
+    if (s + 2 < 8) lds_reads(s + 2);
+    __builtin_amdgcn_sched_barrier(0);
+    if (s + 1 < 8) mfmas(s + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    scale(s);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // additive part of the slice's 8 blocks (see slice_mac)
+  const uint32_t upper = 0u - (g & 1u);  // all ones in the lanes that take blocks 4..7
+  constexpr float kAdd = (FMT == MGN_FMT_Q4 ? 32.0f : -4096.0f) / kOpScale;
+  half8 bm[kSide];
+#pragma unroll
+  for (int u = 0; u < kSide; u++) {
+    uint32_t bw[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const uint32_t w = mw[u][j] ^ ((mw[u][j] ^ mw[u][4 + j]) & upper);
+      bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
+    }
+    bm[u] = as_half8(bw[0], bw[1], bw[2], bw[3]);
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    const uint8_t* const ir = ib + lane * 16 + r * rstride + 8 * HL * 64 * 16;
+    const half8 am = __builtin_bit_cast(half8, *(const u32x4_t*)ir);
+    float4 inv = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+    if constexpr (F32A) inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);  // the rows' inverse slice scales (times 2^20 or 2^24)
+#pragma unroll
+    for (int u = 0; u < kSide; u++) {
+      const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm[u], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+      if constexpr (F32A) {
+        acc[u][r][0] = __fmaf_rn(__fmaf_rn(kAdd, d[0], P[u][r][0]), inv.x, acc[u][r][0]);
+        acc[u][r][1] = __fmaf_rn(__fmaf_rn(kAdd, d[1], P[u][r][1]), inv.y, acc[u][r][1]);
+        acc[u][r][2] = __fmaf_rn(__fmaf_rn(kAdd, d[2], P[u][r][2]), inv.z, acc[u][r][2]);
+        acc[u][r][3] = __fmaf_rn(__fmaf_rn(kAdd, d[3], P[u][r][3]), inv.w, acc[u][r][3]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[u][r][i] += __fmaf_rn(kAdd, d[i], P[u][r][i]);
+      }
+    }
+  }
+}
+
+// Slices of a part: what fits in LDS beside the waves' scale words.
+constexpr int resident_slices(bool f32a, int r) { return f32a && r == 2 ? 2 : 4; }
+
+// Bytes of one column's scale words for the nsl slices of a part, padded so that the 16 columns of
+// a tile fall into different LDS banks.
+__host__ __device__ constexpr uint32_t meta_stride(int fmt, uint32_t nsl) { return nsl * kSliceBlocks * (fmt == MGN_FMT_Q4 ? 4 : 2) + 16; }
+
+template <int FMT, bool F32A, int R, int Q>
+__global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restrict__ a, const void* __restrict__ meta_arg,
+                                                             const void* __restrict__ quants_arg, uint32_t m, uint32_t kdim,
+                                                             uint32_t n, uint32_t parts, uint32_t nslices, TileTail tail) {
+  constexpr uint32_t UNITS = image_units(F32A);
+  constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;
+  constexpr int QB = FMT == MGN_FMT_Q4 ? 16 : 32;
+  constexpr int MB = FMT == MGN_FMT_Q4 ? 4 : 2;
+  constexpr int NLQ = QB / 8;
+  constexpr int NSL = resident_slices(F32A, R);
+  constexpr int STEPS = NSL * Q;  // step f of the walk = (pair f / NSL, slice f % NSL)
+  constexpr int DEPTH = 2;        // steps whose quants are in flight ahead of the one in use
+  constexpr int SLOTS = DEPTH + 1;
+  constexpr int NT = NSL * R;     // conversion tasks per half-wave
+  // 16-byte units of scale words a lane stages: Q pairs x 32 columns x NSL slices x (32 or 16) bytes / 64 lanes
+  constexpr int MU = Q * NSL * MB / 4;
+  constexpr uint32_t kUnitsPerColumn = NSL * kSliceBlocks * MB / 16;
+  constexpr uint32_t mstride = meta_stride(FMT, NSL);
+  extern __shared__ uint4 lds4[];
+  const uint32_t tid = threadIdx.x, lane = tid & 63;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t c = lane & 15, g = lane >> 4;
+  const uint32_t part = blockIdx.x, cg = blockIdx.y;
+  const uint32_t bpc = kdim / 32;
+  const uint32_t pair0 = (cg * 8 + wave) * Q;  // this wave's first pair of column tiles
+  const uint32_t sl0 = part * NSL;             // first slice of this part
+  uint4* const img = lds4;                     // [NSL][R][UNITS]
+  // this wave's scale words: [Q pairs x 32 columns][mstride bytes]
+  uint8_t* const wmeta = (uint8_t*)(lds4 + NSL * R * UNITS) + wave * (Q * 32 * mstride);
+
+  // ---- the part's activations: loads first, so that nothing queues in front of them ----
+  // Task (s, rr): half-wave r converts row 16 rr + r of slice sl0 + s.
+  const uint32_t cr = tid >> 5, cl = tid & 31;
+  float xin[NT][8];
+  bool xok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; t++) {
+    const uint32_t s = t / R, rr = t % R;
+    const uint32_t row = rr * 16 + cr, k0 = (sl0 + s) * 256 + cl * 8;
+    xok[t] = row < m && k0 < kdim;
+    load_task<F32A>(a, xok[t] ? (size_t)row * kdim + k0 : (size_t)0, xin[t]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- the scale words of all the wave's columns and slices: one pass, through LDS ----
+  // A column's words for the part's slices are contiguous (kUnitsPerColumn 16-byte units).  Unit
+  // id = 64 j + lane: column id / kUnitsPerColumn (of the wave's Q x 32), unit id % kUnitsPerColumn.
+  // Every lane of a column's tile reads them back slice by slice during the walk.
+  u32x4_t mu[MU];
+#pragma unroll
+  for (int j = 0; j < MU; j++) {
+    const uint32_t id = 64 * j + lane;
+    const uint32_t wcol = id / kUnitsPerColumn, unit = id % kUnitsPerColumn;
+    const uint32_t col = min(pair0 * (kSide * 16) + wcol, n - 1);
+    const uint8_t* src = (const uint8_t*)meta_arg + ((size_t)col * bpc + (size_t)sl0 * kSliceBlocks) * MB + unit * 16;
+    typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+    const u32x4_a2 v = *(const u32x4_a2*)src;
+    mu[j] = u32x4_t{v.x, v.y, v.z, v.w};
+  }
+
+  // ---- weight slices ----
+  // Slices past the end of K (last part) and columns past N read the pad behind the weights or
+  // a neighbour's data; their products are dropped.
+  u32x4_t wq[SLOTS][kSide][NLQ];
+  const uint32_t lane_part = FMT == MGN_FMT_Q4 ? g * 16 : (g & 1) * 32 + (g >> 1) * 16;
+  uint32_t q_off[Q][kSide];
+#pragma unroll
+  for (int p = 0; p < Q; p++)
+#pragma unroll
+    for (int u = 0; u < kSide; u++) q_off[p][u] = min(((pair0 + p) * kSide + u) * 16 + c, n - 1) * bpc * QB + lane_part;
+  auto fetch = [&](int f) {  // step f into slot f % SLOTS
+    const uint8_t* const qb = (const uint8_t*)quants_arg + (size_t)((sl0 + f % NSL) * kSliceBlocks) * QB;
+#pragma unroll
+    for (int u = 0; u < kSide; u++)
+#pragma unroll
+      for (int j = 0; j < NLQ; j++)
+        wq[f % SLOTS][u][j] = __builtin_nontemporal_load((const u32x4_t*)(qb + q_off[f / NSL][u] + 64 * j));
+  };
+#pragma unroll
+  for (int f = 0; f < DEPTH && f < STEPS; f++) fetch(f);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- activations -> images in LDS; scale words -> LDS ----
+#pragma unroll
+  for (int t = 0; t < NT; t++) convert_task<FMT, F32A>(xin[t], xok[t], img + t * UNITS, cr, cl);
+#pragma unroll
+  for (int j = 0; j < MU; j++) {
+    const uint32_t id = 64 * j + lane;
+    *(u32x4_t*)(wmeta + (id / kUnitsPerColumn) * mstride + (id % kUnitsPerColumn) * 16) = mu[j];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  lds_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+
+  floatx4 res[Q][kSide][R];
+#pragma unroll
+  for (int p = 0; p < Q; p++)
+#pragma unroll
+    for (int u = 0; u < kSide; u++)
+#pragma unroll
+      for (int r = 0; r < R; r++) res[p][u][r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+  const bool pair_live[2] = {pair0 * (kSide * 16) < n, (pair0 + Q - 1) * (kSide * 16) < n};  // uniform over the wave
+#pragma unroll
+  for (int f = 0; f < STEPS; f++) {
+    const int slot = f % SLOTS, wp = f / NSL, ws = f % NSL;
+    __builtin_amdgcn_sched_barrier(0);
+    if (f + DEPTH < STEPS) fetch(f + DEPTH);
+    __builtin_amdgcn_sched_barrier(0);
+    // the slot's quants into B operand order, the step's scale words from LDS
+    uint32_t mw[kSide][8];
+#pragma unroll
+    for (int u = 0; u < kSide; u++) {
+      const uint8_t* const ms = wmeta + ((wp * kSide + u) * 16 + c) * mstride + ws * (kSliceBlocks * MB);
+      if constexpr (FMT == MGN_FMT_Q4) {
+        const u32x4_t m0 = *(const u32x4_t*)ms, m1 = *(const u32x4_t*)(ms + 16);
+        mw[u][0] = m0.x, mw[u][1] = m0.y, mw[u][2] = m0.z, mw[u][3] = m0.w;
+        mw[u][4] = m1.x, mw[u][5] = m1.y, mw[u][6] = m1.z, mw[u][7] = m1.w;
+        transpose_rows(wq[slot][u][0]);
+        transpose_rows(wq[slot][u][1]);
+      } else {
+        const u32x4_t m0 = *(const u32x4_t*)ms;
+        const uint32_t v[4] = {m0.x, m0.y, m0.z, m0.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) mw[u][2 * e] = v[e] & 0xFFFFu, mw[u][2 * e + 1] = v[e] >> 16;
+#pragma unroll
+        for (int j = 0; j < NLQ; j++) swap_row_pairs(wq[slot][u][j]);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const uint32_t sl_raw = sl0 + ws;
+    if (pair_live[wp == 0 ? 0 : 1] && sl_raw < nslices) {  // (with Q = 2, wp is 0 or 1)
+      const uint32_t kb0 = sl_raw * kSliceBlocks;
+      if (kb0 + kSliceBlocks > bpc) {  // last slice of a K that is no multiple of 256
+#pragma unroll
+        for (int u = 0; u < kSide; u++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) mw[u][e] = kb0 + e < bpc ? mw[u][e] : 0u;
+      }
+      slice_mac_side<FMT, F32A, R>(wq[slot], mw, (const uint8_t*)(img + ws * R * UNITS), UNITS * 16, g, lane, res[wp]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if constexpr (!F32A) {
+#pragma unroll
+    for (int p = 0; p < Q; p++)
+#pragma unroll
+      for (int u = 0; u < kSide; u++)
+#pragma unroll
+        for (int r = 0; r < R; r++) res[p][u][r] *= kOpScale;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  if (parts > 1) {
+    // K parts of other workgroups: the last one to arrive adds them up in part order (see above)
+    const size_t plane = (size_t)R * 16 * n;  // floats per part
+#pragma unroll
+    for (int p = 0; p < Q; p++)
+#pragma unroll
+      for (int u = 0; u < kSide; u++) {
+        const uint32_t col = ((pair0 + p) * kSide + u) * 16 + c;
+        if (col < n) {
+          float* const mine = tail.scratch + (size_t)part * plane + col;
+#pragma unroll
+          for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+              __hip_atomic_store(mine + (size_t)(r * 16 + 4 * g + i) * n, res[p][u][r][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    uint32_t* const flag = (uint32_t*)lds4;
+    if (tid == 0) {
+      uint32_t* const ctr = tail.counters + cg;
+      const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = seen == parts - 1;
+      if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+      *flag = last ? 1u : 0u;
+    }
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    if (*flag == 0u) return;
+    // the parts' tiles, several parts in flight at a time, added in part order
+    const float* base[Q][kSide];
+#pragma unroll
+    for (int p = 0; p < Q; p++)
+#pragma unroll
+      for (int u = 0; u < kSide; u++) {
+        base[p][u] = tail.scratch + min(((pair0 + p) * kSide + u) * 16 + c, n - 1) + (size_t)(4 * g) * n;
+#pragma unroll
+        for (int r = 0; r < R; r++) res[p][u][r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+    auto add_parts = [&](auto group) {
+      constexpr int PG = decltype(group)::value;
+      for (uint32_t pp0 = 0; pp0 < parts; pp0 += PG) {
+        float v[PG][Q][kSide][R][4];
+#pragma unroll
+        for (int j = 0; j < PG; j++) {
+          const size_t po = (size_t)min(pp0 + j, parts - 1) * plane;  // (the surplus repeats the last part)
+#pragma unroll
+          for (int p = 0; p < Q; p++)
+#pragma unroll
+            for (int u = 0; u < kSide; u++)
+#pragma unroll
+              for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                  v[j][p][u][r][i] = __hip_atomic_load(base[p][u] + po + (size_t)(r * 16 + i) * n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int j = 0; j < PG; j++) {
+          const bool live = pp0 + j < parts;
+#pragma unroll
+          for (int p = 0; p < Q; p++)
+#pragma unroll
+            for (int u = 0; u < kSide; u++)
+#pragma unroll
+              for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) res[p][u][r][i] = live ? res[p][u][r][i] + v[j][p][u][r][i] : res[p][u][r][i];
+        }
+      }
+    };
+    if (parts <= 4) add_parts(std::integral_constant<int, 4>{});
+    else add_parts(std::integral_constant<int, 16 / (Q * R)>{});
+  }
+#pragma unroll
+  for (int p = 0; p < Q; p++)
+#pragma unroll
+    for (int u = 0; u < kSide; u++) {
+      const uint32_t col = ((pair0 + p) * kSide + u) * 16 + c;
+      if (col < n) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const uint32_t row = r * 16 + 4 * g + i;
+            if (row < m) {
+              const size_t o = (size_t)row * n + col;
+              tail.c[o] = apply_epilogue(tail.dres ? res[p][u][r][i] + tail.dres[o] : res[p][u][r][i], tail.epilogue);
+            }
+          }
+      }
+    }
+}
+
+struct ResidentPlan {
+  uint32_t r, q, nsl, parts, colgroups, nslices;
+  size_t lds, partial_bytes;
+};
+
+size_t resident_lds_bytes(int fmt, bool f32a, uint32_t r, uint32_t q) {
+  const uint32_t nsl = resident_slices(f32a, r);
+  return (size_t)nsl * r * image_units(f32a) * 16 + (size_t)8 * q * 32 * meta_stride(fmt, nsl);
+}
+
+// M <= 32.  Q = 1 or 2 pairs of tiles per wave: the one whose grid fills the CUs better.
+bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
+  if (x.m == 0 || x.m > 32 || x.w.k < 32) return false;
+  const uint32_t bpc = x.w.k / 32;
+  if ((uint64_t)x.w.n * bpc * 32 >= (1ull << 32)) return false;  // a lane's weight offsets are 32-bit
+  const bool f32a = !x.a_is_f16;
+  const uint32_t r = x.m <= 16 ? 1 : 2;
+  if (r == 2 && x.w.fmt == MGN_FMT_Q8) return false;  // would not fit the register file
+  const uint32_t nsl = resident_slices(f32a, r);
+  const uint32_t nslices = (bpc + kSliceBlocks - 1) / kSliceBlocks, n_tiles = (x.w.n + 15) / 16;
+  const uint32_t parts = (nslices + nsl - 1) / nsl;
+  const size_t partial = parts > 1 ? (size_t)parts * r * 16 * x.w.n * 4 : 0;
+  if (partial > x.scratch_bytes) return false;
+  double best = 0;
+  ResidentPlan bp{};
+  for (uint32_t q = 1; q <= (r == 1 ? 2u : 1u); q++) {
+    const uint32_t per_wg = 8 * kSide * q;
+    const uint32_t colgroups = (n_tiles + per_wg - 1) / per_wg;
+    if (colgroups > 65535 || (parts > 1 && colgroups > x.n_counters)) continue;
+    const uint64_t wgs = (uint64_t)parts * colgroups;
+    // time ~ rounds of workgroups x work of one (a fixed part + the steps of its waves)
+    const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q);
+    if (best == 0 || cost < best) {
+      best = cost;
+      bp.r = r, bp.q = q, bp.nsl = nsl, bp.parts = parts, bp.colgroups = colgroups, bp.nslices = nslices;
+      bp.partial_bytes = partial;
+      bp.lds = resident_lds_bytes(x.w.fmt, f32a, r, q);
+    }
+  }
+  if (best == 0) return false;
+  *out = bp;
+  return true;
+}
+
+template <int FMT, bool F32A, int R, int Q>
+int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& p) {
+  auto kern = tile_resident_kernel<FMT, F32A, R, Q>;
+  static std::atomic<uint64_t> big_lds_done{0};
+  if (p.lds > 64 * 1024)
+    if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
+  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue};
+  hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups), dim3(512), p.lds, s, x.a, x.w.meta, x.w.quants, x.m, x.w.k, x.w.n, p.parts,
+                     p.nslices, tail);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int FMT, bool F32A>
+int launch_resident_fa(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& p) {
+  if constexpr (FMT == MGN_FMT_Q4) {
+    if (p.r == 2) return launch_resident_q<FMT, F32A, 2, 1>(s, x, p);
+  }
+  return p.q == 1 ? launch_resident_q<FMT, F32A, 1, 1>(s, x, p) : launch_resident_q<FMT, F32A, 1, 2>(s, x, p);
 }
 
 struct TilePlan {
@@ -637,12 +1160,37 @@ size_t tile_workspace_bytes(const TilePlan& p) { return ((p.partial_bytes + 255)
 }  // namespace
 
 bool tile_mfma_supported(const LaunchArgs& x) {
+  ResidentPlan rp;
+  if (plan_resident(x, &rp)) return true;
   TilePlan p;
   if (!plan_tile(x, &p)) return false;
   return tile_workspace_bytes(p) <= x.scratch_bytes;
 }
 
+// Up to 16 rows, K >= 544, at most four K parts and one round of workgroups that fills at least
+// three quarters of the CUs (e.g. 4096 x 14336 at M = 5..16: 15.0 us against 17.2 us on the 32x32 tiled
+// kernel).  On smaller shapes the conversion of the activations in every workgroup and the
+// parts' hand-over cost more than the tiled kernel's whole call; with more parts or rounds the
+// two are level or the tiled kernel wins.
+bool tile_mfma_preferred(const LaunchArgs& x) {
+  ResidentPlan rp;
+  if (!plan_resident(x, &rp) || rp.r != 1 || rp.parts > 4 || rp.nslices < 3) return false;
+  const uint64_t wgs = (uint64_t)rp.parts * rp.colgroups;
+  return wgs <= (uint64_t)x.num_cus && 4 * wgs >= 3 * (uint64_t)x.num_cus;
+}
+
 bool describe_tile_mfma(const LaunchArgs& x, mgn_plan_info* out) {
+  ResidentPlan rp;
+  if (plan_resident(x, &rp)) {
+    out->route = MGN_ROUTE_TILE_MFMA;
+    out->grid[0] = rp.parts, out->grid[1] = rp.colgroups, out->grid[2] = 1;
+    out->threads = 512;
+    out->lds_bytes = (uint32_t)rp.lds;
+    out->waves_n = 8 * kSide * rp.q, out->k_splits = 1, out->k_parts = rp.parts, out->steps = rp.nsl;
+    out->quads_per_wave = 0, out->full_steps = 0, out->tail_blocks = 0;
+    out->workspace_bytes = rp.partial_bytes;
+    return true;
+  }
   TilePlan p;
   if (!plan_tile(x, &p) || tile_workspace_bytes(p) > x.scratch_bytes) return false;
   out->route = MGN_ROUTE_TILE_MFMA;
@@ -656,6 +1204,12 @@ bool describe_tile_mfma(const LaunchArgs& x, mgn_plan_info* out) {
 }
 
 int launch_matmul_tile_mfma(ihipStream_t* s, const LaunchArgs& x) {
+  ResidentPlan rp;
+  if (plan_resident(x, &rp)) {
+    if (x.w.fmt == MGN_FMT_Q4)
+      return x.a_is_f16 ? launch_resident_fa<MGN_FMT_Q4, false>(s, x, rp) : launch_resident_fa<MGN_FMT_Q4, true>(s, x, rp);
+    return x.a_is_f16 ? launch_resident_fa<MGN_FMT_Q8, false>(s, x, rp) : launch_resident_fa<MGN_FMT_Q8, true>(s, x, rp);
+  }
   TilePlan p;
   if (!plan_tile(x, &p) || tile_workspace_bytes(p) > x.scratch_bytes) return (int)hipErrorInvalidValue;
   if (x.w.fmt == MGN_FMT_Q4) return x.a_is_f16 ? launch_fa<MGN_FMT_Q4, false>(s, x, p) : launch_fa<MGN_FMT_Q4, true>(s, x, p);

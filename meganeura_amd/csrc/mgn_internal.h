@@ -101,6 +101,8 @@ constexpr uint32_t kWorkspaceCounters = 4096;
 int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& a);
 // kernels_tile.hip: the 16x16x32 tiled kernel (activation image + weight streaming)
 bool tile_mfma_supported(const LaunchArgs& a);
+// shapes on which the automatic route takes this kernel ahead of the 32x32 tiled one
+bool tile_mfma_preferred(const LaunchArgs& a);
 bool describe_tile_mfma(const LaunchArgs& a, mgn_plan_info* out);
 int launch_matmul_tile_mfma(ihipStream_t* s, const LaunchArgs& a);
 

@@ -9,7 +9,7 @@ import pytest
 from meganeura_amd import capi
 
 Q4, Q8 = 0, 1
-GENERIC, GEMV_VALU, GEMV_MFMA, GEMM_MFMA = 1, 2, 3, 4
+GENERIC, GEMV_VALU, GEMV_MFMA, GEMM_MFMA, TILE_MFMA = 1, 2, 3, 4, 5
 WORKSPACE = 16 << 20
 COUNTERS = 4096
 
@@ -78,6 +78,24 @@ def check_gemm(p, fmt, m, k, n, f16):
         assert p.workspace_bytes == 0
 
 
+def check_tile_resident(p, fmt, m, k, n, f16):
+    """The automatic route only takes the 16x16x32 kernel in its form for up to 16 rows with the
+    activation images resident in LDS: grid = (K parts, column groups), 8 waves, each with one or
+    two pairs of 16-column tiles, parts of `steps` slices of 256 elements."""
+    assert 5 <= m <= 16 and p.grid[2] == 1 and p.threads == 512
+    assert p.lds_bytes <= 160 * 1024
+    nslices, n_tiles = ceil_div(k, 256), ceil_div(n, 16)
+    assert p.steps == 4 and p.waves_n in (16, 32)  # slices per part; tiles per workgroup
+    assert p.grid[0] == p.k_parts == ceil_div(nslices, p.steps) <= 4 and nslices >= 3
+    assert p.grid[1] * p.waves_n >= n_tiles and (p.grid[1] - 1) * p.waves_n < n_tiles
+    wgs = p.grid[0] * p.grid[1]
+    assert 192 <= wgs <= 256  # one round of workgroups over the 256 CUs, at least three quarters of them busy
+    if p.k_parts > 1:
+        assert p.workspace_bytes == p.k_parts * 16 * n * 4 <= WORKSPACE and p.grid[1] <= COUNTERS
+    else:
+        assert p.workspace_bytes == 0
+
+
 @pytest.mark.parametrize("fmt", [Q4, Q8])
 def test_plans_cover_the_problem_and_respect_the_limits(fmt):
     routes = set()
@@ -89,18 +107,20 @@ def test_plans_cover_the_problem_and_respect_the_limits(fmt):
             where = f"fmt={fmt} m={m} k={k} n={n} f16={f16} route={p.route}"
             routes.add(p.route)
             try:
-                assert p.route in (GENERIC, GEMV_VALU, GEMV_MFMA, GEMM_MFMA)
+                assert p.route in (GENERIC, GEMV_VALU, GEMV_MFMA, GEMM_MFMA, TILE_MFMA)
                 if m > 4:
-                    assert p.route in (GEMM_MFMA, GENERIC)
+                    assert p.route in (GEMM_MFMA, TILE_MFMA, GENERIC)
                 if f16:
                     assert p.route != GEMV_VALU  # the vector-ALU GEMV reads f32 activations only
                 if p.route == GEMV_MFMA:
                     check_gemv(p, fmt, m, k, n)
                 elif p.route == GEMM_MFMA:
                     check_gemm(p, fmt, m, k, n, f16)
+                elif p.route == TILE_MFMA:
+                    check_tile_resident(p, fmt, m, k, n, f16)
             except AssertionError as e:
                 raise AssertionError(where) from e
-    assert {GEMV_MFMA, GEMM_MFMA} <= routes
+    assert {GEMV_MFMA, GEMM_MFMA, TILE_MFMA} <= routes
 
 
 def test_baseline_configurations_take_the_kernels_built_for_them():
@@ -112,8 +132,9 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
     for fmt, m, k, n in gemv:
         assert capi.matmul_plan(fmt, m, k, n).route == GEMV_MFMA, (fmt, m, k, n)
     for fmt in (Q4, Q8):
-        for k, n in ((4096, 14336), (14336, 4096)):
-            assert capi.matmul_plan(fmt, 16, k, n).route == GEMM_MFMA
+        assert capi.matmul_plan(fmt, 16, 4096, 14336).route == TILE_MFMA   # one round of workgroups, 4 K parts
+        assert capi.matmul_plan(fmt, 16, 14336, 4096).route == GEMM_MFMA   # would be 14 K parts
+        assert capi.matmul_plan(fmt, 17, 4096, 14336).route == GEMM_MFMA
     for k, n in ((1024, 3072), (3072, 1024)):
         assert capi.matmul_plan(Q4, 512, k, n, True).route == GEMM_MFMA
     head = capi.matmul_plan(Q4, 1, 4096, 14336)
