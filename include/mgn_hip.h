@@ -41,7 +41,7 @@ typedef enum mgn_status {
   MGN_EUNSUPPORTED = 6, /* a fused entry point asked for a shape its kernel does not serve */
   MGN_ERANGE = 7 /* reported by the next synchronising call: an f32 activation too large for the kernel
                     that ran (|x| >= 65504 on MGN_ROUTE_GEMM_MFMA, M >= 5); outputs of that call are wrong;
-                    MGN_ROUTE_TILE_MFMA takes such data */
+                    see mgn_ctx_set_activation_range */
 } mgn_status;
 
 /* compile::WeightFormat::{Q4,Q8} (src/compile.rs:8-29), graph::DType::{Q4_0,Q8_0}
@@ -77,6 +77,16 @@ void mgn_ctx_destroy(mgn_ctx* ctx);
 const char* mgn_last_error(const mgn_ctx* ctx);
 /* Session::wait (src/runtime.rs:2835-2841). */
 mgn_status mgn_sync(mgn_ctx* ctx);
+/* What the context may assume about f32 activations of matmuls with M >= 5.  By default
+ * (any_magnitude == 0) it assumes |x| < 65504, the range an fp16 pair splits exactly, which its
+ * fastest tiled kernel relies on; a call that meets a larger value is reported as MGN_ERANGE by
+ * the next synchronising call.  With any_magnitude != 0 those matmuls run on the kernel that
+ * rescales every 256-element slice of a row by a power of two: every finite f32 is exact input,
+ * inf and NaN stay in their rows, at the price of a slower call on most shapes.  fp16 activations
+ * and M <= 4 never depend on this.  The reference multiplies in f32 on the scalar ALUs
+ * (src/shaders/matmul.wgsl:43-90) and has no such limit, so a drop-in that cannot bound its
+ * activations sets this once after mgn_ctx_create. */
+mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, int any_magnitude);
 /* ---- plain device buffers: the reference allocates every plan buffer
  *      zero-filled (src/runtime.rs:1737-1755) and moves data with memcpy
  *      through mapped memory (upload_buffer 2552-2558, read_buffer 2623-2629). */

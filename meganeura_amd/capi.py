@@ -19,7 +19,7 @@ ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA, RO
 # every symbol include/mgn_hip.h, include/mgn_bench.h and include/mgn_session.h declare
 BENCH_SYMBOLS = ["mgn_ctx_set_route", "mgn_matmul_q_loop", "mgn_weight_read_loop"]
 HIP_SYMBOLS = [
-    "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync",
+    "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync", "mgn_ctx_set_activation_range",
     "mgn_buf_alloc", "mgn_buf_free", "mgn_buf_size", "mgn_buf_device_ptr", "mgn_buf_upload",
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
@@ -83,6 +83,7 @@ def load():
         "mgn_last_error": (C.c_char_p, [vp]),
         "mgn_sync": (C.c_int, [vp]),
         "mgn_ctx_set_route": (C.c_int, [vp, C.c_int]),
+        "mgn_ctx_set_activation_range": (C.c_int, [vp, C.c_int]),
         "mgn_buf_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
         "mgn_buf_free": (None, [vp, vp]),
         "mgn_buf_size": (sz, [vp]),
@@ -255,6 +256,10 @@ class Context:
 
     def __exit__(self, *exc):
         self.close()
+
+    def set_activation_range(self, any_magnitude):
+        """f32 activations of M >= 5: False (default) promises |x| < 65504, True takes any finite value."""
+        self.check(self.lib.mgn_ctx_set_activation_range(self.h, 1 if any_magnitude else 0))
 
     def set_route(self, route):
         self.check(self.lib.mgn_ctx_set_route(self.h, route))

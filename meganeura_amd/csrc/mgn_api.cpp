@@ -121,7 +121,7 @@ mgn_status check_range_flag(mgn_ctx* ctx) {
   *(volatile uint32_t*)ctx->range_flag_host = 0;
   return fail(ctx, MGN_ERANGE,
               "an f32 activation of magnitude >= 65504 reached the tiled MFMA kernel (M >= 5), which splits activations "
-              "into fp16 pairs: the affected outputs are wrong; select MGN_ROUTE_TILE_MFMA for such data");
+              "into fp16 pairs: the affected outputs are wrong; mgn_ctx_set_activation_range(ctx, 1) takes such data");
 }
 
 // Looks at every block's scale (and minimum) once, right after a weight's blocks are on the
@@ -236,6 +236,12 @@ mgn_status mgn_sync(mgn_ctx* ctx) {
   if (!ctx) return MGN_EINVAL;
   MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
   return check_range_flag(ctx);
+}
+
+mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, int any_magnitude) {
+  if (!ctx) return MGN_EINVAL;
+  ctx->any_magnitude = any_magnitude != 0;
+  return MGN_OK;
 }
 
 mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route) {
@@ -582,6 +588,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   if (route == MGN_ROUTE_AUTO) {
     if (mgn::gemv_mfma_supported(x)) route = MGN_ROUTE_GEMV_MFMA;
     else if (mgn::tile_mfma_preferred(x)) route = MGN_ROUTE_TILE_MFMA;  // measured faster than the kernel below
+    else if (ctx->any_magnitude && !a_is_f16 && mgn::tile_mfma_supported(x)) route = MGN_ROUTE_TILE_MFMA;
     else if (mgn::gemm_mfma_supported(x)) route = MGN_ROUTE_GEMM_MFMA;
     else if (mgn::tile_mfma_supported(x)) route = MGN_ROUTE_TILE_MFMA;  // e.g. a weight whose block minima the kernel above cannot hold
     else if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV_VALU;

@@ -698,6 +698,12 @@ def test_activations_of_any_magnitude_on_the_rescaling_tiled_kernel(ctx, orc, fm
         run_matmul(ctx, fmt, x, wt, ROUTES["gemm_mfma"])
     assert e.value.status == capi.ERANGE
     ctx.sync()  # reported once; the context keeps working
+    # a context told that activations may have any magnitude keeps such matmuls off that kernel
+    ctx.set_activation_range(True)
+    try:
+        assert_close_rowwise(run_matmul(ctx, fmt, x, wt, capi.ROUTE_AUTO), want, x)
+    finally:
+        ctx.set_activation_range(False)
     # non-finite activations give non-finite outputs in their own rows only
     x[1, 5] = np.float32(np.inf)
     x[3, 700] = np.float32(np.nan)
