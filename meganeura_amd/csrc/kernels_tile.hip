@@ -582,8 +582,8 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
 // What a call costs outside the multiplication is what these choices are about: a CU's vector
 // memory pipeline takes about three cycles per cache line a load instruction touches, so the
 // loads of the prologue (activations, scale words, the first slices) hold the waves for
-// thousands of cycles before the first multiplication; only DEPTH slices are requested ahead, the
-// rest step by step.  The walk is written out step by step (NSL and Q are compile-time) with
+// thousands of cycles before the first multiplication; quants are requested one slice ahead and
+// not before the conversion is under way.  The walk is written out step by step (NSL and Q are compile-time) with
 // scheduling fences between its stages: left to itself the compiler moves the loads of later
 // steps behind the multiplications and the call takes a third longer.
 // K is cut into parts of NSL slices; the parts' partial tiles meet as in the kernel above.
@@ -729,7 +729,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   constexpr int NLQ = QB / 8;
   constexpr int NSL = resident_slices(F32A, R);
   constexpr int STEPS = NSL * Q;  // step f of the walk = (pair f / NSL, slice f % NSL)
-  constexpr int DEPTH = 2;        // steps whose quants are in flight ahead of the one in use
+  constexpr int DEPTH = 1;        // steps whose quants are in flight ahead of the one in use
   constexpr int SLOTS = DEPTH + 1;
   constexpr int NT = NSL * R;     // conversion tasks per half-wave
   // 16-byte units of scale words a lane stages: Q pairs x 32 columns x NSL slices x (32 or 16) bytes / 64 lanes
@@ -767,16 +767,19 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   // id = 64 j + lane: column id / kUnitsPerColumn (of the wave's Q x 32), unit id % kUnitsPerColumn.
   // Every lane of a column's tile reads them back slice by slice during the walk.
   u32x4_t mu[MU];
+  auto load_scale_words = [&]() {
 #pragma unroll
-  for (int j = 0; j < MU; j++) {
-    const uint32_t id = 64 * j + lane;
-    const uint32_t wcol = id / kUnitsPerColumn, unit = id % kUnitsPerColumn;
-    const uint32_t col = min(pair0 * (kSide * 16) + wcol, n - 1);
-    const uint8_t* src = (const uint8_t*)meta_arg + ((size_t)col * bpc + (size_t)sl0 * kSliceBlocks) * MB + unit * 16;
-    typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
-    const u32x4_a2 v = *(const u32x4_a2*)src;
-    mu[j] = u32x4_t{v.x, v.y, v.z, v.w};
-  }
+    for (int j = 0; j < MU; j++) {
+      const uint32_t id = 64 * j + lane;
+      const uint32_t wcol = id / kUnitsPerColumn, unit = id % kUnitsPerColumn;
+      const uint32_t col = min(pair0 * (kSide * 16) + wcol, n - 1);
+      const uint8_t* src = (const uint8_t*)meta_arg + ((size_t)col * bpc + (size_t)sl0 * kSliceBlocks) * MB + unit * 16;
+      typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+      const u32x4_a2 v = *(const u32x4_a2*)src;
+      mu[j] = u32x4_t{v.x, v.y, v.z, v.w};
+    }
+  };
+  load_scale_words();
 
   // ---- weight slices ----
   // Slices past the end of K (last part) and columns past N read the pad behind the weights or
@@ -796,13 +799,22 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
       for (int j = 0; j < NLQ; j++)
         wq[f % SLOTS][u][j] = __builtin_nontemporal_load((const u32x4_t*)(qb + q_off[f / NSL][u] + 64 * j));
   };
-#pragma unroll
-  for (int f = 0; f < DEPTH && f < STEPS; f++) fetch(f);
-  __builtin_amdgcn_sched_barrier(0);
-
   // ---- activations -> images in LDS; scale words -> LDS ----
+  // The first slices of quants are requested between the conversion tasks, not before them: a
+  // CU's memory pipeline is busy with the activations until then, and every load queued in
+  // front of them delays the conversion that all waves wait for (first request after the second
+  // task, one slice ahead from there on: 15.0 -> 14.0 us at M = 16 on 4096 x 14336; two slices
+  // ahead or any request before the conversion measured 0.3-2.3 us slower).
+  constexpr int kFirstFetchAfterTask = NT > 1 ? 1 : 0;
 #pragma unroll
-  for (int t = 0; t < NT; t++) convert_task<FMT, F32A>(xin[t], xok[t], img + t * UNITS, cr, cl);
+  for (int t = 0; t < NT; t++) {
+    convert_task<FMT, F32A>(xin[t], xok[t], img + t * UNITS, cr, cl);
+    __builtin_amdgcn_sched_barrier(0);
+    if (t >= kFirstFetchAfterTask && t - kFirstFetchAfterTask < DEPTH && t - kFirstFetchAfterTask < STEPS) fetch(t - kFirstFetchAfterTask);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int f = NT - kFirstFetchAfterTask; f < DEPTH && f < STEPS; f++) fetch(f);
 #pragma unroll
   for (int j = 0; j < MU; j++) {
     const uint32_t id = 64 * j + lane;
@@ -1168,7 +1180,7 @@ bool tile_mfma_supported(const LaunchArgs& x) {
 }
 
 // Up to 16 rows, K >= 544, at most four K parts and one round of workgroups that fills at least
-// three quarters of the CUs (e.g. 4096 x 14336 at M = 5..16: 15.0 us against 17.2 us on the 32x32 tiled
+// three quarters of the CUs (e.g. 4096 x 14336 at M = 5..16: 14.0 us against 17.0 us on the 32x32 tiled
 // kernel).  On smaller shapes the conversion of the activations in every workgroup and the
 // parts' hand-over cost more than the tiled kernel's whole call; with more parts or rounds the
 // two are level or the tiled kernel wins.
