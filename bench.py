@@ -262,6 +262,20 @@ def config_table(ctx, sets, steps=200, repeats=5, preheat_ms=20.0):
         table[name] = {"us": r["median"] * 1e3, "us_min": r["min"] * 1e3, "us_max": r["max"] * 1e3,
                        "bound": roof["bound"], "achieved": roof["achieved"], "unit": roof["unit"], "frac": roof["frac"],
                        "algorithmic_bytes": wl.bytes}
+        if m > 4 and not f16:
+            # f32 activations at M >= 5: the figure above is the context's default (activations of any
+            # magnitude, the rescaling kernels); beside it, the same call on a context that was promised
+            # activations in the fp16 range (mgn_ctx_set_activation_range), where the plans differ
+            from meganeura_amd import capi
+            if capi.matmul_plan(fmt, m, k, n).route != capi.matmul_plan(fmt, m, k, n, fp16_range=True).route:
+                ctx.set_activation_range(True)
+                try:
+                    rp = wl.measure(steps, 20, repeats, preheat_ms)
+                    wl.check()
+                finally:
+                    ctx.set_activation_range(False)
+                table[name]["us_fp16_range"] = rp["median"] * 1e3
+                table[name]["frac_fp16_range"] = wl.roofline(rp["median"])["frac"]
         wl.free()
     if last_key is not None:
         sets.drop(*last_key)

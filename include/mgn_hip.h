@@ -40,8 +40,8 @@ typedef enum mgn_status {
   MGN_ENODEVICE = 5, /* no usable gfx950 device */
   MGN_EUNSUPPORTED = 6, /* a fused entry point asked for a shape its kernel does not serve */
   MGN_ERANGE = 7 /* reported by the next synchronising call: an f32 activation too large for the kernel
-                    that ran (|x| >= 65504 on MGN_ROUTE_GEMM_MFMA, M >= 5); outputs of that call are wrong;
-                    see mgn_ctx_set_activation_range */
+                    that ran (|x| >= 65504 on MGN_ROUTE_GEMM_MFMA, M >= 5, which only a context set to
+                    MGN_ACT_FP16_RANGE or a forced route uses for f32); outputs of that call are wrong */
 } mgn_status;
 
 /* compile::WeightFormat::{Q4,Q8} (src/compile.rs:8-29), graph::DType::{Q4_0,Q8_0}
@@ -77,16 +77,19 @@ void mgn_ctx_destroy(mgn_ctx* ctx);
 const char* mgn_last_error(const mgn_ctx* ctx);
 /* Session::wait (src/runtime.rs:2835-2841). */
 mgn_status mgn_sync(mgn_ctx* ctx);
-/* What the context may assume about f32 activations of matmuls with M >= 5.  By default
- * (any_magnitude == 0) it assumes |x| < 65504, the range an fp16 pair splits exactly, which its
- * fastest tiled kernel relies on; a call that meets a larger value is reported as MGN_ERANGE by
- * the next synchronising call.  With any_magnitude != 0 those matmuls run on the kernel that
- * rescales every 256-element slice of a row by a power of two: every finite f32 is exact input,
- * inf and NaN stay in their rows, at the price of a slower call on most shapes.  fp16 activations
- * and M <= 4 never depend on this.  The reference multiplies in f32 on the scalar ALUs
- * (src/shaders/matmul.wgsl:43-90) and has no such limit, so a drop-in that cannot bound its
- * activations sets this once after mgn_ctx_create. */
-mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, int any_magnitude);
+/* What the context may assume about f32 activations of matmuls with M >= 5.
+ *   MGN_ACT_ANY (default): nothing.  Those matmuls run on the kernels that rescale every
+ *     256-element slice of a row by a power of two before splitting it into fp16 pairs: every
+ *     finite f32 is exact input whatever its magnitude, inf and NaN stay in their rows -- what the
+ *     reference's f32 arithmetic on the scalar ALUs gives (src/shaders/matmul.wgsl:43-90).
+ *   MGN_ACT_FP16_RANGE: the caller promises |x| < 65504 and accepts that values below 2^-4 are
+ *     carried with an absolute step of 2^-25 instead of a relative one.  The matmuls may then run
+ *     on the 32x32 tiled kernel, which splits without rescaling and is faster on most shapes
+ *     (about 1.8x at M = 512); an activation that breaks the promise is detected while it is
+ *     staged and the next synchronising call returns MGN_ERANGE.
+ * fp16 activations (mgn_matmul_q_f16a) and M <= 4 never depend on this. */
+typedef enum mgn_act_range { MGN_ACT_ANY = 0, MGN_ACT_FP16_RANGE = 1 } mgn_act_range;
+mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, mgn_act_range range);
 /* ---- plain device buffers: the reference allocates every plan buffer
  *      zero-filled (src/runtime.rs:1737-1755) and moves data with memcpy
  *      through mapped memory (upload_buffer 2552-2558, read_buffer 2623-2629). */
@@ -220,18 +223,23 @@ mgn_status mgn_matmul_q_at(mgn_ctx* ctx, const mgn_buf* a_t, const mgn_weight* w
  * automatic choice takes (the analogue of reading compile.rs:1390 and runtime.rs:1634 for the
  * reference) and the launch geometry.  For logs, and for checking the planner on the host.
  * `num_cus` is the device's compute-unit count (256 on MI355X); the workspace is assumed to be
- * the one every context owns.  MGN_EINVAL for shapes no weight can have. */
+ * the one every context owns.  a_is_f16: 0 = f32 activations of any magnitude (a context's
+ * default), 1 = fp16 activations, 2 = f32 activations promised to lie in the fp16 range
+ * (MGN_ACT_FP16_RANGE).  MGN_EINVAL for shapes no weight can have. */
 typedef struct mgn_plan_info {
   int route;              /* mgn_route (never MGN_ROUTE_AUTO) */
   uint32_t grid[3];       /* workgroups */
   uint32_t threads;       /* per workgroup */
   uint32_t lds_bytes;     /* dynamic LDS per workgroup */
-  uint32_t waves_n;       /* column quads (GEMV) or 32-column tiles (tiled) per workgroup */
+  uint32_t waves_n;       /* column quads (GEMV), 32-column tiles (MGN_ROUTE_GEMM_MFMA) or 16-column tiles
+                           * (MGN_ROUTE_TILE_MFMA) per workgroup */
   uint32_t k_splits;      /* waves that share a quad / tile inside a workgroup */
   uint32_t k_parts;       /* workgroups that share a column group; > 1: partial sums through the workspace */
-  uint32_t steps;         /* GEMV: 16-block steps per wave; tiled: 8-block chunks per wave */
-  uint32_t quads_per_wave; /* GEMV only */
-  uint32_t full_steps;    /* GEMV only: 1 when no step needs masking */
+  uint32_t steps;         /* GEMV: 16-block steps per wave; tiled: 8-block chunks (slices of 256 elements) per wave and part */
+  uint32_t quads_per_wave; /* GEMV: column quads per wave; MGN_ROUTE_TILE_MFMA: 0 for the form that keeps the
+                            * activation images in LDS (M <= 32), else the launches the rows are spread over
+                            * (more than one when their activation images exceed the workspace) */
+  uint32_t full_steps;    /* GEMV: 1 when no step needs masking; MGN_ROUTE_TILE_MFMA: row tiles of 16 rows per workgroup */
   uint32_t tail_blocks;   /* GEMV only: 0, or the K blocks per column beyond `steps` full steps that the wave's
                            * quads share one more step for (K = 32 * (16 * steps + tail_blocks)) */
   uint64_t workspace_bytes; /* partial sums held in the context's workspace */

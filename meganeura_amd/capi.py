@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_DIR, "libmgn_hip.so")
 
 OK, EINVAL, ENOMEM, EHIP, ENOTFOUND, ENODEVICE, EUNSUPPORTED, ERANGE = range(8)
 FMT_Q4, FMT_Q8 = 0, 1
+ACT_ANY, ACT_FP16_RANGE = 0, 1
 STATIC_WORKSPACE_BYTES = 4 << 20  # MGN_STATIC_WORKSPACE_BYTES
 ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA, ROUTE_TILE_MFMA = range(6)
 
@@ -182,10 +183,11 @@ class PlanInfo(C.Structure):
                 ("workspace_bytes", C.c_uint64)]
 
 
-def matmul_plan(fmt, m, k, n, a_is_f16=False, num_cus=256):
-    """What mgn_matmul_q would launch for this shape (no device needed)."""
+def matmul_plan(fmt, m, k, n, a_is_f16=False, num_cus=256, fp16_range=False):
+    """What mgn_matmul_q would launch for this shape (no device needed).  fp16_range: f32
+    activations on a context set to ACT_FP16_RANGE."""
     info = PlanInfo()
-    st = load().mgn_matmul_q_plan(fmt, m, k, n, 1 if a_is_f16 else 0, num_cus, C.byref(info))
+    st = load().mgn_matmul_q_plan(fmt, m, k, n, 1 if a_is_f16 else 2 if fp16_range else 0, num_cus, C.byref(info))
     if st != OK:
         raise MgnError(st, "matmul_plan: no weight has this shape")
     return info
@@ -257,9 +259,10 @@ class Context:
     def __exit__(self, *exc):
         self.close()
 
-    def set_activation_range(self, any_magnitude):
-        """f32 activations of M >= 5: False (default) promises |x| < 65504, True takes any finite value."""
-        self.check(self.lib.mgn_ctx_set_activation_range(self.h, 1 if any_magnitude else 0))
+    def set_activation_range(self, fp16_range):
+        """f32 activations of M >= 5: False (default, ACT_ANY) takes any value; True (ACT_FP16_RANGE)
+        promises |x| < 65504 and lets the faster unscaled tiled kernel run."""
+        self.check(self.lib.mgn_ctx_set_activation_range(self.h, ACT_FP16_RANGE if fp16_range else ACT_ANY))
 
     def set_route(self, route):
         self.check(self.lib.mgn_ctx_set_route(self.h, route))

@@ -1092,6 +1092,9 @@ bool plan_tile(const LaunchArgs& x, TilePlan* out) {
           if ((phases + nph - 1) / nph != parts) continue;  // same split, already seen
           const size_t partial = parts > 1 ? (size_t)parts * rowgroups * r * 16 * x.w.n * 4 : 0;
           if (partial > x.scratch_bytes) break;
+          // the images of every row tile and slice sit behind the partial tiles in the workspace
+          const size_t images = (size_t)rowgroups * r * parts * nph * ksc * units * 16;
+          if (((partial + 255) & ~(size_t)255) + images > x.scratch_bytes) continue;
           if (parts > 1 && (uint64_t)rowgroups * colgroups > x.n_counters) break;
           const uint64_t wgs = (uint64_t)rowgroups * colgroups * parts;
           const uint32_t per_cu = std::max<uint32_t>(1, std::min<uint32_t>((uint32_t)(160 * 1024 / lds), 16 / waves));
@@ -1169,14 +1172,30 @@ int launch_fa(ihipStream_t* s, const LaunchArgs& x, const TilePlan& p) {
 
 size_t tile_workspace_bytes(const TilePlan& p) { return ((p.partial_bytes + 255) & ~(size_t)255) + p.image_bytes; }
 
+// The general kernel's plan for as many rows per launch as the workspace has room for (partial
+// tiles + activation images): all of them, or blocks of a multiple of 16 rows launched one after
+// the other.  False if not even 16 rows fit.
+bool plan_tile_rows(const LaunchArgs& x, TilePlan* p, uint32_t* rows) {
+  LaunchArgs y = x;
+  for (uint32_t mc = x.m;;) {
+    y.m = mc;
+    if (plan_tile(y, p) && tile_workspace_bytes(*p) <= x.scratch_bytes) {
+      *rows = mc;
+      return true;
+    }
+    if (mc <= 16) return false;
+    mc = mc > 128 ? (mc / 2 + 63) / 64 * 64 : (mc / 2 + 15) / 16 * 16;
+  }
+}
+
 }  // namespace
 
 bool tile_mfma_supported(const LaunchArgs& x) {
   ResidentPlan rp;
   if (plan_resident(x, &rp)) return true;
   TilePlan p;
-  if (!plan_tile(x, &p)) return false;
-  return tile_workspace_bytes(p) <= x.scratch_bytes;
+  uint32_t rows;
+  return plan_tile_rows(x, &p, &rows);
 }
 
 // Up to 16 rows, K >= 544, at most four K parts and one round of workgroups that fills at least
@@ -1199,18 +1218,20 @@ bool describe_tile_mfma(const LaunchArgs& x, mgn_plan_info* out) {
     out->threads = 512;
     out->lds_bytes = (uint32_t)rp.lds;
     out->waves_n = 8 * kSide * rp.q, out->k_splits = 1, out->k_parts = rp.parts, out->steps = rp.nsl;
-    out->quads_per_wave = 0, out->full_steps = 0, out->tail_blocks = 0;
+    out->quads_per_wave = 0, out->full_steps = rp.r, out->tail_blocks = 0;
     out->workspace_bytes = rp.partial_bytes;
     return true;
   }
   TilePlan p;
-  if (!plan_tile(x, &p) || tile_workspace_bytes(p) > x.scratch_bytes) return false;
+  uint32_t rows;
+  if (!plan_tile_rows(x, &p, &rows)) return false;
   out->route = MGN_ROUTE_TILE_MFMA;
   out->grid[0] = p.parts, out->grid[1] = p.colgroups, out->grid[2] = p.rowgroups;
   out->threads = 64 * p.ksc * p.wnc;
   out->lds_bytes = (uint32_t)p.lds;
   out->waves_n = p.wnc, out->k_splits = p.ksc, out->k_parts = p.parts, out->steps = p.nph;
-  out->quads_per_wave = 0, out->full_steps = 0, out->tail_blocks = 0;
+  out->quads_per_wave = (x.m + rows - 1) / rows;  // launches
+  out->full_steps = p.r, out->tail_blocks = 0;
   out->workspace_bytes = tile_workspace_bytes(p);
   return true;
 }
@@ -1223,9 +1244,23 @@ int launch_matmul_tile_mfma(ihipStream_t* s, const LaunchArgs& x) {
     return x.a_is_f16 ? launch_resident_fa<MGN_FMT_Q8, false>(s, x, rp) : launch_resident_fa<MGN_FMT_Q8, true>(s, x, rp);
   }
   TilePlan p;
-  if (!plan_tile(x, &p) || tile_workspace_bytes(p) > x.scratch_bytes) return (int)hipErrorInvalidValue;
-  if (x.w.fmt == MGN_FMT_Q4) return x.a_is_f16 ? launch_fa<MGN_FMT_Q4, false>(s, x, p) : launch_fa<MGN_FMT_Q4, true>(s, x, p);
-  return x.a_is_f16 ? launch_fa<MGN_FMT_Q8, false>(s, x, p) : launch_fa<MGN_FMT_Q8, true>(s, x, p);
+  uint32_t rows;
+  if (!plan_tile_rows(x, &p, &rows)) return (int)hipErrorInvalidValue;
+  // blocks of rows, one launch pair (images, multiplication) each; they share the workspace and
+  // follow each other on the stream
+  for (uint32_t r0 = 0; r0 < x.m; r0 += rows) {
+    LaunchArgs y = x;
+    y.m = std::min(rows, x.m - r0);
+    y.a = (const char*)x.a + (size_t)r0 * x.w.k * (x.a_is_f16 ? 2 : 4);
+    y.c = x.c + (size_t)r0 * x.w.n;
+    y.d = x.d ? x.d + (size_t)r0 * x.w.n : nullptr;
+    if (y.m != rows && !plan_tile(y, &p)) return (int)hipErrorInvalidValue;  // the last, shorter block
+    int e;
+    if (x.w.fmt == MGN_FMT_Q4) e = x.a_is_f16 ? launch_fa<MGN_FMT_Q4, false>(s, y, p) : launch_fa<MGN_FMT_Q4, true>(s, y, p);
+    else e = x.a_is_f16 ? launch_fa<MGN_FMT_Q8, false>(s, y, p) : launch_fa<MGN_FMT_Q8, true>(s, y, p);
+    if (e) return e;
+  }
+  return 0;
 }
 
 }  // namespace mgn

@@ -115,13 +115,27 @@ mgn_status weight_alloc(mgn_ctx* ctx, mgn_fmt fmt, size_t rows, size_t cols, mgn
   return MGN_OK;
 }
 
+// The automatic choice of a kernel family.  M <= 4: the MFMA GEMV.  Larger M: the resident
+// 16x16x32 kernel where it measured faster; the 32x32 tiled kernel for fp16 activations and
+// for f32 activations the caller has promised to keep in the fp16 range (it splits them
+// without rescaling), if the weight's block constants are in its range too; the rescaling
+// 16x16x32 kernels for everything else.
+mgn_route auto_route(const mgn::LaunchArgs& x, bool any_magnitude) {
+  if (mgn::gemv_mfma_supported(x)) return MGN_ROUTE_GEMV_MFMA;
+  if (mgn::tile_mfma_preferred(x)) return MGN_ROUTE_TILE_MFMA;
+  if ((x.a_is_f16 || !any_magnitude) && mgn::gemm_mfma_supported(x)) return MGN_ROUTE_GEMM_MFMA;
+  if (mgn::tile_mfma_supported(x)) return MGN_ROUTE_TILE_MFMA;
+  if (mgn::gemv_supported(x)) return MGN_ROUTE_GEMV_VALU;
+  return MGN_ROUTE_GENERIC;
+}
+
 // After the stream has been synchronised: did a kernel meet activations outside its range?
 mgn_status check_range_flag(mgn_ctx* ctx) {
   if (!ctx->range_flag_host || *(volatile uint32_t*)ctx->range_flag_host == 0) return MGN_OK;
   *(volatile uint32_t*)ctx->range_flag_host = 0;
   return fail(ctx, MGN_ERANGE,
               "an f32 activation of magnitude >= 65504 reached the tiled MFMA kernel (M >= 5), which splits activations "
-              "into fp16 pairs: the affected outputs are wrong; mgn_ctx_set_activation_range(ctx, 1) takes such data");
+              "into fp16 pairs without rescaling: the affected outputs are wrong (the context was set to MGN_ACT_FP16_RANGE, or the route was forced)");
 }
 
 // Looks at every block's scale (and minimum) once, right after a weight's blocks are on the
@@ -238,9 +252,10 @@ mgn_status mgn_sync(mgn_ctx* ctx) {
   return check_range_flag(ctx);
 }
 
-mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, int any_magnitude) {
+mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, mgn_act_range range) {
   if (!ctx) return MGN_EINVAL;
-  ctx->any_magnitude = any_magnitude != 0;
+  if (range != MGN_ACT_ANY && range != MGN_ACT_FP16_RANGE) return fail(ctx, MGN_EINVAL, "unknown activation range");
+  ctx->any_magnitude = range == MGN_ACT_ANY;
   return MGN_OK;
 }
 
@@ -585,15 +600,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
       return fail(ctx, MGN_EUNSUPPORTED, "fused prologue needs the GEMV_MFMA route (f32 activations, M <= 4)");
     route = MGN_ROUTE_GEMV_MFMA;
   }
-  if (route == MGN_ROUTE_AUTO) {
-    if (mgn::gemv_mfma_supported(x)) route = MGN_ROUTE_GEMV_MFMA;
-    else if (mgn::tile_mfma_preferred(x)) route = MGN_ROUTE_TILE_MFMA;  // measured faster than the kernel below
-    else if (ctx->any_magnitude && !a_is_f16 && mgn::tile_mfma_supported(x)) route = MGN_ROUTE_TILE_MFMA;
-    else if (mgn::gemm_mfma_supported(x)) route = MGN_ROUTE_GEMM_MFMA;
-    else if (mgn::tile_mfma_supported(x)) route = MGN_ROUTE_TILE_MFMA;  // e.g. a weight whose block minima the kernel above cannot hold
-    else if (mgn::gemv_supported(x)) route = MGN_ROUTE_GEMV_VALU;
-    else route = MGN_ROUTE_GENERIC;
-  }
+  if (route == MGN_ROUTE_AUTO) route = auto_route(x, ctx->any_magnitude);
   if (static_workspace) {
     // Same plan as the allocating entry point (the planners see the same workspace limits), run
     // on the library's static array if the plan's partial sums fit it; refused otherwise.
@@ -769,7 +776,7 @@ mgn_status mgn_matmul_q_plan(mgn_fmt fmt, uint32_t m, uint64_t k, uint64_t n, in
   mgn::LaunchArgs x{};
   x.w = mgn::WeightView{nullptr, nullptr, (uint32_t)k, (uint32_t)n, (int)fmt, true};
   x.m = m;
-  x.a_is_f16 = a_is_f16 != 0;
+  x.a_is_f16 = a_is_f16 == 1;
   x.num_cus = num_cus;
   // the planners only look at whether a workspace exists, never through the pointers
   static char workspace_stand_in;
@@ -777,11 +784,12 @@ mgn_status mgn_matmul_q_plan(mgn_fmt fmt, uint32_t m, uint64_t k, uint64_t n, in
   x.scratch_bytes = mgn::kWorkspaceBytes;
   x.counters = (uint32_t*)&workspace_stand_in;
   x.n_counters = mgn::kWorkspaceCounters;
-  if (mgn::describe_gemv_mfma(x, out)) return MGN_OK;
-  if (mgn::tile_mfma_preferred(x) && mgn::describe_tile_mfma(x, out)) return MGN_OK;
-  if (mgn::describe_gemm_mfma(x, out)) return MGN_OK;
-  if (mgn::describe_tile_mfma(x, out)) return MGN_OK;
-  out->route = mgn::gemv_supported(x) ? MGN_ROUTE_GEMV_VALU : MGN_ROUTE_GENERIC;
+  if (a_is_f16 < 0 || a_is_f16 > 2) return MGN_EINVAL;
+  const mgn_route route = auto_route(x, a_is_f16 == 0);
+  if (route == MGN_ROUTE_GEMV_MFMA && mgn::describe_gemv_mfma(x, out)) return MGN_OK;
+  if (route == MGN_ROUTE_GEMM_MFMA && mgn::describe_gemm_mfma(x, out)) return MGN_OK;
+  if (route == MGN_ROUTE_TILE_MFMA && mgn::describe_tile_mfma(x, out)) return MGN_OK;
+  out->route = route;
   return MGN_OK;
 }
 

@@ -115,7 +115,7 @@ struct mgn_ctx {
   ihipEvent_t* ev_start = nullptr;
   ihipEvent_t* ev_stop = nullptr;
   mgn_route route = MGN_ROUTE_AUTO;
-  bool any_magnitude = false;  // f32 activations of M >= 5 may exceed the fp16 range (mgn_ctx_set_activation_range)
+  bool any_magnitude = true;  // f32 activations of M >= 5 may have any magnitude (mgn_ctx_set_activation_range)
   void* scratch = nullptr;  // split-K partial results + arrival counters, one allocation
   size_t scratch_bytes = 0;
   uint32_t* counters = nullptr;

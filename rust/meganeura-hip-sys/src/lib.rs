@@ -39,6 +39,10 @@ pub type mgn_fmt = c_int;
 pub const MGN_FMT_Q4: mgn_fmt = 0;
 pub const MGN_FMT_Q8: mgn_fmt = 1;
 
+pub type mgn_act_range = c_int;
+pub const MGN_ACT_ANY: mgn_act_range = 0;
+pub const MGN_ACT_FP16_RANGE: mgn_act_range = 1;
+
 /// `mgn_route`: kernel family; a runtime leaves it at `MGN_ROUTE_AUTO`.
 pub type mgn_route = c_int;
 pub const MGN_ROUTE_AUTO: mgn_route = 0;
@@ -96,7 +100,7 @@ extern "C" {
     pub fn mgn_ctx_destroy(ctx: *mut mgn_ctx);
     pub fn mgn_last_error(ctx: *const mgn_ctx) -> *const c_char;
     pub fn mgn_sync(ctx: *mut mgn_ctx) -> mgn_status;
-    pub fn mgn_ctx_set_activation_range(ctx: *mut mgn_ctx, any_magnitude: c_int) -> mgn_status;
+    pub fn mgn_ctx_set_activation_range(ctx: *mut mgn_ctx, range: mgn_act_range) -> mgn_status;
     pub fn mgn_buf_alloc(ctx: *mut mgn_ctx, bytes: usize, out: *mut *mut mgn_buf) -> mgn_status;
     pub fn mgn_buf_free(ctx: *mut mgn_ctx, buf: *mut mgn_buf);
     pub fn mgn_buf_size(buf: *const mgn_buf) -> usize;

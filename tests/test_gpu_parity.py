@@ -673,6 +673,37 @@ def test_weights_with_huge_minima_and_scales_stay_on_the_matrix_cores(ctx, orc, 
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
+def test_rows_whose_activation_images_exceed_the_workspace_run_in_blocks(ctx, orc, fmt):
+    """The general 16x16x32 kernel keeps the converted activations of a launch in the context's 16 MiB
+    workspace (17.25 KiB per 16 rows x 256 elements of f32 activations).  300 rows of K = 16384 need
+    21 MB: the rows go out in blocks, one launch pair each, with the residual and the epilogue
+    applied per block.  The last block is shorter than the others and ends off a multiple of 16."""
+    m, k, n = 300, 16384, 48
+    plan = capi.matmul_plan(fmt, m, k, n)
+    assert plan.route == capi.ROUTE_TILE_MFMA and plan.quads_per_wave >= 2
+    w = synth.normal(980 + fmt, k * n, 0.02).reshape(k, n)
+    x = synth.normal(981, m * k, 1.0).reshape(m, k)
+    x[7] *= np.float32(3.0e7)   # a row far outside the fp16 range, in the first block
+    x[299] *= np.float32(1e-9)  # and a tiny one in the last
+    d = synth.normal(982, m * n, 1.0).reshape(m, n)
+    packed = orc.quantize(fmt, w)
+    want = np.asarray(orc.matmul_f64(x, orc.dequantize(fmt, packed, k, n)), np.float64)
+    wt = ctx.weight(fmt, w)
+    a, dd, c = ctx.upload(x), ctx.upload(d), ctx.buffer(m * n * 4)
+    ctx.matmul_q(a, wt, c, m)
+    assert_close_rowwise(c.download(np.float32, m * n).reshape(m, n), want, x)
+    ctx.matmul_q(a, wt, c, m, d=dd)
+    got = c.download(np.float32, m * n).reshape(m, n)
+    rows = np.ones(m, bool)
+    rows[[7, 299]] = False  # (their products dwarf or vanish beside a residual of order one)
+    assert_close_rowwise(got[rows], want[rows] + d[rows], x[rows])
+    assert np.allclose(got[299], d[299], rtol=0, atol=1e-6)
+    for b in (a, dd, c):
+        b.free()
+    wt.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
 @pytest.mark.parametrize("m", [5, 16, 40])
 def test_activations_of_any_magnitude_on_the_rescaling_tiled_kernel(ctx, orc, fmt, m):
     """f32 activations are scaled per (row, 256-element slice) by a power of two before they are
@@ -698,10 +729,18 @@ def test_activations_of_any_magnitude_on_the_rescaling_tiled_kernel(ctx, orc, fm
         run_matmul(ctx, fmt, x, wt, ROUTES["gemm_mfma"])
     assert e.value.status == capi.ERANGE
     ctx.sync()  # reported once; the context keeps working
-    # a context told that activations may have any magnitude keeps such matmuls off that kernel
+    # the automatic route assumes nothing about f32 activations and keeps them off that kernel ...
+    assert_close_rowwise(run_matmul(ctx, fmt, x, wt, capi.ROUTE_AUTO), want, x)
+    # ... unless the context was promised that they lie in the fp16 range: then the promise is checked
     ctx.set_activation_range(True)
     try:
-        assert_close_rowwise(run_matmul(ctx, fmt, x, wt, capi.ROUTE_AUTO), want, x)
+        with pytest.raises(capi.MgnError) as e:
+            run_matmul(ctx, fmt, x, wt, capi.ROUTE_AUTO)
+        assert e.value.status == capi.ERANGE
+        ctx.sync()
+        tame = synth.normal(997 + m, m * k, 1.0).reshape(m, k)
+        oracle_tame = orc.matmul_f64(tame, orc.dequantize(fmt, packed, k, n))
+        assert_close_rowwise(run_matmul(ctx, fmt, tame, wt, capi.ROUTE_AUTO), oracle_tame, tame)
     finally:
         ctx.set_activation_range(False)
     # non-finite activations give non-finite outputs in their own rows only

@@ -78,22 +78,34 @@ def check_gemm(p, fmt, m, k, n, f16):
         assert p.workspace_bytes == 0
 
 
-def check_tile_resident(p, fmt, m, k, n, f16):
-    """The automatic route only takes the 16x16x32 kernel in its form for up to 16 rows with the
-    activation images resident in LDS: grid = (K parts, column groups), 8 waves, each with one or
-    two pairs of 16-column tiles, parts of `steps` slices of 256 elements."""
-    assert 5 <= m <= 16 and p.grid[2] == 1 and p.threads == 512
-    assert p.lds_bytes <= 160 * 1024
+def check_tile(p, fmt, m, k, n, f16):
+    """MGN_ROUTE_TILE_MFMA: tiles of 16 columns, K in slices of 256 elements, `full_steps` row tiles of 16 rows
+    per workgroup.  quads_per_wave == 0: the form for M <= 32 that keeps the activation images in LDS (grid =
+    (K parts, column groups), 8 waves with one or two pairs of tiles each, parts of 4 slices, or of 2 with f32
+    activations beyond 16 rows); otherwise the general form (grid = (K parts, column groups, row groups),
+    `k_splits` waves per tile) in `quads_per_wave` launches over blocks of rows."""
     nslices, n_tiles = ceil_div(k, 256), ceil_div(n, 16)
-    assert p.steps == 4 and p.waves_n in (16, 32)  # slices per part; tiles per workgroup
-    assert p.grid[0] == p.k_parts == ceil_div(nslices, p.steps) <= 4 and nslices >= 3
+    assert p.lds_bytes <= 160 * 1024 and p.threads <= 512
+    rows = 16 * p.full_steps
     assert p.grid[1] * p.waves_n >= n_tiles and (p.grid[1] - 1) * p.waves_n < n_tiles
-    wgs = p.grid[0] * p.grid[1]
-    assert 192 <= wgs <= 256  # one round of workgroups over the 256 CUs, at least three quarters of them busy
-    if p.k_parts > 1:
-        assert p.workspace_bytes == p.k_parts * 16 * n * 4 <= WORKSPACE and p.grid[1] <= COUNTERS
+    assert p.grid[0] == p.k_parts >= 1
+    if p.quads_per_wave == 0:
+        assert m <= 32 and p.grid[2] == 1 and p.threads == 512 and rows >= m and p.full_steps == (1 if m <= 16 else 2)
+        assert p.steps == (2 if (not f16 and m > 16) else 4) and p.waves_n in (16, 32)
+        assert p.k_parts == ceil_div(nslices, p.steps)
+        partial = p.k_parts * rows * n * 4 if p.k_parts > 1 else 0
+        assert p.workspace_bytes == partial <= WORKSPACE
+        if p.k_parts > 1:
+            assert p.grid[1] <= COUNTERS
     else:
-        assert p.workspace_bytes == 0
+        assert p.full_steps in (1, 2, 4) and p.k_splits in (1, 2, 4) and p.threads == 64 * p.k_splits * p.waves_n
+        assert p.k_parts * p.steps * p.k_splits >= nslices
+        assert p.quads_per_wave * p.grid[2] * rows >= m          # the launches' row groups cover every row
+        if p.quads_per_wave == 1:
+            assert (p.grid[2] - 1) * rows < m
+        assert p.workspace_bytes <= WORKSPACE
+        if p.k_parts > 1:
+            assert p.grid[1] * p.grid[2] <= COUNTERS
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
@@ -102,14 +114,19 @@ def test_plans_cover_the_problem_and_respect_the_limits(fmt):
     for m, k, n in itertools.product(MS, KS, NS):
         if (k // 32) * n >= 0x7FFFFFFF:
             continue
-        for f16 in (False, True):
-            p = capi.matmul_plan(fmt, m, k, n, f16)
-            where = f"fmt={fmt} m={m} k={k} n={n} f16={f16} route={p.route}"
+        # activations: f32 of any magnitude (a context's default), fp16, f32 promised to lie in the fp16 range
+        for f16, promised in ((False, False), (True, False), (False, True)):
+            p = capi.matmul_plan(fmt, m, k, n, f16, fp16_range=promised)
+            where = f"fmt={fmt} m={m} k={k} n={n} f16={f16} promised={promised} route={p.route}"
             routes.add(p.route)
             try:
                 assert p.route in (GENERIC, GEMV_VALU, GEMV_MFMA, GEMM_MFMA, TILE_MFMA)
-                if m > 4:
-                    assert p.route in (GEMM_MFMA, TILE_MFMA, GENERIC)
+                if m > 4 and not f16 and not promised:
+                    # nothing is assumed about f32 activations: the rescaling kernels (their lanes address the
+                    # weight with 32-bit offsets; beyond 2^32 elements the scalar route is the one left)
+                    assert p.route == (TILE_MFMA if k * n < 1 << 32 else GENERIC)
+                elif m > 4:
+                    assert p.route in (GEMM_MFMA, TILE_MFMA)
                 if f16:
                     assert p.route != GEMV_VALU  # the vector-ALU GEMV reads f32 activations only
                 if p.route == GEMV_MFMA:
@@ -117,7 +134,7 @@ def test_plans_cover_the_problem_and_respect_the_limits(fmt):
                 elif p.route == GEMM_MFMA:
                     check_gemm(p, fmt, m, k, n, f16)
                 elif p.route == TILE_MFMA:
-                    check_tile_resident(p, fmt, m, k, n, f16)
+                    check_tile(p, fmt, m, k, n, f16)
             except AssertionError as e:
                 raise AssertionError(where) from e
     assert {GEMV_MFMA, GEMM_MFMA, TILE_MFMA} <= routes
@@ -132,9 +149,16 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
     for fmt, m, k, n in gemv:
         assert capi.matmul_plan(fmt, m, k, n).route == GEMV_MFMA, (fmt, m, k, n)
     for fmt in (Q4, Q8):
-        assert capi.matmul_plan(fmt, 16, 4096, 14336).route == TILE_MFMA   # one round of workgroups, 4 K parts
-        assert capi.matmul_plan(fmt, 16, 14336, 4096).route == GEMM_MFMA   # would be 14 K parts
-        assert capi.matmul_plan(fmt, 17, 4096, 14336).route == GEMM_MFMA
+        # the LDS-resident form is the faster kernel here whatever the activations (one round of workgroups, 4 K parts)
+        for promised in (False, True):
+            p = capi.matmul_plan(fmt, 16, 4096, 14336, fp16_range=promised)
+            assert p.route == TILE_MFMA and p.quads_per_wave == 0 and list(p.grid) == [4, 56, 1]
+        # elsewhere the 32x32 kernel is ahead, and runs when the activations are fp16 or promised to be in its range
+        assert capi.matmul_plan(fmt, 16, 14336, 4096, fp16_range=True).route == GEMM_MFMA   # would be 14 K parts
+        assert capi.matmul_plan(fmt, 17, 4096, 14336, fp16_range=True).route == GEMM_MFMA
+        assert capi.matmul_plan(fmt, 16, 14336, 4096).route == TILE_MFMA
+    big = capi.matmul_plan(Q4, 512, 14336, 4096)   # images of 512 rows x 14336 exceed the 16 MiB workspace: several launches
+    assert big.route == TILE_MFMA and big.quads_per_wave > 1
     for k, n in ((1024, 3072), (3072, 1024)):
         assert capi.matmul_plan(Q4, 512, k, n, True).route == GEMM_MFMA
     head = capi.matmul_plan(Q4, 1, 4096, 14336)
