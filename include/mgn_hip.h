@@ -84,9 +84,9 @@ mgn_status mgn_sync(mgn_ctx* ctx);
  *     reference's f32 arithmetic on the scalar ALUs gives (src/shaders/matmul.wgsl:43-90).
  *   MGN_ACT_FP16_RANGE: the caller promises |x| < 65504 and accepts that values below 2^-4 are
  *     carried with an absolute step of 2^-25 instead of a relative one.  The matmuls may then run
- *     on the 32x32 tiled kernel, which splits without rescaling and is faster on most shapes
- *     (about 1.8x at M = 512); an activation that breaks the promise is detected while it is
- *     staged and the next synchronising call returns MGN_ERANGE.
+ *     on the 32x32 tiled kernel, which splits without rescaling and is faster on some shapes
+ *     (up to 1.3x, mostly long K at many rows); an activation that breaks the promise is
+ *     detected while it is staged and the next synchronising call returns MGN_ERANGE.
  * fp16 activations (mgn_matmul_q_f16a) and M <= 4 never depend on this. */
 typedef enum mgn_act_range { MGN_ACT_ANY = 0, MGN_ACT_FP16_RANGE = 1 } mgn_act_range;
 mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, mgn_act_range range);

@@ -741,6 +741,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t c = lane & 15, g = lane >> 4;
   const uint32_t part = blockIdx.x, cg = blockIdx.y;
+  const uint32_t row0 = blockIdx.z * (R * 16);  // first row of this workgroup's row group
   const uint32_t bpc = kdim / 32;
   const uint32_t pair0 = (cg * 8 + wave) * Q;  // this wave's first pair of column tiles
   const uint32_t sl0 = part * NSL;             // first slice of this part
@@ -756,7 +757,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
 #pragma unroll
   for (int t = 0; t < NT; t++) {
     const uint32_t s = t / R, rr = t % R;
-    const uint32_t row = rr * 16 + cr, k0 = (sl0 + s) * 256 + cl * 8;
+    const uint32_t row = row0 + rr * 16 + cr, k0 = (sl0 + s) * 256 + cl * 8;
     xok[t] = row < m && k0 < kdim;
     load_task<F32A>(a, xok[t] ? (size_t)row * kdim + k0 : (size_t)0, xin[t]);
   }
@@ -884,14 +885,14 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
 
   if (parts > 1) {
     // K parts of other workgroups: the last one to arrive adds them up in part order (see above)
-    const size_t plane = (size_t)R * 16 * n;  // floats per part
+    const size_t plane = (size_t)gridDim.z * (R * 16) * n;  // floats per part
 #pragma unroll
     for (int p = 0; p < Q; p++)
 #pragma unroll
       for (int u = 0; u < kSide; u++) {
         const uint32_t col = ((pair0 + p) * kSide + u) * 16 + c;
         if (col < n) {
-          float* const mine = tail.scratch + (size_t)part * plane + col;
+          float* const mine = tail.scratch + (size_t)part * plane + (size_t)row0 * n + col;
 #pragma unroll
           for (int r = 0; r < R; r++)
 #pragma unroll
@@ -903,7 +904,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
     __syncthreads();
     uint32_t* const flag = (uint32_t*)lds4;
     if (tid == 0) {
-      uint32_t* const ctr = tail.counters + cg;
+      uint32_t* const ctr = tail.counters + blockIdx.z * gridDim.y + cg;
       const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const bool last = seen == parts - 1;
       if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
@@ -918,7 +919,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
     for (int p = 0; p < Q; p++)
 #pragma unroll
       for (int u = 0; u < kSide; u++) {
-        base[p][u] = tail.scratch + min(((pair0 + p) * kSide + u) * 16 + c, n - 1) + (size_t)(4 * g) * n;
+        base[p][u] = tail.scratch + min(((pair0 + p) * kSide + u) * 16 + c, n - 1) + (size_t)(row0 + 4 * g) * n;
 #pragma unroll
         for (int r = 0; r < R; r++) res[p][u][r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
       }
@@ -966,7 +967,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
         for (int r = 0; r < R; r++)
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            const uint32_t row = r * 16 + 4 * g + i;
+            const uint32_t row = row0 + r * 16 + 4 * g + i;
             if (row < m) {
               const size_t o = (size_t)row * n + col;
               tail.c[o] = apply_epilogue(tail.dres ? res[p][u][r][i] + tail.dres[o] : res[p][u][r][i], tail.epilogue);
@@ -977,8 +978,9 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
 }
 
 struct ResidentPlan {
-  uint32_t r, q, nsl, parts, colgroups, nslices;
+  uint32_t r, q, nsl, parts, colgroups, rowgroups, nslices;
   size_t lds, partial_bytes;
+  double cost;
 };
 
 size_t resident_lds_bytes(int fmt, bool f32a, uint32_t r, uint32_t q) {
@@ -986,33 +988,38 @@ size_t resident_lds_bytes(int fmt, bool f32a, uint32_t r, uint32_t q) {
   return (size_t)nsl * r * image_units(f32a) * 16 + (size_t)8 * q * 32 * meta_stride(fmt, nsl);
 }
 
-// M <= 32.  Q = 1 or 2 pairs of tiles per wave: the one whose grid fills the CUs better.
+// Row groups of 16 or 32 rows (32 only beyond 16 rows, and not for Q8: registers), Q = 1 or 2 pairs
+// of tiles per wave: the combination whose grid takes the fewest rounds over the CUs, weighted by
+// what a workgroup does (a fixed part for the conversion and the hand-over, its waves' steps).
 bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
-  if (x.m == 0 || x.m > 32 || x.w.k < 32) return false;
+  if (x.m == 0 || x.w.k < 32) return false;
   const uint32_t bpc = x.w.k / 32;
   if ((uint64_t)x.w.n * bpc * 32 >= (1ull << 32)) return false;  // a lane's weight offsets are 32-bit
   const bool f32a = !x.a_is_f16;
-  const uint32_t r = x.m <= 16 ? 1 : 2;
-  if (r == 2 && x.w.fmt == MGN_FMT_Q8) return false;  // would not fit the register file
-  const uint32_t nsl = resident_slices(f32a, r);
   const uint32_t nslices = (bpc + kSliceBlocks - 1) / kSliceBlocks, n_tiles = (x.w.n + 15) / 16;
-  const uint32_t parts = (nslices + nsl - 1) / nsl;
-  const size_t partial = parts > 1 ? (size_t)parts * r * 16 * x.w.n * 4 : 0;
-  if (partial > x.scratch_bytes) return false;
   double best = 0;
   ResidentPlan bp{};
-  for (uint32_t q = 1; q <= (r == 1 ? 2u : 1u); q++) {
-    const uint32_t per_wg = 8 * kSide * q;
-    const uint32_t colgroups = (n_tiles + per_wg - 1) / per_wg;
-    if (colgroups > 65535 || (parts > 1 && colgroups > x.n_counters)) continue;
-    const uint64_t wgs = (uint64_t)parts * colgroups;
-    // time ~ rounds of workgroups x work of one (a fixed part + the steps of its waves)
-    const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q);
-    if (best == 0 || cost < best) {
-      best = cost;
-      bp.r = r, bp.q = q, bp.nsl = nsl, bp.parts = parts, bp.colgroups = colgroups, bp.nslices = nslices;
-      bp.partial_bytes = partial;
-      bp.lds = resident_lds_bytes(x.w.fmt, f32a, r, q);
+  for (uint32_t r = 1; r <= 2; r++) {
+    if (r == 2 && (x.m <= 16 || x.w.fmt == MGN_FMT_Q8)) continue;
+    if (r == 1 && x.m > 16 && x.m <= 32 && x.w.fmt == MGN_FMT_Q4) continue;  // one row group of 32 instead of two of 16
+    const uint32_t nsl = resident_slices(f32a, r);
+    const uint32_t parts = (nslices + nsl - 1) / nsl;
+    const uint32_t rowgroups = (x.m + 16 * r - 1) / (16 * r);
+    if (rowgroups > 65535) continue;
+    const size_t partial = parts > 1 ? (size_t)parts * rowgroups * r * 16 * x.w.n * 4 : 0;
+    if (partial > x.scratch_bytes) continue;
+    for (uint32_t q = 1; q <= (r == 1 ? 2u : 1u); q++) {
+      const uint32_t per_wg = 8 * kSide * q;
+      const uint32_t colgroups = (n_tiles + per_wg - 1) / per_wg;
+      if (colgroups > 65535 || (parts > 1 && (uint64_t)colgroups * rowgroups > x.n_counters)) continue;
+      const uint64_t wgs = (uint64_t)parts * colgroups * rowgroups;
+      const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q * r * nsl / 4.0) + (parts > 1 ? 1.0 : 0.0);
+      if (best == 0 || cost < best) {
+        best = cost;
+        bp.r = r, bp.q = q, bp.nsl = nsl, bp.parts = parts, bp.colgroups = colgroups, bp.rowgroups = rowgroups;
+        bp.nslices = nslices, bp.partial_bytes = partial, bp.cost = cost;
+        bp.lds = resident_lds_bytes(x.w.fmt, f32a, r, q);
+      }
     }
   }
   if (best == 0) return false;
@@ -1027,8 +1034,8 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
   const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue};
-  hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups), dim3(512), p.lds, s, x.a, x.w.meta, x.w.quants, x.m, x.w.k, x.w.n, p.parts,
-                     p.nslices, tail);
+  hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups, p.rowgroups), dim3(512), p.lds, s, x.a, x.w.meta, x.w.quants, x.m, x.w.k,
+                     x.w.n, p.parts, p.nslices, tail);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }
@@ -1172,6 +1179,18 @@ int launch_fa(ihipStream_t* s, const LaunchArgs& x, const TilePlan& p) {
 
 size_t tile_workspace_bytes(const TilePlan& p) { return ((p.partial_bytes + 255) & ~(size_t)255) + p.image_bytes; }
 
+// Which of the two kernels takes a call.  Up to 32 rows: the one with LDS-resident images.  Beyond,
+// it runs row groups side by side and still wins where K is short enough for at most four K parts
+// and their partial tiles stay small (f32 512 x 1024 x 3072: 16.5 us against 29 us with images
+// through the workspace; 128 x 4096 x 4096: 21.8 against 28.8), except for Q8 below 128 rows,
+// where too few workgroups carry too much each (64 x 1024 x 3072: 13.9 against 11.2 us), and for
+// wide outputs whose partial tiles dominate (64 x 4096 x 14336: 43 against 40 us).
+bool use_resident(const LaunchArgs& x, ResidentPlan* rp) {
+  if (!plan_resident(x, rp)) return false;
+  if (x.m <= 32) return true;
+  return rp->parts <= 4 && rp->partial_bytes <= ((size_t)8 << 20) && (x.w.fmt == MGN_FMT_Q4 || x.m >= 128);
+}
+
 // The general kernel's plan for as many rows per launch as the workspace has room for (partial
 // tiles + activation images): all of them, or blocks of a multiple of 16 rows launched one after
 // the other.  False if not even 16 rows fit.
@@ -1192,29 +1211,35 @@ bool plan_tile_rows(const LaunchArgs& x, TilePlan* p, uint32_t* rows) {
 
 bool tile_mfma_supported(const LaunchArgs& x) {
   ResidentPlan rp;
-  if (plan_resident(x, &rp)) return true;
+  if (use_resident(x, &rp)) return true;
   TilePlan p;
   uint32_t rows;
   return plan_tile_rows(x, &p, &rows);
 }
 
-// Up to 16 rows, K >= 544, at most four K parts and one round of workgroups that fills at least
-// three quarters of the CUs (e.g. 4096 x 14336 at M = 5..16: 14.0 us against 17.0 us on the 32x32 tiled
-// kernel).  On smaller shapes the conversion of the activations in every workgroup and the
-// parts' hand-over cost more than the tiled kernel's whole call; with more parts or rounds the
-// two are level or the tiled kernel wins.
+// Where the resident kernel measured faster than the 32x32 tiled one, whatever is known about
+// the activations.  Up to 16 rows: K >= 544, at most four K parts and one round of workgroups that
+// fills at least three quarters of the CUs (4096 x 14336 at M = 5..16: 14.0 us against 17.0 us;
+// on smaller shapes the conversion in every workgroup and the parts' hand-over cost more than
+// the tiled kernel's whole call; with more parts or rounds the two are level or the tiled kernel
+// wins).  Beyond 32 rows: Q4 with f32 activations and K short enough for a single part
+// (128 x 1024 x 3072: 9.2 against 13.3 us, 256 x 576 x 1536: 8.9 against 13.3, 512 x 1024 x 3072:
+// 16.8 against 17.6); fp16 activations stay with the tiled kernel (512 x 1024 x 3072: 13.1
+// against 15.6 us) and so does Q8 (level or up to 1.2x slower here).
 bool tile_mfma_preferred(const LaunchArgs& x) {
   ResidentPlan rp;
-  if (!plan_resident(x, &rp) || rp.r != 1 || rp.parts > 4 || rp.nslices < 3) return false;
+  if (!use_resident(x, &rp)) return false;
+  if (x.m > 32) return x.w.fmt == MGN_FMT_Q4 && !x.a_is_f16 && rp.parts == 1;
+  if (x.m > 16 || rp.r != 1 || rp.parts > 4 || rp.nslices < 3) return false;
   const uint64_t wgs = (uint64_t)rp.parts * rp.colgroups;
   return wgs <= (uint64_t)x.num_cus && 4 * wgs >= 3 * (uint64_t)x.num_cus;
 }
 
 bool describe_tile_mfma(const LaunchArgs& x, mgn_plan_info* out) {
   ResidentPlan rp;
-  if (plan_resident(x, &rp)) {
+  if (use_resident(x, &rp)) {
     out->route = MGN_ROUTE_TILE_MFMA;
-    out->grid[0] = rp.parts, out->grid[1] = rp.colgroups, out->grid[2] = 1;
+    out->grid[0] = rp.parts, out->grid[1] = rp.colgroups, out->grid[2] = rp.rowgroups;
     out->threads = 512;
     out->lds_bytes = (uint32_t)rp.lds;
     out->waves_n = 8 * kSide * rp.q, out->k_splits = 1, out->k_parts = rp.parts, out->steps = rp.nsl;
@@ -1238,7 +1263,7 @@ bool describe_tile_mfma(const LaunchArgs& x, mgn_plan_info* out) {
 
 int launch_matmul_tile_mfma(ihipStream_t* s, const LaunchArgs& x) {
   ResidentPlan rp;
-  if (plan_resident(x, &rp)) {
+  if (use_resident(x, &rp)) {
     if (x.w.fmt == MGN_FMT_Q4)
       return x.a_is_f16 ? launch_resident_fa<MGN_FMT_Q4, false>(s, x, rp) : launch_resident_fa<MGN_FMT_Q4, true>(s, x, rp);
     return x.a_is_f16 ? launch_resident_fa<MGN_FMT_Q8, false>(s, x, rp) : launch_resident_fa<MGN_FMT_Q8, true>(s, x, rp);

@@ -80,9 +80,9 @@ def check_gemm(p, fmt, m, k, n, f16):
 
 def check_tile(p, fmt, m, k, n, f16):
     """MGN_ROUTE_TILE_MFMA: tiles of 16 columns, K in slices of 256 elements, `full_steps` row tiles of 16 rows
-    per workgroup.  quads_per_wave == 0: the form for M <= 32 that keeps the activation images in LDS (grid =
-    (K parts, column groups), 8 waves with one or two pairs of tiles each, parts of 4 slices, or of 2 with f32
-    activations beyond 16 rows); otherwise the general form (grid = (K parts, column groups, row groups),
+    per workgroup.  quads_per_wave == 0: the form that keeps the activation images in LDS (grid =
+    (K parts, column groups, row groups of 16 or 32 rows), 8 waves with one or two pairs of tiles each, parts of
+    4 slices, or of 2 with f32 activations in row groups of 32); otherwise the general form (grid = (K parts, column groups, row groups),
     `k_splits` waves per tile) in `quads_per_wave` launches over blocks of rows."""
     nslices, n_tiles = ceil_div(k, 256), ceil_div(n, 16)
     assert p.lds_bytes <= 160 * 1024 and p.threads <= 512
@@ -90,13 +90,16 @@ def check_tile(p, fmt, m, k, n, f16):
     assert p.grid[1] * p.waves_n >= n_tiles and (p.grid[1] - 1) * p.waves_n < n_tiles
     assert p.grid[0] == p.k_parts >= 1
     if p.quads_per_wave == 0:
-        assert m <= 32 and p.grid[2] == 1 and p.threads == 512 and rows >= m and p.full_steps == (1 if m <= 16 else 2)
-        assert p.steps == (2 if (not f16 and m > 16) else 4) and p.waves_n in (16, 32)
+        assert p.threads == 512 and p.full_steps in (1, 2)
+        if m > 32:  # beyond 32 rows only with few K parts and small partial tiles
+            assert p.k_parts <= 4 and p.workspace_bytes <= 8 << 20 and (fmt == Q4 or m >= 128)
+        assert p.grid[2] * rows >= m and (p.grid[2] - 1) * rows < m
+        assert p.steps == (2 if (not f16 and p.full_steps == 2) else 4) and p.waves_n in (16, 32)
         assert p.k_parts == ceil_div(nslices, p.steps)
-        partial = p.k_parts * rows * n * 4 if p.k_parts > 1 else 0
+        partial = p.k_parts * p.grid[2] * rows * n * 4 if p.k_parts > 1 else 0
         assert p.workspace_bytes == partial <= WORKSPACE
         if p.k_parts > 1:
-            assert p.grid[1] <= COUNTERS
+            assert p.grid[1] * p.grid[2] <= COUNTERS
     else:
         assert p.full_steps in (1, 2, 4) and p.k_splits in (1, 2, 4) and p.threads == 64 * p.k_splits * p.waves_n
         assert p.k_parts * p.steps * p.k_splits >= nslices
@@ -159,6 +162,12 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
         assert capi.matmul_plan(fmt, 16, 14336, 4096).route == TILE_MFMA
     big = capi.matmul_plan(Q4, 512, 14336, 4096)   # images of 512 rows x 14336 exceed the 16 MiB workspace: several launches
     assert big.route == TILE_MFMA and big.quads_per_wave > 1
+    # prefill with f32 activations (what the reference's Session hands over): row groups on the LDS-resident form,
+    # also on a context that was promised the fp16 range (it measured faster than the 32x32 kernel there)
+    for promised in (False, True):
+        p = capi.matmul_plan(Q4, 512, 1024, 3072, fp16_range=promised)
+        assert p.route == TILE_MFMA and p.quads_per_wave == 0 and p.k_parts == 1 and p.grid[2] == 32
+    assert capi.matmul_plan(Q4, 512, 1024, 3072, True).route == GEMM_MFMA  # fp16 activations: the 32x32 kernel
     for k, n in ((1024, 3072), (3072, 1024)):
         assert capi.matmul_plan(Q4, 512, k, n, True).route == GEMM_MFMA
     head = capi.matmul_plan(Q4, 1, 4096, 14336)
