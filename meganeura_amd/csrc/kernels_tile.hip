@@ -990,7 +990,9 @@ size_t resident_lds_bytes(int fmt, bool f32a, uint32_t r, uint32_t q) {
 
 // Row groups of 16 or 32 rows (32 only beyond 16 rows, and not for Q8: registers), Q = 1 or 2 pairs
 // of tiles per wave: the combination whose grid takes the fewest rounds over the CUs, weighted by
-// what a workgroup does (a fixed part for the conversion and the hand-over, its waves' steps).
+// what a workgroup does (a fixed part for the conversion and the hand-over, its waves' steps; row
+// groups of 32 share every unpacked B operand between two row tiles and win a tie: fp16
+// 512 x 1024 x 3072 11.9 us against 15.5 us in row groups of 16).
 bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
   if (x.m == 0 || x.w.k < 32) return false;
   const uint32_t bpc = x.w.k / 32;
@@ -1013,7 +1015,7 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
       const uint32_t colgroups = (n_tiles + per_wg - 1) / per_wg;
       if (colgroups > 65535 || (parts > 1 && (uint64_t)colgroups * rowgroups > x.n_counters)) continue;
       const uint64_t wgs = (uint64_t)parts * colgroups * rowgroups;
-      const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q * r * nsl / 4.0) + (parts > 1 ? 1.0 : 0.0);
+      const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q * r * nsl / 4.0) * (r == 2 ? 0.9 : 1.0) + (parts > 1 ? 1.0 : 0.0);
       if (best == 0 || cost < best) {
         best = cost;
         bp.r = r, bp.q = q, bp.nsl = nsl, bp.parts = parts, bp.colgroups = colgroups, bp.rowgroups = rowgroups;
@@ -1222,14 +1224,15 @@ bool tile_mfma_supported(const LaunchArgs& x) {
 // fills at least three quarters of the CUs (4096 x 14336 at M = 5..16: 14.0 us against 17.0 us;
 // on smaller shapes the conversion in every workgroup and the parts' hand-over cost more than
 // the tiled kernel's whole call; with more parts or rounds the two are level or the tiled kernel
-// wins).  Beyond 32 rows: Q4 with f32 activations and K short enough for a single part
-// (128 x 1024 x 3072: 9.2 against 13.3 us, 256 x 576 x 1536: 8.9 against 13.3, 512 x 1024 x 3072:
-// 16.8 against 17.6); fp16 activations stay with the tiled kernel (512 x 1024 x 3072: 13.1
-// against 15.6 us) and so does Q8 (level or up to 1.2x slower here).
+// wins).  Beyond 32 rows: Q4 with K short enough for a single part (f32 activations:
+// 128 x 1024 x 3072 9.2 against 13.3 us, 256 x 576 x 1536 8.9 against 13.3, 512 x 1024 x 3072 16.8
+// against 17.6; fp16 activations, in row groups of 32: 512 x 1024 x 3072 11.9 against 13.1 us,
+// 128 x 1024 x 3072 8.5 against 9.8); with K parts the tiled kernel is ahead (fp16 512 x 3072 x 1024:
+// 15.1 against 16.8 us) and Q8 is level or up to 1.4x slower on this kernel.
 bool tile_mfma_preferred(const LaunchArgs& x) {
   ResidentPlan rp;
   if (!use_resident(x, &rp)) return false;
-  if (x.m > 32) return x.w.fmt == MGN_FMT_Q4 && !x.a_is_f16 && rp.parts == 1;
+  if (x.m > 32) return x.w.fmt == MGN_FMT_Q4 && rp.parts == 1;
   if (x.m > 16 || rp.r != 1 || rp.parts > 4 || rp.nslices < 3) return false;
   const uint64_t wgs = (uint64_t)rp.parts * rp.colgroups;
   return wgs <= (uint64_t)x.num_cus && 4 * wgs >= 3 * (uint64_t)x.num_cus;

@@ -167,9 +167,10 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
     for promised in (False, True):
         p = capi.matmul_plan(Q4, 512, 1024, 3072, fp16_range=promised)
         assert p.route == TILE_MFMA and p.quads_per_wave == 0 and p.k_parts == 1 and p.grid[2] == 32
-    assert capi.matmul_plan(Q4, 512, 1024, 3072, True).route == GEMM_MFMA  # fp16 activations: the 32x32 kernel
-    for k, n in ((1024, 3072), (3072, 1024)):
-        assert capi.matmul_plan(Q4, 512, k, n, True).route == GEMM_MFMA
+    up = capi.matmul_plan(Q4, 512, 1024, 3072, True)  # fp16 activations, C4 up-projection: row groups of 32
+    assert up.route == TILE_MFMA and up.quads_per_wave == 0 and up.full_steps == 2 and list(up.grid) == [1, 12, 16]
+    assert capi.matmul_plan(Q4, 512, 3072, 1024, True).route == GEMM_MFMA   # K parts: the 32x32 kernel
+    assert capi.matmul_plan(Q8, 512, 1024, 3072, True).route == GEMM_MFMA
     head = capi.matmul_plan(Q4, 1, 4096, 14336)
     assert (head.grid[0], head.threads, head.steps, head.k_splits, head.full_steps) == (256, 896, 8, 1, 1)
     tall = capi.matmul_plan(Q4, 4, 14336, 4096)
