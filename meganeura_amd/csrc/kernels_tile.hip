@@ -126,18 +126,37 @@ __device__ __forceinline__ uint32_t image_slot(uint32_t row, uint32_t g, uint32_
 }
 constexpr uint32_t image_units(bool f32a) { return kSliceBlocks * (f32a ? 2u : 1u) * 64u + 64u + 16u; }
 
+// Eight consecutive activations of a row as they come from memory: 8 f32 words or 4 words of fp16 pairs.
+template <bool F32A>
+struct TaskWords {
+  uint32_t w[F32A ? 8 : 4];
+};
+
+template <bool F32A>
+__device__ __forceinline__ void load_task(const void* __restrict__ a, size_t elem, TaskWords<F32A>& x) {
+  if constexpr (F32A) {
+    const uint4* src = (const uint4*)((const float*)a + elem);
+    const uint4 v0 = src[0], v1 = src[1];
+    x.w[0] = v0.x, x.w[1] = v0.y, x.w[2] = v0.z, x.w[3] = v0.w, x.w[4] = v1.x, x.w[5] = v1.y, x.w[6] = v1.z, x.w[7] = v1.w;
+  } else {
+    const uint4 v = *(const uint4*)((const _Float16*)a + elem);
+    x.w[0] = v.x, x.w[1] = v.y, x.w[2] = v.z, x.w[3] = v.w;
+  }
+}
+
 // One task of the conversion: half-wave lane l = kb * 4 + g turns the 8 activations k0 .. k0 + 7
 // (k0 = 256 slice + 32 kb + 8 g) of row `row` into its piece of the image `img` of that (row tile,
 // slice); r = row % 16.  All 32 lanes of the half-wave (one row of one slice) must call it together.
 template <int FMT, bool F32A>
-__device__ __forceinline__ void convert_task(const float (&xin)[8], bool ok, uint4* __restrict__ img, uint32_t r, uint32_t l) {
+__device__ __forceinline__ void convert_task(const TaskWords<F32A>& xin, bool ok, uint4* __restrict__ img, uint32_t r, uint32_t l) {
   constexpr uint32_t HL = F32A ? 2 : 1;
   const uint32_t kb = l >> 2, g = l & 3;
-  float x[8];
-#pragma unroll
-  for (int e = 0; e < 8; e++) x[e] = ok ? xin[e] : 0.0f;
-  float inv = 1.0f;
+  const uint32_t alane = image_slot(r, g, kb & 1);
+  float s, inv = 1.0f;
   if constexpr (F32A) {
+    float x[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) x[e] = ok ? __builtin_bit_cast(float, xin.w[e]) : 0.0f;
     // NaN never wins fmaxf; an infinity does and switches scaling off
     float am = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))),
                      fmaxf(fmaxf(fabsf(x[4]), fabsf(x[5])), fmaxf(fabsf(x[6]), fabsf(x[7]))));
@@ -146,18 +165,15 @@ __device__ __forceinline__ void convert_task(const float (&xin)[8], bool ok, uin
     const float scale = slice_scale<kSplit ? 7 : 11>(am, &inv);
 #pragma unroll
     for (int e = 0; e < 8; e++) x[e] *= (kSplit && e % 2 == 0) ? scale * 16.0f : scale;
-  }
-  float p[8];
-  if constexpr (FMT == MGN_FMT_Q4) {
-    p[0] = x[0], p[1] = x[4], p[2] = x[1], p[3] = x[5], p[4] = x[2], p[5] = x[6], p[6] = x[3], p[7] = x[7];
-  } else {
+    float p[8];
+    if constexpr (FMT == MGN_FMT_Q4) {
+      p[0] = x[0], p[1] = x[4], p[2] = x[1], p[3] = x[5], p[4] = x[2], p[5] = x[6], p[6] = x[3], p[7] = x[7];
+    } else {
 #pragma unroll
-    for (int e = 0; e < 8; e++) p[e] = x[e];
-  }
-  const uint32_t alane = image_slot(r, g, kb & 1);
-  const uint32_t hp[4] = {pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7])};
-  img[(kb * HL) * 64 + alane] = make_uint4(hp[0], hp[1], hp[2], hp[3]);  // fp16 inputs convert back exactly
-  if constexpr (F32A) {
+      for (int e = 0; e < 8; e++) p[e] = x[e];
+    }
+    const uint32_t hp[4] = {pack_rtz(p[0], p[1]), pack_rtz(p[2], p[3]), pack_rtz(p[4], p[5]), pack_rtz(p[6], p[7])};
+    img[(kb * HL) * 64 + alane] = make_uint4(hp[0], hp[1], hp[2], hp[3]);
     float res[8];
 #pragma unroll
     for (int e = 0; e < 4; e++) {
@@ -166,10 +182,23 @@ __device__ __forceinline__ void convert_task(const float (&xin)[8], bool ok, uin
     }
     img[(kb * HL + 1) * 64 + alane] =
         make_uint4(pack_rtz(res[0], res[1]), pack_rtz(res[2], res[3]), pack_rtz(res[4], res[5]), pack_rtz(res[6], res[7]));
+    if constexpr (FMT == MGN_FMT_Q4) s = ((x[0] + x[2]) + (x[4] + x[6])) * 0.0625f + ((x[1] + x[3]) + (x[5] + x[7]));
+    else s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+  } else {
+    // fp16 activations are operands as they are: only their order changes (Q4 pairs k with k + 4)
+    const uint32_t v[4] = {ok ? xin.w[0] : 0u, ok ? xin.w[1] : 0u, ok ? xin.w[2] : 0u, ok ? xin.w[3] : 0u};
+    if constexpr (FMT == MGN_FMT_Q4) {
+      img[kb * 64 + alane] = make_uint4(__builtin_amdgcn_perm(v[2], v[0], 0x05040100u), __builtin_amdgcn_perm(v[2], v[0], 0x07060302u),
+                                        __builtin_amdgcn_perm(v[3], v[1], 0x05040100u), __builtin_amdgcn_perm(v[3], v[1], 0x07060302u));
+    } else {
+      img[kb * 64 + alane] = make_uint4(v[0], v[1], v[2], v[3]);
+    }
+    const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v[0]), ones, 0.0f, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v[1]), ones, s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v[2]), ones, s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v[3]), ones, s, false);
   }
-  float s;
-  if constexpr (F32A && FMT == MGN_FMT_Q4) s = ((x[0] + x[2]) + (x[4] + x[6])) * 0.0625f + ((x[1] + x[3]) + (x[5] + x[7]));
-  else s = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
   s += dpp_move<kDppQuadXor1>(s);
   s += dpp_move<kDppQuadXor2>(s);
   uint32_t* const extra = (uint32_t*)(img + kSliceBlocks * HL * 64);
@@ -184,20 +213,6 @@ __device__ __forceinline__ void convert_task(const float (&xin)[8], bool ok, uin
   if (l == 0) ((float*)extra)[64 * 4 + r] = inv * (FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f);
 }
 
-// eight consecutive activations of a row, as float
-template <bool F32A>
-__device__ __forceinline__ void load_task(const void* __restrict__ a, size_t elem, float (&x)[8]) {
-  if constexpr (F32A) {
-    const float4* src = (const float4*)((const float*)a + elem);
-    const float4 v0 = src[0], v1 = src[1];
-    x[0] = v0.x, x[1] = v0.y, x[2] = v0.z, x[3] = v0.w, x[4] = v1.x, x[5] = v1.y, x[6] = v1.z, x[7] = v1.w;
-  } else {
-    const uint4 v = *(const uint4*)((const _Float16*)a + elem);
-    x[0] = half_lo(v.x), x[1] = half_hi(v.x), x[2] = half_lo(v.y), x[3] = half_hi(v.y);
-    x[4] = half_lo(v.z), x[5] = half_hi(v.z), x[6] = half_lo(v.w), x[7] = half_hi(v.w);
-  }
-}
-
 // grid.x = row tiles * slices; 512 threads: half-wave r (0..15) converts row r of the tile,
 // lane l = kb * 4 + g of it the 8 elements k = 32 kb + 8 g .. + 7 of the slice.
 template <int FMT, bool F32A>
@@ -208,7 +223,7 @@ __global__ __launch_bounds__(512) void image_kernel(const void* __restrict__ a, 
   const uint32_t r = threadIdx.x >> 5, l = threadIdx.x & 31;
   const uint32_t row = rt * 16 + r, k0 = sl * 256 + l * 8;
   const bool ok = row < m && k0 < k;  // K is a multiple of 32: a task lies inside or outside as a whole
-  float x[8];
+  TaskWords<F32A> x;
   load_task<F32A>(a, ok ? (size_t)row * a_stride + k0 : (size_t)0, x);
   convert_task<FMT, F32A>(x, ok, image + ((size_t)rt * nslices + sl) * UNITS, r, l);
 }
@@ -752,7 +767,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   // ---- the part's activations: loads first, so that nothing queues in front of them ----
   // Task (s, rr): half-wave r converts row 16 rr + r of slice sl0 + s.
   const uint32_t cr = tid >> 5, cl = tid & 31;
-  float xin[NT][8];
+  TaskWords<F32A> xin[NT];
   bool xok[NT];
 #pragma unroll
   for (int t = 0; t < NT; t++) {
