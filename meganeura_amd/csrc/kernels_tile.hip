@@ -1017,8 +1017,8 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
   double best = 0;
   ResidentPlan bp{};
   for (uint32_t r = 1; r <= 2; r++) {
-    if (r == 2 && (x.m <= 16 || x.w.fmt == MGN_FMT_Q8)) continue;
-    if (r == 1 && x.m > 16 && x.m <= 32 && x.w.fmt == MGN_FMT_Q4) continue;  // one row group of 32 instead of two of 16
+    if (r == 2 && x.m <= 16) continue;
+    if (r == 1 && x.m > 16 && x.m <= 32) continue;  // one row group of 32 instead of two of 16
     const uint32_t nsl = resident_slices(f32a, r);
     const uint32_t parts = (nslices + nsl - 1) / nsl;
     const uint32_t rowgroups = (x.m + 16 * r - 1) / (16 * r);
@@ -1059,9 +1059,7 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
 
 template <int FMT, bool F32A>
 int launch_resident_fa(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& p) {
-  if constexpr (FMT == MGN_FMT_Q4) {
-    if (p.r == 2) return launch_resident_q<FMT, F32A, 2, 1>(s, x, p);
-  }
+  if (p.r == 2) return launch_resident_q<FMT, F32A, 2, 1>(s, x, p);
   return p.q == 1 ? launch_resident_q<FMT, F32A, 1, 1>(s, x, p) : launch_resident_q<FMT, F32A, 1, 2>(s, x, p);
 }
 
