@@ -34,8 +34,8 @@
 //     grid = (K parts, column groups, row groups): a workgroup owns wnc column tiles of 16
 //     columns, R row tiles of 16 rows and a range of K slices; ksc waves share a column tile and
 //     take the slices of a phase side by side (their sums meet in LDS, in a fixed order).
-//   tile_resident_kernel (M <= 32): every workgroup converts its own K part and keeps the
-//     images in LDS; no second launch, no image traffic (see there).
+//   tile_resident_kernel (row groups of 16 or 32 rows): every workgroup converts its own rows
+//     of its K part and keeps the images in LDS; no second launch, no image traffic (see there).
 // With too few tiles to fill the chip K is also cut into parts for different workgroups, whose
 // partial tiles the last one to finish adds in part order (deterministic).
 #include <algorithm>
@@ -574,9 +574,9 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
   }
 }
 
-// ---- few activation rows (M <= 32): the images stay in LDS ----
-// grid = (K parts, column groups); 512 threads.  A workgroup converts the activations of its K
-// part (all M rows, NSL slices of 256 elements) into images in LDS itself, once; after one barrier
+// ---- the images stay in LDS ----
+// grid = (K parts, column groups, row groups); 512 threads.  A workgroup converts the activations
+// of its K part (its 16 or 32 rows, NSL slices of 256 elements) into images in LDS itself, once; after one barrier
 // every wave walks its own Q pairs of column tiles down the part's slices, pair after pair, with
 // whole slices of both tiles in flight in registers and no further synchronisation.  The two
 // tiles of a pair are multiplied side by side, so every A operand read from LDS serves both (LDS
@@ -1003,7 +1003,7 @@ size_t resident_lds_bytes(int fmt, bool f32a, uint32_t r, uint32_t q) {
   return (size_t)nsl * r * image_units(f32a) * 16 + (size_t)8 * q * 32 * meta_stride(fmt, nsl);
 }
 
-// Row groups of 16 or 32 rows (32 only beyond 16 rows, and not for Q8: registers), Q = 1 or 2 pairs
+// Row groups of 16 or 32 rows (32 only beyond 16 rows, and then with one pair per wave: registers), Q = 1 or 2 pairs
 // of tiles per wave: the combination whose grid takes the fewest rounds over the CUs, weighted by
 // what a workgroup does (a fixed part for the conversion and the hand-over, its waves' steps; row
 // groups of 32 share every unpacked B operand between two row tiles and win a tie: fp16
