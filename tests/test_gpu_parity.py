@@ -182,7 +182,8 @@ def test_small_m_fp16_activations(ctx, orc, fmt, m, k, n):
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
-@pytest.mark.parametrize("m,k,n", [(5, 64, 70), (6, 1024, 2048), (16, 576, 130), (17, 256, 64), (64, 128, 96), (130, 96, 67)])
+@pytest.mark.parametrize("m,k,n", [(5, 64, 70), (6, 1024, 2048), (16, 576, 130), (17, 256, 64), (64, 128, 96), (130, 96, 67),
+                                   (70, 2048, 200), (40, 4128, 48), (33, 1056, 530)])  # row groups with K parts, ragged K
 def test_larger_m(ctx, orc, fmt, m, k, n):
     x = synth.normal(11 + m + k + n, m * k).reshape(m, k)
     w = synth.normal(12 + m + k + n, k * n, 0.02).reshape(k, n)
