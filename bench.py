@@ -86,7 +86,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c4_q4_prefill_down_512x3072x1024": 25.5e6,
     "c5_q4_m1_14336x4096": 37.4e6,
     "c5_q4_m4_4096x14336": 37.8e6,
-    "c5_q8_m16_4096x14336": 77.4e6,
+    "c5_q8_m16_4096x14336": 75.2e6,
 }
 
 

@@ -582,13 +582,20 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
 // tiles of a pair are multiplied side by side, so every A operand read from LDS serves both (LDS
 // bandwidth is what limits a wave that reads each operand for one tile only).
 //
-// The quants reach the B operand's lane order without LDS: lane (c, g) loads 16 bytes of
-// column c, and the four lanes of a column exchange dwords with the row swap instructions
-// (v_permlane32_swap, v_permlane16_swap: rows of 16 lanes).
+// The quants reach the B operand's lane order in one of two ways.
+// Through LDS (PARK, whenever a strip per wave fits beside the images): the wave loads whole
+// cache lines, 8 (Q8: 16) lanes per column, parks them in its own strip with a padded column
+// stride and every lane reads its operands back block by block.
+// Without LDS: lane (c, g) loads 16 bytes of column c, and the four lanes of a column exchange
+// dwords with the row swap instructions (v_permlane32_swap, v_permlane16_swap: rows of 16 lanes).
 //   Q4: lane (c, g) loads block g (then 4 + g) of the slice; a 4x4 transpose over (row, dword)
 //       leaves dword g of blocks 0..3 (4..7): the block's elements 8g..8g+7.
 //   Q8: load j, lane (c, g): half g / 2 of block 2j + g % 2; swapping (x, z) and (y, w) between
 //       the odd and even rows leaves dwords 2g, 2g+1 of block 2j in (x, y), of 2j+1 in (z, w).
+// That form touches half a cache line per column and instruction, twice as many lines per byte,
+// and the CU's memory pipeline charges per line: M = 16 on 4096 x 14336 takes 14.0 us with it and
+// 13.3 us parked (Q8: 18.9 and 16.6 us).  It remains for the plans whose LDS is full (two pairs
+// of tiles per wave with f32 activations).
 // The scale words are wanted by all four lanes of a column; loading them per lane would ask the
 // memory pipeline for every word four times.  Each wave instead loads the words of all its
 // columns and slices once, in whole cache lines, parks them in its own LDS strip and reads a
@@ -628,14 +635,17 @@ __device__ __forceinline__ void swap_row_pairs(u32x4_t& v) {
 // One slice (8 K blocks) of kSide column tiles against R row tiles: the tiles' quants in B operand
 // order (q, see above), their 8 scale words (mw), the slice's image at ib (row tile 0, row tiles
 // rstride bytes apart).
-template <int FMT, bool F32A, int R>
-__device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == MGN_FMT_Q4 ? 2 : 4], const uint32_t (&mw)[kSide][8],
-                                               const uint8_t* ib, uint32_t rstride, uint32_t g, uint32_t lane,
-                                               floatx4 (&acc)[kSide][R]) {
+// PARK: the quants are not in q but parked in LDS, column by column (park_stride apart, tile u
+// 16 columns on): park_rd is this lane's piece of block 0 of its column of tile 0.
+template <int FMT, bool F32A, int R, bool PARK>
+__device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == MGN_FMT_Q4 ? 2 : 4], const uint8_t* park_rd,
+                                               const uint32_t (&mw)[kSide][8], const uint8_t* ib, uint32_t rstride, uint32_t g,
+                                               uint32_t lane, floatx4 (&acc)[kSide][R]) {
   constexpr uint32_t HL = F32A ? 2 : 1;
   constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;  // 2^20, 2^24
   const uint32_t slot_off[2] = {image_slot(lane & 15, g, 0) * 16, image_slot(lane & 15, g, 1) * 16};
   u32x4_t aop[3][R][HL];
+  uint32_t bq[3][kSide][FMT == MGN_FMT_Q4 ? 1 : 2];  // PARK: the lane's quants of a block
   floatx4 dsum[2][kSide][R];
   floatx4 P[kSide][R];
 #pragma unroll
@@ -647,12 +657,27 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
     for (int r = 0; r < R; r++)
 #pragma unroll
       for (uint32_t h = 0; h < HL; h++) aop[s % 3][r][h] = *(const u32x4_t*)(ib + slot_off[s & 1] + r * rstride + (s * HL + h) * 64 * 16);
+    if constexpr (PARK) {
+#pragma unroll
+      for (int u = 0; u < kSide; u++) {
+        const uint8_t* src = park_rd + u * 16 * park_stride(FMT) + s * (FMT == MGN_FMT_Q4 ? 16 : 32);
+        if constexpr (FMT == MGN_FMT_Q4) {
+          bq[s % 3][u][0] = *(const uint32_t*)src;
+        } else {
+          const uint2 v = *(const uint2*)src;
+          bq[s % 3][u][0] = v.x, bq[s % 3][u][1] = v.y;
+        }
+      }
+    }
   };
   auto mfmas = [&](int s) {
 #pragma unroll
     for (int u = 0; u < kSide; u++) {
       half8 bop;
-      if constexpr (FMT == MGN_FMT_Q4) {
+      if constexpr (PARK) {
+        if constexpr (FMT == MGN_FMT_Q4) bop = nibbles_to_operand<F32A>(bq[s % 3][u][0]);
+        else bop = bytes_to_operand(bq[s % 3][u][0], bq[s % 3][u][1]);
+      } else if constexpr (FMT == MGN_FMT_Q4) {
         bop = nibbles_to_operand<F32A>(q[u][s >> 2][s & 3]);
       } else {
         bop = (s & 1) ? bytes_to_operand(q[u][s >> 1].z, q[u][s >> 1].w) : bytes_to_operand(q[u][s >> 1].x, q[u][s >> 1].y);
@@ -733,7 +758,7 @@ constexpr int resident_slices(bool f32a, int r) { return f32a && r == 2 ? 2 : 4;
 // a tile fall into different LDS banks.
 __host__ __device__ constexpr uint32_t meta_stride(int fmt, uint32_t nsl) { return nsl * kSliceBlocks * (fmt == MGN_FMT_Q4 ? 4 : 2) + 16; }
 
-template <int FMT, bool F32A, int R, int Q>
+template <int FMT, bool F32A, int R, int Q, bool PARK>
 __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restrict__ a, const void* __restrict__ meta_arg,
                                                              const void* __restrict__ quants_arg, uint32_t m, uint32_t kdim,
                                                              uint32_t n, uint32_t parts, uint32_t nslices, TileTail tail) {
@@ -763,6 +788,9 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   uint4* const img = lds4;                     // [NSL][R][UNITS]
   // this wave's scale words: [Q pairs x 32 columns][mstride bytes]
   uint8_t* const wmeta = (uint8_t*)(lds4 + NSL * R * UNITS) + wave * (Q * 32 * mstride);
+  // PARK: this wave's strip for the quants of the step at hand, kSide x 16 columns
+  constexpr int kStride = park_stride(FMT);
+  uint8_t* const wpark = (uint8_t*)(lds4 + NSL * R * UNITS) + 8 * (Q * 32 * mstride) + wave * (kSide * 16 * kStride);
 
   // ---- the part's activations: loads first, so that nothing queues in front of them ----
   // Task (s, rr): half-wave r converts row 16 rr + r of slice sl0 + s.
@@ -801,19 +829,29 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   // Slices past the end of K (last part) and columns past N read the pad behind the weights or
   // a neighbour's data; their products are dropped.
   u32x4_t wq[SLOTS][kSide][NLQ];
+  constexpr uint32_t LPC = QB / 2, CPL = 64 / LPC;  // PARK: lanes per column, columns per load
   const uint32_t lane_part = FMT == MGN_FMT_Q4 ? g * 16 : (g & 1) * 32 + (g >> 1) * 16;
-  uint32_t q_off[Q][kSide];
+  uint32_t q_off[Q][kSide][PARK ? NLQ : 1];
 #pragma unroll
   for (int p = 0; p < Q; p++)
 #pragma unroll
-    for (int u = 0; u < kSide; u++) q_off[p][u] = min(((pair0 + p) * kSide + u) * 16 + c, n - 1) * bpc * QB + lane_part;
+    for (int u = 0; u < kSide; u++) {
+      if constexpr (PARK) {
+#pragma unroll
+        for (int j = 0; j < NLQ; j++)
+          q_off[p][u][j] = min(((pair0 + p) * kSide + u) * 16 + CPL * j + lane / LPC, n - 1) * bpc * QB + (lane % LPC) * 16;
+      } else {
+        q_off[p][u][0] = min(((pair0 + p) * kSide + u) * 16 + c, n - 1) * bpc * QB + lane_part;
+      }
+    }
   auto fetch = [&](int f) {  // step f into slot f % SLOTS
     const uint8_t* const qb = (const uint8_t*)quants_arg + (size_t)((sl0 + f % NSL) * kSliceBlocks) * QB;
 #pragma unroll
     for (int u = 0; u < kSide; u++)
 #pragma unroll
       for (int j = 0; j < NLQ; j++)
-        wq[f % SLOTS][u][j] = __builtin_nontemporal_load((const u32x4_t*)(qb + q_off[f / NSL][u] + 64 * j));
+        wq[f % SLOTS][u][j] = __builtin_nontemporal_load(
+            (const u32x4_t*)(qb + (PARK ? q_off[f / NSL][u][PARK ? j : 0] : q_off[f / NSL][u][0] + 64 * j)));
   };
   // ---- activations -> images in LDS; scale words -> LDS ----
   // The first slices of quants are requested between the conversion tasks, not before them: a
@@ -863,13 +901,20 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
         const u32x4_t m0 = *(const u32x4_t*)ms, m1 = *(const u32x4_t*)(ms + 16);
         mw[u][0] = m0.x, mw[u][1] = m0.y, mw[u][2] = m0.z, mw[u][3] = m0.w;
         mw[u][4] = m1.x, mw[u][5] = m1.y, mw[u][6] = m1.z, mw[u][7] = m1.w;
-        transpose_rows(wq[slot][u][0]);
-        transpose_rows(wq[slot][u][1]);
       } else {
         const u32x4_t m0 = *(const u32x4_t*)ms;
         const uint32_t v[4] = {m0.x, m0.y, m0.z, m0.w};
 #pragma unroll
         for (int e = 0; e < 4; e++) mw[u][2 * e] = v[e] & 0xFFFFu, mw[u][2 * e + 1] = v[e] >> 16;
+      }
+      if constexpr (PARK) {
+#pragma unroll
+        for (int j = 0; j < NLQ; j++)
+          *(u32x4_t*)(wpark + (u * 16 + CPL * j + lane / LPC) * kStride + (lane % LPC) * 16) = wq[slot][u][j];
+      } else if constexpr (FMT == MGN_FMT_Q4) {
+        transpose_rows(wq[slot][u][0]);
+        transpose_rows(wq[slot][u][1]);
+      } else {
 #pragma unroll
         for (int j = 0; j < NLQ; j++) swap_row_pairs(wq[slot][u][j]);
       }
@@ -884,7 +929,8 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
 #pragma unroll
           for (int e = 0; e < 8; e++) mw[u][e] = kb0 + e < bpc ? mw[u][e] : 0u;
       }
-      slice_mac_side<FMT, F32A, R>(wq[slot], mw, (const uint8_t*)(img + ws * R * UNITS), UNITS * 16, g, lane, res[wp]);
+      slice_mac_side<FMT, F32A, R, PARK>(wq[slot], wpark + c * kStride + g * (QB / 4), mw, (const uint8_t*)(img + ws * R * UNITS),
+                                         UNITS * 16, g, lane, res[wp]);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -994,13 +1040,15 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
 
 struct ResidentPlan {
   uint32_t r, q, nsl, parts, colgroups, rowgroups, nslices;
+  bool park;  // quants through a wave-private LDS strip (if there is room) instead of row swaps
   size_t lds, partial_bytes;
   double cost;
 };
 
-size_t resident_lds_bytes(int fmt, bool f32a, uint32_t r, uint32_t q) {
+size_t resident_lds_bytes(int fmt, bool f32a, uint32_t r, uint32_t q, bool park) {
   const uint32_t nsl = resident_slices(f32a, r);
-  return (size_t)nsl * r * image_units(f32a) * 16 + (size_t)8 * q * 32 * meta_stride(fmt, nsl);
+  return (size_t)nsl * r * image_units(f32a) * 16 + (size_t)8 * q * 32 * meta_stride(fmt, nsl) +
+         (park ? (size_t)8 * kSide * 16 * park_stride(fmt) : 0);
 }
 
 // Row groups of 16 or 32 rows (32 only beyond 16 rows, and then with one pair per wave: registers), Q = 1 or 2 pairs
@@ -1035,7 +1083,8 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
         best = cost;
         bp.r = r, bp.q = q, bp.nsl = nsl, bp.parts = parts, bp.colgroups = colgroups, bp.rowgroups = rowgroups;
         bp.nslices = nslices, bp.partial_bytes = partial, bp.cost = cost;
-        bp.lds = resident_lds_bytes(x.w.fmt, f32a, r, q);
+        bp.park = resident_lds_bytes(x.w.fmt, f32a, r, q, true) <= 160 * 1024;
+        bp.lds = resident_lds_bytes(x.w.fmt, f32a, r, q, bp.park);
       }
     }
   }
@@ -1044,9 +1093,9 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
   return true;
 }
 
-template <int FMT, bool F32A, int R, int Q>
+template <int FMT, bool F32A, int R, int Q, bool PARK>
 int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& p) {
-  auto kern = tile_resident_kernel<FMT, F32A, R, Q>;
+  auto kern = tile_resident_kernel<FMT, F32A, R, Q, PARK>;
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
@@ -1059,8 +1108,11 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
 
 template <int FMT, bool F32A>
 int launch_resident_fa(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& p) {
-  if (p.r == 2) return launch_resident_q<FMT, F32A, 2, 1>(s, x, p);
-  return p.q == 1 ? launch_resident_q<FMT, F32A, 1, 1>(s, x, p) : launch_resident_q<FMT, F32A, 1, 2>(s, x, p);
+  if (p.r == 2)
+    return p.park ? launch_resident_q<FMT, F32A, 2, 1, true>(s, x, p) : launch_resident_q<FMT, F32A, 2, 1, false>(s, x, p);
+  if (p.q == 1)
+    return p.park ? launch_resident_q<FMT, F32A, 1, 1, true>(s, x, p) : launch_resident_q<FMT, F32A, 1, 1, false>(s, x, p);
+  return p.park ? launch_resident_q<FMT, F32A, 1, 2, true>(s, x, p) : launch_resident_q<FMT, F32A, 1, 2, false>(s, x, p);
 }
 
 struct TilePlan {
