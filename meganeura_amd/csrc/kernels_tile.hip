@@ -751,7 +751,8 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
   }
 }
 
-// Slices of a part: what fits in LDS beside the waves' scale words.
+// Slices of a part: what fits in LDS beside the waves' scale words (f32 activations in row groups
+// of 16, fp16 activations in row groups of 16 or 32).
 constexpr int resident_slices(bool f32a, int r) { return f32a && r == 2 ? 2 : 4; }
 
 // Bytes of one column's scale words for the nsl slices of a part, padded so that the 16 columns of
@@ -1065,8 +1066,11 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
   double best = 0;
   ResidentPlan bp{};
   for (uint32_t r = 1; r <= 2; r++) {
-    if (r == 2 && x.m <= 16) continue;
-    if (r == 1 && x.m > 16 && x.m <= 32) continue;  // one row group of 32 instead of two of 16
+    // Row groups of 32 are for fp16 activations: with f32 only two slices of 32 rows fit in LDS, K falls
+    // into twice as many parts, and two row groups of 16 are faster throughout (M = 32 on 4096 x 14336:
+    // 22.7 against 33.0 us, 576 x 576: 8.1 against 11.6 us)
+    if (r == 2 && (x.m <= 16 || f32a)) continue;
+    if (r == 1 && !f32a && x.m > 16 && x.m <= 32) continue;  // fp16: one row group of 32 instead of two of 16
     const uint32_t nsl = resident_slices(f32a, r);
     const uint32_t parts = (nslices + nsl - 1) / nsl;
     const uint32_t rowgroups = (x.m + 16 * r - 1) / (16 * r);
@@ -1108,8 +1112,11 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
 
 template <int FMT, bool F32A>
 int launch_resident_fa(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& p) {
-  if (p.r == 2)
-    return p.park ? launch_resident_q<FMT, F32A, 2, 1, true>(s, x, p) : launch_resident_q<FMT, F32A, 2, 1, false>(s, x, p);
+  if constexpr (!F32A) {
+    if (p.r == 2)
+      return p.park ? launch_resident_q<FMT, F32A, 2, 1, true>(s, x, p) : launch_resident_q<FMT, F32A, 2, 1, false>(s, x, p);
+  }
+  if (p.r != 1) return (int)hipErrorInvalidValue;
   if (p.q == 1)
     return p.park ? launch_resident_q<FMT, F32A, 1, 1, true>(s, x, p) : launch_resident_q<FMT, F32A, 1, 1, false>(s, x, p);
   return p.park ? launch_resident_q<FMT, F32A, 1, 2, true>(s, x, p) : launch_resident_q<FMT, F32A, 1, 2, false>(s, x, p);
@@ -1289,7 +1296,13 @@ bool tile_mfma_supported(const LaunchArgs& x) {
 // fills at least three quarters of the CUs (4096 x 14336 at M = 5..16: 14.0 us against 17.0 us;
 // on smaller shapes the conversion in every workgroup and the parts' hand-over cost more than
 // the tiled kernel's whole call; with more parts or rounds the two are level or the tiled kernel
-// wins).  Beyond 32 rows: Q4 with K short enough for a single part (f32 activations:
+// wins).  17 to 32 rows of f32 activations, where the tiled kernel runs twice the MFMAs: whenever
+// the two row groups' workgroups fit one round (576 x 576: 8.1 against 11.7 us, 4096 x 4096: 12.5
+// against 16.5, 14336 x 1536: 17.6 against 23.2; with more workgroups the weights' second pass
+// costs more: 576 x 49152 16.5 against 15.2, 14336 x 4096 29.4 against 27.1, and so do many K
+// parts that fill the chip: 14336 x 4096 at two pairs per wave 28.6 against 26.9; Q8 with two pairs
+// of tiles per wave has no room to park its quants and loses too: 4096 x 14336 31.3 against
+// 28.0).  Beyond 32 rows: Q4 with K short enough for a single part (f32 activations:
 // 128 x 1024 x 3072 9.2 against 13.3 us, 256 x 576 x 1536 8.9 against 13.3, 512 x 1024 x 3072 16.8
 // against 17.6; fp16 activations, in row groups of 32: 512 x 1024 x 3072 11.9 against 13.1 us,
 // 128 x 1024 x 3072 8.5 against 9.8); with K parts the tiled kernel is ahead (fp16 512 x 3072 x 1024:
@@ -1298,8 +1311,11 @@ bool tile_mfma_preferred(const LaunchArgs& x) {
   ResidentPlan rp;
   if (!use_resident(x, &rp)) return false;
   if (x.m > 32) return x.w.fmt == MGN_FMT_Q4 && rp.parts == 1;
-  if (x.m > 16 || rp.r != 1 || rp.parts > 4 || rp.nslices < 3) return false;
-  const uint64_t wgs = (uint64_t)rp.parts * rp.colgroups;
+  const uint64_t wgs = (uint64_t)rp.parts * rp.colgroups * rp.rowgroups;
+  if (x.m > 16)
+    return !x.a_is_f16 && wgs <= (uint64_t)x.num_cus && (x.w.fmt == MGN_FMT_Q4 || rp.q == 1) &&
+           (rp.parts <= 4 || 2 * wgs <= (uint64_t)x.num_cus);
+  if (rp.r != 1 || rp.parts > 4 || rp.nslices < 3) return false;
   return wgs <= (uint64_t)x.num_cus && 4 * wgs >= 3 * (uint64_t)x.num_cus;
 }
 

@@ -82,7 +82,7 @@ def check_tile(p, fmt, m, k, n, f16):
     """MGN_ROUTE_TILE_MFMA: tiles of 16 columns, K in slices of 256 elements, `full_steps` row tiles of 16 rows
     per workgroup.  quads_per_wave == 0: the form that keeps the activation images in LDS (grid =
     (K parts, column groups, row groups of 16 or 32 rows), 8 waves with one or two pairs of tiles each, parts of
-    4 slices, or of 2 with f32 activations in row groups of 32); otherwise the general form (grid = (K parts, column groups, row groups),
+    4 slices; row groups of 32 only with fp16 activations); otherwise the general form (grid = (K parts, column groups, row groups),
     `k_splits` waves per tile) in `quads_per_wave` launches over blocks of rows."""
     nslices, n_tiles = ceil_div(k, 256), ceil_div(n, 16)
     assert p.lds_bytes <= 160 * 1024 and p.threads <= 512
@@ -94,7 +94,8 @@ def check_tile(p, fmt, m, k, n, f16):
         if m > 32:  # beyond 32 rows only with few K parts and small partial tiles
             assert p.k_parts <= 4 and p.workspace_bytes <= 8 << 20 and (fmt == Q4 or m >= 128)
         assert p.grid[2] * rows >= m and (p.grid[2] - 1) * rows < m
-        assert p.steps == (2 if (not f16 and p.full_steps == 2) else 4) and p.waves_n in (16, 32)
+        assert p.steps == 4 and p.waves_n in (16, 32)
+        assert p.full_steps == 1 or f16  # row groups of 32 are for fp16 activations
         assert p.k_parts == ceil_div(nslices, p.steps)
         partial = p.k_parts * p.grid[2] * rows * n * 4 if p.k_parts > 1 else 0
         assert p.workspace_bytes == partial <= WORKSPACE
@@ -158,7 +159,8 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
             assert p.route == TILE_MFMA and p.quads_per_wave == 0 and list(p.grid) == [4, 56, 1]
         # elsewhere the 32x32 kernel is ahead, and runs when the activations are fp16 or promised to be in its range
         assert capi.matmul_plan(fmt, 16, 14336, 4096, fp16_range=True).route == GEMM_MFMA   # would be 14 K parts
-        assert capi.matmul_plan(fmt, 17, 4096, 14336, fp16_range=True).route == GEMM_MFMA
+        assert capi.matmul_plan(fmt, 17, 14336, 4096, fp16_range=True).route == GEMM_MFMA  # two rounds of workgroups
+        assert capi.matmul_plan(fmt, 17, 4096, 4096, fp16_range=True).route == TILE_MFMA   # two row groups of 16, one round
         assert capi.matmul_plan(fmt, 16, 14336, 4096).route == TILE_MFMA
     big = capi.matmul_plan(Q4, 512, 14336, 4096)   # images of 512 rows x 14336 exceed the 16 MiB workspace: several launches
     assert big.route == TILE_MFMA and big.quads_per_wave > 1
