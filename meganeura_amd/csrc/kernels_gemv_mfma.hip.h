@@ -520,8 +520,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         float scale = block_scale(am, &inv);
         if constexpr (I8) {
           // |x| * scale < 2^20 (block_scale leaves 2^12), so that rounding cannot reach 2^21 and the top
-          // digit stays within int8
-          if (scale != 1.0f || inv != 1.0f) scale *= 256.0f, inv *= 0.00390625f;
+          // digit stays within int8.  Blocks that block_scale leaves alone take the factor too: all
+          // zero stays zero, below 2^-100 rounds to zero, beyond 2^100 gets the NaN factor below.
+          scale *= 256.0f, inv *= 0.00390625f;
           if (!(am < 1.0e30f)) inv = __builtin_nanf("");
           const float x[8] = {v0.x * scale, v0.y * scale, v0.z * scale, v0.w * scale,
                               v1.x * scale, v1.y * scale, v1.z * scale, v1.w * scale};

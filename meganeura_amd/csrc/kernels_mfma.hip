@@ -25,10 +25,10 @@
 //   Per quant block: two MFMAs (K = 32) into a fresh accumulator D, then
 //     acc += d * D on the vector ALU (16 FMAs per lane).  The format's additive part
 //     (m * sum(x) for Q4, -128 * scale * sum(x) for Q8's byte bias) is one more MFMA
-//     per step into a second accumulator: its A operand is the block's mean
-//     activation (hi, lo), its B operand 32*m (or -4096*scale) taken from the scale
-//     word, so |m| < 2048 and scale < 16 are required.  Both accumulators are f32;
-//     their sum is taken once at the end.
+//     per step into a second accumulator: its A operand is the block's activation sum
+//     as (mean, sum - 32 mean), its B operand (32 m, m) (or (-4096, -128) * scale) taken
+//     from the scale word, so |m| < 2048 and scale < 16 are required.  Both accumulators
+//     are f32; their sum is taken once at the end.
 //
 // Work split: grid.y = row tiles; a workgroup owns `wnc` column tiles; K is cut into
 // chunks of 8*ksc blocks which the workgroup walks in order (ksc waves share a chunk),
@@ -82,7 +82,7 @@ __device__ __forceinline__ half8 bytes_to_operand(uint32_t w0, uint32_t w1) {
 //   aimg[b][(lb * 2 + h) * 64 + lane]  (uint4): A operand of the MFMA that covers k = 16h..16h+15
 //                                      of local block lb, for A lane `lane` = row + 32 * g
 //   simg[b][(lb / 2) * 64 + lane]      (uint4): A operand of a step's additive MFMA; lanes < 32 hold
-//                                      (mean_hi, mean_lo) of blocks 2p and 2p+1 in the first two
+//                                      (mean, sum - 32 mean) of blocks 2p and 2p+1 in the first two
 //                                      dwords, everything else stays zero
 // The element order inside an A operand follows the B side: Q4 pairs k with k+4, Q8 is natural.
 constexpr int kSteps = 4;  // steps per wave per chunk; a step is two K blocks
@@ -100,6 +100,18 @@ struct GemmTail {  // arguments first needed in the epilogue
   uint32_t row_tiles;
   uint32_t epilogue;  // unary operations on the output (apply_epilogue)
 };
+
+// B operand pair of a block's additive part from its scale word: (32 c, c) with c = m (Q4: the
+// word's high half) or -128 scale (Q8: the low half).  The A side pairs them with the block's mean
+// activation and with what the sum has beyond 32 * mean.
+template <int FMT>
+__device__ __forceinline__ uint32_t additive_pair(uint32_t w) {
+  const half2_t h = __builtin_bit_cast(half2_t, w);
+  const _Float16 c = h[FMT == MGN_FMT_Q4 ? 1 : 0];
+  const half2_t pair = {c, c};
+  const half2_t weights = FMT == MGN_FMT_Q4 ? half2_t{(_Float16)32.0f, (_Float16)1.0f} : half2_t{(_Float16)-4096.0f, (_Float16)-128.0f};
+  return __builtin_bit_cast(uint32_t, pair * weights);
+}
 
 template <int FMT>
 __device__ __forceinline__ uint4 f16_operand(uint4 v) {
@@ -254,7 +266,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
         s_hi = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, v.w), ones, s_hi, false);
         op_hi = f16_operand<FMT>(v);
       }
-      // block mean (sum over the lane quad's 32 values / 32), split into two fp16
+      // block sum (over the lane quad's 32 values)
       s_hi += dpp_move<kDppQuadXor1>(s_hi);
       s_hi += dpp_move<kDppQuadXor2>(s_hi);
       if constexpr (F32A) {
@@ -266,13 +278,14 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
         if constexpr (F32A) ab[t_slot[tt] + (CHAIN ? 64 : 16)] = op_lo;  // lo: an operand of its own, or rows 16-31
         if ((tid & 3) == 0) {
           uint32_t* sdst = sb + (lb >> 1) * 256 + (lb & 1);
-          const float mean = (CHAIN ? s_hi + s_lo : s_hi) * 0.03125f;
-          const uint32_t mh = pack_rtz(mean, 0.0f);
-          sdst[r * 4] = (mh & 0xFFFFu) | (pack_rtz(mean - half_lo(mh), 0.0f) << 16);
+          // the sum as 32 * mean + rest: the mean alone, as hi + lo, would lose the sum's low bits
+          // where fp16 runs out of exponent (activations around 1e-3 and below)
+          const float sum = CHAIN ? s_hi + s_lo : s_hi;
+          const uint32_t mh = pack_rtz(sum * 0.03125f, 0.0f);
+          sdst[r * 4] = (mh & 0xFFFFu) | (pack_rtz(sum - 32.0f * half_lo(mh), 0.0f) << 16);
           if constexpr (AM == 1) {
-            const float mean_l = s_lo * 0.03125f;
-            const uint32_t ml = pack_rtz(mean_l, 0.0f);
-            sdst[(16 + r) * 4] = (ml & 0xFFFFu) | (pack_rtz(mean_l - half_lo(ml), 0.0f) << 16);
+            const uint32_t ml = pack_rtz(s_lo * 0.03125f, 0.0f);
+            sdst[(16 + r) * 4] = (ml & 0xFFFFu) | (pack_rtz(s_lo - 32.0f * half_lo(ml), 0.0f) << 16);
           }
         }
       }
@@ -386,23 +399,10 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
         bop[0][1] = bytes_to_operand(r4, r5);
         bop[1][1] = bytes_to_operand(r6, r7);
       }
-      // additive part of both blocks: mean(x) * (32 * m), into its own accumulator so that this
-      // MFMA chain and the vector ALU's chain never wait for each other
-      uint32_t add0, add1;
-      if constexpr (FMT == MGN_FMT_Q4) {
-        add0 = __builtin_amdgcn_perm(meta0, meta0, 0x07060706u);  // (m, m) of block 0
-        add1 = __builtin_amdgcn_perm(meta1, meta1, 0x07060706u);
-        const half2_t k32 = {(_Float16)32.0f, (_Float16)32.0f};
-        add0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add0) * k32);
-        add1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add1) * k32);
-      } else {
-        // bytes carry q + 128: take 128 * scale * sum(x) back out
-        add0 = __builtin_amdgcn_perm(meta0, meta0, 0x05040504u);  // (scale, scale)
-        add1 = __builtin_amdgcn_perm(meta1, meta1, 0x05040504u);
-        const half2_t kb = {(_Float16)-4096.0f, (_Float16)-4096.0f};
-        add0 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add0) * kb);
-        add1 = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, add1) * kb);
-      }
+      // additive part of both blocks: (mean(x), sum(x) - 32 mean(x)) x (32 m, m), into its own
+      // accumulator so that this MFMA chain and the vector ALU's chain never wait for each other
+      // (Q8: bytes carry q + 128, so 128 * scale * sum(x) is taken back out)
+      const uint32_t add0 = additive_pair<FMT>(meta0), add1 = additive_pair<FMT>(meta1);
       uint4 aop[2][2], lop[2][2];  // [block][k half]; lop: the low halves' operands (CHAIN)
 #pragma unroll
       for (int t = 0; t < 2; t++) {

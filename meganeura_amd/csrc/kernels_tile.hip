@@ -21,8 +21,8 @@
 //     activations are used as they are.
 //   Per block: D = sum n x on the matrix cores, then P += d * D on the vector ALU (4 FMAs per
 //     lane).  The format's additive part (m * sum(x) for Q4, -128 * scale * sum(x) for Q8's byte
-//     bias) is one more MFMA per slice of 8 blocks: its A operand holds the blocks' mean
-//     activations (hi, lo), its B operand the blocks' m (or scale), both exact fp16 values.
+//     bias) is one more MFMA per slice of 8 blocks: its A operand holds the blocks' activation
+//     sums as (mean, sum - 32 mean), its B operand the blocks' (c, c / 32), c = m or the scale.
 //     A slice's P is multiplied by the rows' inverse power-of-two scales and added to the
 //     accumulators.
 //
@@ -79,6 +79,19 @@ __device__ __forceinline__ half8 bytes_to_operand(uint32_t w0, uint32_t w1) {
                   __builtin_amdgcn_perm(0u, u1, 0x0c010c00u), __builtin_amdgcn_perm(0u, u1, 0x0c030c02u));
 }
 
+// B operand pair of a block's additive part from its scale word: (c, c / 32) with c = m (Q4: the
+// word's high half) or the scale (Q8: the low half).  The A side pairs them with the block's mean
+// activation and with what the sum has beyond 32 * mean (convert_task).  c / 32 only rounds where
+// c is below 2^-9, against a partner that is 2^-10 of the sum at most.
+template <int FMT>
+__device__ __forceinline__ uint32_t additive_pair(uint32_t w) {
+  const half2_t h = __builtin_bit_cast(half2_t, w);
+  const _Float16 c = h[FMT == MGN_FMT_Q4 ? 1 : 0];
+  const half2_t pair = {c, c};
+  const half2_t weights = {(_Float16)1.0f, (_Float16)0.03125f};
+  return __builtin_bit_cast(uint32_t, pair * weights);
+}
+
 // max over aligned groups of 32 consecutive lanes (every lane ends with the group's maximum)
 __device__ __forceinline__ float group_max32(float v) {
   v = fmaxf(v, dpp_move<kDppQuadXor1>(v));
@@ -113,7 +126,7 @@ __device__ __forceinline__ float slice_scale(float amax, float* inv) {
 //                                that write together during the conversion (one row, two blocks, four
 //                                g) then fall into different LDS banks, and so do the readers'.
 //   [8 * HL * 64 + lane]         A operand of the slice's additive MFMA: lanes (row, g' < 2) hold
-//                                (mean_hi | mean_lo << 16) of blocks 4g'..4g'+3, the rest is zero
+//                                (mean | (sum - 32 mean) << 16) of blocks 4g'..4g'+3, the rest is zero
 //   [8 * HL * 64 + 64 + 0..15]   (as float) the rows' inverse scales times the quants' operand scale
 //                                (2^20 for Q4, 2^24 for Q8; f32 activations only)
 // The element order inside an operand follows the B side: Q4 pairs k with k + 4, Q8 is natural.
@@ -202,9 +215,10 @@ __device__ __forceinline__ void convert_task(const TaskWords<F32A>& xin, bool ok
   s += dpp_move<kDppQuadXor2>(s);
   uint32_t* const extra = (uint32_t*)(img + kSliceBlocks * HL * 64);
   if (g == 0) {
-    const float mean = s * 0.03125f;
-    const uint32_t mh = pack_rtz(mean, 0.0f);
-    extra[(r + 16 * (kb >> 2)) * 4 + (kb & 3)] = (mh & 0xFFFFu) | (pack_rtz(mean - half_lo(mh), 0.0f) << 16);
+    // the block's sum as 32 * mean + rest: the mean alone, as hi + lo, would lose the sum's low bits
+    // where fp16 runs out of exponent (fp16 activations around 1e-3 and below)
+    const uint32_t mh = pack_rtz(s * 0.03125f, 0.0f);
+    extra[(r + 16 * (kb >> 2)) * 4 + (kb & 3)] = (mh & 0xFFFFu) | (pack_rtz(s - 32.0f * half_lo(mh), 0.0f) << 16);
   }
   // lanes (row, g' >= 2) of the additive operand stay zero (8 dwords per half-wave lane... 16 rows x 32
   // lanes cover the 128 dwords); the rows' inverse scales follow
@@ -298,7 +312,7 @@ __device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t*
       // (bit arithmetic, not a select between array elements: that would be turned into an
       // indexed load from a stack copy of the array)
       const uint32_t w = mw[j] ^ ((mw[j] ^ mw[4 + j]) & upper);
-      bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
+      bw[j] = additive_pair<FMT>(w);
     }
     const half8 bm = as_half8(bw[0], bw[1], bw[2], bw[3]);
     constexpr float kAdd = (FMT == MGN_FMT_Q4 ? 32.0f : -4096.0f) / kOpScale;
@@ -724,7 +738,7 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const uint32_t w = mw[u][j] ^ ((mw[u][j] ^ mw[u][4 + j]) & upper);
-      bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
+      bw[j] = additive_pair<FMT>(w);
     }
     bm[u] = as_half8(bw[0], bw[1], bw[2], bw[3]);
   }

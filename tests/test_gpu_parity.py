@@ -705,6 +705,33 @@ def test_rows_whose_activation_images_exceed_the_workspace_run_in_blocks(ctx, or
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("f16", [False, True])
+@pytest.mark.parametrize("m,route", [(1, "gemv_mfma"), (2, "gemv_mfma"), (4, "gemv_mfma"), (16, "tile_mfma"), (40, "tile_mfma"),
+                                     (16, "gemm_mfma"), (40, "gemm_mfma"), (1, "auto"), (16, "auto"), (40, "auto")])
+def test_the_error_scales_with_the_activations(ctx, orc, fmt, f16, m, route):
+    """The same activations times 1e-4 .. 3e3 stay within the bar scaled by that factor, on every
+    matrix-core kernel.  Two things this pins: block sums of small fp16 activations (a mean kept as
+    an fp16 pair loses the sum's low bits from about 1e-3 down), and the one-row Q4 kernel's
+    integer digits for blocks whose largest magnitude lies in [2^11, 2^12), where the block's own
+    power of two is 1 (1000 and 3000 put most blocks there).  f32 activations on the 32x32x16
+    kernel are left out below 1e-2: it does not rescale them and says so."""
+    k, n = 1280, 208
+    w = synth.normal(1201, k * n, 0.02).reshape(k, n)
+    base = synth.normal(1202 + m, m * k, 1.0).reshape(m, k)
+    deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
+    wt = ctx.weight(fmt, w)
+    for mag in (1e-4, 1e-3, 1e-2, 1.0, 1000.0, 3000.0):
+        if route == "gemm_mfma" and not f16 and mag < 1e-2:
+            continue
+        x = base * np.float32(mag)
+        if f16:
+            x = x.astype(np.float16).astype(np.float32)
+        got = run_matmul(ctx, fmt, x, wt, ROUTES[route], f16=f16)
+        assert_close_rowwise(got, orc.matmul_f64(x, deq), x)
+    wt.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
 @pytest.mark.parametrize("m", [5, 16, 40])
 def test_activations_of_any_magnitude_on_the_rescaling_tiled_kernel(ctx, orc, fmt, m):
     """f32 activations are scaled per (row, 256-element slice) by a power of two before they are
