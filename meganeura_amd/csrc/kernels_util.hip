@@ -9,6 +9,16 @@
 namespace mgn {
 namespace {
 
+// A Q8 block whose 32 quants are all zero holds a scale that multiplies nothing.  The reference's
+// quantizer writes 1.0 there (src/runtime.rs:2171), a thousand times the scales around it, and
+// the matrix-core kernels, which form scale * (sum (q + 128) x - 128 sum x), would leave that
+// scale's share of rounding in an output that is exactly zero.  In device memory such a block
+// carries -0.0 instead: 0x3C00 and 0x8000 trade places on the way in and on the way out, so every
+// input still exports to the bytes it came from and dequantizes as the reference does.
+__device__ __forceinline__ uint32_t q8_device_scale(uint32_t bits, bool all_zero) {
+  return all_zero && (bits == 0x3C00u || bits == 0x8000u) ? bits ^ 0xBC00u : bits;
+}
+
 // One thread per (block row kb, column n), n fastest, so the f32 side is
 // coalesced across the wave while each thread owns one whole block.
 // dequantize_q4_0 / dequantize_q8_0 (src/runtime.rs:2105-2138, 2191-2215):
@@ -31,10 +41,11 @@ __global__ __launch_bounds__(256) void dequantize_kernel(WeightView w, float* __
       for (int j = 0; j < 8; j++)
         dst[(size_t)(t * 8 + j) * w.n] = __fmaf_rn((float)((words[t] >> (4 * j)) & 0xFu), d, m);
   } else {
-    const float s = half_bits_to_float(((const uint16_t*)w.meta)[b]);
     const uint4* qp = (const uint4*)w.quants + b * 2;
     const uint4 q0 = qp[0], q1 = qp[1];
     const uint32_t words[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    const bool all_zero = (q0.x | q0.y | q0.z | q0.w | q1.x | q1.y | q1.z | q1.w) == 0;
+    const float s = half_bits_to_float(q8_device_scale(((const uint16_t*)w.meta)[b], all_zero));
 #pragma unroll
     for (int t = 0; t < 8; t++)
 #pragma unroll
@@ -50,9 +61,12 @@ __global__ __launch_bounds__(256) void export_q8_kernel(const uint16_t* __restri
                                                         uint32_t* __restrict__ out) {
   const size_t b = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (b >= nb) return;
-  out[b * 9] = scales[b];
+  uint32_t q[8], any = 0;
 #pragma unroll
-  for (int i = 0; i < 8; i++) out[b * 9 + 1 + i] = quants[b * 8 + i];
+  for (int i = 0; i < 8; i++) any |= q[i] = quants[b * 8 + i];
+  out[b * 9] = q8_device_scale(scales[b], any == 0);
+#pragma unroll
+  for (int i = 0; i < 8; i++) out[b * 9 + 1 + i] = q[i];
 }
 
 __global__ __launch_bounds__(256) void import_q8_kernel(const uint32_t* __restrict__ ref, size_t nb,
@@ -60,9 +74,12 @@ __global__ __launch_bounds__(256) void import_q8_kernel(const uint32_t* __restri
                                                         uint32_t* __restrict__ quants) {
   const size_t b = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (b >= nb) return;
-  scales[b] = (uint16_t)ref[b * 9];
+  uint32_t q[8], any = 0;
 #pragma unroll
-  for (int i = 0; i < 8; i++) quants[b * 8 + i] = ref[b * 9 + 1 + i];
+  for (int i = 0; i < 8; i++) any |= q[i] = ref[b * 9 + 1 + i];
+  scales[b] = (uint16_t)q8_device_scale(ref[b * 9] & 0xFFFFu, any == 0);
+#pragma unroll
+  for (int i = 0; i < 8; i++) quants[b * 8 + i] = q[i];
 }
 
 // Largest |scale| and largest |min| over all blocks, as f32 bit patterns (for non-negative
@@ -155,7 +172,6 @@ __global__ __launch_bounds__(256) void quantize_kernel(int fmt, const float* __r
     }
     const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
     const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
-    ((uint16_t*)meta)[b] = __builtin_bit_cast(uint16_t, (_Float16)scale);
     uint32_t words[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < 32; i++) {
@@ -163,6 +179,8 @@ __global__ __launch_bounds__(256) void quantize_kernel(int fmt, const float* __r
       int q = (t != t) ? 0 : (int)t;
       words[i / 4] |= (uint32_t)(q & 0xFF) << (8 * (i % 4));
     }
+    const bool all_zero = (words[0] | words[1] | words[2] | words[3] | words[4] | words[5] | words[6] | words[7]) == 0;
+    ((uint16_t*)meta)[b] = (uint16_t)q8_device_scale(__builtin_bit_cast(uint16_t, (_Float16)scale), all_zero);
     uint4* qp = (uint4*)quants + b * 2;
     qp[0] = make_uint4(words[0], words[1], words[2], words[3]);
     qp[1] = make_uint4(words[4], words[5], words[6], words[7]);

@@ -705,6 +705,65 @@ def test_rows_whose_activation_images_exceed_the_workspace_run_in_blocks(ctx, or
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
+def test_all_zero_columns_give_exactly_the_residual(ctx, orc, fmt):
+    """Columns of zeros (the padding of an lm_head, a pruned unit) come out as the residual, bit
+    for bit, on every kernel, and zero blocks inside live columns leave those within the bar.  The
+    reference's Q8 quantizer gives an all-zero block the scale 1.0 (src/runtime.rs:2171), about a
+    thousand times its neighbours': a kernel that forms scale * (sum (q + 128) x - 128 sum x) with
+    that scale leaves rounding of the size of an ordinary output there.  Such weights still export
+    to the bytes they were made from and dequantize as the oracle does."""
+    k, n = 2080, 150
+    w = synth.normal(1301, k * n, 0.02).reshape(k, n)
+    zero_cols = [0, 77, n - 1]
+    for j in zero_cols:
+        w[:, j] = 0.0
+    w[64:96, 5] = 0.0
+    w[2048:2080, 140] = 0.0
+    w[0:512, 33] = 0.0
+    packed = orc.quantize(fmt, w)
+    deq = orc.dequantize(fmt, packed, k, n)
+    weights = [ctx.weight_from_packed(fmt, packed, k, n), ctx.weight(fmt, w)]
+    src = ctx.upload(w)
+    weights.append(ctx.weight_from_device(fmt, src, k, n))
+    for wt in weights:
+        assert (wt.export_ref() == packed).all()
+        assert (bits(wt.dequantize()) == bits(deq)).all()
+    wt = weights[0]
+    for m in (1, 3, 6, 16, 40, 70):
+        x = synth.normal(1302 + m, m * k, 1.0).reshape(m, k)
+        d = synth.normal(1303 + m, m * n).reshape(m, n)
+        for f16 in (False, True):
+            xin = x.astype(np.float16).astype(np.float32) if f16 else x
+            want = orc.matmul_f64(xin, deq, d)
+            for route in ("generic", "gemv_mfma", "gemm_mfma", "tile_mfma", "auto"):
+                if (route == "gemv_mfma" and m > 4) or (route in ("gemm_mfma", "tile_mfma") and m < 5):
+                    continue
+                got = run_matmul(ctx, fmt, x, wt, ROUTES[route], d=d, f16=f16)
+                assert (bits(got[:, zero_cols]) == bits(d[:, zero_cols])).all(), (m, f16, route)
+                orc.assert_close(got, want, REL, ABS)
+    for wt in weights:
+        wt.free()
+    src.free()
+
+
+def test_q8_zero_blocks_with_foreign_scales_round_trip(ctx, orc):
+    """All-zero Q8 blocks with scales the reference's quantizer never writes (0, -0, anything)
+    come back byte for byte and dequantize to zeros."""
+    k, n = 64, 8
+    w = synth.normal(1311, k * n, 0.02).reshape(k, n)
+    w[:, :6] = 0.0
+    packed = orc.quantize(Q8, w).copy()
+    blocks = packed.reshape(-1, 36)
+    for b, scale_bits in enumerate([0x0000, 0x8000, 0x3C00, 0x1234, 0x3555, 0xBC00]):
+        assert not blocks[b, 4:].any()
+        blocks[b, 0], blocks[b, 1] = scale_bits & 0xFF, scale_bits >> 8
+    wt = ctx.weight_from_packed(Q8, packed, k, n)
+    assert (wt.export_ref() == packed).all()
+    assert (bits(wt.dequantize()) == bits(orc.dequantize(Q8, packed, k, n))).all()
+    wt.free()
+
+
+@pytest.mark.parametrize("fmt", [Q4, Q8])
 @pytest.mark.parametrize("f16", [False, True])
 @pytest.mark.parametrize("m,route", [(1, "gemv_mfma"), (2, "gemv_mfma"), (4, "gemv_mfma"), (16, "tile_mfma"), (40, "tile_mfma"),
                                      (16, "gemm_mfma"), (40, "gemm_mfma"), (1, "auto"), (16, "auto"), (40, "auto")])
