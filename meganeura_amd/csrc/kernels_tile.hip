@@ -21,8 +21,9 @@
 //     activations are used as they are.
 //   Per block: D = sum n x on the matrix cores, then P += d * D on the vector ALU (4 FMAs per
 //     lane).  The format's additive part (m * sum(x) for Q4, -128 * scale * sum(x) for Q8's byte
-//     bias) is one more MFMA per slice of 8 blocks: its A operand holds the blocks' activation
-//     sums as (mean, sum - 32 mean), its B operand the blocks' (c, c / 32), c = m or the scale.
+//     bias) is one more MFMA per slice of 8 blocks: its A operand holds the blocks' mean
+//     activations (hi, lo; with fp16 activations scaled per (row, slice) by a power of two like
+//     the f32 activations themselves), its B operand the blocks' m (or scale), exact fp16 values.
 //     A slice's P is multiplied by the rows' inverse power-of-two scales and added to the
 //     accumulators.
 //
@@ -79,18 +80,10 @@ __device__ __forceinline__ half8 bytes_to_operand(uint32_t w0, uint32_t w1) {
                   __builtin_amdgcn_perm(0u, u1, 0x0c010c00u), __builtin_amdgcn_perm(0u, u1, 0x0c030c02u));
 }
 
-// B operand pair of a block's additive part from its scale word: (c, c / 32) with c = m (Q4: the
-// word's high half) or the scale (Q8: the low half).  The A side pairs them with the block's mean
-// activation and with what the sum has beyond 32 * mean (convert_task).  c / 32 only rounds where
-// c is below 2^-9, against a partner that is 2^-10 of the sum at most.
+// What the additive MFMA's result (block means times m, or times the Q8 scale) is multiplied by:
+// 32 for the means and, for Q8, -128 for the byte bias, over the quants' operand scale.
 template <int FMT>
-__device__ __forceinline__ uint32_t additive_pair(uint32_t w) {
-  const half2_t h = __builtin_bit_cast(half2_t, w);
-  const _Float16 c = h[FMT == MGN_FMT_Q4 ? 1 : 0];
-  const half2_t pair = {c, c};
-  const half2_t weights = {(_Float16)1.0f, (_Float16)0.03125f};
-  return __builtin_bit_cast(uint32_t, pair * weights);
-}
+constexpr float additive_constant() { return FMT == MGN_FMT_Q4 ? 32.0f / 1048576.0f : -4096.0f / 16777216.0f; }
 
 // max over aligned groups of 32 consecutive lanes (every lane ends with the group's maximum)
 __device__ __forceinline__ float group_max32(float v) {
@@ -126,9 +119,10 @@ __device__ __forceinline__ float slice_scale(float amax, float* inv) {
 //                                that write together during the conversion (one row, two blocks, four
 //                                g) then fall into different LDS banks, and so do the readers'.
 //   [8 * HL * 64 + lane]         A operand of the slice's additive MFMA: lanes (row, g' < 2) hold
-//                                (mean | (sum - 32 mean) << 16) of blocks 4g'..4g'+3, the rest is zero
-//   [8 * HL * 64 + 64 + 0..15]   (as float) the rows' inverse scales times the quants' operand scale
-//                                (2^20 for Q4, 2^24 for Q8; f32 activations only)
+//                                (mean_hi | mean_lo << 16) of blocks 4g'..4g'+3, the rest is zero
+//   [8 * HL * 64 + 64 + 0..15]   (as float) f32 activations: the rows' inverse scales times the quants'
+//                                operand scale (2^20 for Q4, 2^24 for Q8); fp16 activations: the inverse
+//                                scales of the rows' block sums times the additive part's constant
 // The element order inside an operand follows the B side: Q4 pairs k with k + 4, Q8 is natural.
 // Q4 with f32 activations: the even elements are stored times 16 (see nibbles_to_operand) and the
 // slice scale aims at 2^7 instead of 2^11 to leave room for that.
@@ -213,17 +207,28 @@ __device__ __forceinline__ void convert_task(const TaskWords<F32A>& xin, bool ok
   }
   s += dpp_move<kDppQuadXor1>(s);
   s += dpp_move<kDppQuadXor2>(s);
+  if constexpr (!F32A) {
+    // The block sums of fp16 activations span 2^-24 .. 2^21: the slice's largest is brought to
+    // [2^15, 2^16) (its mean to [2^10, 2^11)) before the means are split into fp16 pairs, so that
+    // neither large sums overflow nor small ones lose their low bits; the additive MFMA's result
+    // is multiplied by the inverse.  (f32 activations were scaled before they were summed.)
+    float am = fabsf(s);
+    am = fmaxf(am, dpp_move<kDppRowHalfMirror>(am));
+    am = fmaxf(am, dpp_move<kDppRowMirror>(am));
+    am = fmaxf(am, __shfl_xor(am, 16, 64));
+    s *= slice_scale<15>(am, &inv);
+  }
   uint32_t* const extra = (uint32_t*)(img + kSliceBlocks * HL * 64);
   if (g == 0) {
-    // the block's sum as 32 * mean + rest: the mean alone, as hi + lo, would lose the sum's low bits
-    // where fp16 runs out of exponent (fp16 activations around 1e-3 and below)
-    const uint32_t mh = pack_rtz(s * 0.03125f, 0.0f);
-    extra[(r + 16 * (kb >> 2)) * 4 + (kb & 3)] = (mh & 0xFFFFu) | (pack_rtz(s - 32.0f * half_lo(mh), 0.0f) << 16);
+    const float mean = s * 0.03125f;
+    const uint32_t mh = pack_rtz(mean, 0.0f);
+    extra[(r + 16 * (kb >> 2)) * 4 + (kb & 3)] = (mh & 0xFFFFu) | (pack_rtz(mean - half_lo(mh), 0.0f) << 16);
   }
   // lanes (row, g' >= 2) of the additive operand stay zero (8 dwords per half-wave lane... 16 rows x 32
-  // lanes cover the 128 dwords); the rows' inverse scales follow
+  // lanes cover the 128 dwords); the rows' inverse scales follow: of the activations, times the
+  // quants' operand scale (f32), or of the block sums, times the additive part's constant (fp16)
   if (l < 8) extra[32 * 4 + r * 8 + l] = 0u;
-  if (l == 0) ((float*)extra)[64 * 4 + r] = inv * (FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f);
+  if (l == 0) ((float*)extra)[64 * 4 + r] = inv * (F32A ? (FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f) : additive_constant<FMT>());
 }
 
 // grid.x = row tiles * slices; 512 threads: half-wave r (0..15) converts row r of the tile,
@@ -248,7 +253,6 @@ template <int FMT, bool F32A, int R>
 __device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t* ib, uint32_t rstride, const uint32_t (&mw)[8],
                                           uint32_t g, uint32_t lane, floatx4 (&acc)[R]) {
   constexpr uint32_t HL = F32A ? 2 : 1;
-  constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;  // 2^20, 2^24
     // Software pipeline over the 8 blocks: LDS reads two blocks ahead, unpack and MFMAs one
     // block ahead of the scaling FMAs that consume the previous block's products.
     const uint32_t slot_off[2] = {image_slot(lane & 15, g, 0) * 16, image_slot(lane & 15, g, 1) * 16};
@@ -312,25 +316,28 @@ __device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t*
       // (bit arithmetic, not a select between array elements: that would be turned into an
       // indexed load from a stack copy of the array)
       const uint32_t w = mw[j] ^ ((mw[j] ^ mw[4 + j]) & upper);
-      bw[j] = additive_pair<FMT>(w);
+      bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
     }
     const half8 bm = as_half8(bw[0], bw[1], bw[2], bw[3]);
-    constexpr float kAdd = (FMT == MGN_FMT_Q4 ? 32.0f : -4096.0f) / kOpScale;
+    constexpr float kAdd = additive_constant<FMT>();
 #pragma unroll
     for (int r = 0; r < R; r++) {
       const uint8_t* const ir = ib + lane * 16 + r * rstride + 8 * HL * 64 * 16;
       const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, *(const u32x4_t*)ir), bm,
                                                                floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+      // f32 activations: the rows' inverse slice scales (times 2^20 or 2^24: the operand scale of the
+      // quants); fp16 activations: the inverse scales of the rows' block sums times kAdd
+      const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
       if constexpr (F32A) {
-        // the rows' inverse slice scales (times 2^20 or 2^24: the operand scale of the quants)
-        const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
         acc[r][0] = __fmaf_rn(__fmaf_rn(kAdd, d[0], P[r][0]), inv.x, acc[r][0]);
         acc[r][1] = __fmaf_rn(__fmaf_rn(kAdd, d[1], P[r][1]), inv.y, acc[r][1]);
         acc[r][2] = __fmaf_rn(__fmaf_rn(kAdd, d[2], P[r][2]), inv.z, acc[r][2]);
         acc[r][3] = __fmaf_rn(__fmaf_rn(kAdd, d[3], P[r][3]), inv.w, acc[r][3]);
       } else {
-#pragma unroll
-        for (int i = 0; i < 4; i++) acc[r][i] += __fmaf_rn(kAdd, d[i], P[r][i]);
+        acc[r][0] += __fmaf_rn(inv.x, d[0], P[r][0]);
+        acc[r][1] += __fmaf_rn(inv.y, d[1], P[r][1]);
+        acc[r][2] += __fmaf_rn(inv.z, d[2], P[r][2]);
+        acc[r][3] += __fmaf_rn(inv.w, d[3], P[r][3]);
       }
     }
   }
@@ -655,7 +662,6 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
                                                const uint32_t (&mw)[kSide][8], const uint8_t* ib, uint32_t rstride, uint32_t g,
                                                uint32_t lane, floatx4 (&acc)[kSide][R]) {
   constexpr uint32_t HL = F32A ? 2 : 1;
-  constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;  // 2^20, 2^24
   const uint32_t slot_off[2] = {image_slot(lane & 15, g, 0) * 16, image_slot(lane & 15, g, 1) * 16};
   u32x4_t aop[3][R][HL];
   uint32_t bq[3][kSide][FMT == MGN_FMT_Q4 ? 1 : 2];  // PARK: the lane's quants of a block
@@ -730,7 +736,7 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
   }
   // additive part of the slice's 8 blocks (see slice_mac)
   const uint32_t upper = 0u - (g & 1u);  // all ones in the lanes that take blocks 4..7
-  constexpr float kAdd = (FMT == MGN_FMT_Q4 ? 32.0f : -4096.0f) / kOpScale;
+  constexpr float kAdd = additive_constant<FMT>();
   half8 bm[kSide];
 #pragma unroll
   for (int u = 0; u < kSide; u++) {
@@ -738,7 +744,7 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const uint32_t w = mw[u][j] ^ ((mw[u][j] ^ mw[u][4 + j]) & upper);
-      bw[j] = additive_pair<FMT>(w);
+      bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
     }
     bm[u] = as_half8(bw[0], bw[1], bw[2], bw[3]);
   }
@@ -746,8 +752,9 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
   for (int r = 0; r < R; r++) {
     const uint8_t* const ir = ib + lane * 16 + r * rstride + 8 * HL * 64 * 16;
     const half8 am = __builtin_bit_cast(half8, *(const u32x4_t*)ir);
-    float4 inv = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
-    if constexpr (F32A) inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);  // the rows' inverse slice scales (times 2^20 or 2^24)
+    // f32 activations: the rows' inverse slice scales (times 2^20 or 2^24); fp16 activations: the
+    // inverse scales of the rows' block sums times kAdd
+    const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
 #pragma unroll
     for (int u = 0; u < kSide; u++) {
       const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm[u], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
@@ -757,8 +764,10 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
         acc[u][r][2] = __fmaf_rn(__fmaf_rn(kAdd, d[2], P[u][r][2]), inv.z, acc[u][r][2]);
         acc[u][r][3] = __fmaf_rn(__fmaf_rn(kAdd, d[3], P[u][r][3]), inv.w, acc[u][r][3]);
       } else {
-#pragma unroll
-        for (int i = 0; i < 4; i++) acc[u][r][i] += __fmaf_rn(kAdd, d[i], P[u][r][i]);
+        acc[u][r][0] += __fmaf_rn(inv.x, d[0], P[u][r][0]);
+        acc[u][r][1] += __fmaf_rn(inv.y, d[1], P[u][r][1]);
+        acc[u][r][2] += __fmaf_rn(inv.z, d[2], P[u][r][2]);
+        acc[u][r][3] += __fmaf_rn(inv.w, d[3], P[u][r][3]);
       }
     }
   }
