@@ -19,6 +19,38 @@ __device__ __forceinline__ uint32_t q8_device_scale(uint32_t bits, bool all_zero
   return all_zero && (bits == 0x3C00u || bits == 0x8000u) ? bits ^ 0xBC00u : bits;
 }
 
+// ---- the range of a weight's block constants ----
+// Largest |scale| and largest |min| over all blocks, as f32 bit patterns (for non-negative
+// floats the unsigned order is the numeric order, and inf / NaN sort above every finite value),
+// in two words that must be zero before the first launch that adds to them.  The scan runs where
+// the blocks are written (the device quantizer, the Q8 import); only Q4 bytes that are uploaded as
+// they are need a kernel of its own (scale_range_kernel).
+
+// |x| of an fp16 bit pattern as the bit pattern of an f32
+__device__ __forceinline__ uint32_t abs_bits(uint32_t half_bits) {
+  return __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(half_bits & 0xFFFFu)));
+}
+
+// Every thread of a 256-thread workgroup brings its maxima; one atomic pair per workgroup at most
+// (thousands of atomics on one address would take longer than the scan), and none when the
+// published maximum, which only grows, is already as large.
+__device__ __forceinline__ void publish_range(uint32_t smax, uint32_t mmax, uint32_t* __restrict__ out) {
+  __shared__ uint32_t part[2][4];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    smax = max(smax, (uint32_t)__shfl_xor((int)smax, off, 64));
+    mmax = max(mmax, (uint32_t)__shfl_xor((int)mmax, off, 64));
+  }
+  if ((threadIdx.x & 63) == 0) part[0][threadIdx.x >> 6] = smax, part[1][threadIdx.x >> 6] = mmax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    smax = max(max(part[0][0], part[0][1]), max(part[0][2], part[0][3]));
+    mmax = max(max(part[1][0], part[1][1]), max(part[1][2], part[1][3]));
+    if (smax > __hip_atomic_load(out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(out, smax);
+    if (mmax > __hip_atomic_load(out + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(out + 1, mmax);
+  }
+}
+
 // One thread per (block row kb, column n), n fastest, so the f32 side is
 // coalesced across the wave while each thread owns one whole block.
 // dequantize_q4_0 / dequantize_q8_0 (src/runtime.rs:2105-2138, 2191-2215):
@@ -71,23 +103,25 @@ __global__ __launch_bounds__(256) void export_q8_kernel(const uint16_t* __restri
 
 __global__ __launch_bounds__(256) void import_q8_kernel(const uint32_t* __restrict__ ref, size_t nb,
                                                         uint16_t* __restrict__ scales,
-                                                        uint32_t* __restrict__ quants) {
+                                                        uint32_t* __restrict__ quants, uint32_t* __restrict__ range) {
   const size_t b = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (b >= nb) return;
-  uint32_t q[8], any = 0;
+  uint32_t smax = 0;
+  if (b < nb) {
+    uint32_t q[8], any = 0;
 #pragma unroll
-  for (int i = 0; i < 8; i++) any |= q[i] = ref[b * 9 + 1 + i];
-  scales[b] = (uint16_t)q8_device_scale(ref[b * 9] & 0xFFFFu, any == 0);
+    for (int i = 0; i < 8; i++) any |= q[i] = ref[b * 9 + 1 + i];
+    const uint32_t bits = q8_device_scale(ref[b * 9] & 0xFFFFu, any == 0);
+    scales[b] = (uint16_t)bits;
+    smax = abs_bits(bits);
 #pragma unroll
-  for (int i = 0; i < 8; i++) quants[b * 8 + i] = q[i];
+    for (int i = 0; i < 8; i++) quants[b * 8 + i] = q[i];
+  }
+  publish_range(smax, 0u, range);
 }
 
-// Largest |scale| and largest |min| over all blocks, as f32 bit patterns (for non-negative
-// floats the unsigned order is the numeric order, and inf / NaN sort above every finite value).
-// out[0], out[1] must be zero before the launch.
+// The range scan as a pass of its own over the scale words.
 __global__ __launch_bounds__(256) void scale_range_kernel(int fmt, const void* __restrict__ meta, size_t nb,
                                                           uint32_t* __restrict__ out) {
-  __shared__ uint32_t part[2][4];
   uint32_t smax = 0, mmax = 0;
   // four scale words (Q8: eight scales) per load; the tail past a multiple of four reads the
   // all-zero blocks that follow the real ones
@@ -97,27 +131,13 @@ __global__ __launch_bounds__(256) void scale_range_kernel(int fmt, const void* _
     const uint32_t w[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-      const uint32_t lo = __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(w[e] & 0xFFFFu)));
-      const uint32_t hi = __builtin_bit_cast(uint32_t, fabsf(half_bits_to_float(w[e] >> 16)));
+      const uint32_t lo = abs_bits(w[e]), hi = abs_bits(w[e] >> 16);
       smax = max(smax, lo);
       if (fmt == MGN_FMT_Q4) mmax = max(mmax, hi);
       else smax = max(smax, hi);
     }
   }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    smax = max(smax, (uint32_t)__shfl_xor((int)smax, off, 64));
-    mmax = max(mmax, (uint32_t)__shfl_xor((int)mmax, off, 64));
-  }
-  // one atomic pair per workgroup: thousands of atomics on one address would take longer than the scan
-  if ((threadIdx.x & 63) == 0) part[0][threadIdx.x >> 6] = smax, part[1][threadIdx.x >> 6] = mmax;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    smax = max(max(part[0][0], part[0][1]), max(part[0][2], part[0][3]));
-    mmax = max(max(part[1][0], part[1][1]), max(part[1][2], part[1][3]));
-    if (smax) atomicMax(out, smax);
-    if (mmax) atomicMax(out + 1, mmax);
-  }
+  publish_range(smax, mmax, out);
 }
 
 __device__ __forceinline__ float clamp_keep_nan(float v, float lo, float hi) {
@@ -132,59 +152,65 @@ __device__ __forceinline__ float clamp_keep_nan(float v, float lo, float hi) {
 #pragma clang fp contract(off)
 __global__ __launch_bounds__(256) void quantize_kernel(int fmt, const float* __restrict__ w, uint32_t k,
                                                        uint32_t n_cols, void* __restrict__ meta,
-                                                       void* __restrict__ quants) {
+                                                       void* __restrict__ quants, uint32_t* __restrict__ range) {
   const uint32_t n = blockIdx.x * 256 + threadIdx.x;
   const uint32_t kb = blockIdx.y;
-  if (n >= n_cols) return;
-  const uint32_t bpc = k / 32;
-  const size_t b = (size_t)n * bpc + kb;
-  const float* src = w + (size_t)kb * 32 * n_cols + n;
-  float v[32];
+  uint32_t smax = 0, mmax = 0;  // this block's |scale| and |min| as stored (see publish_range)
+  if (n < n_cols) {
+    const uint32_t bpc = k / 32;
+    const size_t b = (size_t)n * bpc + kb;
+    const float* src = w + (size_t)kb * 32 * n_cols + n;
+    float v[32];
 #pragma unroll
-  for (int i = 0; i < 32; i++) v[i] = src[(size_t)i * n_cols];
-  if (fmt == MGN_FMT_Q4) {
-    float bmin = INFINITY, bmax = -INFINITY;
+    for (int i = 0; i < 32; i++) v[i] = src[(size_t)i * n_cols];
+    if (fmt == MGN_FMT_Q4) {
+      float bmin = INFINITY, bmax = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 32; i++) {
-      if (v[i] < bmin) bmin = v[i];
-      if (v[i] > bmax) bmax = v[i];
+      for (int i = 0; i < 32; i++) {
+        if (v[i] < bmin) bmin = v[i];
+        if (v[i] > bmax) bmax = v[i];
+      }
+      const float d = bmax > bmin ? (bmax - bmin) / 15.0f : 1.0f;
+      const float m = bmin;
+      const float d_inv = d > 0.0f ? 1.0f / d : 0.0f;
+      const uint32_t dbits = __builtin_bit_cast(uint16_t, (_Float16)d);
+      const uint32_t mbits = __builtin_bit_cast(uint16_t, (_Float16)m);
+      ((uint32_t*)meta)[b] = dbits | (mbits << 16);
+      smax = abs_bits(dbits), mmax = abs_bits(mbits);
+      uint32_t words[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 32; i++) {
+        float t = clamp_keep_nan(roundf((v[i] - m) * d_inv), 0.0f, 15.0f);
+        uint32_t nib = (t != t) ? 0u : (uint32_t)t;
+        words[i / 8] |= nib << (4 * (i % 8));
+      }
+      ((uint4*)quants)[b] = make_uint4(words[0], words[1], words[2], words[3]);
+    } else {
+      float amax = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 32; i++) {
+        float a = fabsf(v[i]);
+        if (a > amax) amax = a;
+      }
+      const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+      const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+      uint32_t words[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 32; i++) {
+        float t = clamp_keep_nan(roundf(v[i] * inv), -128.0f, 127.0f);
+        int q = (t != t) ? 0 : (int)t;
+        words[i / 4] |= (uint32_t)(q & 0xFF) << (8 * (i % 4));
+      }
+      const bool all_zero = (words[0] | words[1] | words[2] | words[3] | words[4] | words[5] | words[6] | words[7]) == 0;
+      const uint32_t sbits = q8_device_scale(__builtin_bit_cast(uint16_t, (_Float16)scale), all_zero);
+      ((uint16_t*)meta)[b] = (uint16_t)sbits;
+      smax = abs_bits(sbits);
+      uint4* qp = (uint4*)quants + b * 2;
+      qp[0] = make_uint4(words[0], words[1], words[2], words[3]);
+      qp[1] = make_uint4(words[4], words[5], words[6], words[7]);
     }
-    const float d = bmax > bmin ? (bmax - bmin) / 15.0f : 1.0f;
-    const float m = bmin;
-    const float d_inv = d > 0.0f ? 1.0f / d : 0.0f;
-    const uint32_t dbits = __builtin_bit_cast(uint16_t, (_Float16)d);
-    const uint32_t mbits = __builtin_bit_cast(uint16_t, (_Float16)m);
-    ((uint32_t*)meta)[b] = dbits | (mbits << 16);
-    uint32_t words[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < 32; i++) {
-      float t = clamp_keep_nan(roundf((v[i] - m) * d_inv), 0.0f, 15.0f);
-      uint32_t nib = (t != t) ? 0u : (uint32_t)t;
-      words[i / 8] |= nib << (4 * (i % 8));
-    }
-    ((uint4*)quants)[b] = make_uint4(words[0], words[1], words[2], words[3]);
-  } else {
-    float amax = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 32; i++) {
-      float a = fabsf(v[i]);
-      if (a > amax) amax = a;
-    }
-    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
-    const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
-    uint32_t words[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < 32; i++) {
-      float t = clamp_keep_nan(roundf(v[i] * inv), -128.0f, 127.0f);
-      int q = (t != t) ? 0 : (int)t;
-      words[i / 4] |= (uint32_t)(q & 0xFF) << (8 * (i % 4));
-    }
-    const bool all_zero = (words[0] | words[1] | words[2] | words[3] | words[4] | words[5] | words[6] | words[7]) == 0;
-    ((uint16_t*)meta)[b] = (uint16_t)q8_device_scale(__builtin_bit_cast(uint16_t, (_Float16)scale), all_zero);
-    uint4* qp = (uint4*)quants + b * 2;
-    qp[0] = make_uint4(words[0], words[1], words[2], words[3]);
-    qp[1] = make_uint4(words[4], words[5], words[6], words[7]);
   }
+  publish_range(smax, mmax, range);
 }
 
 // ---- pointwise companions of the matmul in a decode layer ----
@@ -355,17 +381,17 @@ int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev)
   return 0;
 }
 
-int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* meta, void* quants) {
+int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* meta, void* quants, uint32_t* range2_dev) {
   hipLaunchKernelGGL(import_q8_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s,
-                     (const uint32_t*)ref_dev, nb, (uint16_t*)meta, (uint32_t*)quants);
+                     (const uint32_t*)ref_dev, nb, (uint16_t*)meta, (uint32_t*)quants, range2_dev);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }
 
 int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, uint32_t n, void* meta,
-                    void* quants) {
+                    void* quants, uint32_t* range2_dev) {
   dim3 grid((n + 255) / 256, k / 32);
-  hipLaunchKernelGGL(quantize_kernel, grid, dim3(256), 0, s, fmt, w_dev, k, n, meta, quants);
+  hipLaunchKernelGGL(quantize_kernel, grid, dim3(256), 0, s, fmt, w_dev, k, n, meta, quants, range2_dev);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

@@ -138,16 +138,20 @@ mgn_status check_range_flag(mgn_ctx* ctx) {
               "into fp16 pairs without rescaling: the affected outputs are wrong (the context was set to MGN_ACT_FP16_RANGE, or the route was forced)");
 }
 
-// Looks at every block's scale (and minimum) once, right after a weight's blocks are on the
-// device, and records whether the tiled MFMA kernel may take this weight.  Synchronises.
-mgn_status scan_weight_range(mgn_ctx* ctx, mgn_weight* w) {
-  uint32_t* dev = (uint32_t*)((char*)ctx->scratch + ctx->scratch_bytes) + ctx->n_counters;  // two spare words
-  hipError_t e = hipMemsetAsync(dev, 0, 8, ctx->stream);
-  if (e == hipSuccess) e = (hipError_t)mgn::launch_scale_range(ctx->stream, view_of(w), dev);
+// Whether the 32x32 MFMA kernel may take a weight depends on the largest |scale| and |min| over
+// its blocks.  The kernels that put the blocks on the device reduce them on the way into two spare
+// words of the context (range_words), which are zeroed before and read back after, in stream
+// order; the one synchronisation a weight's creation needs anyway then covers the read-back.
+uint32_t* range_words(mgn_ctx* ctx) { return (uint32_t*)((char*)ctx->scratch + ctx->scratch_bytes) + ctx->n_counters; }
+
+hipError_t clear_range_words(mgn_ctx* ctx) { return hipMemsetAsync(range_words(ctx), 0, 8, ctx->stream); }
+
+// Enqueues the read-back, synchronises and records the verdict in the weight.
+mgn_status finish_weight_range(mgn_ctx* ctx, mgn_weight* w, const char* what) {
   uint32_t host[2] = {0, 0};
-  if (e == hipSuccess) e = hipMemcpyAsync(host, dev, 8, hipMemcpyDeviceToHost, ctx->stream);
+  hipError_t e = hipMemcpyAsync(host, range_words(ctx), 8, hipMemcpyDeviceToHost, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
-  if (e != hipSuccess) return hip_fail(ctx, "weight range scan", e);
+  if (e != hipSuccess) return hip_fail(ctx, what, e);
   float smax, mmax;
   std::memcpy(&smax, &host[0], 4);
   std::memcpy(&mmax, &host[1], 4);
@@ -368,29 +372,29 @@ mgn_status mgn_weight_create_packed(mgn_ctx* ctx, mgn_fmt fmt, const uint8_t* pa
   mgn_weight* w = nullptr;
   mgn_status st = weight_alloc(ctx, fmt, rows, cols, &w);
   if (st != MGN_OK) return st;
-  hipError_t e = hipSuccess;
+  hipError_t e = clear_range_words(ctx);
   void* tmp = nullptr;
   if (fmt == MGN_FMT_Q4) {
-    // the reference layout is already "all scale|min words, then all nibbles"
-    e = hipMemcpyAsync(w->meta, packed, w->meta_bytes, hipMemcpyHostToDevice, ctx->stream);
+    // the reference layout is already "all scale|min words, then all nibbles": plain copies, and
+    // a pass over the scale words for their range
+    if (e == hipSuccess) e = hipMemcpyAsync(w->meta, packed, w->meta_bytes, hipMemcpyHostToDevice, ctx->stream);
     if (e == hipSuccess)
       e = hipMemcpyAsync(w->quants, packed + w->meta_bytes, w->quant_bytes, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = (hipError_t)mgn::launch_scale_range(ctx->stream, view_of(w), range_words(ctx));
   } else {
     const size_t bytes = w->nb * 36;
-    e = hipMalloc(&tmp, bytes);
+    if (e == hipSuccess) e = hipMalloc(&tmp, bytes);
     if (e == hipSuccess) e = hipMemcpyAsync(tmp, packed, bytes, hipMemcpyHostToDevice, ctx->stream);
-    if (e == hipSuccess) e = (hipError_t)mgn::launch_import_q8(ctx->stream, (const uint8_t*)tmp, w->nb, w->meta, w->quants);
+    if (e == hipSuccess)
+      e = (hipError_t)mgn::launch_import_q8(ctx->stream, (const uint8_t*)tmp, w->nb, w->meta, w->quants, range_words(ctx));
   }
-  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  // one synchronisation: the caller's bytes are free again, tmp can go, the range is known
+  if (e == hipSuccess) st = finish_weight_range(ctx, w, "weight upload");
+  else (void)hipStreamSynchronize(ctx->stream);
   if (tmp) (void)hipFree(tmp);
-  if (e != hipSuccess) {
+  if (e != hipSuccess || st != MGN_OK) {
     mgn_weight_free(ctx, w);
-    return hip_fail(ctx, "weight upload", e);
-  }
-  st = scan_weight_range(ctx, w);
-  if (st != MGN_OK) {
-    mgn_weight_free(ctx, w);
-    return st;
+    return e != hipSuccess ? hip_fail(ctx, "weight upload", e) : st;
   }
   *out = w;
   return MGN_OK;
@@ -440,13 +444,15 @@ mgn_status mgn_weight_create_device(mgn_ctx* ctx, mgn_fmt fmt, const mgn_buf* w_
     mgn_weight_free(ctx, w);
     return fail(ctx, MGN_EINVAL, "source buffer smaller than rows*cols floats");
   }
-  hipError_t e = (hipError_t)mgn::launch_quantize(ctx->stream, (int)fmt, (const float*)w_f32->ptr, (uint32_t)rows,
-                                                  (uint32_t)cols, w->meta, w->quants);
+  hipError_t e = clear_range_words(ctx);
+  if (e == hipSuccess)
+    e = (hipError_t)mgn::launch_quantize(ctx->stream, (int)fmt, (const float*)w_f32->ptr, (uint32_t)rows, (uint32_t)cols,
+                                         w->meta, w->quants, range_words(ctx));
   if (e != hipSuccess) {
     mgn_weight_free(ctx, w);
     return hip_fail(ctx, "quantize kernel", e);
   }
-  st = scan_weight_range(ctx, w);
+  st = finish_weight_range(ctx, w, "quantize kernel");
   if (st != MGN_OK) {
     mgn_weight_free(ctx, w);
     return st;

@@ -78,10 +78,12 @@ struct LaunchArgs {
 // kernels.hip
 int launch_dequantize(ihipStream_t* s, const WeightView& w, float* out_dev);  // out [k, n] f32
 int launch_export_q8(ihipStream_t* s, const WeightView& w, uint8_t* out_dev);  // 36-byte blocks
-int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* meta, void* quants);
-int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev);  // out: max |scale|, max |min| bits
+// range2_dev / out2_dev: two words, zero before the launch, that receive the bits of the largest
+// |scale| and the largest |min| (as f32) over the blocks the kernel writes or reads
+int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* meta, void* quants, uint32_t* range2_dev);
+int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev);
 int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, uint32_t n, void* meta,
-                    void* quants);
+                    void* quants, uint32_t* range2_dev);
 // in[rows][cols] -> out[cols][rows] (f32); cols at most 65535 * 32
 int launch_transpose(ihipStream_t* s, const float* in, float* out, uint32_t rows, uint32_t cols);
 // measurement aid: one pass of plain reads over the weight's quants and scales

@@ -671,6 +671,15 @@ def test_weights_with_huge_minima_and_scales_stay_on_the_matrix_cores(ctx, orc, 
         orc.assert_close(got1, want[:1], REL, ABS)
         wt.free()
     src.free()
+    # the verdict is the weight's own: an ordinary weight created next is taken by the 32x32x16 kernel
+    tame = synth.normal(992 + fmt, k * n, 0.02).reshape(k, n)
+    tame_packed = orc.quantize(fmt, tame)
+    tame_want = orc.matmul_f64(x, orc.dequantize(fmt, tame_packed, k, n))
+    src = ctx.upload(tame)
+    for wt in (ctx.weight(fmt, tame), ctx.weight_from_device(fmt, src, k, n), ctx.weight_from_packed(fmt, tame_packed, k, n)):
+        orc.assert_close(run_matmul(ctx, fmt, x, wt, ROUTES["gemm_mfma"]), tame_want, REL, ABS)
+        wt.free()
+    src.free()
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
