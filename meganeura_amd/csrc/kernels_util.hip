@@ -145,69 +145,120 @@ __device__ __forceinline__ float clamp_keep_nan(float v, float lo, float hi) {
 }
 
 // quantize_q4_0 / quantize_q8_0 (src/runtime.rs:2035-2102, 2143-2188) as a
-// kernel, one thread per block.  Every f32 operation rounds separately (no
-// contraction), division and roundf are the correctly rounded device forms,
-// and the f16 stores use round-to-nearest-even conversion, so the bytes equal
-// the host quantizer's.
+// kernel.  Every f32 operation rounds separately (no contraction), division and
+// roundf are the correctly rounded device forms, and the f16 stores use
+// round-to-nearest-even conversion, so the bytes equal the host quantizer's.
+//
+// The source is row-major [K, N], the blocks run down the columns (block n * K/32 + kb): a
+// workgroup takes 64 columns x 16 block rows, reads the source along the rows (256 bytes per
+// wave and load; a wave quantizes four block rows of its 64 columns, one after the other, a
+// thread the 32 values of one block at a time), parks scale words and quants in LDS and writes
+// them out along the columns: 16 consecutive blocks per column, 64 bytes of scale words and 256
+// (Q8: 512) bytes of quants in a run.  Writing each block from the thread that made it would
+// scatter 4- and 16-byte stores K/32 blocks apart.
 #pragma clang fp contract(off)
-__global__ __launch_bounds__(256) void quantize_kernel(int fmt, const float* __restrict__ w, uint32_t k,
-                                                       uint32_t n_cols, void* __restrict__ meta,
-                                                       void* __restrict__ quants, uint32_t* __restrict__ range) {
-  const uint32_t n = blockIdx.x * 256 + threadIdx.x;
-  const uint32_t kb = blockIdx.y;
-  uint32_t smax = 0, mmax = 0;  // this block's |scale| and |min| as stored (see publish_range)
-  if (n < n_cols) {
-    const uint32_t bpc = k / 32;
-    const size_t b = (size_t)n * bpc + kb;
-    const float* src = w + (size_t)kb * 32 * n_cols + n;
-    float v[32];
+constexpr int kQuantCols = 64, kQuantRows = 16;  // a workgroup's tile, in columns and block rows
+
+// Quantizes the 32 values v[] of one block: scale word(s) and quants as they are stored on the
+// device, and the bits of |scale| and |min| for the range (see publish_range).
+template <int FMT>
+__device__ __forceinline__ void quantize_block(const float (&v)[32], uint32_t* __restrict__ meta_word,
+                                               uint32_t (&words)[8], uint32_t* __restrict__ smax, uint32_t* __restrict__ mmax) {
+  if constexpr (FMT == MGN_FMT_Q4) {
+    float bmin = INFINITY, bmax = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 32; i++) v[i] = src[(size_t)i * n_cols];
-    if (fmt == MGN_FMT_Q4) {
-      float bmin = INFINITY, bmax = -INFINITY;
+    for (int i = 0; i < 32; i++) {
+      if (v[i] < bmin) bmin = v[i];
+      if (v[i] > bmax) bmax = v[i];
+    }
+    const float d = bmax > bmin ? (bmax - bmin) / 15.0f : 1.0f;
+    const float m = bmin;
+    const float d_inv = d > 0.0f ? 1.0f / d : 0.0f;
+    const uint32_t dbits = __builtin_bit_cast(uint16_t, (_Float16)d);
+    const uint32_t mbits = __builtin_bit_cast(uint16_t, (_Float16)m);
+    *meta_word = dbits | (mbits << 16);
+    *smax = max(*smax, abs_bits(dbits));
+    *mmax = max(*mmax, abs_bits(mbits));
 #pragma unroll
-      for (int i = 0; i < 32; i++) {
-        if (v[i] < bmin) bmin = v[i];
-        if (v[i] > bmax) bmax = v[i];
+    for (int t = 0; t < 4; t++) words[t] = 0;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      float t = clamp_keep_nan(roundf((v[i] - m) * d_inv), 0.0f, 15.0f);
+      uint32_t nib = (t != t) ? 0u : (uint32_t)t;
+      words[i / 8] |= nib << (4 * (i % 8));
+    }
+  } else {
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      float a = fabsf(v[i]);
+      if (a > amax) amax = a;
+    }
+    const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+    const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+#pragma unroll
+    for (int t = 0; t < 8; t++) words[t] = 0;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      float t = clamp_keep_nan(roundf(v[i] * inv), -128.0f, 127.0f);
+      int q = (t != t) ? 0 : (int)t;
+      words[i / 4] |= (uint32_t)(q & 0xFF) << (8 * (i % 4));
+    }
+    const bool all_zero = (words[0] | words[1] | words[2] | words[3] | words[4] | words[5] | words[6] | words[7]) == 0;
+    const uint32_t sbits = q8_device_scale(__builtin_bit_cast(uint16_t, (_Float16)scale), all_zero);
+    *meta_word = sbits;
+    *smax = max(*smax, abs_bits(sbits));
+  }
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__ w, uint32_t k, uint32_t n_cols,
+                                                       void* __restrict__ meta, void* __restrict__ quants,
+                                                       uint32_t* __restrict__ range) {
+  constexpr int QW = FMT == MGN_FMT_Q4 ? 4 : 8;  // dwords of quants per block
+  // [column][block row], a column's row padded by one entry so that the 64 columns a wave writes
+  // at a time spread over the banks
+  __shared__ uint32_t s_meta[kQuantCols][kQuantRows + 1];
+  __shared__ uint32_t s_quants[kQuantCols][kQuantRows * QW + 1];
+  const uint32_t tid = threadIdx.x, nl = tid & 63, wave = tid >> 6;
+  const uint32_t n0 = blockIdx.x * kQuantCols, kb0 = blockIdx.y * kQuantRows;
+  const uint32_t bpc = k / 32;
+  const uint32_t n = n0 + nl;
+  uint32_t smax = 0, mmax = 0;
+#pragma unroll
+  for (int j = 0; j < kQuantRows / 4; j++) {
+    const uint32_t kbl = 4 * j + wave, kb = kb0 + kbl;  // the same for the whole wave
+    if (kb < bpc && n < n_cols) {
+      const float* src = w + (size_t)kb * 32 * n_cols + n;
+      float v[32];
+#pragma unroll
+      for (int i = 0; i < 32; i++) v[i] = src[(size_t)i * n_cols];
+      uint32_t mword, words[8];
+      quantize_block<FMT>(v, &mword, words, &smax, &mmax);
+      s_meta[nl][kbl] = mword;
+#pragma unroll
+      for (int t = 0; t < QW; t++) s_quants[nl][kbl * QW + t] = words[t];
+    }
+  }
+  __syncthreads();
+  // write-out: 16 consecutive threads take the 16 block rows of one column
+  const uint32_t rows_live = min((uint32_t)kQuantRows, bpc - kb0);
+#pragma unroll
+  for (int j = 0; j < kQuantCols * kQuantRows / 256; j++) {
+    const uint32_t idx = tid + 256 * j, col = idx / kQuantRows, kbl = idx % kQuantRows;
+    if (n0 + col < n_cols && kbl < rows_live) {
+      const size_t b = (size_t)(n0 + col) * bpc + kb0 + kbl;
+      if constexpr (FMT == MGN_FMT_Q4) {
+        ((uint32_t*)meta)[b] = s_meta[col][kbl];
+        ((uint4*)quants)[b] = make_uint4(s_quants[col][kbl * 4], s_quants[col][kbl * 4 + 1], s_quants[col][kbl * 4 + 2],
+                                         s_quants[col][kbl * 4 + 3]);
+      } else {
+        ((uint16_t*)meta)[b] = (uint16_t)s_meta[col][kbl];
+        uint4* qp = (uint4*)quants + b * 2;
+        qp[0] = make_uint4(s_quants[col][kbl * 8], s_quants[col][kbl * 8 + 1], s_quants[col][kbl * 8 + 2], s_quants[col][kbl * 8 + 3]);
+        qp[1] = make_uint4(s_quants[col][kbl * 8 + 4], s_quants[col][kbl * 8 + 5], s_quants[col][kbl * 8 + 6],
+                           s_quants[col][kbl * 8 + 7]);
       }
-      const float d = bmax > bmin ? (bmax - bmin) / 15.0f : 1.0f;
-      const float m = bmin;
-      const float d_inv = d > 0.0f ? 1.0f / d : 0.0f;
-      const uint32_t dbits = __builtin_bit_cast(uint16_t, (_Float16)d);
-      const uint32_t mbits = __builtin_bit_cast(uint16_t, (_Float16)m);
-      ((uint32_t*)meta)[b] = dbits | (mbits << 16);
-      smax = abs_bits(dbits), mmax = abs_bits(mbits);
-      uint32_t words[4] = {0, 0, 0, 0};
-#pragma unroll
-      for (int i = 0; i < 32; i++) {
-        float t = clamp_keep_nan(roundf((v[i] - m) * d_inv), 0.0f, 15.0f);
-        uint32_t nib = (t != t) ? 0u : (uint32_t)t;
-        words[i / 8] |= nib << (4 * (i % 8));
-      }
-      ((uint4*)quants)[b] = make_uint4(words[0], words[1], words[2], words[3]);
-    } else {
-      float amax = 0.0f;
-#pragma unroll
-      for (int i = 0; i < 32; i++) {
-        float a = fabsf(v[i]);
-        if (a > amax) amax = a;
-      }
-      const float scale = amax > 0.0f ? amax / 127.0f : 1.0f;
-      const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
-      uint32_t words[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-      for (int i = 0; i < 32; i++) {
-        float t = clamp_keep_nan(roundf(v[i] * inv), -128.0f, 127.0f);
-        int q = (t != t) ? 0 : (int)t;
-        words[i / 4] |= (uint32_t)(q & 0xFF) << (8 * (i % 4));
-      }
-      const bool all_zero = (words[0] | words[1] | words[2] | words[3] | words[4] | words[5] | words[6] | words[7]) == 0;
-      const uint32_t sbits = q8_device_scale(__builtin_bit_cast(uint16_t, (_Float16)scale), all_zero);
-      ((uint16_t*)meta)[b] = (uint16_t)sbits;
-      smax = abs_bits(sbits);
-      uint4* qp = (uint4*)quants + b * 2;
-      qp[0] = make_uint4(words[0], words[1], words[2], words[3]);
-      qp[1] = make_uint4(words[4], words[5], words[6], words[7]);
     }
   }
   publish_range(smax, mmax, range);
@@ -390,8 +441,10 @@ int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* m
 
 int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, uint32_t n, void* meta,
                     void* quants, uint32_t* range2_dev) {
-  dim3 grid((n + 255) / 256, k / 32);
-  hipLaunchKernelGGL(quantize_kernel, grid, dim3(256), 0, s, fmt, w_dev, k, n, meta, quants, range2_dev);
+  dim3 grid((n + kQuantCols - 1) / kQuantCols, (k / 32 + kQuantRows - 1) / kQuantRows);
+  if (grid.y > 65535) return (int)hipErrorInvalidValue;
+  if (fmt == MGN_FMT_Q4) hipLaunchKernelGGL(quantize_kernel<MGN_FMT_Q4>, grid, dim3(256), 0, s, w_dev, k, n, meta, quants, range2_dev);
+  else hipLaunchKernelGGL(quantize_kernel<MGN_FMT_Q8>, grid, dim3(256), 0, s, w_dev, k, n, meta, quants, range2_dev);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }
