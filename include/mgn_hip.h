@@ -121,7 +121,9 @@ mgn_status mgn_dequantize_ref(mgn_fmt fmt, const uint8_t* in, size_t rows, size_
 /* ---- quantized weights on the device
  * Session::set_parameter for a Q4/Q8 parameter (src/runtime.rs:2327-2345):
  * quantize f32 [rows, cols] and place it in device memory.  The device layout
- * is private; mgn_weight_export_ref gives back the reference's bytes. */
+ * is private; mgn_weight_export_ref gives back the reference's bytes.  (The values are
+ * uploaded and packed by the device quantizer, whose bytes equal mgn_quantize_ref's; when the
+ * device has no room for the f32 copy, the host packs and the bytes are uploaded.) */
 mgn_status mgn_weight_create(mgn_ctx* ctx, mgn_fmt fmt, const float* w, size_t rows, size_t cols,
                              mgn_weight** out);
 /* Same from bytes already in the reference layout (what load_checkpoint copies
