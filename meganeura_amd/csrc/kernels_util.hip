@@ -264,6 +264,36 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* __restrict__
   publish_range(smax, mmax, range);
 }
 
+// The same for a weight stored [N, K] row-major (the table of a matmul_bt): block b = n * K/32 + kb
+// is the 32 consecutive floats from 32 b on, so a thread reads its block as eight float4 and the
+// blocks leave in the order they are stored.
+template <int FMT>
+__global__ __launch_bounds__(256) void quantize_nk_kernel(const float4* __restrict__ w_nk, size_t nb, void* __restrict__ meta,
+                                                          void* __restrict__ quants, uint32_t* __restrict__ range) {
+  const size_t b = (size_t)blockIdx.x * 256 + threadIdx.x;
+  uint32_t smax = 0, mmax = 0;
+  if (b < nb) {
+    float v[32];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const float4 x = w_nk[b * 8 + i];
+      v[4 * i] = x.x, v[4 * i + 1] = x.y, v[4 * i + 2] = x.z, v[4 * i + 3] = x.w;
+    }
+    uint32_t mword, words[8];
+    quantize_block<FMT>(v, &mword, words, &smax, &mmax);
+    if constexpr (FMT == MGN_FMT_Q4) {
+      ((uint32_t*)meta)[b] = mword;
+      ((uint4*)quants)[b] = make_uint4(words[0], words[1], words[2], words[3]);
+    } else {
+      ((uint16_t*)meta)[b] = (uint16_t)mword;
+      uint4* qp = (uint4*)quants + b * 2;
+      qp[0] = make_uint4(words[0], words[1], words[2], words[3]);
+      qp[1] = make_uint4(words[4], words[5], words[6], words[7]);
+    }
+  }
+  publish_range(smax, mmax, range);
+}
+
 // ---- pointwise companions of the matmul in a decode layer ----
 
 __global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
@@ -435,6 +465,18 @@ int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev)
 int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* meta, void* quants, uint32_t* range2_dev) {
   hipLaunchKernelGGL(import_q8_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s,
                      (const uint32_t*)ref_dev, nb, (uint16_t*)meta, (uint32_t*)quants, range2_dev);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_quantize_nk(ihipStream_t* s, int fmt, const float* w_nk_dev, uint32_t k, uint32_t n, void* meta, void* quants,
+                       uint32_t* range2_dev) {
+  const size_t nb = (size_t)(k / 32) * n;
+  const dim3 grid((unsigned)((nb + 255) / 256));
+  if (fmt == MGN_FMT_Q4)
+    hipLaunchKernelGGL(quantize_nk_kernel<MGN_FMT_Q4>, grid, dim3(256), 0, s, (const float4*)w_nk_dev, nb, meta, quants, range2_dev);
+  else
+    hipLaunchKernelGGL(quantize_nk_kernel<MGN_FMT_Q8>, grid, dim3(256), 0, s, (const float4*)w_nk_dev, nb, meta, quants, range2_dev);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

@@ -400,6 +400,52 @@ mgn_status mgn_weight_create_packed(mgn_ctx* ctx, mgn_fmt fmt, const uint8_t* pa
   return MGN_OK;
 }
 
+// A weight from f32 values on the device, stored [rows, cols] (K major) or, nk, [cols, rows]: the
+// quantizer kernel packs them and reduces the range of the block constants on the way.  Synchronises.
+static mgn_status weight_from_device_f32(mgn_ctx* ctx, mgn_fmt fmt, const void* src, size_t src_bytes, size_t rows,
+                                         size_t cols, bool nk, mgn_weight** out) {
+  mgn_weight* w = nullptr;
+  mgn_status st = weight_alloc(ctx, fmt, rows, cols, &w);
+  if (st != MGN_OK) return st;
+  if (src_bytes / sizeof(float) < rows * cols) {
+    mgn_weight_free(ctx, w);
+    return fail(ctx, MGN_EINVAL, "source buffer smaller than rows*cols floats");
+  }
+  hipError_t e = clear_range_words(ctx);
+  if (e == hipSuccess)
+    e = (hipError_t)(nk ? mgn::launch_quantize_nk : mgn::launch_quantize)(ctx->stream, (int)fmt, (const float*)src, (uint32_t)rows,
+                                                                          (uint32_t)cols, w->meta, w->quants, range_words(ctx));
+  if (e != hipSuccess) {
+    mgn_weight_free(ctx, w);
+    return hip_fail(ctx, "quantize kernel", e);
+  }
+  st = finish_weight_range(ctx, w, "quantize kernel");
+  if (st != MGN_OK) {
+    mgn_weight_free(ctx, w);
+    return st;
+  }
+  *out = w;
+  return MGN_OK;
+}
+
+// Uploads host f32 values into a staging buffer and packs them there (see mgn_weight_create).
+// MGN_ENOMEM: no room for the staging copy or the weight; the caller may pack on the host instead.
+static mgn_status weight_from_host_f32(mgn_ctx* ctx, mgn_fmt fmt, const float* wdata, size_t rows, size_t cols, bool nk,
+                                       mgn_weight** out) {
+  void* staged = nullptr;
+  const size_t bytes = rows * cols * sizeof(float);
+  if (hipMalloc(&staged, bytes) != hipSuccess) {
+    (void)hipGetLastError();  // out of device memory for the staging copy: not an error of the call
+    return MGN_ENOMEM;
+  }
+  const hipError_t e = hipMemcpyAsync(staged, wdata, bytes, hipMemcpyHostToDevice, ctx->stream);
+  const mgn_status st = e == hipSuccess ? weight_from_device_f32(ctx, fmt, staged, bytes, rows, cols, nk, out)
+                                        : hip_fail(ctx, "weight upload", e);
+  if (e != hipSuccess) (void)hipStreamSynchronize(ctx->stream);
+  (void)hipFree(staged);
+  return st;
+}
+
 mgn_status mgn_weight_create(mgn_ctx* ctx, mgn_fmt fmt, const float* wdata, size_t rows, size_t cols,
                              mgn_weight** out) {
   if (!ctx || !out || !wdata) return fail(ctx, MGN_EINVAL, "null argument");
@@ -410,17 +456,8 @@ mgn_status mgn_weight_create(mgn_ctx* ctx, mgn_fmt fmt, const float* wdata, size
   // The f32 values go up as they are and the device quantizer packs them (the same bytes as the
   // host quantizer's, three to four times sooner on a 4096 x 14336 weight: 9 ms against 28-35 ms)
   // when there is device memory for them; otherwise the host packs and the bytes go up.
-  void* staged = nullptr;
-  if (hipMalloc(&staged, rows * cols * sizeof(float)) == hipSuccess) {
-    mgn_buf src{staged, rows * cols * sizeof(float)};
-    hipError_t e = hipMemcpyAsync(staged, wdata, src.bytes, hipMemcpyHostToDevice, ctx->stream);
-    mgn_status st = e == hipSuccess ? mgn_weight_create_device(ctx, fmt, &src, rows, cols, out)  // synchronises
-                                    : hip_fail(ctx, "weight upload", e);
-    if (e != hipSuccess) (void)hipStreamSynchronize(ctx->stream);
-    (void)hipFree(staged);
-    if (st != MGN_ENOMEM) return st;  // (without the staging copy the packed bytes may still fit)
-  }
-  (void)hipGetLastError();  // out of device memory for the staging copy: not an error of this call
+  const mgn_status direct = weight_from_host_f32(ctx, fmt, wdata, rows, cols, false, out);
+  if (direct != MGN_ENOMEM) return direct;
   std::vector<uint8_t> packed;
   try {
     packed.resize(mgn_packed_size(fmt, rows, cols));
@@ -438,6 +475,8 @@ mgn_status mgn_weight_create_nk(mgn_ctx* ctx, mgn_fmt fmt, const float* w_nk, si
   if (!valid_fmt(fmt)) return fail(ctx, MGN_EINVAL, "unknown weight format");
   if (k_cols % 32 != 0) return fail(ctx, MGN_EINVAL, "quantized weights require the K dim to be a multiple of 32");
   if (n_rows == 0 || k_cols == 0) return fail(ctx, MGN_EINVAL, "empty weight");
+  const mgn_status direct = weight_from_host_f32(ctx, fmt, w_nk, k_cols, n_rows, true, out);  // as mgn_weight_create
+  if (direct != MGN_ENOMEM) return direct;
   std::vector<uint8_t> packed;
   try {
     packed.resize(mgn_packed_size(fmt, k_cols, n_rows));
@@ -451,28 +490,7 @@ mgn_status mgn_weight_create_nk(mgn_ctx* ctx, mgn_fmt fmt, const float* w_nk, si
 mgn_status mgn_weight_create_device(mgn_ctx* ctx, mgn_fmt fmt, const mgn_buf* w_f32, size_t rows, size_t cols,
                                     mgn_weight** out) {
   if (!w_f32) return fail(ctx, MGN_EINVAL, "null argument");
-  mgn_weight* w = nullptr;
-  mgn_status st = weight_alloc(ctx, fmt, rows, cols, &w);
-  if (st != MGN_OK) return st;
-  if (w_f32->bytes / sizeof(float) < rows * cols) {
-    mgn_weight_free(ctx, w);
-    return fail(ctx, MGN_EINVAL, "source buffer smaller than rows*cols floats");
-  }
-  hipError_t e = clear_range_words(ctx);
-  if (e == hipSuccess)
-    e = (hipError_t)mgn::launch_quantize(ctx->stream, (int)fmt, (const float*)w_f32->ptr, (uint32_t)rows, (uint32_t)cols,
-                                         w->meta, w->quants, range_words(ctx));
-  if (e != hipSuccess) {
-    mgn_weight_free(ctx, w);
-    return hip_fail(ctx, "quantize kernel", e);
-  }
-  st = finish_weight_range(ctx, w, "quantize kernel");
-  if (st != MGN_OK) {
-    mgn_weight_free(ctx, w);
-    return st;
-  }
-  *out = w;
-  return MGN_OK;
+  return weight_from_device_f32(ctx, fmt, w_f32->ptr, w_f32->bytes, rows, cols, false, out);
 }
 
 void mgn_weight_free(mgn_ctx* ctx, mgn_weight* w) {

@@ -84,6 +84,9 @@ int launch_import_q8(ihipStream_t* s, const uint8_t* ref_dev, size_t nb, void* m
 int launch_scale_range(ihipStream_t* s, const WeightView& w, uint32_t* out2_dev);
 int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, uint32_t n, void* meta,
                     void* quants, uint32_t* range2_dev);
+// the same from a matrix stored [n, k] row-major (16-byte aligned)
+int launch_quantize_nk(ihipStream_t* s, int fmt, const float* w_nk_dev, uint32_t k, uint32_t n, void* meta, void* quants,
+                       uint32_t* range2_dev);
 // in[rows][cols] -> out[cols][rows] (f32); cols at most 65535 * 32
 int launch_transpose(ihipStream_t* s, const float* in, float* out, uint32_t rows, uint32_t cols);
 // measurement aid: one pass of plain reads over the weight's quants and scales

@@ -63,6 +63,10 @@ def test_device_weight_is_bit_exact(ctx, orc, fmt, shape):
     wt = ctx.weight_from_device(fmt, src, k, n)
     assert (wt.export_ref() == want_packed).all()
     wt.free(); src.free()
+    # and from the same matrix stored [N, K], as a matmul_bt operand keeps it
+    wt = ctx.weight_nk(fmt, np.ascontiguousarray(w.T))
+    assert (wt.export_ref() == want_packed).all()
+    wt.free()
 
 
 def test_device_quantizer_matches_golden_vectors(ctx):
