@@ -345,7 +345,7 @@ __device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t*
 struct TileTail {  // arguments first needed in the epilogue
   const float* dres;
   float* c;
-  float* scratch;      // [parts][row groups * R * 16][n] partial results when parts > 1
+  float* scratch;      // partial results when parts > 1 (general kernel: [parts][row groups * R * 16][n])
   uint32_t* counters;  // one arrival counter per (row group, column group), zero between launches
   uint32_t epilogue;   // unary operations on the output (apply_epilogue)
 };
@@ -784,7 +784,8 @@ __host__ __device__ constexpr uint32_t meta_stride(int fmt, uint32_t nsl) { retu
 template <int FMT, bool F32A, int R, int Q, bool PARK>
 __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restrict__ a, const void* __restrict__ meta_arg,
                                                              const void* __restrict__ quants_arg, uint32_t m, uint32_t kdim,
-                                                             uint32_t n, uint32_t parts, uint32_t nslices, TileTail tail) {
+                                                             uint32_t n, uint32_t parts, uint32_t nslices, uint32_t colgroups,
+                                                             TileTail tail) {
   constexpr uint32_t UNITS = image_units(F32A);
   constexpr float kOpScale = FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f;
   constexpr int QB = FMT == MGN_FMT_Q4 ? 16 : 32;
@@ -803,8 +804,14 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t c = lane & 15, g = lane >> 4;
-  const uint32_t part = blockIdx.x, cg = blockIdx.y;
-  const uint32_t row0 = blockIdx.z * (R * 16);  // first row of this workgroup's row group
+  // grid = (column groups x row groups, rounded up to a multiple of 8; K parts): workgroups go to the
+  // eight XCDs in turn by their linear index, so the K parts of a (column group, row group) run on
+  // one XCD, which their hand-over below measures 0.5 us better than spread over all eight
+  const uint32_t part = blockIdx.y;
+  const uint32_t rg = blockIdx.x / colgroups, cg = blockIdx.x - rg * colgroups;
+  const uint32_t rowgroups = (m + R * 16 - 1) / (R * 16);
+  if (rg >= rowgroups) return;            // padding of the grid
+  const uint32_t row0 = rg * (R * 16);    // first row of this workgroup's row group
   const uint32_t bpc = kdim / 32;
   const uint32_t pair0 = (cg * 8 + wave) * Q;  // this wave's first pair of column tiles
   const uint32_t sl0 = part * NSL;             // first slice of this part
@@ -968,27 +975,33 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   __builtin_amdgcn_sched_barrier(0);
 
   if (parts > 1) {
-    // K parts of other workgroups: the last one to arrive adds them up in part order (see above)
-    const size_t plane = (size_t)gridDim.z * (R * 16) * n;  // floats per part
+    // K parts of other workgroups: the last one to arrive adds them up in part order (see above).
+    // The partial tiles travel in register order: the float4 a lane holds for (pair, side, row tile)
+    // goes out and comes back as one 128-bit access, 1 KiB per wave and instruction, at
+    //   (((part * row groups + row group) * column groups + column group) * 8 + wave) * Q * kSide * R + slot
+    // Every XCD has its own L2, so both directions carry sc1 (device scope).  What the read-back costs
+    // is one trip to the tiles (about 1 us) plus 0.15 us for every further part: a CU takes in about
+    // 100 GB/s, wherever the tiles sit (14 parts of 14336 x 4096 at M = 16: 3 us of 16.2).
+    constexpr uint32_t kSlots = Q * kSide * R;
+    constexpr int kDeviceScope = 16;  // the sc1 bit of a buffer instruction's cache policy
+    const uint32_t wgs_per_part = rowgroups * colgroups;
+    const __amdgpu_buffer_rsrc_t partials =
+        __builtin_amdgcn_make_buffer_rsrc(tail.scratch, 0, parts * wgs_per_part * (8u * kSlots * 1024u), 0x00020000);
+    const uint32_t my_off = ((rg * colgroups + cg) * 8u + wave) * (kSlots * 1024u) + lane * 16u;
+    const uint32_t part_stride = wgs_per_part * (8u * kSlots * 1024u);
 #pragma unroll
     for (int p = 0; p < Q; p++)
 #pragma unroll
-      for (int u = 0; u < kSide; u++) {
-        const uint32_t col = ((pair0 + p) * kSide + u) * 16 + c;
-        if (col < n) {
-          float* const mine = tail.scratch + (size_t)part * plane + (size_t)row0 * n + col;
+      for (int u = 0; u < kSide; u++)
 #pragma unroll
-          for (int r = 0; r < R; r++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-              __hip_atomic_store(mine + (size_t)(r * 16 + 4 * g + i) * n, res[p][u][r][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-      }
+        for (int r = 0; r < R; r++)
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, res[p][u][r]), partials,
+                                                 part * part_stride + my_off + ((p * kSide + u) * R + r) * 1024u, 0, kDeviceScope);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     uint32_t* const flag = (uint32_t*)lds4;
     if (tid == 0) {
-      uint32_t* const ctr = tail.counters + blockIdx.z * gridDim.y + cg;
+      uint32_t* const ctr = tail.counters + rg * colgroups + cg;
       const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const bool last = seen == parts - 1;
       if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
@@ -998,31 +1011,21 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
     __builtin_amdgcn_sched_barrier(0);
     if (*flag == 0u) return;
     // the parts' tiles, several parts in flight at a time, added in part order
-    const float* base[Q][kSide];
 #pragma unroll
     for (int p = 0; p < Q; p++)
 #pragma unroll
-      for (int u = 0; u < kSide; u++) {
-        base[p][u] = tail.scratch + min(((pair0 + p) * kSide + u) * 16 + c, n - 1) + (size_t)(row0 + 4 * g) * n;
+      for (int u = 0; u < kSide; u++)
 #pragma unroll
         for (int r = 0; r < R; r++) res[p][u][r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-      }
     auto add_parts = [&](auto group) {
       constexpr int PG = decltype(group)::value;
       for (uint32_t pp0 = 0; pp0 < parts; pp0 += PG) {
-        float v[PG][Q][kSide][R][4];
+        u32x4_t v[PG][kSlots];
 #pragma unroll
         for (int j = 0; j < PG; j++) {
-          const size_t po = (size_t)min(pp0 + j, parts - 1) * plane;  // (the surplus repeats the last part)
+          const uint32_t po = min(pp0 + j, parts - 1) * part_stride + my_off;  // (the surplus repeats the last part)
 #pragma unroll
-          for (int p = 0; p < Q; p++)
-#pragma unroll
-            for (int u = 0; u < kSide; u++)
-#pragma unroll
-              for (int r = 0; r < R; r++)
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-                  v[j][p][u][r][i] = __hip_atomic_load(base[p][u] + po + (size_t)(r * 16 + i) * n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (uint32_t t = 0; t < kSlots; t++) v[j][t] = __builtin_amdgcn_raw_buffer_load_b128(partials, po + t * 1024u, 0, kDeviceScope);
         }
 #pragma unroll
         for (int j = 0; j < PG; j++) {
@@ -1032,9 +1035,11 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
 #pragma unroll
             for (int u = 0; u < kSide; u++)
 #pragma unroll
-              for (int r = 0; r < R; r++)
+              for (int r = 0; r < R; r++) {
+                const floatx4 t = __builtin_bit_cast(floatx4, v[j][(p * kSide + u) * R + r]);
 #pragma unroll
-                for (int i = 0; i < 4; i++) res[p][u][r][i] = live ? res[p][u][r][i] + v[j][p][u][r][i] : res[p][u][r][i];
+                for (int i = 0; i < 4; i++) res[p][u][r][i] = live ? res[p][u][r][i] + t[i] : res[p][u][r][i];
+              }
         }
       }
     };
@@ -1097,12 +1102,14 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
     const uint32_t parts = (nslices + nsl - 1) / nsl;
     const uint32_t rowgroups = (x.m + 16 * r - 1) / (16 * r);
     if (rowgroups > 65535) continue;
-    const size_t partial = parts > 1 ? (size_t)parts * rowgroups * r * 16 * x.w.n * 4 : 0;
-    if (partial > x.scratch_bytes) continue;
     for (uint32_t q = 1; q <= (r == 1 ? 2u : 1u); q++) {
       const uint32_t per_wg = 8 * kSide * q;
       const uint32_t colgroups = (n_tiles + per_wg - 1) / per_wg;
-      if (colgroups > 65535 || (parts > 1 && (uint64_t)colgroups * rowgroups > x.n_counters)) continue;
+      if (parts > 65535 || (uint64_t)colgroups * rowgroups > 0x7FFFFFF0ull) continue;
+      if (parts > 1 && (uint64_t)colgroups * rowgroups > x.n_counters) continue;
+      // a workgroup's partial tile: 8 waves x (q kSide r) float4 per lane
+      const uint64_t partial = parts > 1 ? (uint64_t)parts * rowgroups * colgroups * (8u * q * kSide * r * 1024u) : 0;
+      if (partial > x.scratch_bytes || partial >= (1ull << 32)) continue;
       const uint64_t wgs = (uint64_t)parts * colgroups * rowgroups;
       const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q * r * nsl / 4.0) * (r == 2 ? 0.9 : 1.0) + (parts > 1 ? 1.0 : 0.0);
       if (best == 0 || cost < best) {
@@ -1126,8 +1133,11 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
   const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue};
-  hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups, p.rowgroups), dim3(512), p.lds, s, x.a, x.w.meta, x.w.quants, x.m, x.w.k,
-                     x.w.n, p.parts, p.nslices, tail);
+  // (column groups x row groups, K parts); with K parts the first is rounded up to a multiple of 8 (see the kernel)
+  const uint64_t groups = (uint64_t)p.colgroups * p.rowgroups;
+  const dim3 grid((unsigned)(p.parts > 1 ? (groups + 7) / 8 * 8 : groups), p.parts, 1);
+  hipLaunchKernelGGL(kern, grid, dim3(512), p.lds, s, x.a, x.w.meta, x.w.quants, x.m, x.w.k, x.w.n, p.parts, p.nslices,
+                     p.colgroups, tail);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

@@ -80,8 +80,9 @@ def check_gemm(p, fmt, m, k, n, f16):
 
 def check_tile(p, fmt, m, k, n, f16):
     """MGN_ROUTE_TILE_MFMA: tiles of 16 columns, K in slices of 256 elements, `full_steps` row tiles of 16 rows
-    per workgroup.  quads_per_wave == 0: the form that keeps the activation images in LDS (grid =
-    (K parts, column groups, row groups of 16 or 32 rows), 8 waves with one or two pairs of tiles each, parts of
+    per workgroup.  quads_per_wave == 0: the form that keeps the activation images in LDS (grid, as the plan
+    reports it: (K parts, column groups, row groups of 16 or 32 rows); launched with the groups in x, rounded
+    up to a multiple of 8, and the parts in y), 8 waves with one or two pairs of tiles each, parts of
     4 slices; row groups of 32 only with fp16 activations); otherwise the general form (grid = (K parts, column groups, row groups),
     `k_splits` waves per tile) in `quads_per_wave` launches over blocks of rows."""
     nslices, n_tiles = ceil_div(k, 256), ceil_div(n, 16)
@@ -97,7 +98,9 @@ def check_tile(p, fmt, m, k, n, f16):
         assert p.steps == 4 and p.waves_n in (16, 32)
         assert p.full_steps == 1 or f16  # row groups of 32 are for fp16 activations
         assert p.k_parts == ceil_div(nslices, p.steps)
-        partial = p.k_parts * p.grid[2] * rows * n * 4 if p.k_parts > 1 else 0
+        # partial tiles in whole workgroup slots: 8 waves x (pairs x 2 tiles x row tiles) float4 per lane
+        slot = 8 * (p.waves_n // 16) * 2 * p.full_steps * 1024
+        partial = p.k_parts * p.grid[2] * p.grid[1] * slot if p.k_parts > 1 else 0
         assert p.workspace_bytes == partial <= WORKSPACE
         if p.k_parts > 1:
             assert p.grid[1] * p.grid[2] <= COUNTERS
