@@ -77,7 +77,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c5_q4_m1_4096x14336": 37.01e6,
     "c5_q8_m1_4096x14336": 63.59e6,
     "c5_q4_m4_14336x4096": 39.6e6,
-    "c5_q4_m16_4096x14336": 45.8e6,
+    "c5_q4_m16_4096x14336": 47.4e6,
     "c4_q4_prefill_up_512x1024x3072": 19.1e6,
     "c3_q4_lm_head_576x49152": 18.03e6,
     "c1_q8_up_576x1536": 1.17e6,
@@ -86,7 +86,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c4_q4_prefill_down_512x3072x1024": 25.5e6,
     "c5_q4_m1_14336x4096": 37.4e6,
     "c5_q4_m4_4096x14336": 37.8e6,
-    "c5_q8_m16_4096x14336": 75.2e6,
+    "c5_q8_m16_4096x14336": 73.1e6,
 }
 
 
