@@ -1324,11 +1324,14 @@ bool tile_mfma_supported(const LaunchArgs& x) {
 }
 
 // Where the resident kernel measured faster than the 32x32 tiled one, whatever is known about
-// the activations.  Up to 16 rows: K >= 544 and one round of workgroups that fills at least three
-// quarters of the CUs (4096 x 14336 at M = 5..16: 12.5 us against 17.0 us; 14336 x 4096, 14 K parts:
-// 15.5-15.9 against 17.6-18.0, Q8 18.3-19.2 against 21.3-22.9; on smaller shapes the conversion in
-// every workgroup and the parts' hand-over cost more than the tiled kernel's whole call, and so
-// does a second round: 5120 x 14336 22.6 against 19.5).  17 to 32 rows of f32 activations, where the tiled kernel runs twice the MFMAs: whenever
+// the activations.  Up to 16 rows: K >= 544 and workgroups that fill at least three quarters of
+// their rounds over the CUs (4096 x 14336 at M = 5..16: 12.5 us against 17.0 us; 14336 x 4096, 14 K
+// parts: 15.5-15.9 against 17.6-18.0, Q8 18.3-19.2 against 21.3-22.9; 4096 x 49152, 1.5 rounds: 36.3
+// against 43.7, Q8 55.2 against 55.9; 8192 x 28672, 1.75 rounds: 39.9 against 47.8, Q8 59.9 against
+// 65.1; on smaller shapes the conversion in every workgroup and the parts' hand-over cost more than
+// the tiled kernel's whole call, and so does a round that stays half empty: 5120 x 14336, 0.55 of a
+// round, 22.9 against 20.3, Q8 34.3 against 25.1; 6144 x 14336, 0.66: 23.0 against 22.2, Q8 33.4
+// against 28.7).  17 to 32 rows of f32 activations, where the tiled kernel runs twice the MFMAs: whenever
 // the two row groups' workgroups fit one round (576 x 576: 8.1 against 11.7 us, 4096 x 4096: 12.5
 // against 16.5, 14336 x 1536: 17.6 against 23.2; with more workgroups the weights' second pass
 // costs more: 576 x 49152 16.5 against 15.2, 14336 x 4096 29.4 against 27.1, and so do many K
@@ -1348,7 +1351,8 @@ bool tile_mfma_preferred(const LaunchArgs& x) {
     return !x.a_is_f16 && wgs <= (uint64_t)x.num_cus && (x.w.fmt == MGN_FMT_Q4 || rp.q == 1) &&
            (rp.parts <= 4 || 2 * wgs <= (uint64_t)x.num_cus);
   if (rp.r != 1 || rp.nslices < 3) return false;
-  return wgs <= (uint64_t)x.num_cus && 4 * wgs >= 3 * (uint64_t)x.num_cus;
+  const uint64_t rounds = (wgs + x.num_cus - 1) / x.num_cus;
+  return 4 * wgs >= 3 * rounds * (uint64_t)x.num_cus;
 }
 
 bool describe_tile_mfma(const LaunchArgs& x, mgn_plan_info* out) {

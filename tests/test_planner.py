@@ -163,7 +163,8 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
             p = capi.matmul_plan(fmt, 16, 14336, 4096, fp16_range=promised)   # 14 K parts, still one round
             assert p.route == TILE_MFMA and p.quads_per_wave == 0 and list(p.grid) == [14, 16, 1]
         # elsewhere the 32x32 kernel is ahead, and runs when the activations are fp16 or promised to be in its range
-        assert capi.matmul_plan(fmt, 16, 5120, 14336, fp16_range=True).route == GEMM_MFMA  # two rounds of workgroups
+        assert capi.matmul_plan(fmt, 16, 5120, 14336, fp16_range=True).route == GEMM_MFMA  # 0.55 of a round of workgroups
+        assert capi.matmul_plan(fmt, 16, 4096, 49152, fp16_range=True).route == TILE_MFMA  # 1.5 rounds, all but full
         assert capi.matmul_plan(fmt, 16, 4096, 4096, fp16_range=True).route == GEMM_MFMA   # a quarter of the CUs
         assert capi.matmul_plan(fmt, 17, 14336, 4096, fp16_range=True).route == GEMM_MFMA  # two rounds of workgroups
         assert capi.matmul_plan(fmt, 17, 4096, 4096, fp16_range=True).route == TILE_MFMA   # two row groups of 16, one round
