@@ -83,7 +83,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c1_q8_up_576x1536": 1.17e6,
     "c2_q4_gate_up_576x3072": 1.32e6,
     "c2_q4_down_1536x576_add": 0.72e6,
-    "c4_q4_prefill_down_512x3072x1024": 25.5e6,
+    "c4_q4_prefill_down_512x3072x1024": 31.7e6,
     "c5_q4_m1_14336x4096": 37.4e6,
     "c5_q4_m4_4096x14336": 37.8e6,
     "c5_q8_m16_4096x14336": 73.1e6,

@@ -1340,18 +1340,24 @@ bool tile_mfma_supported(const LaunchArgs& x) {
 // 28.0).  Beyond 32 rows: Q4 with K short enough for a single part (f32 activations:
 // 128 x 1024 x 3072 9.2 against 13.3 us, 256 x 576 x 1536 8.9 against 13.3, 512 x 1024 x 3072 16.8
 // against 17.6; fp16 activations, in row groups of 32: 512 x 1024 x 3072 11.9 against 13.1 us,
-// 128 x 1024 x 3072 8.5 against 9.8); with K parts the tiled kernel is ahead (fp16 512 x 3072 x 1024:
-// 15.1 against 16.8 us) and Q8 is level or up to 1.4x slower on this kernel.
+// 128 x 1024 x 3072 8.5 against 9.8), and with up to four K parts (which is where the resident form
+// ends beyond 32 rows) when the workgroups fill three quarters of their rounds or, with the quants
+// parked, fit one (fp16 512 x 3072 x 1024: 14.8-15.6 against 15.3-15.9 us, 512 x 4096 x 1024 15.9
+// against 18.6, 48 x 3072 x 4096 10.3 against 13.2; f32 128 x 4096 x 4096 20.1 against 23.2, but
+// 128 x 3072 x 3072, two pairs of tiles per wave without room to park the quants on 0.56 of the CUs,
+// 20.4 against 19.0);
+// Q8 is between 0.8 and 1.4 of the tiled kernel's time on this one and stays where it was.
 bool tile_mfma_preferred(const LaunchArgs& x) {
   ResidentPlan rp;
   if (!use_resident(x, &rp)) return false;
-  if (x.m > 32) return x.w.fmt == MGN_FMT_Q4 && rp.parts == 1;
   const uint64_t wgs = (uint64_t)rp.parts * rp.colgroups * rp.rowgroups;
+  const uint64_t rounds = (wgs + x.num_cus - 1) / x.num_cus;
+  if (x.m > 32)
+    return x.w.fmt == MGN_FMT_Q4 && (rp.parts == 1 || (rp.park && rounds == 1) || 4 * wgs >= 3 * rounds * (uint64_t)x.num_cus);
   if (x.m > 16)
     return !x.a_is_f16 && wgs <= (uint64_t)x.num_cus && (x.w.fmt == MGN_FMT_Q4 || rp.q == 1) &&
            (rp.parts <= 4 || 2 * wgs <= (uint64_t)x.num_cus);
   if (rp.r != 1 || rp.nslices < 3) return false;
-  const uint64_t rounds = (wgs + x.num_cus - 1) / x.num_cus;
   return 4 * wgs >= 3 * rounds * (uint64_t)x.num_cus;
 }
 

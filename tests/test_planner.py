@@ -178,7 +178,9 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
         assert p.route == TILE_MFMA and p.quads_per_wave == 0 and p.k_parts == 1 and p.grid[2] == 32
     up = capi.matmul_plan(Q4, 512, 1024, 3072, True)  # fp16 activations, C4 up-projection: row groups of 32
     assert up.route == TILE_MFMA and up.quads_per_wave == 0 and up.full_steps == 2 and list(up.grid) == [1, 12, 16]
-    assert capi.matmul_plan(Q4, 512, 3072, 1024, True).route == GEMM_MFMA   # K parts: the 32x32 kernel
+    down = capi.matmul_plan(Q4, 512, 3072, 1024, True)  # C4 down-projection: three K parts, three quarters of a round
+    assert down.route == TILE_MFMA and down.quads_per_wave == 0 and list(down.grid) == [3, 4, 16]
+    assert capi.matmul_plan(Q4, 128, 3072, 3072, fp16_range=True).route == GEMM_MFMA  # a second round would stay half empty
     assert capi.matmul_plan(Q8, 512, 1024, 3072, True).route == GEMM_MFMA
     head = capi.matmul_plan(Q4, 1, 4096, 14336)
     assert (head.grid[0], head.threads, head.steps, head.k_splits, head.full_steps) == (256, 896, 8, 1, 1)
