@@ -1332,12 +1332,14 @@ bool tile_mfma_supported(const LaunchArgs& x) {
 // the tiled kernel's whole call, and so does a round that stays half empty: 5120 x 14336, 0.55 of a
 // round, 22.9 against 20.3, Q8 34.3 against 25.1; 6144 x 14336, 0.66: 23.0 against 22.2, Q8 33.4
 // against 28.7).  17 to 32 rows of f32 activations, where the tiled kernel runs twice the MFMAs: whenever
-// the two row groups' workgroups fit one round (576 x 576: 8.1 against 11.7 us, 4096 x 4096: 12.5
-// against 16.5, 14336 x 1536: 17.6 against 23.2; with more workgroups the weights' second pass
-// costs more: 576 x 49152 16.5 against 15.2, 14336 x 4096 29.4 against 27.1, and so do many K
-// parts that fill the chip: 14336 x 4096 at two pairs per wave 28.6 against 26.9; Q8 with two pairs
-// of tiles per wave has no room to park its quants and loses too: 4096 x 14336 31.3 against
-// 28.0).  Beyond 32 rows: Q4 with K short enough for a single part (f32 activations:
+// the two row groups' workgroups fit one round (576 x 576: 8.0 against 11.4 us, 4096 x 4096: 11.5
+// against 15.8, 8192 x 4096, 8 K parts: 15.0 against 21.6, 14336 x 1536, 14 parts: 15.0 against 22.9,
+// 14336 x 4096 at two pairs of tiles per wave 24.2 against 26.4; with more workgroups the weights'
+// second pass costs more: 1536 x 49152 33.2 against 24.6, 8192 x 14336 39.7 against 36.1), except
+// Q4 at two pairs per wave with K in one part (576 x 49152: 16.2 against 14.5), Q8 at two pairs per
+// wave, which has no room to park its quants (4096 x 14336 31.8 against 27.4, 14336 x 4096 33.5
+// against 29.8), and Q8 with K parts below K = 2048, where the hand-over is a third of the call
+// (1536 x 576 11.9 against 10.5).  Beyond 32 rows: Q4 with K short enough for a single part (f32 activations:
 // 128 x 1024 x 3072 9.2 against 13.3 us, 256 x 576 x 1536 8.9 against 13.3, 512 x 1024 x 3072 16.8
 // against 17.6; fp16 activations, in row groups of 32: 512 x 1024 x 3072 11.9 against 13.1 us,
 // 128 x 1024 x 3072 8.5 against 9.8), and with up to four K parts (which is where the resident form
@@ -1354,9 +1356,11 @@ bool tile_mfma_preferred(const LaunchArgs& x) {
   const uint64_t rounds = (wgs + x.num_cus - 1) / x.num_cus;
   if (x.m > 32)
     return x.w.fmt == MGN_FMT_Q4 && (rp.parts == 1 || (rp.park && rounds == 1) || 4 * wgs >= 3 * rounds * (uint64_t)x.num_cus);
-  if (x.m > 16)
-    return !x.a_is_f16 && wgs <= (uint64_t)x.num_cus && (x.w.fmt == MGN_FMT_Q4 || rp.q == 1) &&
-           (rp.parts <= 4 || 2 * wgs <= (uint64_t)x.num_cus);
+  if (x.m > 16) {
+    if (x.a_is_f16 || wgs > (uint64_t)x.num_cus) return false;
+    if (x.w.fmt == MGN_FMT_Q4) return !(rp.q == 2 && rp.parts == 1);
+    return rp.q == 1 && (rp.parts == 1 || rp.nslices >= 8);
+  }
   if (rp.r != 1 || rp.nslices < 3) return false;
   return 4 * wgs >= 3 * rounds * (uint64_t)x.num_cus;
 }

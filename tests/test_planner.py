@@ -166,7 +166,10 @@ def test_baseline_configurations_take_the_kernels_built_for_them():
         assert capi.matmul_plan(fmt, 16, 5120, 14336, fp16_range=True).route == GEMM_MFMA  # 0.55 of a round of workgroups
         assert capi.matmul_plan(fmt, 16, 4096, 49152, fp16_range=True).route == TILE_MFMA  # 1.5 rounds, all but full
         assert capi.matmul_plan(fmt, 16, 4096, 4096, fp16_range=True).route == GEMM_MFMA   # a quarter of the CUs
-        assert capi.matmul_plan(fmt, 17, 14336, 4096, fp16_range=True).route == GEMM_MFMA  # two rounds of workgroups
+        # 17 rows on 14336 x 4096: two pairs of tiles per wave keep it to one round; Q8 cannot park its quants then
+        assert capi.matmul_plan(fmt, 17, 14336, 4096, fp16_range=True).route == (TILE_MFMA if fmt == Q4 else GEMM_MFMA)
+        assert capi.matmul_plan(fmt, 17, 8192, 14336, fp16_range=True).route == GEMM_MFMA  # two rounds of workgroups
+        assert capi.matmul_plan(fmt, 17, 8192, 4096, fp16_range=True).route == TILE_MFMA   # 8 K parts, one round
         assert capi.matmul_plan(fmt, 17, 4096, 4096, fp16_range=True).route == TILE_MFMA   # two row groups of 16, one round
         assert capi.matmul_plan(fmt, 16, 14336, 4096).route == TILE_MFMA
     big = capi.matmul_plan(Q4, 512, 14336, 4096)   # images of 512 rows x 14336 exceed the 16 MiB workspace: several launches
