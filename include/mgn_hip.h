@@ -230,7 +230,9 @@ mgn_status mgn_matmul_q_at(mgn_ctx* ctx, const mgn_buf* a_t, const mgn_weight* w
  * (MGN_ACT_FP16_RANGE).  MGN_EINVAL for shapes no weight can have. */
 typedef struct mgn_plan_info {
   int route;              /* mgn_route (never MGN_ROUTE_AUTO) */
-  uint32_t grid[3];       /* workgroups */
+  uint32_t grid[3];       /* workgroups: GEMV (column groups, K parts, 1); tiled routes (K parts, column groups, row
+                           * groups) -- the LDS-resident MGN_ROUTE_TILE_MFMA form launches them as (column groups x
+                           * row groups, rounded up to a multiple of 8 when K is in parts; K parts) */
   uint32_t threads;       /* per workgroup */
   uint32_t lds_bytes;     /* dynamic LDS per workgroup */
   uint32_t waves_n;       /* column quads (GEMV), 32-column tiles (MGN_ROUTE_GEMM_MFMA) or 16-column tiles
@@ -239,7 +241,7 @@ typedef struct mgn_plan_info {
   uint32_t k_parts;       /* workgroups that share a column group; > 1: partial sums through the workspace */
   uint32_t steps;         /* GEMV: 16-block steps per wave; tiled: 8-block chunks (slices of 256 elements) per wave and part */
   uint32_t quads_per_wave; /* GEMV: column quads per wave; MGN_ROUTE_TILE_MFMA: 0 for the form that keeps the
-                            * activation images in LDS (M <= 32), else the launches the rows are spread over
+                            * activation images in LDS, else the launches the rows are spread over
                             * (more than one when their activation images exceed the workspace) */
   uint32_t full_steps;    /* GEMV: 1 when no step needs masking; MGN_ROUTE_TILE_MFMA: row tiles of 16 rows per workgroup */
   uint32_t tail_blocks;   /* GEMV only: 0, or the K blocks per column beyond `steps` full steps that the wave's
