@@ -519,6 +519,7 @@ def main():
         layer = decode_layer_times(200, 20)
         line["configs"]["c2_q4_decode_layer_session"] = {
             "us": layer["fused_us_per_layer"], "unfused_us": layer["unfused_us_per_layer"],
+            "graph_replay_us": layer["fused_graph_us_per_layer"],  # the fused step captured once and replayed
             "launches": layer["fused_launches_per_layer"], "dispatches": layer["dispatches_per_layer"],
             "what": "one SmolLM2-135M decode layer's matmuls, norms and SwiGLU through the Graph/Session surface, per layer"}
 
