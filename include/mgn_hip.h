@@ -39,9 +39,13 @@ typedef enum mgn_status {
   MGN_ENOTFOUND = 4, /* unknown name (session layer) */
   MGN_ENODEVICE = 5, /* no usable gfx950 device */
   MGN_EUNSUPPORTED = 6, /* a fused entry point asked for a shape its kernel does not serve */
-  MGN_ERANGE = 7 /* reported by the next synchronising call: an f32 activation too large for the kernel
+  MGN_ERANGE = 7, /* reported by the next synchronising call: an f32 activation too large for the kernel
                     that ran (|x| >= 65504 on MGN_ROUTE_GEMM_MFMA, M >= 5, which only a context set to
                     MGN_ACT_FP16_RANGE or a forced route uses for f32); outputs of that call are wrong */
+  MGN_ETIMEOUT = 8 /* reported by the next synchronising call: a workgroup that adds up the partial sums of a
+                    matmul whose K is cut into parts gave up waiting for another part (its wait is bounded, so
+                    every kernel ends); outputs since the last synchronisation are not valid.  The library
+                    has emptied its hand-over workspace again when the call returns. */
 } mgn_status;
 
 /* compile::WeightFormat::{Q4,Q8} (src/compile.rs:8-29), graph::DType::{Q4_0,Q8_0}

@@ -33,7 +33,7 @@ bool describe_gemv_mfma(const LaunchArgs& x, mgn_plan_info* out) {
   out->lds_bytes = (uint32_t)p.lds;
   out->waves_n = p.wnc, out->k_splits = p.ksc, out->k_parts = p.kparts, out->steps = p.steps;
   out->quads_per_wave = p.qpw, out->full_steps = p.exact ? 1 : 0, out->tail_blocks = p.tail;
-  out->workspace_bytes = p.kparts > 1 ? (uint64_t)p.kparts * mrows * x.w.n * sizeof(float) : 0;
+  out->workspace_bytes = (uint64_t)(p.kparts - 1) * mrows * x.w.n * sizeof(float);
   return true;
 }
 

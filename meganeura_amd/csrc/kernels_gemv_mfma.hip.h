@@ -104,8 +104,9 @@ struct GemvBatch {
 struct GemvSplit {
   uint32_t k_full;     // the weight's K: column stride of its blocks, row stride of the activations
   uint32_t kparts;
-  float* scratch;      // [kparts][MROWS][n] partial sums
-  uint32_t* counters;  // one arrival counter per blockIdx.x, zero between launches
+  float* handover;     // [kparts - 1][MROWS][n] partial sums of all parts but the last; kHandoverEmpty between launches
+  uint32_t spin_limit; // polls after which the adding workgroup stops waiting for a partial sum
+  uint32_t* fault_flag;  // set when it did
   uint32_t epilogue;   // unary operations on the output (apply_epilogue); needed with or without K parts
 };
 template <typename T>
@@ -254,8 +255,13 @@ __device__ __forceinline__ float block_scale(float amax, float* inv) {
 // of all of K would not fit in LDS (M = 4 with K > ~9000) or need more threads to prepare than a
 // workgroup has (K > 16384), so grid.y workgroups share a quad group, each with a part of K
 // that is a whole number of steps (the last part may reach past the end of K).  Their partial
-// sums meet in a workspace; the last workgroup to arrive adds them in part order (bit-identical
-// from run to run) and writes C.
+// sums meet in the hand-over workspace, whose words all hold kHandoverEmpty between launches: every
+// part but the last stores its sums there and is done; the last part (dispatched last, when the
+// others are running or done; grid.x is a multiple of 8, so a quad group's parts share an XCD and
+// its L2) polls each word it needs until it is no longer empty, adds the parts in part order, its
+// own last (bit-identical from run to run), puts the empty pattern back and writes C.  No counter,
+// no barrier, one trip to the L2 per poll; the wait is bounded (spin_limit polls, then the
+// context's fault word is set and the next synchronising call reports it).
 template <int FMT, int MROWS, int STEPS, int QPW, int PRO, int TASKS, bool EXACT, bool KSPLIT, bool TAIL = false>
 __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // The leading scalar arguments are what a wave needs before it can issue its first loads;
@@ -267,6 +273,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     uint32_t ksc, uint32_t wnc, uint32_t kdim, uint32_t n0, uint32_t first_quad1, uint32_t first_quad2,
     uint32_t ksc_recip,  // ceil(4096 / ksc): wave / ksc == (wave * ksc_recip) >> 12 for the 16 waves there can be
     const float* __restrict__ norm_weight, float eps, GemvBatch bt, GemvSplit sp) {
+  if (KSPLIT && blockIdx.x * wnc >= (n0 + 3) / 4) return;  // padding of the grid to a multiple of 8 quad groups
   const uint32_t m = m_flags & 0xFFu;
   const bool a_f16 = PRO == kProNone && (m_flags >> 31) != 0;
   const GemvPrologue pro{norm_weight, eps};
@@ -779,49 +786,47 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot;
   }
   lds_barrier();
-  // ---- combine the K splits, add the residual, store ----
-  uint32_t* const last_flag = (uint32_t*)nrm;  // (KSPLIT comes without the prologue that uses nrm)
-  for (int pass = 0; pass < (KSPLIT ? 2 : 1); pass++) {
-    if (KSPLIT && pass == 1) {
-      // Each XCD has its own L2: the partial sums travel as device-scope relaxed atomics
-      // (write-through stores, L2-coherent loads).  Every wave waits until its stores have
-      // been acknowledged (they are in memory then), the barrier orders all of them before
-      // the count; a release fence instead would write back the XCD's whole L2 (4 us).
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-      if (tid == 0) {
-        uint32_t* const ctr = sp.counters + blockIdx.x;
-        const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const bool last = seen == sp.kparts - 1;
-        if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-        *last_flag = last ? 1u : 0u;
-      }
-      __syncthreads();
-      if (*last_flag == 0u) break;
-    }
-    for (uint32_t t = tid; t < wnc * MROWS * 4; t += nthreads) {
-      const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
-      // the quads of a workgroup may belong to different weights of the batch
-      const uint32_t gq = quad0 + ql;
-      const uint32_t wi = (gq >= first_quad1 ? 1u : 0u) + (gq >= first_quad2 ? 1u : 0u);
-      const uint32_t wn_cols = pick3(wi, n0, bt.w[1].n, bt.w[2].n);
-      const uint32_t n = (gq - pick3(wi, 0u, first_quad1, first_quad2)) * 4 + col;
-      if (r < m && n < wn_cols) {
-        float v = 0.0f;
-        if (!KSPLIT || pass == 0) {
-          for (uint32_t s = 0; s < ksc; s++) v += red[((ql * ksc + s) * MROWS + r) * 4 + col];
-        } else {  // the last workgroup: every part from memory, its own included, in part order
-          for (uint32_t p = 0; p < sp.kparts; p++)
-            v += __hip_atomic_load(sp.scratch + ((size_t)p * MROWS + r) * wn_cols + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // ---- combine the K splits, then the K parts, add the residual, store ----
+  for (uint32_t t = tid; t < wnc * MROWS * 4; t += nthreads) {
+    const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
+    // the quads of a workgroup may belong to different weights of the batch
+    const uint32_t gq = quad0 + ql;
+    const uint32_t wi = (gq >= first_quad1 ? 1u : 0u) + (gq >= first_quad2 ? 1u : 0u);
+    const uint32_t wn_cols = pick3(wi, n0, bt.w[1].n, bt.w[2].n);
+    const uint32_t n = (gq - pick3(wi, 0u, first_quad1, first_quad2)) * 4 + col;
+    if (r < m && n < wn_cols) {
+      float v = 0.0f;
+      for (uint32_t s = 0; s < ksc; s++) v += red[((ql * ksc + s) * MROWS + r) * 4 + col];
+      if constexpr (KSPLIT) {
+        float* const slot0 = sp.handover + (size_t)r * wn_cols + n;  // part p's word: slot0 + p * MROWS * wn_cols
+        const size_t pstride = (size_t)MROWS * wn_cols;
+        if (kpart + 1 < sp.kparts) {
+          const uint32_t bits = __builtin_bit_cast(uint32_t, v);
+          __hip_atomic_store(slot0 + kpart * pstride, __builtin_bit_cast(float, bits == kHandoverEmpty ? 0x7FC00000u : bits),
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          continue;
         }
-        if (KSPLIT && pass == 0) {
-          __hip_atomic_store(sp.scratch + ((size_t)kpart * MROWS + r) * wn_cols + n, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        } else {
-          const size_t o = (size_t)r * wn_cols + n;
-          const float* const dd = pick3(wi, bt.d[0], bt.d[1], bt.d[2]);
-          pick3(wi, bt.c[0], bt.c[1], bt.c[2])[o] = apply_epilogue(dd ? v + dd[o] : v, sp.epilogue);
+        float acc = 0.0f;
+        bool gave_up = false;
+        for (uint32_t p = 0; p + 1 < sp.kparts; p++) {
+          float x = __hip_atomic_load(slot0 + p * pstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (uint32_t polls = 0; __builtin_bit_cast(uint32_t, x) == kHandoverEmpty; polls++) {
+            if (polls >= sp.spin_limit) {
+              gave_up = true;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+            x = __hip_atomic_load(slot0 + p * pstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          acc += x;
+          __hip_atomic_store(slot0 + p * pstride, __builtin_bit_cast(float, kHandoverEmpty), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        v = acc + v;
+        if (gave_up && sp.fault_flag) *sp.fault_flag = 1u;
       }
+      const size_t o = (size_t)r * wn_cols + n;
+      const float* const dd = pick3(wi, bt.d[0], bt.d[1], bt.d[2]);
+      pick3(wi, bt.c[0], bt.c[1], bt.c[2])[o] = apply_epilogue(dd ? v + dd[o] : v, sp.epilogue);
     }
   }
 }
@@ -914,7 +919,7 @@ bool plan_mfma_gemv(const LaunchArgs& x, uint32_t mrows, MfmaGemvPlan* out) {
   const bool plain = x.pro_kind == kProNone && x.n_more == 0;
   const uint32_t nquads = total_quads(x);
   if (plan_one_part(x.w.fmt, x.w.k, nquads, mrows, x.num_cus, !plain, out)) return true;
-  if (!plain || !x.scratch || !x.counters) return false;
+  if (!plain || !x.handover) return false;
   const uint32_t steps_total = (x.w.k / 32 + 15) / 16;
   // Four parts first: a workgroup then prepares a quarter of the activations and mostly needs no
   // K split of its own, which outweighs the two further partial sums per output (measured on
@@ -925,10 +930,10 @@ bool plan_mfma_gemv(const LaunchArgs& x, uint32_t mrows, MfmaGemvPlan* out) {
     // parts of a whole number of 16-block steps; the last one may be short, never empty
     const uint32_t part_steps = (steps_total + kp - 1) / kp;
     if ((kp - 1) * part_steps >= steps_total) continue;
-    if ((size_t)kp * mrows * x.w.n * sizeof(float) > x.scratch_bytes) continue;
+    if ((size_t)(kp - 1) * mrows * x.w.n * sizeof(float) > x.handover_bytes) continue;  // the last part keeps its own sums
     MfmaGemvPlan p;
     if (!plan_one_part(x.w.fmt, part_steps * 512, nquads, mrows, std::max(1, x.num_cus / (int)kp), true, &p)) continue;
-    if (p.qpw != 1 || p.grid > x.n_counters) continue;
+    if (p.qpw != 1) continue;
     p.kparts = kp;
     p.part_k = part_steps * 512;
     p.exact = false;  // the K-part kernels always mask (the last part may reach past the end of K)
@@ -958,8 +963,9 @@ int launch_tasks(ihipStream_t* s, const LaunchArgs& x, const MfmaGemvPlan& p) {
       bt.first_quad[j] = 0xFFFFFFFFu;
     }
   }
-  const GemvSplit sp{x.w.k, p.kparts, (float*)x.scratch, x.counters, x.epilogue};
-  hipLaunchKernelGGL(kern, dim3(p.grid, p.kparts), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants,
+  const GemvSplit sp{x.w.k, p.kparts, (float*)x.handover, x.spin_limit, x.fault_flag, x.epilogue};
+  // (with K parts: a multiple of 8 quad groups, so that the parts of a group run on one XCD)
+  hipLaunchKernelGGL(kern, dim3(p.kparts > 1 ? (p.grid + 7) / 8 * 8 : p.grid, p.kparts), dim3(64 * p.ksc * p.wnc), p.lds, s, (const float*)x.a, x.w.meta, x.w.quants,
                      x.m | (x.a_is_f16 ? 0x80000000u : 0u), p.ksc, p.wnc, p.kparts > 1 ? p.part_k : x.w.k, x.w.n,
                      bt.first_quad[1], bt.first_quad[2],
                      (4096u + p.ksc - 1) / p.ksc, x.pro_weight, x.pro_eps, bt, sp);

@@ -42,43 +42,10 @@
 #include <algorithm>
 #include <type_traits>
 
-#include "kernels_common.hip.h"
+#include "kernels_operand.hip.h"
 
 namespace mgn {
 namespace {
-
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
-  const u32x4_t v = {a, b, c, d};
-  return __builtin_bit_cast(half8, v);
-}
-__device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
-  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
-}
-__device__ __forceinline__ float half_lo(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[0]; }
-__device__ __forceinline__ float half_hi(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[1]; }
-
-// one dword of nibbles -> B operand (8 fp16): (n0,n4),(n1,n5),(n2,n6),(n3,n7), each n * 2^-20.
-// SPLIT: the even nibbles stay in bits 0-3 of their halves, n * 2^-24 (two shifts fewer); the
-// activations they meet are stored times 16 in the image.
-template <bool SPLIT>
-__device__ __forceinline__ half8 nibbles_to_operand(uint32_t wd) {
-  if constexpr (SPLIT) {
-    const uint32_t hi = wd >> 8;
-    return as_half8(wd & 0x000F000Fu, wd & 0x00F000F0u, hi & 0x000F000Fu, hi & 0x00F000F0u);
-  }
-  return as_half8((wd << 4) & 0x00F000F0u, wd & 0x00F000F0u, (wd >> 4) & 0x00F000F0u, (wd >> 8) & 0x00F000F0u);
-}
-// two dwords of int8 -> B operand: (b0,b1),(b2,b3),(b4,b5),(b6,b7), each (q + 128) * 2^-24
-__device__ __forceinline__ half8 bytes_to_operand(uint32_t w0, uint32_t w1) {
-  const uint32_t u0 = w0 ^ 0x80808080u, u1 = w1 ^ 0x80808080u;
-  return as_half8(__builtin_amdgcn_perm(0u, u0, 0x0c010c00u), __builtin_amdgcn_perm(0u, u0, 0x0c030c02u),
-                  __builtin_amdgcn_perm(0u, u1, 0x0c010c00u), __builtin_amdgcn_perm(0u, u1, 0x0c030c02u));
-}
 
 // What the additive MFMA's result (block means times m, or times the Q8 scale) is multiplied by:
 // 32 for the means and, for Q8, -128 for the byte bias, over the quants' operand scale.
@@ -93,21 +60,6 @@ __device__ __forceinline__ float group_max32(float v) {
   v = fmaxf(v, dpp_move<kDppRowMirror>(v));
   v = fmaxf(v, __shfl_xor(v, 16, 64));
   return v;
-}
-
-// Power of two that brings a row slice's largest magnitude into [2^TOP, 2^(TOP+1)) (1 if the
-// slice is all zero, tiny, huge or not finite).  *inv gets the reciprocal.
-template <int TOP>
-__device__ __forceinline__ float slice_scale(float amax, float* inv) {
-  const uint32_t bits = __builtin_bit_cast(uint32_t, amax);
-  const int e = (int)(bits >> 23) - 127;  // floor(log2(amax)) for normal values
-  if (bits == 0 || e >= 100 || e <= -100) {
-    *inv = 1.0f;
-    return 1.0f;
-  }
-  const int sh = TOP - e;
-  *inv = __builtin_bit_cast(float, (uint32_t)(127 - sh) << 23);
-  return __builtin_bit_cast(float, (uint32_t)(127 + sh) << 23);
 }
 
 // ---- the activation image ----
@@ -348,6 +300,11 @@ struct TileTail {  // arguments first needed in the epilogue
   float* scratch;      // partial results when parts > 1 (general kernel: [parts][row groups * R * 16][n])
   uint32_t* counters;  // one arrival counter per (row group, column group), zero between launches
   uint32_t epilogue;   // unary operations on the output (apply_epilogue)
+  // the resident kernel's K parts: the counter-free hand-over workspace (kHandoverEmpty between
+  // launches), the polls a reading wave makes at most, the word it sets when it gives up
+  float* handover;
+  uint32_t spin_limit;
+  uint32_t* fault_flag;
 };
 
 constexpr int park_stride(int fmt) { return fmt == MGN_FMT_Q4 ? 8 * 16 + 16 : 8 * 32 + 16; }  // bytes per parked column
@@ -630,27 +587,6 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
 // steps behind the multiplications and the call takes a third longer.
 // K is cut into parts of NSL slices; the parts' partial tiles meet as in the kernel above.
 constexpr int kSide = 2;            // column tiles a wave multiplies side by side
-
-typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-
-// component j of lane (c, g) <- component g of lane (c, j)
-__device__ __forceinline__ void transpose_rows(u32x4_t& v) {
-  u32x2_t s = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);
-  v.x = s.x, v.z = s.y;
-  s = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
-  v.y = s.x, v.w = s.y;
-  s = __builtin_amdgcn_permlane16_swap(v.x, v.y, false, false);
-  v.x = s.x, v.y = s.y;
-  s = __builtin_amdgcn_permlane16_swap(v.z, v.w, false, false);
-  v.z = s.x, v.w = s.y;
-}
-// odd rows of (x, y) <-> even rows of (z, w)
-__device__ __forceinline__ void swap_row_pairs(u32x4_t& v) {
-  u32x2_t s = __builtin_amdgcn_permlane16_swap(v.x, v.z, false, false);
-  v.x = s.x, v.z = s.y;
-  s = __builtin_amdgcn_permlane16_swap(v.y, v.w, false, false);
-  v.y = s.x, v.w = s.y;
-}
 
 // One slice (8 K blocks) of kSide column tiles against R row tiles: the tiles' quants in B operand
 // order (q, see above), their 8 scale words (mw), the slice's image at ib (row tile 0, row tiles
@@ -975,76 +911,94 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   __builtin_amdgcn_sched_barrier(0);
 
   if (parts > 1) {
-    // K parts of other workgroups: the last one to arrive adds them up in part order (see above).
+    // K parts of other workgroups.  The parts of a (column group, row group) run on one XCD (see the
+    // grid above) and the part with the highest index is dispatched last, when the others are
+    // already running or done; it is the one that adds them up, in part order, its own sums last.
+    // There is no counter and no barrier: the hand-over workspace holds kHandoverEmpty in every word
+    // between launches, a part stores its tiles over it and is done (write-through stores, device
+    // scope), and every wave of the adding workgroup polls the slots of its own tiles until none of
+    // their words is empty any more, then puts the pattern back for the next launch.  A wait costs
+    // one trip to the XCD's L2 per poll, not the three dependent trips through memory of a counted
+    // hand-over (stores acknowledged, count returned, tiles read): M = 16 on 4096 x 14336, 4 parts,
+    // 12.8 -> 10.6 us.  The wait is bounded: after spin_limit polls the wave sets the context's
+    // fault word, which the next synchronising call reports, and goes on with what it has.
     // The partial tiles travel in register order: the float4 a lane holds for (pair, side, row tile)
     // goes out and comes back as one 128-bit access, 1 KiB per wave and instruction, at
     //   (((part * row groups + row group) * column groups + column group) * 8 + wave) * Q * kSide * R + slot
-    // Every XCD has its own L2, so both directions carry sc1 (device scope).  What the read-back costs
-    // is one trip to the tiles (about 1 us) plus 0.15 us for every further part: a CU takes in about
-    // 100 GB/s, wherever the tiles sit (14 parts of 14336 x 4096 at M = 16: 3 us of 16.2).
     constexpr uint32_t kSlots = Q * kSide * R;
     constexpr int kDeviceScope = 16;  // the sc1 bit of a buffer instruction's cache policy
     const uint32_t wgs_per_part = rowgroups * colgroups;
-    const __amdgpu_buffer_rsrc_t partials =
-        __builtin_amdgcn_make_buffer_rsrc(tail.scratch, 0, parts * wgs_per_part * (8u * kSlots * 1024u), 0x00020000);
-    const uint32_t my_off = ((rg * colgroups + cg) * 8u + wave) * (kSlots * 1024u) + lane * 16u;
     const uint32_t part_stride = wgs_per_part * (8u * kSlots * 1024u);
+    const __amdgpu_buffer_rsrc_t partials =
+        __builtin_amdgcn_make_buffer_rsrc(tail.handover, 0, (parts - 1) * part_stride, 0x00020000);
+    const uint32_t my_off = ((rg * colgroups + cg) * 8u + wave) * (kSlots * 1024u) + lane * 16u;
+    if (part + 1 < parts) {
 #pragma unroll
-    for (int p = 0; p < Q; p++)
+      for (int p = 0; p < Q; p++)
 #pragma unroll
-      for (int u = 0; u < kSide; u++)
+        for (int u = 0; u < kSide; u++)
 #pragma unroll
-        for (int r = 0; r < R; r++)
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, res[p][u][r]), partials,
-                                                 part * part_stride + my_off + ((p * kSide + u) * R + r) * 1024u, 0, kDeviceScope);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    uint32_t* const flag = (uint32_t*)lds4;
-    if (tid == 0) {
-      uint32_t* const ctr = tail.counters + rg * colgroups + cg;
-      const uint32_t seen = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const bool last = seen == parts - 1;
-      if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-      *flag = last ? 1u : 0u;
+          for (int r = 0; r < R; r++) {
+            u32x4_t v = __builtin_bit_cast(u32x4_t, res[p][u][r]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = v[i] == kHandoverEmpty ? 0x7FC00000u : v[i];
+            __builtin_amdgcn_raw_buffer_store_b128(v, partials, part * part_stride + my_off + ((p * kSide + u) * R + r) * 1024u, 0,
+                                                   kDeviceScope);
+          }
+      return;
     }
-    __syncthreads();
-    __builtin_amdgcn_sched_barrier(0);
-    if (*flag == 0u) return;
-    // the parts' tiles, several parts in flight at a time, added in part order
+    floatx4 sum[kSlots];
 #pragma unroll
-    for (int p = 0; p < Q; p++)
-#pragma unroll
-      for (int u = 0; u < kSide; u++)
-#pragma unroll
-        for (int r = 0; r < R; r++) res[p][u][r] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t t = 0; t < kSlots; t++) sum[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    bool gave_up = false;
     auto add_parts = [&](auto group) {
       constexpr int PG = decltype(group)::value;
-      for (uint32_t pp0 = 0; pp0 < parts; pp0 += PG) {
+      const u32x4_t empty4 = {kHandoverEmpty, kHandoverEmpty, kHandoverEmpty, kHandoverEmpty};
+      for (uint32_t pp0 = 0; pp0 + 1 < parts; pp0 += PG) {
         u32x4_t v[PG][kSlots];
+        for (uint32_t polls = 0;; polls++) {
+          bool missing = false;
 #pragma unroll
-        for (int j = 0; j < PG; j++) {
-          const uint32_t po = min(pp0 + j, parts - 1) * part_stride + my_off;  // (the surplus repeats the last part)
+          for (int j = 0; j < PG; j++) {
+            const uint32_t po = min(pp0 + j, parts - 2) * part_stride + my_off;  // (the surplus repeats the last part)
 #pragma unroll
-          for (uint32_t t = 0; t < kSlots; t++) v[j][t] = __builtin_amdgcn_raw_buffer_load_b128(partials, po + t * 1024u, 0, kDeviceScope);
+            for (uint32_t t = 0; t < kSlots; t++) v[j][t] = __builtin_amdgcn_raw_buffer_load_b128(partials, po + t * 1024u, 0, kDeviceScope);
+          }
+#pragma unroll
+          for (int j = 0; j < PG; j++)
+#pragma unroll
+            for (uint32_t t = 0; t < kSlots; t++)
+              missing |= v[j][t].x == kHandoverEmpty || v[j][t].y == kHandoverEmpty || v[j][t].z == kHandoverEmpty || v[j][t].w == kHandoverEmpty;
+          if (!__builtin_amdgcn_ballot_w64(missing)) break;
+          if (polls >= tail.spin_limit) {
+            gave_up = true;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+          asm volatile("" ::: "memory");  // the loads are issued anew on every round
         }
 #pragma unroll
         for (int j = 0; j < PG; j++) {
-          const bool live = pp0 + j < parts;
+          const bool live = pp0 + j + 1 < parts;
+          if (live) {  // uniform
 #pragma unroll
-          for (int p = 0; p < Q; p++)
-#pragma unroll
-            for (int u = 0; u < kSide; u++)
-#pragma unroll
-              for (int r = 0; r < R; r++) {
-                const floatx4 t = __builtin_bit_cast(floatx4, v[j][(p * kSide + u) * R + r]);
-#pragma unroll
-                for (int i = 0; i < 4; i++) res[p][u][r][i] = live ? res[p][u][r][i] + t[i] : res[p][u][r][i];
-              }
+            for (uint32_t t = 0; t < kSlots; t++) {
+              sum[t] += __builtin_bit_cast(floatx4, v[j][t]);
+              __builtin_amdgcn_raw_buffer_store_b128(empty4, partials, (pp0 + j) * part_stride + my_off + t * 1024u, 0, kDeviceScope);
+            }
+          }
         }
       }
     };
-    if (parts <= 4) add_parts(std::integral_constant<int, 4>{});
+    if (parts <= 5) add_parts(std::integral_constant<int, 4>{});
     else add_parts(std::integral_constant<int, 16 / (Q * R)>{});
+#pragma unroll
+    for (int p = 0; p < Q; p++)
+#pragma unroll
+      for (int u = 0; u < kSide; u++)
+#pragma unroll
+        for (int r = 0; r < R; r++) res[p][u][r] = sum[(p * kSide + u) * R + r] + res[p][u][r];
+    if (gave_up && lane == 0 && tail.fault_flag) *tail.fault_flag = 1u;
   }
 #pragma unroll
   for (int p = 0; p < Q; p++)
@@ -1106,10 +1060,9 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
       const uint32_t per_wg = 8 * kSide * q;
       const uint32_t colgroups = (n_tiles + per_wg - 1) / per_wg;
       if (parts > 65535 || (uint64_t)colgroups * rowgroups > 0x7FFFFFF0ull) continue;
-      if (parts > 1 && (uint64_t)colgroups * rowgroups > x.n_counters) continue;
-      // a workgroup's partial tile: 8 waves x (q kSide r) float4 per lane
-      const uint64_t partial = parts > 1 ? (uint64_t)parts * rowgroups * colgroups * (8u * q * kSide * r * 1024u) : 0;
-      if (partial > x.scratch_bytes || partial >= (1ull << 32)) continue;
+      // a workgroup's partial tile: 8 waves x (q kSide r) float4 per lane; the last part keeps its own
+      const uint64_t partial = parts > 1 ? (uint64_t)(parts - 1) * rowgroups * colgroups * (8u * q * kSide * r * 1024u) : 0;
+      if (partial > x.handover_bytes || partial >= (1ull << 32)) continue;
       const uint64_t wgs = (uint64_t)parts * colgroups * rowgroups;
       const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q * r * nsl / 4.0) * (r == 2 ? 0.9 : 1.0) + (parts > 1 ? 1.0 : 0.0);
       if (best == 0 || cost < best) {
@@ -1132,7 +1085,7 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
-  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue};
+  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, (float*)x.handover, x.spin_limit, x.fault_flag};
   // (column groups x row groups, K parts); with K parts the first is rounded up to a multiple of 8 (see the kernel)
   const uint64_t groups = (uint64_t)p.colgroups * p.rowgroups;
   const dim3 grid((unsigned)(p.parts > 1 ? (groups + 7) / 8 * 8 : groups), p.parts, 1);
@@ -1251,7 +1204,7 @@ int launch_cpt(ihipStream_t* s, const LaunchArgs& x, const TilePlan& p, uint4* i
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
-  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue};
+  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, nullptr, 0, nullptr};
   hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups, p.rowgroups), dim3(64 * p.ksc * p.wnc), p.lds, s, image, x.w.meta, x.w.quants,
                      x.m, x.w.k, x.w.n, p.wnc, p.ksc, p.nph, p.parts, p.nslices, tail);
   MGN_HIP_LAUNCH_CHECK();

@@ -18,11 +18,13 @@
 // once per device (every device holds its own copy), and only that pointer is passed on.
 constexpr size_t kStaticPartialBytes = MGN_STATIC_WORKSPACE_BYTES;  // partial sums of K parts
 constexpr uint32_t kStaticCounters = mgn::kWorkspaceCounters;      // arrival counters behind them
-static __device__ __align__(256) unsigned char scratch[kStaticPartialBytes + kStaticCounters * sizeof(uint32_t)];
+// ... and, behind the counters, as many bytes again for the kernels whose K parts meet without counters
+constexpr size_t kStaticHandoverOffset = kStaticPartialBytes + kStaticCounters * sizeof(uint32_t);
+static __device__ __align__(256) unsigned char scratch[kStaticHandoverOffset + kStaticPartialBytes];
 
-__global__ void clear_words_kernel(uint32_t* p, uint32_t n) {
+__global__ void fill_words_kernel(uint32_t* p, uint32_t n, uint32_t value) {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = 0u;
+  if (i < n) p[i] = value;
 }
 
 namespace {
@@ -129,10 +131,26 @@ mgn_route auto_route(const mgn::LaunchArgs& x, bool any_magnitude) {
   return MGN_ROUTE_GENERIC;
 }
 
-// After the stream has been synchronised: did a kernel meet activations outside its range?
+// After the stream has been synchronised: did a wave give up waiting for another workgroup's
+// partial sums, or did a kernel meet activations outside its range?
 mgn_status check_range_flag(mgn_ctx* ctx) {
-  if (!ctx->range_flag_host || *(volatile uint32_t*)ctx->range_flag_host == 0) return MGN_OK;
-  *(volatile uint32_t*)ctx->range_flag_host = 0;
+  if (!ctx->range_flag_host) return MGN_OK;
+  volatile uint32_t* const flags = (volatile uint32_t*)ctx->range_flag_host;
+  if (flags[1] != 0) {
+    // what the parts of that launch stored after the reader had given up is still in the hand-over
+    // workspace: make it empty again before anything else runs
+    flags[0] = flags[1] = 0;
+    hipError_t e = ctx->handover ? hipMemsetAsync(ctx->handover, 0xFF, ctx->handover_bytes, ctx->stream) : hipSuccess;
+    if (e == hipSuccess && ctx->static_scratch)
+      e = hipMemsetAsync((char*)ctx->static_scratch + kStaticHandoverOffset, 0xFF, kStaticPartialBytes, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, "hand-over workspace reset", e);
+    return fail(ctx, MGN_ETIMEOUT,
+                "a workgroup gave up waiting for the partial sums of the other K parts of its matmul (spin limit reached): "
+                "outputs of the matmuls since the last synchronisation are not valid");
+  }
+  if (flags[0] == 0) return MGN_OK;
+  flags[0] = 0;
   return fail(ctx, MGN_ERANGE,
               "an f32 activation of magnitude >= 65504 reached the tiled MFMA kernel (M >= 5), which splits activations "
               "into fp16 pairs without rescaling: the affected outputs are wrong (the context was set to MGN_ACT_FP16_RANGE, or the route was forced)");
@@ -222,14 +240,23 @@ mgn_status mgn_ctx_create(int device_id, mgn_ctx** out) {
   ctx->scratch_bytes = kScratchBytes;
   ctx->counters = (uint32_t*)((char*)ctx->scratch + kScratchBytes);
   ctx->n_counters = kCounters;
+  // the counter-free hand-over workspace: every word "empty" between launches.  The static array's
+  // share is set up here too (once per context: cheap, and whatever an earlier process state left is gone)
+  if ((e = hipMalloc(&ctx->handover, mgn::kHandoverBytes)) != hipSuccess ||
+      (e = hipMemsetAsync(ctx->handover, 0xFF, mgn::kHandoverBytes, ctx->stream)) != hipSuccess ||
+      (e = hipMemsetAsync((char*)ctx->static_scratch + kStaticHandoverOffset, 0xFF, kStaticPartialBytes, ctx->stream)) != hipSuccess) {
+    mgn_ctx_destroy(ctx);
+    return hip_fail(nullptr, "hand-over workspace allocation", e);
+  }
+  ctx->handover_bytes = mgn::kHandoverBytes;
   // one pinned, device-mapped word: a kernel that meets activations it cannot represent sets it
   // and the next synchronising call reports MGN_ERANGE
-  if ((e = hipHostMalloc((void**)&ctx->range_flag_host, sizeof(uint32_t), hipHostMallocMapped)) != hipSuccess ||
+  if ((e = hipHostMalloc((void**)&ctx->range_flag_host, 2 * sizeof(uint32_t), hipHostMallocMapped)) != hipSuccess ||
       (e = hipHostGetDevicePointer((void**)&ctx->range_flag_dev, ctx->range_flag_host, 0)) != hipSuccess) {
     mgn_ctx_destroy(ctx);
     return hip_fail(nullptr, "pinned flag allocation", e);
   }
-  *ctx->range_flag_host = 0;
+  ctx->range_flag_host[0] = ctx->range_flag_host[1] = 0;
   *out = ctx;
   return MGN_OK;
 }
@@ -241,6 +268,7 @@ void mgn_ctx_destroy(mgn_ctx* ctx) {
     (void)hipStreamDestroy(ctx->stream);
   }
   if (ctx->scratch) (void)hipFree(ctx->scratch);
+  if (ctx->handover) (void)hipFree(ctx->handover);
   if (ctx->at_stage) (void)hipFree(ctx->at_stage);
   if (ctx->range_flag_host) (void)hipHostFree(ctx->range_flag_host);
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
@@ -260,6 +288,12 @@ mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, mgn_act_range range) {
   if (!ctx) return MGN_EINVAL;
   if (range != MGN_ACT_ANY && range != MGN_ACT_FP16_RANGE) return fail(ctx, MGN_EINVAL, "unknown activation range");
   ctx->any_magnitude = range == MGN_ACT_ANY;
+  return MGN_OK;
+}
+
+mgn_status mgn_ctx_set_spin_limit(mgn_ctx* ctx, uint32_t polls) {
+  if (!ctx) return MGN_EINVAL;
+  ctx->spin_limit = polls;
   return MGN_OK;
 }
 
@@ -623,10 +657,14 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus};
   x.device = ctx->device;
   x.range_flag = ctx->range_flag_dev;
+  x.fault_flag = ctx->range_flag_dev + 1;
+  x.spin_limit = ctx->spin_limit;
   x.scratch = ctx->scratch;
   x.scratch_bytes = ctx->scratch_bytes;
   x.counters = ctx->counters;
   x.n_counters = ctx->n_counters;
+  x.handover = ctx->handover;
+  x.handover_bytes = ctx->handover_bytes;
   x.pro_kind = pro_kind;
   x.pro_weight = norm_weight ? (const float*)norm_weight->ptr : nullptr;
   x.pro_eps = eps;
@@ -654,14 +692,20 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
                       " bytes of workspace, the static one holds " + std::to_string(kStaticPartialBytes) +
                       "; use mgn_matmul_q");
     x.scratch = ctx->static_scratch;
+    x.scratch_capacity = kStaticPartialBytes;  // a launch that would need more than was checked above is refused, not run
     x.counters = (uint32_t*)((char*)ctx->static_scratch + kStaticPartialBytes);
+    x.handover = (char*)ctx->static_scratch + kStaticHandoverOffset;
     if (need > 0) {
-      // every call on this device shares the array: the arrival counters must start at zero
-      // whatever an earlier call left (a fill kernel, not a memset node: safe under graph capture)
-      hipLaunchKernelGGL(clear_words_kernel, dim3((kStaticCounters + 255) / 256), dim3(256), 0, ctx->stream, x.counters,
-                         kStaticCounters);
+      // every call on this device shares the array: the arrival counters must start at zero and
+      // the hand-over words the plan uses must be empty, whatever an earlier call left (fill
+      // kernels, not memset nodes: safe under graph capture)
+      hipLaunchKernelGGL(fill_words_kernel, dim3((kStaticCounters + 255) / 256), dim3(256), 0, ctx->stream, x.counters,
+                         kStaticCounters, 0u);
+      const uint32_t words = (uint32_t)((need + 3) / 4);
+      hipLaunchKernelGGL(fill_words_kernel, dim3((words + 255) / 256), dim3(256), 0, ctx->stream, (uint32_t*)x.handover, words,
+                         mgn::kHandoverEmpty);
       const hipError_t le = hipGetLastError();
-      if (le != hipSuccess) return hip_fail(ctx, "counter clear launch", le);
+      if (le != hipSuccess) return hip_fail(ctx, "workspace fill launch", le);
     }
   }
   int rc;
@@ -747,6 +791,10 @@ mgn_status mgn_matmul_q_batch(mgn_ctx* ctx, const mgn_buf* a, mgn_prologue prolo
   }
   x.n_more = (int)count - 1;
   x.device = ctx->device;
+  x.fault_flag = ctx->range_flag_dev + 1;
+  x.spin_limit = ctx->spin_limit;
+  x.handover = ctx->handover;
+  x.handover_bytes = ctx->handover_bytes;
   x.scratch = ctx->scratch;
   x.scratch_bytes = ctx->scratch_bytes;
   x.counters = ctx->counters;
@@ -822,6 +870,8 @@ mgn_status mgn_matmul_q_plan(mgn_fmt fmt, uint32_t m, uint64_t k, uint64_t n, in
   x.scratch_bytes = mgn::kWorkspaceBytes;
   x.counters = (uint32_t*)&workspace_stand_in;
   x.n_counters = mgn::kWorkspaceCounters;
+  x.handover = &workspace_stand_in;
+  x.handover_bytes = mgn::kHandoverBytes;
   if (a_is_f16 < 0 || a_is_f16 > 2) return MGN_EINVAL;
   const mgn_route route = auto_route(x, a_is_f16 == 0);
   if (route == MGN_ROUTE_GEMV_MFMA && mgn::describe_gemv_mfma(x, out)) return MGN_OK;

@@ -71,9 +71,22 @@ struct LaunchArgs {
   size_t scratch_bytes = 0;
   uint32_t* counters = nullptr;  // all zero between launches
   uint32_t n_counters = 0;
+  size_t scratch_capacity = 0;   // bytes really behind `scratch` when that is less than the planners are shown (0: scratch_bytes)
+  // Second workspace, for kernels whose K parts meet without counters: every word is kHandoverEmpty
+  // between launches; a part's partial sums are stored over it and the reading workgroup, which
+  // polls until none of the words it needs is empty any more, puts the pattern back.
+  void* handover = nullptr;
+  size_t handover_bytes = 0;
+  uint32_t spin_limit = 1u << 20;  // polls after which a reading wave gives up and sets fault_flag
   // host-visible word a kernel sets when f32 activations leave the range it can represent
   uint32_t* range_flag = nullptr;
+  // host-visible word set by a wave that gave up waiting for another workgroup's partial sums
+  uint32_t* fault_flag = nullptr;
 };
+
+// the bit pattern of a word of the hand-over workspace that holds nothing (a NaN no arithmetic
+// produces; a partial sum that happens to carry it is stored as the default NaN instead)
+constexpr uint32_t kHandoverEmpty = 0xFFFFFFFFu;
 
 // kernels.hip
 int launch_dequantize(ihipStream_t* s, const WeightView& w, float* out_dev);  // out [k, n] f32
@@ -103,6 +116,7 @@ bool describe_gemm_mfma(const LaunchArgs& a, mgn_plan_info* out);
 // the workspace every context owns: partial sums of K parts, then arrival counters
 constexpr size_t kWorkspaceBytes = (size_t)16 << 20;
 constexpr uint32_t kWorkspaceCounters = 4096;
+constexpr size_t kHandoverBytes = (size_t)16 << 20;  // the counter-free hand-over workspace of a context
 int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& a);
 // kernels_tile.hip: the 16x16x32 tiled kernel (activation image + weight streaming)
 bool tile_mfma_supported(const LaunchArgs& a);
@@ -125,8 +139,11 @@ struct mgn_ctx {
   size_t scratch_bytes = 0;
   uint32_t* counters = nullptr;
   uint32_t n_counters = 0;
-  uint32_t* range_flag_host = nullptr;  // pinned, mapped: written by kernels, read at sync points
-  uint32_t* range_flag_dev = nullptr;   // the same word as the device sees it
+  void* handover = nullptr;  // counter-free hand-over workspace (LaunchArgs::handover), kHandoverEmpty between launches
+  size_t handover_bytes = 0;
+  uint32_t spin_limit = 1u << 20;
+  uint32_t* range_flag_host = nullptr;  // pinned, mapped, two words: [0] range, [1] hand-over gave up; written by kernels, read at sync points
+  uint32_t* range_flag_dev = nullptr;   // the same words as the device sees them
   void* static_scratch = nullptr;       // this device's copy of the library's static workspace (mgn_matmul_q_static)
   void* at_stage = nullptr;             // transposed activations of the A^T matmul forms, grown on demand
   size_t at_stage_bytes = 0;

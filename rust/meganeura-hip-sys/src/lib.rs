@@ -33,6 +33,7 @@ pub const MGN_ENOTFOUND: mgn_status = 4;
 pub const MGN_ENODEVICE: mgn_status = 5;
 pub const MGN_EUNSUPPORTED: mgn_status = 6;
 pub const MGN_ERANGE: mgn_status = 7;
+pub const MGN_ETIMEOUT: mgn_status = 8;
 
 /// `mgn_fmt` = `compile::WeightFormat::{Q4, Q8}` (src/compile.rs:8-29).
 pub type mgn_fmt = c_int;
@@ -145,6 +146,7 @@ pub mod bench {
     #[link(name = "mgn_hip")]
     extern "C" {
         pub fn mgn_ctx_set_route(ctx: *mut mgn_ctx, route: mgn_route) -> mgn_status;
+        pub fn mgn_ctx_set_spin_limit(ctx: *mut mgn_ctx, polls: u32) -> mgn_status;
         pub fn mgn_matmul_q_loop(ctx: *mut mgn_ctx, a: *const mgn_buf, a_is_f16: c_int, weights: *const *const mgn_weight, count: usize, d: *const mgn_buf, c: *mut mgn_buf, m: u32, steps: u32) -> mgn_status;
         pub fn mgn_weight_read_loop(ctx: *mut mgn_ctx, weights: *const *const mgn_weight, count: usize, steps: u32) -> mgn_status;
     }
