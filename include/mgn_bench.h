@@ -21,8 +21,9 @@ mgn_status mgn_ctx_set_route(mgn_ctx* ctx, mgn_route route);
 
 /* How many times a wave polls for another workgroup's partial sums before it gives up (kernels whose
  * K parts meet without counters; default 2^20, far beyond any wait of a healthy launch).  With 0 a
- * reading wave does not wait at all, which is how a test makes the give-up path run: the kernels
- * all end, and the next synchronising call returns MGN_ETIMEOUT. */
+ * reading wave looks at nothing and gives up at once, which is how a test makes that path run: the
+ * kernels all end, the matmul's outputs are not valid and the next synchronising call returns
+ * MGN_ETIMEOUT. */
 mgn_status mgn_ctx_set_spin_limit(mgn_ctx* ctx, uint32_t polls);
 
 /* `steps` matmuls (mgn_matmul_q, or mgn_matmul_q_f16a when a_is_f16 != 0) enqueued back to back,

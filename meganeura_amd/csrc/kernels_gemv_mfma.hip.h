@@ -809,14 +809,15 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         float acc = 0.0f;
         bool gave_up = false;
         for (uint32_t p = 0; p + 1 < sp.kparts; p++) {
-          float x = __hip_atomic_load(slot0 + p * pstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          for (uint32_t polls = 0; __builtin_bit_cast(uint32_t, x) == kHandoverEmpty; polls++) {
-            if (polls >= sp.spin_limit) {
+          float x = __builtin_bit_cast(float, kHandoverEmpty);
+          for (uint32_t polls = 0;; polls++) {
+            if (polls >= sp.spin_limit) {  // (a limit of 0 looks at nothing: the give-up path, for tests)
               gave_up = true;
               break;
             }
-            __builtin_amdgcn_s_sleep(1);
             x = __hip_atomic_load(slot0 + p * pstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (__builtin_bit_cast(uint32_t, x) != kHandoverEmpty) break;
+            __builtin_amdgcn_s_sleep(1);
           }
           acc += x;
           __hip_atomic_store(slot0 + p * pstride, __builtin_bit_cast(float, kHandoverEmpty), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -956,7 +956,15 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
       const u32x4_t empty4 = {kHandoverEmpty, kHandoverEmpty, kHandoverEmpty, kHandoverEmpty};
       for (uint32_t pp0 = 0; pp0 + 1 < parts; pp0 += PG) {
         u32x4_t v[PG][kSlots];
+#pragma unroll
+        for (int j = 0; j < PG; j++)
+#pragma unroll
+          for (uint32_t t = 0; t < kSlots; t++) v[j][t] = empty4;
         for (uint32_t polls = 0;; polls++) {
+          if (polls >= tail.spin_limit) {  // (a limit of 0 looks at nothing: the give-up path, for tests)
+            gave_up = true;
+            break;
+          }
           bool missing = false;
 #pragma unroll
           for (int j = 0; j < PG; j++) {
@@ -970,10 +978,6 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
             for (uint32_t t = 0; t < kSlots; t++)
               missing |= v[j][t].x == kHandoverEmpty || v[j][t].y == kHandoverEmpty || v[j][t].z == kHandoverEmpty || v[j][t].w == kHandoverEmpty;
           if (!__builtin_amdgcn_ballot_w64(missing)) break;
-          if (polls >= tail.spin_limit) {
-            gave_up = true;
-            break;
-          }
           __builtin_amdgcn_s_sleep(1);
           asm volatile("" ::: "memory");  // the loads are issued anew on every round
         }

@@ -85,4 +85,13 @@ def test_c5_llama_ffn(ctx, orc, fmt, k, n):
         want = orc.matmul_packed(fmt, x, packed, n)
         got = run_matmul(ctx, fmt, x, wt)
         orc.assert_close(got, want, REL, ABS)
+        if m == 16:
+            # a context that was promised activations in the fp16 range may take the 32x32x16 kernel:
+            # that route on the same shape, forced so that it runs whatever the planner prefers
+            ctx.set_activation_range(True)
+            try:
+                orc.assert_close(run_matmul(ctx, fmt, x, wt), want, REL, ABS)
+                orc.assert_close(run_matmul(ctx, fmt, x, wt, ROUTES["gemm_mfma"]), want, REL, ABS)
+            finally:
+                ctx.set_activation_range(False)
     wt.free()

@@ -16,6 +16,15 @@ def ctx():
     c.close()
 
 
+def free_device_bytes():
+    """hipMemGetInfo's free figure, straight from the HIP runtime the library itself is linked to."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
 def both(ctx, orc, fmt, m, k, n, seed, with_d):
     x = synth.normal(seed, m * k).reshape(m, k)
     w = synth.normal(seed + 1, k * n, 0.02).reshape(k, n)
@@ -25,7 +34,11 @@ def both(ctx, orc, fmt, m, k, n, seed, with_d):
     c_ref, c_new = ctx.buffer(m * n * 4), ctx.buffer(m * n * 4)
     ctx.matmul_q(a, wt, c_ref, m, db)
     ref = c_ref.download(np.float32, m * n).reshape(m, n)
+    ctx.sync()
+    before = free_device_bytes()
     ctx.matmul_q_static(a, wt, c_new, m, db)
+    ctx.sync()
+    assert free_device_bytes() == before, "the static entry point must not change the device's free memory"
     got = c_new.download(np.float32, m * n).reshape(m, n)
     want = orc.matmul_f32(x, orc.dequantize(fmt, orc.quantize(fmt, w), k, n), d)
     for buf in (a, c_ref, c_new, wt) + ((db,) if with_d else ()):
@@ -50,6 +63,28 @@ def test_static_workspace_matches_the_allocating_entry_point(ctx, orc, first, se
     assert capi.matmul_plan(*first).workspace_bytes <= capi.STATIC_WORKSPACE_BYTES
     both(ctx, orc, *first, seed=901, with_d=True)
     both(ctx, orc, *second, seed=907, with_d=False)
+
+
+def test_static_workspace_tolerates_what_an_earlier_call_left(ctx, orc):
+    """All contexts of a device share the static array and it keeps the last call's contents.  A
+    call that gave up half-way (forced here with a zero spin limit) leaves partial sums behind and
+    counters that may not be zero; the next call must still come out right."""
+    fmt, m, k, n = Q4, 16, 14336, 4096
+    w = synth.normal(931, k * n, 0.02).reshape(k, n)
+    x = synth.normal(932, m * k).reshape(m, k)
+    wt, a, c = ctx.weight(fmt, w), ctx.upload(x), ctx.buffer(m * n * 4)
+    ctx.set_spin_limit(0)
+    try:
+        ctx.matmul_q_static(a, wt, c, m)
+        with pytest.raises(capi.MgnError) as e:
+            ctx.sync()
+        assert e.value.status == capi.ETIMEOUT
+    finally:
+        ctx.set_spin_limit(1 << 20)
+    for h in (wt, a, c):
+        h.free()
+    both(ctx, orc, Q8, 16, 4096, 2048, seed=941, with_d=False)   # tiled kernel, K parts
+    both(ctx, orc, Q4, 4, 14336, 518, seed=943, with_d=True)     # decode kernel, K parts
 
 
 def test_static_workspace_refuses_what_does_not_fit(ctx):
