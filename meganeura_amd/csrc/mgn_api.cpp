@@ -180,6 +180,26 @@ mgn_status finish_weight_range(mgn_ctx* ctx, mgn_weight* w, const char* what) {
 }  // namespace
 
 namespace mgn {
+// The staging area of the A^T matmul forms holds at least `bytes` afterwards (allocates or grows it;
+// a session does this for its whole plan when it is built, so that no step allocates).
+mgn_status reserve_at_stage(mgn_ctx* ctx, size_t bytes) {
+  if (!ctx) return MGN_EINVAL;
+  if (ctx->at_stage_bytes >= bytes) return MGN_OK;
+  // earlier launches may still read the old area
+  MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  if (ctx->at_stage) (void)hipFree(ctx->at_stage);
+  ctx->at_stage = nullptr;
+  ctx->at_stage_bytes = 0;
+  const size_t grown = align_up(bytes, (size_t)1 << 20);
+  const hipError_t e = hipMalloc(&ctx->at_stage, grown);
+  if (e != hipSuccess) {
+    ctx->at_stage = nullptr;
+    return e == hipErrorOutOfMemory ? fail(ctx, MGN_ENOMEM, "out of device memory") : hip_fail(ctx, "hipMalloc", e);
+  }
+  ctx->at_stage_bytes = grown;
+  return MGN_OK;
+}
+
 // Would one launch serve these weights together (mgn_matmul_q_batch's own check)?  The plan
 // depends on the column count of the whole batch, so a weight that plans alone need not plan
 // next to its siblings.
@@ -463,20 +483,27 @@ static mgn_status weight_from_device_f32(mgn_ctx* ctx, mgn_fmt fmt, const void* 
 }
 
 // Uploads host f32 values into a staging buffer and packs them there (see mgn_weight_create).
-// MGN_ENOMEM: no room for the staging copy or the weight; the caller may pack on the host instead.
+// The staging copy costs 4 bytes per element of device memory until the call returns.  *no_staging
+// is set when there was no room for it, or none for the weight while it was held: the caller then
+// packs on the host, which needs the weight's own bytes only.
 static mgn_status weight_from_host_f32(mgn_ctx* ctx, mgn_fmt fmt, const float* wdata, size_t rows, size_t cols, bool nk,
-                                       mgn_weight** out) {
+                                       mgn_weight** out, bool* no_staging) {
+  *no_staging = false;
   void* staged = nullptr;
   const size_t bytes = rows * cols * sizeof(float);
   if (hipMalloc(&staged, bytes) != hipSuccess) {
     (void)hipGetLastError();  // out of device memory for the staging copy: not an error of the call
+    *no_staging = true;
     return MGN_ENOMEM;
   }
   const hipError_t e = hipMemcpyAsync(staged, wdata, bytes, hipMemcpyHostToDevice, ctx->stream);
   const mgn_status st = e == hipSuccess ? weight_from_device_f32(ctx, fmt, staged, bytes, rows, cols, nk, out)
                                         : hip_fail(ctx, "weight upload", e);
-  if (e != hipSuccess) (void)hipStreamSynchronize(ctx->stream);
+  if (e != hipSuccess || st != MGN_OK) (void)hipStreamSynchronize(ctx->stream);
   (void)hipFree(staged);
+  // the weight itself found no room while the staging copy was held: the host path, which holds
+  // none, gets its try
+  if (st == MGN_ENOMEM) *no_staging = true;
   return st;
 }
 
@@ -490,8 +517,9 @@ mgn_status mgn_weight_create(mgn_ctx* ctx, mgn_fmt fmt, const float* wdata, size
   // The f32 values go up as they are and the device quantizer packs them (the same bytes as the
   // host quantizer's, three to four times sooner on a 4096 x 14336 weight: 9 ms against 28-35 ms)
   // when there is device memory for them; otherwise the host packs and the bytes go up.
-  const mgn_status direct = weight_from_host_f32(ctx, fmt, wdata, rows, cols, false, out);
-  if (direct != MGN_ENOMEM) return direct;
+  bool no_staging = false;
+  const mgn_status direct = weight_from_host_f32(ctx, fmt, wdata, rows, cols, false, out, &no_staging);
+  if (!no_staging) return direct;
   std::vector<uint8_t> packed;
   try {
     packed.resize(mgn_packed_size(fmt, rows, cols));
@@ -509,8 +537,9 @@ mgn_status mgn_weight_create_nk(mgn_ctx* ctx, mgn_fmt fmt, const float* w_nk, si
   if (!valid_fmt(fmt)) return fail(ctx, MGN_EINVAL, "unknown weight format");
   if (k_cols % 32 != 0) return fail(ctx, MGN_EINVAL, "quantized weights require the K dim to be a multiple of 32");
   if (n_rows == 0 || k_cols == 0) return fail(ctx, MGN_EINVAL, "empty weight");
-  const mgn_status direct = weight_from_host_f32(ctx, fmt, w_nk, k_cols, n_rows, true, out);  // as mgn_weight_create
-  if (direct != MGN_ENOMEM) return direct;
+  bool no_staging = false;
+  const mgn_status direct = weight_from_host_f32(ctx, fmt, w_nk, k_cols, n_rows, true, out, &no_staging);  // as mgn_weight_create
+  if (!no_staging) return direct;
   std::vector<uint8_t> packed;
   try {
     packed.resize(mgn_packed_size(fmt, k_cols, n_rows));
@@ -830,20 +859,7 @@ mgn_status mgn_matmul_q_at(mgn_ctx* ctx, const mgn_buf* a_t, const mgn_weight* w
   if (a_t->bytes < need) return fail(ctx, MGN_EINVAL, "A^T is smaller than K rows of m floats");
   if (c->ptr == a_t->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
   if (((size_t)m + 31) / 32 > 65535) return fail(ctx, MGN_EINVAL, "m is too large for the transposed form");
-  if (ctx->at_stage_bytes < need) {
-    // earlier launches may still read the old area
-    MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    if (ctx->at_stage) (void)hipFree(ctx->at_stage);
-    ctx->at_stage = nullptr;
-    ctx->at_stage_bytes = 0;
-    const size_t grown = align_up(need, (size_t)1 << 20);
-    hipError_t e = hipMalloc(&ctx->at_stage, grown);
-    if (e != hipSuccess) {
-      ctx->at_stage = nullptr;
-      return e == hipErrorOutOfMemory ? fail(ctx, MGN_ENOMEM, "out of device memory") : hip_fail(ctx, "hipMalloc", e);
-    }
-    ctx->at_stage_bytes = grown;
-  }
+  if (const mgn_status st = mgn::reserve_at_stage(ctx, need)) return st;
   const int rc = mgn::launch_transpose(ctx->stream, (const float*)a_t->ptr, (float*)ctx->at_stage, (uint32_t)k, m);
   if (rc != 0) return hip_fail(ctx, "transpose launch", (hipError_t)rc);
   const mgn_buf staged{ctx->at_stage, need};

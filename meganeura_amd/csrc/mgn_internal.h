@@ -151,6 +151,7 @@ struct mgn_ctx {
 };
 
 namespace mgn {
+mgn_status reserve_at_stage(mgn_ctx* ctx, size_t bytes);
 // whether mgn_matmul_q_batch would take these weights in one launch (same K and format assumed checked)
 bool batch_plans(const mgn_ctx* ctx, const mgn_weight* const* ws, size_t count, uint32_t m, int pro_kind);
 }  // namespace mgn

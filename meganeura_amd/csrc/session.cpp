@@ -478,6 +478,12 @@ Session::Session(ExecutionPlan plan, int device_id) : plan_(std::move(plan)) {
     // a quantized parameter gets its device storage when it is first set
     for (size_t i = 0; i < plan_.buffers.size(); i++)
       if (!plan_.weight_buffers.count((int)i)) check(mgn_buf_alloc(ctx_, plan_.buffers[i], &buffers_[i]), "mgn_buf_alloc");
+    // the A^T matmul forms transpose their activations into a staging area of the context: sized
+    // here for the whole plan, so that no step allocates (a step may run under stream capture)
+    size_t at_bytes = 0;
+    for (const Dispatch& d : plan_.dispatches)
+      if (is_at(d.shader)) at_bytes = std::max(at_bytes, (size_t)d.params[0] * matmul_k(d) * sizeof(float));
+    if (at_bytes) check(mgn::reserve_at_stage(ctx_, at_bytes), "A^T staging area");
   } catch (...) {
     release();
     throw;
@@ -737,6 +743,17 @@ void Session::plan_launches() {
 
 void Session::run_dispatches() {
   plan_launches();
+  // A norm or SwiGLU dispatch that was folded into the matmuls behind it, run on its own after all
+  // (into the buffer the plan gave it); returns that buffer.
+  auto run_producer = [&](const Dispatch& p) -> const mgn_buf* {
+    const float* in0 = (const float*)buffers_[p.input_buffers[0]]->ptr;
+    float* dst = (float*)buffers_[p.output_buffer]->ptr;
+    const int e = p.shader == MGN_SHADER_RMS_NORM
+                      ? launch_rms_norm(ctx_->stream, in0, (const float*)buffers_[p.input_buffers[1]]->ptr, dst, p.params[0], p.params[1], p.eps)
+                      : launch_swiglu_concat(ctx_->stream, in0, dst, p.params[0], p.params[1]);
+    if (e != 0) throw std::runtime_error(std::string("kernel launch: ") + hipGetErrorString((hipError_t)e));
+    return buffers_[p.output_buffer];
+  };
   for (size_t di = 0; di < plan_.dispatches.size(); di++) {
     if (skipped_[di]) continue;
     const Dispatch& d = plan_.dispatches[di];
@@ -778,23 +795,22 @@ void Session::run_dispatches() {
           const mgn_buf* nw = f.kind == kProRmsNorm ? buffers_[p->input_buffers[1]] : nullptr;
           mgn_status st = mgn_matmul_q_batch(ctx_, act, (mgn_prologue)f.kind, nw, p ? p->eps : 0.0f, items, count, d.params[0]);
           if (st == MGN_EUNSUPPORTED) {
-            // planned as one launch, refused now (the route was changed since): one launch per weight
+            // planned as one launch, refused now (the route was changed since): the producer's own
+            // dispatch into its own buffer, then one plain matmul per weight
+            const mgn_buf* plain = p ? run_producer(*p) : act;
             st = MGN_OK;
-            for (size_t j = 0; j < count && st == MGN_OK; j++)
-              st = f.kind == kProRmsNorm  ? mgn_matmul_q_rms_norm(ctx_, act, nw, p->eps, items[j].w, items[j].d, items[j].c, d.params[0])
-                   : f.kind == kProSwiglu ? mgn_matmul_q_swiglu(ctx_, act, items[j].w, items[j].d, items[j].c, d.params[0])
-                                          : mgn_matmul_q(ctx_, act, items[j].w, items[j].d, items[j].c, d.params[0]);
+            for (size_t j = 0; j < count && st == MGN_OK; j++) st = mgn_matmul_q(ctx_, plain, items[j].w, items[j].d, items[j].c, d.params[0]);
           }
           check(st, "mgn_matmul_q_batch");
-        } else if (f.kind == kProRmsNorm) {
+        } else if (f.kind == kProRmsNorm || f.kind == kProSwiglu) {
           const Dispatch& p = plan_.dispatches[f.producer];
-          check(mgn_matmul_q_rms_norm(ctx_, buffers_[p.input_buffers[0]], buffers_[p.input_buffers[1]], p.eps, w, addend,
-                                      buffers_[d.output_buffer], d.params[0]),
-                "mgn_matmul_q_rms_norm");
-        } else if (f.kind == kProSwiglu) {
-          const Dispatch& p = plan_.dispatches[f.producer];
-          check(mgn_matmul_q_swiglu(ctx_, buffers_[p.input_buffers[0]], w, addend, buffers_[d.output_buffer], d.params[0]),
-                "mgn_matmul_q_swiglu");
+          mgn_status st = f.kind == kProRmsNorm
+                              ? mgn_matmul_q_rms_norm(ctx_, buffers_[p.input_buffers[0]], buffers_[p.input_buffers[1]], p.eps, w, addend,
+                                                      buffers_[d.output_buffer], d.params[0])
+                              : mgn_matmul_q_swiglu(ctx_, buffers_[p.input_buffers[0]], w, addend, buffers_[d.output_buffer], d.params[0]);
+          if (st == MGN_EUNSUPPORTED)  // as above: the fused kernel no longer takes the call
+            st = mgn_matmul_q(ctx_, run_producer(p), w, addend, buffers_[d.output_buffer], d.params[0]);
+          check(st, f.kind == kProRmsNorm ? "mgn_matmul_q_rms_norm" : "mgn_matmul_q_swiglu");
         } else if (!d.epilogue.empty() || !f.post.empty()) {
           std::vector<mgn_unary> ops = d.epilogue;
           ops.insert(ops.end(), f.post.begin(), f.post.end());
