@@ -36,8 +36,11 @@ mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const
 /* `steps` launches, back to back like mgn_matmul_q_loop's, of a kernel that reads the packed
  * bytes of weights[i % count] (quants and scales) once and computes nothing.  Timed like a
  * matmul it gives the time the device needs for one launch plus one pass over a weight's
- * bytes: the floor a bandwidth-bound matmul on that weight can be held against. */
-mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, size_t count, uint32_t steps);
+ * bytes: the floor a bandwidth-bound matmul on that weight can be held against.
+ * pattern 0: every workgroup reads a contiguous share; pattern 1: the decode kernel's own map of
+ * lanes to addresses (a wave per quad of columns, a lane per quant block, three blocks in flight),
+ * which is the faster of the two on the weights that kernel is built for. */
+mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, size_t count, uint32_t steps, int pattern);
 
 #ifdef __cplusplus
 }

@@ -114,7 +114,7 @@ def load():
         "mgn_matmul_q_at": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32, vp, C.c_size_t]),
         "mgn_matmul_q_plan": (C.c_int, [C.c_int, C.c_uint32, C.c_uint64, C.c_uint64, C.c_int, C.c_int, vp]),
         "mgn_matmul_q_loop": (C.c_int, [vp, vp, C.c_int, vp, C.c_size_t, vp, vp, C.c_uint32, C.c_uint32]),
-        "mgn_weight_read_loop": (C.c_int, [vp, vp, C.c_size_t, C.c_uint32]),
+        "mgn_weight_read_loop": (C.c_int, [vp, vp, C.c_size_t, C.c_uint32, C.c_int]),
         "mgn_matmul_q_rms_norm": (C.c_int, [vp, vp, vp, C.c_float, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_swiglu": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_can_fuse": (C.c_int, [vp, vp, C.c_uint32]),
@@ -364,11 +364,11 @@ class Context:
         self.check(self.lib.mgn_matmul_q_loop(self.h, a.h, 1 if a_is_f16 else 0, start, n,
                                               d.h if d is not None else None, c.h, m, steps))
 
-    def weight_read_loop(self, weights, steps, first=0):
+    def weight_read_loop(self, weights, steps, first=0, pattern=0):
         """`steps` launches of a kernel that only reads the packed bytes of weights[(first + i) % len(weights)]."""
         arr, n = weights if isinstance(weights, tuple) else self.rotation(weights)
         start = C.cast(C.byref(arr, (first % n) * C.sizeof(C.c_void_p)), C.c_void_p) if n else None
-        self.check(self.lib.mgn_weight_read_loop(self.h, start, n, steps))
+        self.check(self.lib.mgn_weight_read_loop(self.h, start, n, steps, pattern))
 
     def matmul_q_rms_norm(self, x, norm_weight, eps, w, c, m, d=None):
         """C = rms_norm(x; norm_weight, eps) x W (+ D) in one launch."""

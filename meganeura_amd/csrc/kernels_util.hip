@@ -491,7 +491,59 @@ int launch_quantize(ihipStream_t* s, int fmt, const float* w_dev, uint32_t k, ui
   return 0;
 }
 
-int launch_read_probe(ihipStream_t* s, const WeightView& w, int num_cus, uint32_t* sink) {
+// The same pass with the decode kernel's own lane -> address map: a wave takes a quad of columns,
+// lane (b, i) = (lane / 4, lane % 4) reads K block 16 s + b of column 4 quad + i (quants and scale
+// word) for s = 0, 1, ..., three blocks in flight ahead of the one consumed; one workgroup of 14
+// waves per CU walks the quads in turn.  On a 4096 x 14336 Q4 weight this reads the 36.7 MB in
+// 6.8 us where the contiguous shares above take 7.3 us.
+template <int QB, int MB>
+__global__ __launch_bounds__(896) void read_probe_gemv_kernel(const char* __restrict__ quants, const char* __restrict__ meta,
+                                                              uint32_t bpc, uint32_t ncols, uint32_t* __restrict__ sink) {
+  const uint32_t lane = threadIdx.x & 63, wpb = blockDim.x >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t b = lane >> 2, i = lane & 3;
+  const uint32_t nquads = (ncols + 3) / 4, steps = (bpc + 15) / 16;
+  u32x4_t acc = {0, 0, 0, 0};
+  uint32_t macc = 0;
+  for (uint32_t quad = blockIdx.x * wpb + wave; quad < nquads; quad += gridDim.x * wpb) {
+    const size_t col_base = (size_t)min(quad * 4 + i, ncols - 1) * bpc;
+    // groups of eight steps, written out; a block past the end of the column re-reads the last one
+    for (uint32_t s0 = 0; s0 < steps; s0 += 8) {
+      u32x4_t v[8][QB / 16];
+      uint32_t mv[8];
+      auto fetch = [&](int s) {
+        const size_t blk = col_base + min((s0 + s) * 16 + b, bpc - 1);
+#pragma unroll
+        for (int h = 0; h < QB / 16; h++) v[s][h] = __builtin_nontemporal_load((const u32x4_t*)(quants + blk * QB) + h);
+        if constexpr (MB == 4) mv[s] = __builtin_nontemporal_load((const uint32_t*)(meta + blk * 4));
+        else mv[s] = __builtin_nontemporal_load((const uint16_t*)(meta + blk * 2));
+      };
+#pragma unroll
+      for (int s = 0; s < 3; s++) fetch(s);
+#pragma unroll
+      for (int s = 0; s < 8; s++) {
+        if (s + 3 < 8) fetch(s + 3);
+#pragma unroll
+        for (int h = 0; h < QB / 16; h++) acc ^= v[s][h];
+        macc ^= mv[s];
+      }
+    }
+  }
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w ^ macc) == 0x9E3779B9u) sink[0] = 1u;
+}
+
+int launch_read_probe(ihipStream_t* s, const WeightView& w, int num_cus, uint32_t* sink, int pattern) {
+  if (pattern == 1) {
+    const uint32_t bpc = w.k / 32;
+    if (w.fmt == MGN_FMT_Q4)
+      hipLaunchKernelGGL((read_probe_gemv_kernel<16, 4>), dim3((unsigned)num_cus), dim3(896), 0, s, (const char*)w.quants,
+                         (const char*)w.meta, bpc, w.n, sink);
+    else
+      hipLaunchKernelGGL((read_probe_gemv_kernel<32, 2>), dim3((unsigned)num_cus), dim3(896), 0, s, (const char*)w.quants,
+                         (const char*)w.meta, bpc, w.n, sink);
+    MGN_HIP_LAUNCH_CHECK();
+    return 0;
+  }
   // A weight's scales and quants share one allocation, scales first, about 1 KiB of padding
   // between them: one span from the first scale to the last quant covers both.
   const size_t nb = (size_t)(w.k / 32) * w.n;

@@ -907,13 +907,14 @@ mgn_status mgn_matmul_q_loop(mgn_ctx* ctx, const mgn_buf* a, int a_is_f16, const
   return MGN_OK;
 }
 
-mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, size_t count, uint32_t steps) {
+mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, size_t count, uint32_t steps, int pattern) {
   if (!ctx || !weights || count == 0) return fail(ctx, MGN_EINVAL, "null argument or no weights");
+  if (pattern != 0 && pattern != 1) return fail(ctx, MGN_EINVAL, "unknown read pattern");
   for (size_t i = 0; i < count; i++)
     if (!weights[i]) return fail(ctx, MGN_EINVAL, "null weight");
   for (uint32_t i = 0; i < steps; i++) {
     // the sink is the first word of the split-K workspace, which holds nothing between launches
-    const int e = mgn::launch_read_probe(ctx->stream, view_of(weights[i % count]), ctx->num_cus, (uint32_t*)ctx->scratch);
+    const int e = mgn::launch_read_probe(ctx->stream, view_of(weights[i % count]), ctx->num_cus, (uint32_t*)ctx->scratch, pattern);
     if (e != 0) return fail(ctx, MGN_EHIP, hipGetErrorString((hipError_t)e));
   }
   return MGN_OK;

@@ -559,6 +559,9 @@ def test_weight_read_loop_leaves_results_alone(ctx, orc):
         ctx.weight_read_loop([], 3)
     tiny = ctx.weight(Q8, synth.normal(975, 32, 0.02).reshape(32, 1))
     ctx.weight_read_loop([tiny], 3)
+    ctx.weight_read_loop([tiny], 3, pattern=1)
+    with pytest.raises(capi.MgnError):
+        ctx.weight_read_loop([tiny], 1, pattern=2)
     m, k, n = 4, 14336, 70
     for fmt in (Q4, Q8):
         w = synth.normal(976 + fmt, k * n, 0.02).reshape(k, n)
@@ -567,8 +570,10 @@ def test_weight_read_loop_leaves_results_alone(ctx, orc):
         a = ctx.upload(x)
         c = ctx.buffer(m * n * 4)
         ctx.weight_read_loop([wt, tiny], 7)
+        ctx.weight_read_loop([wt, tiny], 4, pattern=1)
         ctx.matmul_q(a, wt, c, m)
         ctx.weight_read_loop([wt], 2)
+        ctx.weight_read_loop([wt], 2, pattern=1)
         got = c.download(np.float32, m * n).reshape(m, n)
         orc.assert_close(got, orc.matmul_packed(fmt, x, orc.quantize(fmt, w), n), REL, ABS)
         a.free(); c.free(); wt.free()
