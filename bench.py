@@ -338,9 +338,11 @@ def decode_layer_times(steps, warmup, layers=8):
     sess.set_input("attn", synth.activations(2, 1, hidden, which=1))
     ctx = sess.context()
     res = {"layers": layers, "dispatches_per_layer": len(sess.plan()) // layers}
-    for label, fusion, replay in (("unfused", False, False), ("fused", True, False), ("fused_graph", True, True)):
+    for label, fusion, replay, chains in (("unfused", False, False, False), ("fused", True, False, False),
+                                          ("fused_graph", True, True, False), ("chain", True, False, True)):
         sess.set_fusion(fusion)
         sess.set_graph_replay(replay)
+        sess.set_chains(chains)
         res[label + "_launches_per_layer"] = sess.num_launches() / layers
         for _ in range(warmup + 2):
             sess.step()
@@ -534,10 +536,14 @@ def main():
         line["configs"] = config_table(ctx, sets)
         layer = decode_layer_times(200, 20)
         line["configs"]["c2_q4_decode_layer_session"] = {
-            "us": layer["fused_us_per_layer"], "unfused_us": layer["unfused_us_per_layer"],
-            "graph_replay_us": layer["fused_graph_us_per_layer"],  # the fused step captured once and replayed
-            "launches": layer["fused_launches_per_layer"], "dispatches": layer["dispatches_per_layer"],
-            "what": "one SmolLM2-135M decode layer's matmuls, norms and SwiGLU through the Graph/Session surface, per layer"}
+            "us": layer["chain_us_per_layer"],  # the session's default: the whole step's matmuls as one chain launch
+            "launches": layer["chain_launches_per_layer"],
+            "separate_launches_us": layer["fused_us_per_layer"], "separate_launches": layer["fused_launches_per_layer"],
+            "unfused_us": layer["unfused_us_per_layer"],
+            "graph_replay_us": layer["fused_graph_us_per_layer"],  # the separate launches captured once and replayed
+            "dispatches": layer["dispatches_per_layer"],
+            "what": "one SmolLM2-135M decode layer's matmuls, norms and SwiGLU through the Graph/Session surface, per layer "
+                    "(8 layers chained in one session)"}
 
     if args.sweep:
         rows = []

@@ -287,6 +287,38 @@ typedef struct mgn_matmul_item {
 mgn_status mgn_matmul_q_batch(mgn_ctx* ctx, const mgn_buf* a, mgn_prologue prologue, const mgn_buf* norm_weight,
                               float eps, const mgn_matmul_item* items, size_t count, uint32_t m);
 
+/* ---- a whole chain of dependent decode matmuls in ONE launch.
+ * The reference encodes every dispatch of a step into one command buffer and submits it once
+ * (Session::step, src/runtime.rs:2843-2959); a decode step is a chain of small dependent matmuls
+ * (src/models/smollm2.rs:392-405).  A chain object stands in for a run of such dispatches with
+ * M = 1: stage j computes C_j = f_j(prologue_j(A_j) x W_j + D_j), where A_j and D_j may be outputs
+ * of earlier stages of the same chain (recognised by the buffer handle) or buffers written before
+ * the launch.  One resident launch walks the stages; outputs that later stages read travel through
+ * a workspace of the chain, and a reader polls the data itself (bounded: MGN_ETIMEOUT at the next
+ * synchronising call if it ever gives up).  Every C_j is also written to the caller's buffer.
+ * mgn_chain_create: MGN_EUNSUPPORTED when a stage is not served (m != 1, a Q8 weight, K beyond
+ * 16384, two stages writing one buffer, a stage writing a buffer that the chain also reads as
+ * written before the launch): run the dispatches one by one then.  It allocates (tables and
+ * workspace) and synchronises; mgn_chain_run allocates nothing and is asynchronous on the
+ * context's stream.  The weights and buffers must outlive the chain; free it before them.
+ * A chain must not be recorded into a HIP graph that is replayed: consecutive runs alternate
+ * between two sets of workspace slots. */
+typedef struct mgn_chain mgn_chain;
+typedef struct mgn_chain_stage {
+  const mgn_weight* w;
+  const mgn_buf* a;           /* [1, K] activations ([1, 2K] = gate | up with MGN_PROLOGUE_SWIGLU) */
+  mgn_prologue prologue;      /* what the activations go through first (mgn_matmul_q_rms_norm / _swiglu) */
+  const mgn_buf* norm_weight; /* [K], MGN_PROLOGUE_RMS_NORM only */
+  float eps;
+  const mgn_buf* d;           /* residual [1, N], may be null */
+  mgn_buf* c;                 /* [1, N] */
+  const mgn_unary* ops;       /* unary operations on the output, first to last (mgn_matmul_q_epilogue), may be null */
+  size_t n_ops;               /* at most 8 */
+} mgn_chain_stage;
+mgn_status mgn_chain_create(mgn_ctx* ctx, const mgn_chain_stage* stages, size_t count, uint32_t m, mgn_chain** out);
+mgn_status mgn_chain_run(mgn_ctx* ctx, mgn_chain* chain);
+void mgn_chain_free(mgn_ctx* ctx, mgn_chain* chain);
+
 /* ---- GPU timing on the context's stream: Session::set_profiling +
  *      dump_gpu_timings (src/runtime.rs:1965, 2798-2832) reduced to one
  *      start/stop pair of HIP events. */

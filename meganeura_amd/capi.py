@@ -26,6 +26,7 @@ HIP_SYMBOLS = [
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
     "mgn_weight_info", "mgn_weight_dequantize", "mgn_weight_export_ref", "mgn_weight_save", "mgn_weight_load", "mgn_matmul_q",
     "mgn_matmul_q_f16a", "mgn_matmul_q_static", "mgn_matmul_q_epilogue", "mgn_matmul_q_at", "mgn_matmul_q_plan", "mgn_matmul_q_rms_norm", "mgn_matmul_q_swiglu", "mgn_matmul_q_can_fuse", "mgn_matmul_q_batch",
+    "mgn_chain_create", "mgn_chain_run", "mgn_chain_free",
     "mgn_timer_start", "mgn_timer_stop", "mgn_version", "mgn_built_for",
 ]
 SESSION_SYMBOLS = [
@@ -36,7 +37,7 @@ SESSION_SYMBOLS = [
     "mgn_session_num_dispatches", "mgn_session_dispatch_info", "mgn_session_set_parameter",
     "mgn_session_set_input", "mgn_session_step", "mgn_session_wait", "mgn_session_read_output",
     "mgn_session_read_output_by_index", "mgn_session_ctx", "mgn_session_set_graph_replay",
-    "mgn_session_graph_active", "mgn_session_set_fusion", "mgn_session_num_launches",
+    "mgn_session_graph_active", "mgn_session_set_fusion", "mgn_session_set_chains", "mgn_session_num_launches",
 ]
 
 
@@ -45,6 +46,11 @@ class MatmulItem(C.Structure):
 
 
 PROLOGUE_NONE, PROLOGUE_RMS_NORM, PROLOGUE_SWIGLU = range(3)
+
+
+class ChainStage(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("a", C.c_void_p), ("prologue", C.c_int), ("norm_weight", C.c_void_p), ("eps", C.c_float),
+                ("d", C.c_void_p), ("c", C.c_void_p), ("ops", C.POINTER(C.c_int)), ("n_ops", C.c_size_t)]
 
 
 class DispatchInfo(C.Structure):
@@ -119,6 +125,9 @@ def load():
         "mgn_matmul_q_swiglu": (C.c_int, [vp, vp, vp, vp, vp, C.c_uint32]),
         "mgn_matmul_q_can_fuse": (C.c_int, [vp, vp, C.c_uint32]),
         "mgn_matmul_q_batch": (C.c_int, [vp, vp, C.c_int, vp, C.c_float, C.POINTER(MatmulItem), sz, C.c_uint32]),
+        "mgn_chain_create": (C.c_int, [vp, C.POINTER(ChainStage), sz, C.c_uint32, C.POINTER(vp)]),
+        "mgn_chain_run": (C.c_int, [vp, vp]),
+        "mgn_chain_free": (None, [vp, vp]),
         "mgn_timer_start": (C.c_int, [vp]),
         "mgn_timer_stop": (C.c_int, [vp, C.POINTER(C.c_float)]),
         "mgn_version": (C.c_char_p, []),
@@ -154,6 +163,7 @@ def load():
         "mgn_session_set_graph_replay": (C.c_int, [vp, C.c_int]),
         "mgn_session_graph_active": (C.c_int, [vp]),
         "mgn_session_set_fusion": (C.c_int, [vp, C.c_int]),
+        "mgn_session_set_chains": (C.c_int, [vp, C.c_int]),
         "mgn_session_num_launches": (sz, [vp]),
     }
     for name, (res, args) in sig.items():
@@ -388,6 +398,41 @@ class Context:
 
     def can_fuse(self, w, m):
         return bool(self.lib.mgn_matmul_q_can_fuse(self.h, w.h, m))
+
+    def chain(self, stages, m=1):
+        """One launch for a chain of dependent one-row matmuls.  stages: dicts with w, a, c and
+        optionally prologue, norm_weight, eps, d, ops (mgn_chain_stage)."""
+        return Chain(self, stages, m)
+
+
+class Chain:
+    def __init__(self, ctx, stages, m=1):
+        self.ctx = ctx
+        arr = (ChainStage * len(stages))()
+        self._keep = []
+        for s, st in zip(arr, stages):
+            s.w, s.a, s.c = st["w"].h, st["a"].h, st["c"].h
+            s.prologue = st.get("prologue", PROLOGUE_NONE)
+            s.norm_weight = st["norm_weight"].h if st.get("norm_weight") is not None else None
+            s.eps = st.get("eps", 0.0)
+            s.d = st["d"].h if st.get("d") is not None else None
+            ops = list(st.get("ops", ()))
+            if ops:
+                o = (C.c_int * len(ops))(*ops)
+                self._keep.append(o)
+                s.ops = C.cast(o, C.POINTER(C.c_int))
+            s.n_ops = len(ops)
+        h = C.c_void_p()
+        ctx.check(ctx.lib.mgn_chain_create(ctx.h, arr, len(stages), m, C.byref(h)))
+        self.h = h
+
+    def run(self):
+        self.ctx.check(self.ctx.lib.mgn_chain_run(self.ctx.h, self.h))
+
+    def free(self):
+        if self.h:
+            self.ctx.lib.mgn_chain_free(self.ctx.h, self.h)
+            self.h = None
 
 
 class Buffer:

@@ -42,53 +42,10 @@
 // read consecutive 16-byte chunks.
 #pragma once
 #include "kernels_common.hip.h"
+#include "kernels_gemv_prep.hip.h"
 
 namespace mgn {
 namespace {
-
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
-// fp16 bit patterns used as operands stand for value * 2^-kOperandShift
-template <int FMT>
-constexpr float operand_scale() { return FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f; }  // 2^20, 2^24
-constexpr int kMaxTasks = 2;  // activation chunks a thread prepares at most, per row
-// weight blocks in flight per lane ahead of the one in use (measured: 3 for Q4's 20-byte
-// blocks, 2 for Q8's 34-byte blocks; one more or less costs 0.3-0.4 us on a 4096 x 14336 weight)
-template <int FMT>
-constexpr int prefetch_depth() { return FMT == MGN_FMT_Q8 ? 2 : 3; }
-
-__device__ __forceinline__ half4 as_half4(uint32_t lo, uint32_t hi) {
-  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-  const u32x2 v = {lo, hi};
-  return __builtin_bit_cast(half4, v);
-}
-
-// two floats -> packed fp16 pair, truncating: the low halves computed from the
-// residual make up for the truncation
-__device__ __forceinline__ uint32_t pack_rtz(float a, float b) {
-  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
-}
-__device__ __forceinline__ float half_lo(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[0]; }
-__device__ __forceinline__ float half_hi(uint32_t p) { return (float)__builtin_bit_cast(half2_t, p)[1]; }
-
-constexpr int kRowRor4 = 0x124, kRowRor8 = 0x128;  // rotate right within a row of 16 lanes
-
-// sum over the 16 lanes sharing lane%4 (every such lane ends with the total)
-__device__ __forceinline__ float sum_over_blocks(float v) {
-  v += dpp_move<kRowRor4>(v);
-  v += dpp_move<kRowRor8>(v);
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  return v;
-}
-
-// src/shaders/swiglu_concat.wgsl:20-32: silu(gate) * up with sig = 1 / (1 + exp(-gate))
-__device__ __forceinline__ float swiglu_act(float gate, float up) {
-  const float sig = 1.0f / (1.0f + expf(-gate));
-  return gate * sig * up;
-}
 
 // Up to three weights that share K, the format and the activations, served by one launch
 // (the q, k and v projections of a decode layer): their column quads are numbered one
@@ -181,57 +138,6 @@ __device__ __forceinline__ void make_chunks(const float (&x)[8], uint4& hi, uint
 #pragma unroll
   for (int i = 0; i < 4; i++) l[i] = pack_rtz(p[2 * i] - half_lo(h[i]), p[2 * i + 1] - half_hi(h[i]));
   lo = make_uint4(l[0], l[1], l[2], l[3]);
-}
-
-// ---- one activation row: integer digits on the int8 matrix instruction ----
-// With a single activation row the four A rows of v_mfma_i32_4x4x4_16B_i8 hold the base-128
-// digits of the activations instead of fp16 halves: x, scaled per 32-element block by a power of
-// two to |x| < 2^20 and rounded to an integer, is d0 + 128 d1 + 16384 d2 with d0, d1 in
-// [0, 127] and d2 in [-64, 64] -- three int8 rows (the fourth is not used).  The B operand is
-// then the nibbles as bytes (two mask operations per four weights instead of seven for eight) or,
-// for Q8, the weight bytes as they are; the products are exact integers and the three digit sums
-// are put together with two shift-adds.  The vector ALU work per block drops by a third, which
-// is what bounds the Q4 kernel when the engine clock is low.
-// A block's image is 128 bytes: Q4 [plane i][MFMA 0..7] dwords (MFMA 2c holds elements 8c + 0, 2,
-// 4, 6 and MFMA 2c + 1 elements 8c + 1, 3, 5, 7, as the two nibble masks deliver them); Q8
-// [half][plane i][MFMA 0..3] dwords in natural order.
-
-// eight scaled activations -> their three digit planes, four bytes per dword: lo[i], hi[i] hold
-// plane i of elements (e0, e1, e2, e3) and (e4, e5, e6, e7) of the given order
-__device__ __forceinline__ void make_digits(const float (&x)[8], const int (&order)[8], uint32_t (&lo)[3], uint32_t (&hi)[3], int* sum) {
-  int v[8];
-  int s = 0;
-#pragma unroll
-  for (int e = 0; e < 8; e++) {
-    v[e] = (int)__builtin_rintf(x[e]);
-    s += v[e];
-  }
-  *sum = s;
-#pragma unroll
-  for (int i = 0; i < 3; i++) {
-    uint32_t d[8];
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-      const int val = v[order[e]];
-      d[e] = i == 0 ? (uint32_t)val & 127u : i == 1 ? ((uint32_t)val >> 7) & 127u : (uint32_t)(val >> 14) & 255u;
-    }
-    lo[i] = d[0] | (d[1] << 8) | (d[2] << 16) | (d[3] << 24);
-    hi[i] = d[4] | (d[5] << 8) | (d[6] << 16) | (d[7] << 24);
-  }
-}
-
-// Power of two that brings a block's largest magnitude below 2^12 (1 if the block
-// is all zero, tiny or not finite).  *inv gets the reciprocal.
-__device__ __forceinline__ float block_scale(float amax, float* inv) {
-  const uint32_t amax_bits = __builtin_bit_cast(uint32_t, amax);
-  const int e = (int)(amax_bits >> 23) - 127;  // floor(log2(amax)) for normal values
-  if (amax_bits == 0 || e >= 100 || e <= -100) {
-    *inv = 1.0f;
-    return 1.0f;
-  }
-  const int sh = 11 - e;  // amax * 2^sh in [2^11, 2^12)
-  *inv = __builtin_bit_cast(float, (uint32_t)(127 - sh) << 23);
-  return __builtin_bit_cast(float, (uint32_t)(127 + sh) << 23);
 }
 
 // blockDim.x = 64 * ksc * wnc.  Wave w: K split ks = w % ksc, quad slot wn = w / ksc.

@@ -8,6 +8,7 @@
 #include <mutex>
 #include <new>
 #include <string>
+#include <algorithm>
 #include <vector>
 
 #include "mgn_internal.h"
@@ -138,9 +139,11 @@ mgn_status check_range_flag(mgn_ctx* ctx) {
   volatile uint32_t* const flags = (volatile uint32_t*)ctx->range_flag_host;
   if (flags[1] != 0) {
     // what the parts of that launch stored after the reader had given up is still in the hand-over
-    // workspace: make it empty again before anything else runs
+    // workspace (and in the slots of the chains): make it empty again before anything else runs
     flags[0] = flags[1] = 0;
     hipError_t e = ctx->handover ? hipMemsetAsync(ctx->handover, 0xFF, ctx->handover_bytes, ctx->stream) : hipSuccess;
+    for (mgn_chain* ch : ctx->chains)
+      if (e == hipSuccess && ch->slot_words) e = hipMemsetAsync(ch->slots[0], 0xFF, (size_t)2 * ch->slot_words * 4, ctx->stream);
     if (e == hipSuccess && ctx->static_scratch)
       e = hipMemsetAsync((char*)ctx->static_scratch + kStaticHandoverOffset, 0xFF, kStaticPartialBytes, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
@@ -918,6 +921,174 @@ mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, 
     if (e != 0) return fail(ctx, MGN_EHIP, hipGetErrorString((hipError_t)e));
   }
   return MGN_OK;
+}
+
+// ---- chains ----
+
+mgn_status mgn_chain_create(mgn_ctx* ctx, const mgn_chain_stage* stages, size_t count, uint32_t m, mgn_chain** out) {
+  if (!ctx || !stages || !out) return fail(ctx, MGN_EINVAL, "null argument");
+  *out = nullptr;
+  if (count == 0 || count > 4096) return fail(ctx, MGN_EINVAL, "a chain holds 1 to 4096 stages");
+  if (m != 1) return fail(ctx, MGN_EUNSUPPORTED, "chains serve one activation row (M = 1)");
+  // Small stages are latency-bound: the chain then runs on one XCD (an eighth of the CUs), where a
+  // hand-over is a trip to the shared L2 instead of one through memory.
+  size_t weight_bytes = 0;
+  for (size_t j = 0; j < count; j++)
+    if (stages[j].w) weight_bytes += stages[j].w->meta_bytes + stages[j].w->quant_bytes;
+  uint32_t wg_stride = weight_bytes / count <= ((size_t)2 << 20) && ctx->num_cus % 8 == 0 ? 8u : 1u;
+  if (const char* e = getenv("MGN_CHAIN_XCDS")) wg_stride = e[0] == '1' ? 8u : 1u;
+  const int chain_cus = ctx->num_cus / (int)wg_stride;
+  std::vector<mgn::ChainStageDev> dev(count);
+  std::vector<int> a_from(count, -1), d_from(count, -1);
+  std::vector<char> has_reader(count, 0);
+  size_t lds = 0;
+  uint32_t grid = 1;
+  const mgn_fmt fmt = stages[0].w ? stages[0].w->fmt : MGN_FMT_Q4;
+  for (size_t j = 0; j < count; j++) {
+    const mgn_chain_stage& st = stages[j];
+    if (!st.w || !st.a || !st.c) return fail(ctx, MGN_EINVAL, "a stage lacks its weight, activations or output");
+    if (st.prologue < MGN_PROLOGUE_NONE || st.prologue > MGN_PROLOGUE_SWIGLU) return fail(ctx, MGN_EINVAL, "unknown prologue");
+    if (st.n_ops > 8 || (st.n_ops > 0 && !st.ops)) return fail(ctx, MGN_EINVAL, "an epilogue has at most 8 operations");
+    const size_t k = st.w->rows, n = st.w->cols;
+    if (st.a->bytes / 4 < (st.prologue == MGN_PROLOGUE_SWIGLU ? 2 * k : k)) return fail(ctx, MGN_EINVAL, "A is smaller than its row");
+    if (st.prologue == MGN_PROLOGUE_RMS_NORM && (!st.norm_weight || st.norm_weight->bytes / 4 < k))
+      return fail(ctx, MGN_EINVAL, "norm weight is missing or shorter than K floats");
+    if (st.c->bytes / 4 < n) return fail(ctx, MGN_EINVAL, "C is smaller than N floats");
+    if (st.d && st.d->bytes / 4 < n) return fail(ctx, MGN_EINVAL, "D is smaller than N floats");
+    if (st.c == st.a || st.c->ptr == st.a->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
+    if (st.w->fmt != fmt) return fail(ctx, MGN_EUNSUPPORTED, "the stages of a chain share one weight format");
+    mgn::ChainStageDev& d = dev[j];
+    d = mgn::ChainStageDev{};
+    d.meta = st.w->meta, d.quants = st.w->quants, d.k = (uint32_t)k, d.n = (uint32_t)n;
+    d.pro = (uint32_t)st.prologue, d.eps = st.eps;
+    d.norm_w = st.prologue == MGN_PROLOGUE_RMS_NORM ? (const float*)st.norm_weight->ptr : nullptr;
+    for (size_t i = 0; i < st.n_ops; i++) {
+      if (st.ops[i] < MGN_UNARY_RELU || st.ops[i] > MGN_UNARY_SILU) return fail(ctx, MGN_EINVAL, "unknown unary operation in the epilogue");
+      d.epilogue |= (uint32_t)st.ops[i] << (4 * i);
+    }
+    d.c = (float*)st.c->ptr;
+    // the latest earlier stage that writes what this one reads
+    for (size_t p = 0; p < j; p++) {
+      if (stages[p].c->ptr == st.a->ptr) a_from[j] = (int)p;
+      if (st.d && stages[p].c->ptr == st.d->ptr) d_from[j] = (int)p;
+      if (stages[p].c->ptr == st.c->ptr) return fail(ctx, MGN_EUNSUPPORTED, "two stages of a chain write the same buffer");
+    }
+    if (a_from[j] >= 0) has_reader[a_from[j]] = 1;
+    if (d_from[j] >= 0) has_reader[d_from[j]] = 1;
+  }
+  // Phases: consecutive stages that read nothing from each other share the workgroups between
+  // them (in proportion to their column quads), so a workgroup serves one stage per phase and the
+  // chain's length in hand-overs is its number of phases (a decode layer: q, k, v and o together,
+  // then gate | up, then down).
+  for (size_t p0 = 0; p0 < count;) {
+    size_t p1 = p0 + 1;
+    while (p1 < count && a_from[p1] < (int)p0 && d_from[p1] < (int)p0 && (int)(p1 - p0) < chain_cus) p1++;
+    uint64_t quads = 0;
+    for (size_t j = p0; j < p1; j++) quads += (dev[j].n + 3) / 4;
+    uint32_t first = 0;
+    for (size_t j = p0; j < p1; j++) {
+      const uint64_t mine = (dev[j].n + 3) / 4;
+      const uint32_t left_stages = (uint32_t)(p1 - j - 1);
+      uint32_t share = (uint32_t)std::max<uint64_t>(1, (uint64_t)chain_cus * mine / quads);
+      share = std::min<uint32_t>(share, (uint32_t)chain_cus - first - left_stages);  // every later stage of the phase keeps at least one
+      size_t need = 0;
+      if (!mgn::plan_chain_stage((int)fmt, (int)share, &dev[j], &need))
+        return fail(ctx, MGN_EUNSUPPORTED, "stage " + std::to_string(j) + " is not served by the chain kernel (Q4, K <= 16384)");
+      dev[j].wg_first = first;
+      first += dev[j].wgs;
+      lds = std::max(lds, need);
+      grid = std::max(grid, first);
+    }
+    p0 = p1;
+  }
+  // A buffer that some stage reads as written before the launch must not be written by any stage:
+  // the workgroups are not in step, and one that is ahead would overwrite what another still reads.
+  for (size_t j = 0; j < count; j++) {
+    const void* ext[3] = {a_from[j] < 0 ? stages[j].a->ptr : nullptr, (stages[j].d && d_from[j] < 0) ? stages[j].d->ptr : nullptr,
+                          stages[j].norm_weight ? stages[j].norm_weight->ptr : nullptr};
+    for (size_t p = 0; p < count; p++)
+      for (const void* e : ext)
+        if (e && stages[p].c->ptr == e) return fail(ctx, MGN_EUNSUPPORTED, "a stage writes a buffer that the chain reads as its input");
+  }
+  // slots for the outputs that later stages read
+  std::vector<size_t> slot_at(count, 0);
+  size_t slot_words = 0;
+  for (size_t j = 0; j < count; j++)
+    if (has_reader[j]) {
+      slot_at[j] = slot_words;
+      slot_words += align_up(dev[j].n, 64);
+    }
+  if (slot_words > 0x3FFFFFFFu) return fail(ctx, MGN_EUNSUPPORTED, "chain workspace too large");
+  auto* ch = new (std::nothrow) mgn_chain();
+  if (!ch) return fail(ctx, MGN_ENOMEM, "out of host memory");
+  ch->fmt = (int)fmt, ch->nstages = (uint32_t)count, ch->grid = grid, ch->lds = lds, ch->slot_words = (uint32_t)slot_words;
+  ch->wg_stride = wg_stride;
+  const size_t table_bytes = align_up(count * sizeof(mgn::ChainStageDev), 256);
+  const size_t total = 2 * table_bytes + 2 * slot_words * 4 + 256;
+  hipError_t e = hipMalloc(&ch->dev, total);
+  if (e != hipSuccess) {
+    delete ch;
+    return e == hipErrorOutOfMemory ? fail(ctx, MGN_ENOMEM, "out of device memory") : hip_fail(ctx, "hipMalloc", e);
+  }
+  ch->tables[0] = (mgn::ChainStageDev*)ch->dev;
+  ch->tables[1] = (mgn::ChainStageDev*)((char*)ch->dev + table_bytes);
+  ch->slots[0] = (uint32_t*)((char*)ch->dev + 2 * table_bytes);
+  ch->slots[1] = ch->slots[0] + slot_words;
+  std::vector<mgn::ChainStageDev> both(2 * count);
+  for (int set = 0; set < 2; set++)
+    for (size_t j = 0; j < count; j++) {
+      mgn::ChainStageDev d = dev[j];
+      const mgn_chain_stage& st = stages[j];
+      float* const base = (float*)ch->slots[set];
+      d.a = a_from[j] >= 0 ? base + slot_at[a_from[j]] : (const float*)st.a->ptr;
+      d.a_poll = a_from[j] >= 0;
+      if (const char* dbg = getenv("MGN_CHAIN_DEBUG")) {
+        if (dbg[0] == '1') d.a = (const float*)st.a->ptr, d.a_poll = 0;   // user buffer, no polling (racy)
+        if (dbg[0] == '2') d.a_poll = 0;                                  // slot, no polling (racy)
+        if (dbg[0] == '3' && a_from[j] >= 0) d.a = (const float*)st.a->ptr;  // user buffer, polled loads
+      }
+      d.d = !st.d ? nullptr : d_from[j] >= 0 ? base + slot_at[d_from[j]] : (const float*)st.d->ptr;
+      d.d_poll = st.d && d_from[j] >= 0;
+      d.c_slot = has_reader[j] ? base + slot_at[j] : nullptr;
+      both[set * count + j] = d;
+    }
+  e = hipMemcpyAsync(ch->tables[0], both.data(), count * sizeof(mgn::ChainStageDev), hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(ch->tables[1], both.data() + count, count * sizeof(mgn::ChainStageDev), hipMemcpyHostToDevice, ctx->stream);
+  if (e == hipSuccess && slot_words) e = hipMemsetAsync(ch->slots[0], 0xFF, 2 * slot_words * 4, ctx->stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);  // `both` goes out of scope
+  if (e != hipSuccess) {
+    (void)hipFree(ch->dev);
+    delete ch;
+    return hip_fail(ctx, "chain upload", e);
+  }
+  ctx->chains.push_back(ch);
+  *out = ch;
+  return MGN_OK;
+}
+
+mgn_status mgn_chain_run(mgn_ctx* ctx, mgn_chain* chain) {
+  if (!ctx || !chain) return fail(ctx, MGN_EINVAL, "null argument");
+  const uint32_t set = chain->runs & 1u;
+  const int rc = mgn::launch_chain(ctx->stream, ctx->device, chain->fmt, chain->tables[set], chain->nstages, chain->grid, chain->lds,
+                                   chain->slots[set ^ 1u], chain->slot_words, ctx->spin_limit, ctx->range_flag_dev + 1, chain->wg_stride);
+  if (rc != 0) return hip_fail(ctx, "chain launch", (hipError_t)rc);
+  chain->runs++;
+  return MGN_OK;
+}
+
+void mgn_chain_free(mgn_ctx* ctx, mgn_chain* chain) {
+  if (!chain) return;
+  if (ctx) {
+    (void)hipStreamSynchronize(ctx->stream);
+    for (size_t i = 0; i < ctx->chains.size(); i++)
+      if (ctx->chains[i] == chain) {
+        ctx->chains.erase(ctx->chains.begin() + (long)i);
+        break;
+      }
+  }
+  if (chain->dev) (void)hipFree(chain->dev);
+  delete chain;
 }
 
 // ---- timing ----

@@ -3,6 +3,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <string>
+#include <vector>
 
 #include "../../include/mgn_hip.h"
 #include "../../include/mgn_bench.h"
@@ -119,6 +120,28 @@ constexpr size_t kWorkspaceBytes = (size_t)16 << 20;
 constexpr uint32_t kWorkspaceCounters = 4096;
 constexpr size_t kHandoverBytes = (size_t)16 << 20;  // the counter-free hand-over workspace of a context
 int launch_matmul_gemm_mfma(ihipStream_t* s, const LaunchArgs& a);
+// kernels_chain.hip: a chain of dependent one-row matmuls in one launch.  One stage as the kernel
+// reads it from its table in device memory.
+struct ChainStageDev {
+  const void* meta;
+  const void* quants;
+  const float* a;       // activations [K] (kProSwiglu: [2K] = gate | up); a slot of the chain's workspace when made in the chain
+  const float* d;       // residual [N] or null; likewise
+  const float* norm_w;  // [K] (kProRmsNorm)
+  float* c;             // [N]: the caller's buffer
+  float* c_slot;        // the workspace slot later stages read this output from, or null
+  uint32_t k, n;
+  uint32_t pro, epilogue;
+  float eps;
+  uint32_t a_poll, d_poll;  // that operand is made in the chain: poll until none of its words is empty
+  // plan: workgroups that take part, column quads per workgroup, K splits across waves (log2),
+  // 16-block steps per split, quad slots (waves per K split that take quads)
+  uint32_t wgs, qpw_wg, ksc_log2, steps, nslots;
+  uint32_t wg_first;  // the first of the `wgs` consecutive workgroups that serve this stage
+};
+bool plan_chain_stage(int fmt, int num_cus, ChainStageDev* st, size_t* lds);
+int launch_chain(ihipStream_t* s, int device, int fmt, const ChainStageDev* stages_dev, uint32_t nstages, uint32_t grid, size_t lds,
+                 uint32_t* clear_ptr, uint32_t clear_words, uint32_t spin_limit, uint32_t* fault_flag, uint32_t wg_stride);
 // kernels_tile.hip: the 16x16x32 tiled kernel (activation image + weight streaming)
 bool tile_mfma_supported(const LaunchArgs& a);
 // shapes on which the automatic route takes this kernel ahead of the 32x32 tiled one
@@ -148,7 +171,21 @@ struct mgn_ctx {
   void* static_scratch = nullptr;       // this device's copy of the library's static workspace (mgn_matmul_q_static)
   void* at_stage = nullptr;             // transposed activations of the A^T matmul forms, grown on demand
   size_t at_stage_bytes = 0;
+  std::vector<struct mgn_chain*> chains;  // live chains: their workspaces are emptied again after a fault
   std::string err;
+};
+
+// A chain of dependent one-row matmuls served by one launch (mgn_chain_create).
+struct mgn_chain {
+  int fmt = 0;
+  uint32_t nstages = 0, grid = 0;
+  size_t lds = 0;
+  void* dev = nullptr;  // one allocation: two stage tables, then two sets of slots
+  mgn::ChainStageDev* tables[2] = {nullptr, nullptr};
+  uint32_t* slots[2] = {nullptr, nullptr};
+  uint32_t slot_words = 0;  // per set
+  uint32_t runs = 0;        // launches so far: run r works on set r % 2 and empties the other
+  uint32_t wg_stride = 1;   // 8: the chain runs on the workgroups of one XCD only
 };
 
 namespace mgn {

@@ -496,6 +496,7 @@ void Session::release() {
   if (!ctx_) return;
   (void)mgn_sync(ctx_);  // Drop waits for the GPU first (src/runtime.rs:4339-4345)
   drop_graph();
+  drop_chains();
   for (mgn_buf* b : buffers_) mgn_buf_free(ctx_, b);
   for (mgn_weight* w : weights_) mgn_weight_free(ctx_, w);
   buffers_.clear();
@@ -510,6 +511,7 @@ void Session::upload_weight(int buf, const WeightBufferInfo& info, const float* 
   if (info.nk) check(mgn_weight_create_nk(ctx_, fmt, data, info.rows, info.cols, &fresh), "mgn_weight_create_nk");
   else check(mgn_weight_create(ctx_, fmt, data, info.rows, info.cols, &fresh), "mgn_weight_create");
   drop_graph();  // a captured step holds the old handle's addresses
+  drop_chains();  // ... and so does a chain
   launches_planned_ = false;
   mgn_weight_free(ctx_, weights_[buf]);  // waits for in-flight work that may still read it
   weights_[buf] = fresh;
@@ -577,6 +579,7 @@ void Session::set_input(const std::string& name, const float* data, size_t len) 
 // src/runtime.rs:2843-2959 submits the whole plan as one command buffer; the equivalent here
 // is one captured graph.  Kernel nodes only: nothing on this path records a memset.
 void Session::step() {
+  plan_launches();  // (may free chains and synchronise: never inside a stream capture)
   if (exec_) {
     hipError_t e = hipGraphLaunch(exec_, ctx_->stream);
     if (e != hipSuccess) throw std::runtime_error(std::string("hipGraphLaunch: ") + hipGetErrorString(e));
@@ -620,6 +623,7 @@ void Session::step() {
 }
 
 void Session::set_graph_replay(bool on) {
+  if (on != graph_wanted_) launches_planned_ = false;  // chains are left out of a replayed graph
   graph_wanted_ = on;
   if (!on) drop_graph();
 }
@@ -640,11 +644,94 @@ void Session::set_fusion(bool on) {
   drop_graph();
 }
 
+void Session::set_chains(bool on) {
+  if (on == chains_wanted_) return;
+  chains_wanted_ = on;
+  launches_planned_ = false;
+  drop_graph();
+}
+
+void Session::drop_chains() {
+  for (ChainRun& c : chains_) mgn_chain_free(ctx_, c.chain);
+  chains_.clear();
+  chain_of_.clear();
+}
+
 size_t Session::num_launches() {
   plan_launches();
   size_t n = 0;
-  for (char sk : skipped_) n += sk ? 0 : 1;
+  for (size_t i = 0; i < skipped_.size(); i++) {
+    if (skipped_[i]) continue;
+    const int c = chain_of_.empty() ? -1 : chain_of_[i];
+    n += c < 0 || chains_[c].first == i ? 1 : 0;  // a chain is one launch
+  }
   return n;
+}
+
+// One launch for every run of at least two consecutive launches that the chain kernel serves: M = 1,
+// Q4, no transposed activations (src/runtime.rs:2843-2959 encodes the whole step once; here the
+// runs between other kinds of dispatches are what can go out together).
+void Session::plan_chains() {
+  drop_chains();
+  const size_t nd = plan_.dispatches.size();
+  chain_of_.assign(nd, -1);
+  if (!chains_wanted_ || !fusion_wanted_ || graph_wanted_) return;
+  auto chainable = [&](size_t i) {
+    const Dispatch& d = plan_.dispatches[i];
+    if (!is_matmul(d.shader) || is_at(d.shader) || d.params[0] != 1) return false;
+    mgn_weight* w = weights_[d.input_buffers[1]];
+    return w && w->fmt == MGN_FMT_Q4;
+  };
+  for (size_t i = 0; i < nd;) {
+    if (skipped_[i] || !chainable(i)) {
+      i++;
+      continue;
+    }
+    // the run: launches i .. j-1 (skipped dispatches between them belong to some launch of the run or to none that matters)
+    size_t j = i, launches = 0, last = i;
+    while (j < nd && (skipped_[j] || chainable(j))) {
+      if (!skipped_[j]) launches++, last = j;
+      j++;
+    }
+    if (launches >= 2) {
+      std::vector<mgn_chain_stage> stages;
+      std::vector<std::vector<mgn_unary>> ops;  // kept alive until the chain is made
+      ops.reserve(2 * (last - i + 1));
+      for (size_t di = i; di <= last; di++) {
+        if (skipped_[di]) continue;
+        const Dispatch& d = plan_.dispatches[di];
+        const Fused& f = fused_[di];
+        const Dispatch* p = f.kind != kProNone ? &plan_.dispatches[f.producer] : nullptr;
+        auto add = [&](const Dispatch& md, const Fused* mf) {
+          mgn_chain_stage st{};
+          st.w = weights_[md.input_buffers[1]];
+          st.a = p ? buffers_[p->input_buffers[0]] : buffers_[md.input_buffers[0]];
+          st.prologue = (mgn_prologue)f.kind;
+          st.norm_weight = f.kind == kProRmsNorm ? buffers_[p->input_buffers[1]] : nullptr;
+          st.eps = p ? p->eps : 0.0f;
+          st.d = md.input_buffers.size() > 2 ? buffers_[md.input_buffers[2]] : nullptr;
+          ops.emplace_back(md.epilogue);
+          if (mf) ops.back().insert(ops.back().end(), mf->post.begin(), mf->post.end());
+          st.ops = ops.back().empty() ? nullptr : ops.back().data();
+          st.n_ops = ops.back().size();
+          st.c = buffers_[mf && mf->out_buffer >= 0 ? mf->out_buffer : md.output_buffer];
+          stages.push_back(st);
+        };
+        add(d, &f);
+        for (int sib : f.more)
+          if (sib >= 0) add(plan_.dispatches[sib], nullptr);
+      }
+      mgn_chain* ch = nullptr;
+      const mgn_status st = mgn_chain_create(ctx_, stages.data(), stages.size(), 1, &ch);
+      if (st == MGN_OK) {
+        for (size_t di = i; di <= last; di++) chain_of_[di] = (int)chains_.size();
+        chains_.push_back(ChainRun{i, last, ch});
+      } else if (st != MGN_EUNSUPPORTED) {
+        check(st, "mgn_chain_create");
+      }
+    }
+    i = j;
+  }
 }
 
 // Which RmsNorm / SwiGLUConcat dispatches disappear into the matmuls that read them
@@ -657,6 +744,8 @@ void Session::plan_launches() {
   fused_.assign(nd, Fused{});
   skipped_.assign(nd, 0);
   launches_planned_ = true;
+  drop_chains();
+  chain_of_.assign(nd, -1);
   if (!fusion_wanted_) return;
   std::vector<std::vector<int>> readers(plan_.buffers.size());
   for (size_t i = 0; i < nd; i++)
@@ -739,6 +828,7 @@ void Session::plan_launches() {
     producer_of[u.output_buffer] = pi;
     skipped_[ui] = 1;
   }
+  plan_chains();
 }
 
 void Session::run_dispatches() {
@@ -756,6 +846,11 @@ void Session::run_dispatches() {
   };
   for (size_t di = 0; di < plan_.dispatches.size(); di++) {
     if (skipped_[di]) continue;
+    if (chain_of_[di] >= 0) {  // the whole run goes out with its first launch
+      const ChainRun& run = chains_[chain_of_[di]];
+      if (run.first == di) check(mgn_chain_run(ctx_, run.chain), "mgn_chain_run");
+      continue;
+    }
     const Dispatch& d = plan_.dispatches[di];
     float* out = (float*)buffers_[d.output_buffer]->ptr;
     auto fin = [&](size_t i) { return (const float*)buffers_[d.input_buffers[i]]->ptr; };
@@ -1035,6 +1130,9 @@ mgn_status mgn_session_set_graph_replay(mgn_session* s, int enable) {
 }
 mgn_status mgn_session_set_fusion(mgn_session* s, int enable) {
   return session_call(s, [&] { s->s->set_fusion(enable != 0); });
+}
+mgn_status mgn_session_set_chains(mgn_session* s, int enable) {
+  return session_call(s, [&] { s->s->set_chains(enable != 0); });
 }
 size_t mgn_session_num_launches(mgn_session* s) {
   size_t n = 0;

@@ -159,6 +159,10 @@ class Session {
   // launch apply the unary dispatches that follow it (the compiler folds those into tiled
   // matmul entries only, not into the M = 1 ones) (default on).  The plan keeps the reference's dispatch list; only the launches differ.
   void set_fusion(bool on);
+  // Runs of consecutive launches that are all one-row Q4 matmuls (with whatever was folded into
+  // them) go out as ONE launch each (mgn_chain_*), the dependencies between them carried by the
+  // data (default on; needs launch fusion, and is left out while graph replay is wanted).
+  void set_chains(bool on);
   size_t num_launches();  // kernel launches one step makes with the current settings
   bool graph_active() const { return exec_ != nullptr; }
   void wait();
@@ -180,6 +184,15 @@ class Session {
     std::vector<mgn_unary> post;  // unary dispatches behind an M = 1 matmul, applied by its launch
     int out_buffer = -1;          // ... whose last output buffer the launch then writes
   };
+  struct ChainRun {
+    size_t first, last;  // dispatch indices the chain stands in for (the skipped ones between them included)
+    mgn_chain* chain;
+  };
+  std::vector<ChainRun> chains_;
+  std::vector<int> chain_of_;    // per dispatch: index into chains_ or -1
+  bool chains_wanted_ = true;
+  void plan_chains();
+  void drop_chains();
   std::vector<Fused> fused_;     // per dispatch (matmuls only)
   std::vector<char> skipped_;    // per dispatch: folded into its consumers
   bool launches_planned_ = false;

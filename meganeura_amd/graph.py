@@ -200,6 +200,10 @@ class Session:
         """Fold RmsNorm / SwiGLUConcat dispatches into the decode matmuls reading them (default on)."""
         self._check(self.lib.mgn_session_set_fusion(self.h, 1 if enable else 0))
 
+    def set_chains(self, enable):
+        """Runs of one-row Q4 matmul launches as one launch each (default on)."""
+        self._check(self.lib.mgn_session_set_chains(self.h, 1 if enable else 0))
+
     def num_launches(self):
         return int(self.lib.mgn_session_num_launches(self.h))
 

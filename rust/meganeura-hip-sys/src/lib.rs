@@ -78,6 +78,27 @@ pub struct mgn_matmul_item {
     pub c: *mut mgn_buf,
 }
 
+/// A chain of dependent one-row matmuls served by one launch (`mgn_chain_create`).
+#[repr(C)]
+pub struct mgn_chain {
+    _private: [u8; 0],
+}
+
+/// One stage of a chain: `C = f(prologue(A) x W + D)`.
+#[repr(C)]
+#[derive(Clone, Copy)]
+pub struct mgn_chain_stage {
+    pub w: *const mgn_weight,
+    pub a: *const mgn_buf,
+    pub prologue: mgn_prologue,
+    pub norm_weight: *const mgn_buf,
+    pub eps: f32,
+    pub d: *const mgn_buf,
+    pub c: *mut mgn_buf,
+    pub ops: *const mgn_unary,
+    pub n_ops: usize,
+}
+
 #[repr(C)]
 #[derive(Clone, Copy, Debug, Default)]
 pub struct mgn_plan_info {
@@ -133,6 +154,9 @@ extern "C" {
     pub fn mgn_matmul_q_swiglu(ctx: *mut mgn_ctx, gate_up: *const mgn_buf, w: *const mgn_weight, d: *const mgn_buf, c: *mut mgn_buf, m: u32) -> mgn_status;
     pub fn mgn_matmul_q_can_fuse(ctx: *mut mgn_ctx, w: *const mgn_weight, m: u32) -> c_int;
     pub fn mgn_matmul_q_batch(ctx: *mut mgn_ctx, a: *const mgn_buf, prologue: mgn_prologue, norm_weight: *const mgn_buf, eps: f32, items: *const mgn_matmul_item, count: usize, m: u32) -> mgn_status;
+    pub fn mgn_chain_create(ctx: *mut mgn_ctx, stages: *const mgn_chain_stage, count: usize, m: u32, out: *mut *mut mgn_chain) -> mgn_status;
+    pub fn mgn_chain_run(ctx: *mut mgn_ctx, chain: *mut mgn_chain) -> mgn_status;
+    pub fn mgn_chain_free(ctx: *mut mgn_ctx, chain: *mut mgn_chain);
     pub fn mgn_timer_start(ctx: *mut mgn_ctx) -> mgn_status;
     pub fn mgn_timer_stop(ctx: *mut mgn_ctx, elapsed_ms: *mut f32) -> mgn_status;
     pub fn mgn_version() -> *const c_char;
@@ -226,6 +250,7 @@ pub mod session {
         pub fn mgn_session_wait(s: *mut mgn_session) -> mgn_status;
         pub fn mgn_session_set_graph_replay(s: *mut mgn_session, enable: c_int) -> mgn_status;
         pub fn mgn_session_set_fusion(s: *mut mgn_session, enable: c_int) -> mgn_status;
+        pub fn mgn_session_set_chains(s: *mut mgn_session, enable: c_int) -> mgn_status;
         pub fn mgn_session_num_launches(s: *mut mgn_session) -> usize;
         pub fn mgn_session_graph_active(s: *const mgn_session) -> c_int;
         pub fn mgn_session_read_output(s: *mut mgn_session, out: *mut f32, len: usize) -> mgn_status;

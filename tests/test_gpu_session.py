@@ -238,8 +238,8 @@ def test_graph_replay_matches_individual_launches(orc):
 
 def test_decode_layer_fuses_norm_and_swiglu_into_the_matmuls(orc):
     """9 dispatches in the plan, 4 kernel launches per step: both norms and the SwiGLU ride on
-    the matmuls that read them, and q, k, v share one launch.  Same numbers as the unfused
-    step within the matmul bar."""
+    the matmuls that read them, and q, k, v share one launch; with chains (the default) those
+    four go out as ONE launch.  Same numbers as the unfused step within the matmul bar."""
     hidden, inter = 576, 1536
     g = _decode_layer_graph(hidden, inter, lambda gr, name, shape: gr.parameter_q4(name, shape))
     sess = build_inference_session(g)
@@ -254,10 +254,26 @@ def test_decode_layer_fuses_norm_and_swiglu_into_the_matmuls(orc):
     sizes = [hidden, hidden, hidden // 3, hidden // 3]
     plan = [d.shader for d in sess.plan()]
     assert len(plan) == 9 and plan.count(ShaderEntry.RmsNorm) == 2 and plan.count(ShaderEntry.SwiGLUConcat) == 1
+    assert sess.num_launches() == 1
+    chained = []
+    for _ in range(3):  # consecutive steps alternate between the chain's two sets of hand-over slots
+        sess.step()
+        sess.wait()
+        chained.append([sess.read_output_by_index(i, n) for i, n in enumerate(sizes)])
+    sess.set_chains(False)
     assert sess.num_launches() == 4
     sess.step()
     sess.wait()
     fused = [sess.read_output_by_index(i, n) for i, n in enumerate(sizes)]
+    for step in chained:
+        for a, b in zip(step, fused):
+            assert np.isfinite(a).all()
+            orc.assert_close(a, b, 1e-3, 1e-4)
+    sess.set_graph_replay(True)   # a replayed graph would run a chain on one set of slots every time
+    sess.set_chains(True)
+    assert sess.num_launches() == 4
+    sess.set_graph_replay(False)
+    assert sess.num_launches() == 1
     sess.set_fusion(False)
     assert sess.num_launches() == 9
     sess.step()
