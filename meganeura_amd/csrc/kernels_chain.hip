@@ -15,6 +15,13 @@
 // alternately; a launch empties the other set for the launch after it (by then the launch that
 // used it has ended).  Waits are bounded (spin_limit polls, then the context's fault word is set,
 // the thread goes on with what it has and the next synchronising call reports it).
+// Stages that read nothing from each other (q, k, v and the o-projection of a layer) share the
+// workgroups between them, so the length of a chain in hand-overs is its number of such phases;
+// a hand-over costs about 3.3 us (eight SmolLM2 decode layers, 48 stages in 24 phases: 79 us, against
+// 127 us as 32 separate launches).  Measured and not kept: running the chain on the workgroups of
+// one XCD, so that hand-overs meet in that XCD's L2 (13.0 against 10.2 us per layer: an eighth of
+// the CUs streams the weights), requesting the norm weights and the residual ahead of the polling
+// (+0.1 .. +0.3 us per layer) and the next stage's table entry ahead of its stage (+1.1 us).
 //
 // A stage is the one-row Q4 decode matmul of kernels_gemv_mfma.hip.h in loop form: the
 // activations go through the optional prologue (rms_norm, SwiGLU), are scaled per 32-element block
@@ -83,15 +90,11 @@ __device__ __forceinline__ float load1_polled(const float* p, uint32_t spin_limi
 constexpr int kRing = 3;  // weight blocks in flight per lane ahead of the one in use
 
 // grid = one workgroup per CU (or fewer), 1024 threads.  Every workgroup walks all stages in order.
-// wg_stride: 1, or 8 when the chain is to run on one XCD only: workgroups go to the eight XCDs in
-// turn by their index, so every eighth one shares an XCD (and its L2, where their hand-overs then
-// meet without a trip through memory); the others end at once.
 __global__ __launch_bounds__(1024) void chain_kernel_q4(const ChainStageDev* __restrict__ stages, uint32_t nstages,
                                                         uint32_t* __restrict__ clear_ptr, uint32_t clear_words, uint32_t spin_limit,
-                                                        uint32_t* __restrict__ fault_flag, uint32_t wg_stride) {
+                                                        uint32_t* __restrict__ fault_flag) {
   extern __shared__ uint4 lds4[];
-  if (blockIdx.x % wg_stride != 0) return;
-  const uint32_t wg = blockIdx.x / wg_stride, nwg = gridDim.x / wg_stride;
+  const uint32_t wg = blockIdx.x, nwg = gridDim.x;
   const uint32_t tid = threadIdx.x, lane = tid & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t b = lane >> 2, i = lane & 3;
@@ -323,13 +326,12 @@ bool plan_chain_stage(int fmt, int num_cus, ChainStageDev* st, size_t* lds) {
 }
 
 int launch_chain(ihipStream_t* s, int device, int fmt, const ChainStageDev* stages_dev, uint32_t nstages, uint32_t grid, size_t lds,
-                 uint32_t* clear_ptr, uint32_t clear_words, uint32_t spin_limit, uint32_t* fault_flag, uint32_t wg_stride) {
+                 uint32_t* clear_ptr, uint32_t clear_words, uint32_t spin_limit, uint32_t* fault_flag) {
   if (fmt != MGN_FMT_Q4) return (int)hipErrorInvalidValue;
   static std::atomic<uint64_t> big_lds_done{0};
   if (lds > 64 * 1024)
     if (int e = enable_big_lds(chain_kernel_q4, device, big_lds_done)) return e;
-  hipLaunchKernelGGL(chain_kernel_q4, dim3(grid * wg_stride), dim3(1024), lds, s, stages_dev, nstages, clear_ptr, clear_words, spin_limit,
-                     fault_flag, wg_stride);
+  hipLaunchKernelGGL(chain_kernel_q4, dim3(grid), dim3(1024), lds, s, stages_dev, nstages, clear_ptr, clear_words, spin_limit, fault_flag);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

@@ -930,14 +930,7 @@ mgn_status mgn_chain_create(mgn_ctx* ctx, const mgn_chain_stage* stages, size_t 
   *out = nullptr;
   if (count == 0 || count > 4096) return fail(ctx, MGN_EINVAL, "a chain holds 1 to 4096 stages");
   if (m != 1) return fail(ctx, MGN_EUNSUPPORTED, "chains serve one activation row (M = 1)");
-  // Small stages are latency-bound: the chain then runs on one XCD (an eighth of the CUs), where a
-  // hand-over is a trip to the shared L2 instead of one through memory.
-  size_t weight_bytes = 0;
-  for (size_t j = 0; j < count; j++)
-    if (stages[j].w) weight_bytes += stages[j].w->meta_bytes + stages[j].w->quant_bytes;
-  uint32_t wg_stride = weight_bytes / count <= ((size_t)2 << 20) && ctx->num_cus % 8 == 0 ? 8u : 1u;
-  if (const char* e = getenv("MGN_CHAIN_XCDS")) wg_stride = e[0] == '1' ? 8u : 1u;
-  const int chain_cus = ctx->num_cus / (int)wg_stride;
+  const int chain_cus = ctx->num_cus;
   std::vector<mgn::ChainStageDev> dev(count);
   std::vector<int> a_from(count, -1), d_from(count, -1);
   std::vector<char> has_reader(count, 0);
@@ -1022,7 +1015,6 @@ mgn_status mgn_chain_create(mgn_ctx* ctx, const mgn_chain_stage* stages, size_t 
   auto* ch = new (std::nothrow) mgn_chain();
   if (!ch) return fail(ctx, MGN_ENOMEM, "out of host memory");
   ch->fmt = (int)fmt, ch->nstages = (uint32_t)count, ch->grid = grid, ch->lds = lds, ch->slot_words = (uint32_t)slot_words;
-  ch->wg_stride = wg_stride;
   const size_t table_bytes = align_up(count * sizeof(mgn::ChainStageDev), 256);
   const size_t total = 2 * table_bytes + 2 * slot_words * 4 + 256;
   hipError_t e = hipMalloc(&ch->dev, total);
@@ -1042,11 +1034,6 @@ mgn_status mgn_chain_create(mgn_ctx* ctx, const mgn_chain_stage* stages, size_t 
       float* const base = (float*)ch->slots[set];
       d.a = a_from[j] >= 0 ? base + slot_at[a_from[j]] : (const float*)st.a->ptr;
       d.a_poll = a_from[j] >= 0;
-      if (const char* dbg = getenv("MGN_CHAIN_DEBUG")) {
-        if (dbg[0] == '1') d.a = (const float*)st.a->ptr, d.a_poll = 0;   // user buffer, no polling (racy)
-        if (dbg[0] == '2') d.a_poll = 0;                                  // slot, no polling (racy)
-        if (dbg[0] == '3' && a_from[j] >= 0) d.a = (const float*)st.a->ptr;  // user buffer, polled loads
-      }
       d.d = !st.d ? nullptr : d_from[j] >= 0 ? base + slot_at[d_from[j]] : (const float*)st.d->ptr;
       d.d_poll = st.d && d_from[j] >= 0;
       d.c_slot = has_reader[j] ? base + slot_at[j] : nullptr;
@@ -1071,7 +1058,7 @@ mgn_status mgn_chain_run(mgn_ctx* ctx, mgn_chain* chain) {
   if (!ctx || !chain) return fail(ctx, MGN_EINVAL, "null argument");
   const uint32_t set = chain->runs & 1u;
   const int rc = mgn::launch_chain(ctx->stream, ctx->device, chain->fmt, chain->tables[set], chain->nstages, chain->grid, chain->lds,
-                                   chain->slots[set ^ 1u], chain->slot_words, ctx->spin_limit, ctx->range_flag_dev + 1, chain->wg_stride);
+                                   chain->slots[set ^ 1u], chain->slot_words, ctx->spin_limit, ctx->range_flag_dev + 1);
   if (rc != 0) return hip_fail(ctx, "chain launch", (hipError_t)rc);
   chain->runs++;
   return MGN_OK;

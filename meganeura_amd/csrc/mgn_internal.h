@@ -141,7 +141,7 @@ struct ChainStageDev {
 };
 bool plan_chain_stage(int fmt, int num_cus, ChainStageDev* st, size_t* lds);
 int launch_chain(ihipStream_t* s, int device, int fmt, const ChainStageDev* stages_dev, uint32_t nstages, uint32_t grid, size_t lds,
-                 uint32_t* clear_ptr, uint32_t clear_words, uint32_t spin_limit, uint32_t* fault_flag, uint32_t wg_stride);
+                 uint32_t* clear_ptr, uint32_t clear_words, uint32_t spin_limit, uint32_t* fault_flag);
 // kernels_tile.hip: the 16x16x32 tiled kernel (activation image + weight streaming)
 bool tile_mfma_supported(const LaunchArgs& a);
 // shapes on which the automatic route takes this kernel ahead of the 32x32 tiled one
@@ -185,7 +185,6 @@ struct mgn_chain {
   uint32_t* slots[2] = {nullptr, nullptr};
   uint32_t slot_words = 0;  // per set
   uint32_t runs = 0;        // launches so far: run r works on set r % 2 and empties the other
-  uint32_t wg_stride = 1;   // 8: the chain runs on the workgroups of one XCD only
 };
 
 namespace mgn {

@@ -206,6 +206,7 @@ def test_graph_replay_matches_individual_launches(orc):
         return [sess.read_output_by_index(i, n) for i, n in enumerate(sizes)]
 
     sess.set_graph_replay(False)
+    sess.set_chains(False)      # launch by launch: what the graph records (a chain launch is never recorded)
     want = {seed: run(seed) for seed in (1, 2, 3)}
     assert not sess.graph_active()
     sess.set_graph_replay(True)
