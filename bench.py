@@ -297,6 +297,71 @@ def config_table(ctx, sets, steps=200, repeats=5, preheat_ms=100.0):
     return table
 
 
+def ffn_chain_times(ctx, steps=200, repeats=5, hidden=4096, inter=14336):
+    """The Llama-3-8B-shaped FFN at one token as the dependent pair it is: rms_norm -> gate | up
+    (4096 x 28672) and SwiGLU -> down + residual (14336 x 4096), 110.1 MB of Q4 weights, two launches
+    (each with its neighbour folded in), weights rotating through >= 512 MiB of copies.  Beside it the
+    same pair as ONE chain launch (mgn_chain_*), which is not what the library's Session would do
+    with weights of this size: the chain's looped stage streams them more slowly."""
+    import oracle
+    from meganeura_amd import capi, synth
+
+    x = synth.activations(5, 1, hidden, which=77)
+    g = (1.0 + synth.normal(78, hidden, 0.1)).astype(np.float32)
+    wgu, wd = synth.weights(5, hidden, 2 * inter, which=79), synth.weights(5, inter, hidden, which=80)
+    first = (ctx.weight(Q4, wgu), ctx.weight(Q4, wd))
+    packed = (first[0].export_ref(), first[1].export_ref())
+    nbytes = packed[0].size + packed[1].size
+    copies = max(2, (512 << 20) // nbytes + 1)
+    pairs = [first] + [(ctx.weight_from_packed(Q4, packed[0], hidden, 2 * inter), ctx.weight_from_packed(Q4, packed[1], inter, hidden))
+                       for _ in range(copies - 1)]
+    bx, bg = ctx.upload(x), ctx.upload(g)
+    bgu, by = ctx.buffer(2 * inter * 4), ctx.buffer(hidden * 4)
+
+    def separate(n, at):
+        for i in range(n):
+            wa, wb = pairs[(at + i) % copies]
+            ctx.matmul_q_rms_norm(bx, bg, 1e-5, wa, bgu, 1)
+            ctx.matmul_q_swiglu(bgu, wb, by, 1, bx)
+
+    chains = [ctx.chain([dict(w=wa, a=bx, c=bgu, prologue=capi.PROLOGUE_RMS_NORM, norm_weight=bg, eps=1e-5),
+                         dict(w=wb, a=bgu, c=by, prologue=capi.PROLOGUE_SWIGLU, d=bx)]) for wa, wb in pairs]
+
+    def chained(n, at):
+        for i in range(n):
+            chains[(at + i) % copies].run()
+
+    # the result against numpy pointwise operations + the oracle's matmul (on the first copy)
+    deq = lambda w: oracle.dequantize(Q4, oracle.quantize(Q4, w), *w.shape)
+    x64 = x.astype(np.float64)
+    n1 = (x64 / np.sqrt((x64 ** 2).mean() + 1e-5) * g).astype(np.float32)
+    gu = oracle.matmul_f32(n1, deq(wgu))
+    gg, uu = gu[:, :inter].astype(np.float64), gu[:, inter:].astype(np.float64)
+    want = oracle.matmul_f32((gg / (1.0 + np.exp(-gg)) * uu).astype(np.float32), deq(wd), x)
+    res = {}
+    for name, fn in (("separate", separate), ("chain", chained)):
+        fn(1, 0)
+        oracle.assert_close(by.download(np.float32, hidden).reshape(1, -1), want, 1e-3, 1e-4)
+        fn(600, 0)
+        ctx.sync()
+        t = []
+        for r in range(repeats):
+            ctx.timer_start()
+            fn(steps, r * 3)
+            t.append(ctx.timer_stop() / steps)
+        res[name] = sorted(t)[len(t) // 2] * 1e3
+    bytes_ = nbytes // 20 * 20 + 4 * (hidden + 2 * inter) * 2 + 4 * hidden * 3  # weights + activations in and out of both matmuls + residual
+    for c in chains:
+        c.free()
+    for h in [bx, bg, bgu, by] + [w for p in pairs for w in p]:
+        h.free()
+    return {"us": res["separate"], "chain_us": res["chain"], "algorithmic_bytes": bytes_, "bound": "hbm",
+            "achieved": bytes_ / (res["separate"] * 1e-6) / 1e9, "unit": "GB/s",
+            "frac": bytes_ / (res["separate"] * 1e-6) / 1e9 / HBM_PEAK_GBS,
+            "what": "rms_norm -> gate|up (4096 x 28672) then SwiGLU -> down + residual (14336 x 4096), Q4, one token: two launches, "
+                    "cache-cold; chain_us = the same pair as one chain launch"}
+
+
 def decode_layer_times(steps, warmup, layers=8):
     """C2 as the reference runs it: SmolLM2-135M decode layers' matmuls through the
     Graph/Session surface (models/smollm2.rs:340-414 without the attention core): rms_norm,
@@ -534,6 +599,7 @@ def main():
 
     if not args.no_configs:
         line["configs"] = config_table(ctx, sets)
+        line["configs"]["c5_q4_ffn_m1"] = ffn_chain_times(ctx)
         layer = decode_layer_times(200, 20)
         line["configs"]["c2_q4_decode_layer_session"] = {
             "us": layer["chain_us_per_layer"],  # the session's default: the whole step's matmuls as one chain launch

@@ -118,8 +118,8 @@ mgn_status mgn_session_set_graph_replay(mgn_session* s, int enable);
  * mgn_session_num_launches reports how many kernels a step really launches.  The folded
  * dispatch's own output buffer is then never written. */
 mgn_status mgn_session_set_fusion(mgn_session* s, int enable);
-/* Chains (on by default; with launch fusion on and graph replay off): every run of at least two
- * consecutive launches that are one-row Q4 matmuls goes out as ONE launch (mgn_chain_create /
+/* Chains (on by default; with launch fusion on and graph replay off): every run of at least three
+ * consecutive launches that are one-row Q4 matmuls on weights of at most 4 MiB goes out as ONE launch (mgn_chain_create /
  * mgn_chain_run in mgn_hip.h), which is how the whole step of a decode plan becomes one submission
  * as in Session::step (src/runtime.rs:2843-2959).  Results are those of the separate launches. */
 mgn_status mgn_session_set_chains(mgn_session* s, int enable);

@@ -668,9 +668,15 @@ size_t Session::num_launches() {
   return n;
 }
 
-// One launch for every run of at least two consecutive launches that the chain kernel serves: M = 1,
-// Q4, no transposed activations (src/runtime.rs:2843-2959 encodes the whole step once; here the
-// runs between other kinds of dispatches are what can go out together).
+// One launch for every run of at least three consecutive launches that the chain kernel serves (M = 1,
+// Q4, no transposed activations) and that are launch-bound: every weight at most 4 MiB packed
+// (src/runtime.rs:2843-2959 encodes the whole step once; here the runs between other kinds of
+// dispatches are what can go out together).  Where it pays was measured: a hand-over inside a chain
+// costs about 3.3 us against 3.7-4 us for a dependent launch, so two stages in a chain take what
+// two launches take (576 -> 3072 -> 576: 7.3 us either way; 1024 -> 6144 -> 1024: 8.4 against 7.6),
+// the gain comes from stages that run side by side and from the one launch they all share (eight
+// SmolLM2 decode layers: 9.8 against 15.8 us per layer), and a chain's looped stage streams a large
+// weight more slowly than the kernels written out for it (4096 -> 28672 -> 4096: 28.7 against 25.5 us).
 void Session::plan_chains() {
   drop_chains();
   const size_t nd = plan_.dispatches.size();
@@ -680,7 +686,7 @@ void Session::plan_chains() {
     const Dispatch& d = plan_.dispatches[i];
     if (!is_matmul(d.shader) || is_at(d.shader) || d.params[0] != 1) return false;
     mgn_weight* w = weights_[d.input_buffers[1]];
-    return w && w->fmt == MGN_FMT_Q4;
+    return w && w->fmt == MGN_FMT_Q4 && w->meta_bytes + w->quant_bytes <= ((size_t)4 << 20);
   };
   for (size_t i = 0; i < nd;) {
     if (skipped_[i] || !chainable(i)) {
@@ -693,7 +699,7 @@ void Session::plan_chains() {
       if (!skipped_[j]) launches++, last = j;
       j++;
     }
-    if (launches >= 2) {
+    if (launches >= 3) {
       std::vector<mgn_chain_stage> stages;
       std::vector<std::vector<mgn_unary>> ops;  // kept alive until the chain is made
       ops.reserve(2 * (last - i + 1));
