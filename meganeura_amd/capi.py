@@ -18,7 +18,7 @@ STATIC_WORKSPACE_BYTES = 4 << 20  # MGN_STATIC_WORKSPACE_BYTES
 ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA, ROUTE_TILE_MFMA = range(6)
 
 # every symbol include/mgn_hip.h, include/mgn_bench.h and include/mgn_session.h declare
-BENCH_SYMBOLS = ["mgn_ctx_set_route", "mgn_ctx_set_spin_limit", "mgn_matmul_q_loop", "mgn_weight_read_loop"]
+BENCH_SYMBOLS = ["mgn_ctx_set_route", "mgn_ctx_set_spin_limit", "mgn_engine_clock_mhz", "mgn_matmul_q_loop", "mgn_weight_read_loop"]
 HIP_SYMBOLS = [
     "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync", "mgn_ctx_set_activation_range",
     "mgn_buf_alloc", "mgn_buf_free", "mgn_buf_size", "mgn_buf_device_ptr", "mgn_buf_upload",
@@ -91,6 +91,7 @@ def load():
         "mgn_sync": (C.c_int, [vp]),
         "mgn_ctx_set_route": (C.c_int, [vp, C.c_int]),
         "mgn_ctx_set_spin_limit": (C.c_int, [vp, C.c_uint32]),
+        "mgn_engine_clock_mhz": (C.c_int, [vp, C.POINTER(C.c_float)]),
         "mgn_ctx_set_activation_range": (C.c_int, [vp, C.c_int]),
         "mgn_buf_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
         "mgn_buf_free": (None, [vp, vp]),
@@ -281,6 +282,11 @@ class Context:
     def set_spin_limit(self, polls):
         """Polls a wave makes for another workgroup's partial sums before it gives up (tests only)."""
         self.check(self.lib.mgn_ctx_set_spin_limit(self.h, polls))
+
+    def engine_clock_mhz(self):
+        mhz = C.c_float()
+        self.check(self.lib.mgn_engine_clock_mhz(self.h, C.byref(mhz)))
+        return float(mhz.value)
 
     def sync(self):
         self.check(self.lib.mgn_sync(self.h))

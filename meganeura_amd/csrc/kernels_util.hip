@@ -532,6 +532,24 @@ __global__ __launch_bounds__(896) void read_probe_gemv_kernel(const char* __rest
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w ^ macc) == 0x9E3779B9u) sink[0] = 1u;
 }
 
+// Measurement aid: the engine clock as a kernel sees it.  The shader clock counter against the
+// constant 100 MHz counter over about 20 us of one wave spinning.
+__global__ void clock_probe_kernel(uint64_t* __restrict__ out) {
+  const uint64_t t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+  uint64_t r1 = r0;
+  for (uint32_t i = 0; i < (1u << 22) && r1 - r0 < 2000; i++) {  // (bounded: ends whatever the counters do)
+    __builtin_amdgcn_s_sleep(8);
+    r1 = __builtin_amdgcn_s_memrealtime();
+  }
+  const uint64_t t1 = __builtin_amdgcn_s_memtime();
+  if (threadIdx.x == 0) out[0] = t1 - t0, out[1] = r1 - r0;
+}
+int launch_clock_probe(ihipStream_t* s, uint64_t* out2_dev) {
+  hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, s, out2_dev);
+  MGN_HIP_LAUNCH_CHECK();
+  return 0;
+}
+
 int launch_read_probe(ihipStream_t* s, const WeightView& w, int num_cus, uint32_t* sink, int pattern) {
   if (pattern == 1) {
     const uint32_t bpc = w.k / 32;

@@ -923,6 +923,18 @@ mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, 
   return MGN_OK;
 }
 
+mgn_status mgn_engine_clock_mhz(mgn_ctx* ctx, float* mhz) {
+  if (!ctx || !mhz) return fail(ctx, MGN_EINVAL, "null argument");
+  // (the first 16 bytes of the split-K workspace hold nothing between launches)
+  const int rc = mgn::launch_clock_probe(ctx->stream, (uint64_t*)ctx->scratch);
+  if (rc != 0) return hip_fail(ctx, "clock probe launch", (hipError_t)rc);
+  uint64_t host[2] = {0, 0};
+  MGN_HIP(ctx, hipMemcpyAsync(host, ctx->scratch, sizeof(host), hipMemcpyDeviceToHost, ctx->stream));
+  MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  *mhz = host[1] ? 100.0f * (float)host[0] / (float)host[1] : 0.0f;
+  return MGN_OK;
+}
+
 // ---- chains ----
 
 mgn_status mgn_chain_create(mgn_ctx* ctx, const mgn_chain_stage* stages, size_t count, uint32_t m, mgn_chain** out) {
