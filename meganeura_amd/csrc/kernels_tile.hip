@@ -22,10 +22,10 @@
 //   Per block: D = sum n x on the matrix cores, then P += d * D on the vector ALU (4 FMAs per
 //     lane).  The format's additive part (m * sum(x) for Q4, -128 * scale * sum(x) for Q8's byte
 //     bias) is one more MFMA per slice of 8 blocks: its A operand holds the blocks' mean
-//     activations (hi, lo; with fp16 activations scaled per (row, slice) by a power of two like
-//     the f32 activations themselves), its B operand the blocks' m (or scale), exact fp16 values.
-//     A slice's P is multiplied by the rows' inverse power-of-two scales and added to the
-//     accumulators.
+//     activations (hi, lo), its B operand the blocks' m (or scale), exact fp16 values.  (fp16
+//     activations: two MFMAs, hi and lo apart, because lo is kept times 2^11; see convert_task.)
+//     With f32 activations a slice's P is multiplied by the rows' inverse power-of-two scales
+//     before it is added to the accumulators.
 //
 // Two kernels share this arithmetic.
 //   tile_mfma_kernel (any M): image_kernel converts the activations ONCE per call into images
@@ -71,10 +71,12 @@ __device__ __forceinline__ float group_max32(float v) {
 //                                that write together during the conversion (one row, two blocks, four
 //                                g) then fall into different LDS banks, and so do the readers'.
 //   [8 * HL * 64 + lane]         A operand of the slice's additive MFMA: lanes (row, g' < 2) hold
-//                                (mean_hi | mean_lo << 16) of blocks 4g'..4g'+3, the rest is zero
-//   [8 * HL * 64 + 64 + 0..15]   (as float) f32 activations: the rows' inverse scales times the quants'
-//                                operand scale (2^20 for Q4, 2^24 for Q8); fp16 activations: the inverse
-//                                scales of the rows' block sums times the additive part's constant
+//                                (mean_hi | mean_lo << 16) of blocks 4g'..4g'+3; f32 activations: the
+//                                rest is zero; fp16 activations: the rest is not written, mean_lo is
+//                                the part of the mean below mean_hi TIMES 2^11, and the readers take
+//                                the two halves apart (mean_operands)
+//   [8 * HL * 64 + 64 + 0..15]   (as float) f32 activations only: the rows' inverse scales times the
+//                                quants' operand scale (2^20 for Q4, 2^24 for Q8)
 // The element order inside an operand follows the B side: Q4 pairs k with k + 4, Q8 is natural.
 // Q4 with f32 activations: the even elements are stored times 16 (see nibbles_to_operand) and the
 // slice scale aims at 2^7 instead of 2^11 to leave room for that.
@@ -159,28 +161,32 @@ __device__ __forceinline__ void convert_task(const TaskWords<F32A>& xin, bool ok
   }
   s += dpp_move<kDppQuadXor1>(s);
   s += dpp_move<kDppQuadXor2>(s);
-  if constexpr (!F32A) {
-    // The block sums of fp16 activations span 2^-24 .. 2^21: the slice's largest is brought to
-    // [2^15, 2^16) (its mean to [2^10, 2^11)) before the means are split into fp16 pairs, so that
-    // neither large sums overflow nor small ones lose their low bits; the additive MFMA's result
-    // is multiplied by the inverse.  (f32 activations were scaled before they were summed.)
-    float am = fabsf(s);
-    am = fmaxf(am, dpp_move<kDppRowHalfMirror>(am));
-    am = fmaxf(am, dpp_move<kDppRowMirror>(am));
-    am = fmaxf(am, __shfl_xor(am, 16, 64));
-    s *= slice_scale<15>(am, &inv);
-  }
   uint32_t* const extra = (uint32_t*)(img + kSliceBlocks * HL * 64);
-  if (g == 0) {
-    const float mean = s * 0.03125f;
-    const uint32_t mh = pack_rtz(mean, 0.0f);
-    extra[(r + 16 * (kb >> 2)) * 4 + (kb & 3)] = (mh & 0xFFFFu) | (pack_rtz(mean - half_lo(mh), 0.0f) << 16);
+  const float mean = s * 0.03125f;
+  const uint32_t mh = pack_rtz(mean, 0.0f);
+  if constexpr (!F32A) {
+    // A block of fp16 activations sums to at most 2^21, its mean to at most 65504: no scale is
+    // needed to keep it in range.  hi is the mean cut to fp16 and lo the rest times 2^11, which fp16
+    // holds exactly down to the smallest sums (the rest is a multiple of 2^-29 below 2^-24) and
+    // without overflow at the largest; the readers multiply lo's products by 2^-11.  So the
+    // conversion needs no maximum over the slice, no scale and no inverse: a permutation and a sum.
+    if (g == 0) extra[(r + 16 * (kb >> 2)) * 4 + (kb & 3)] = (mh & 0xFFFFu) | (pack_rtz((mean - half_lo(mh)) * 2048.0f, 0.0f) << 16);
+    return;
   }
+  if (g == 0) extra[(r + 16 * (kb >> 2)) * 4 + (kb & 3)] = (mh & 0xFFFFu) | (pack_rtz(mean - half_lo(mh), 0.0f) << 16);
   // lanes (row, g' >= 2) of the additive operand stay zero (8 dwords per half-wave lane... 16 rows x 32
-  // lanes cover the 128 dwords); the rows' inverse scales follow: of the activations, times the
-  // quants' operand scale (f32), or of the block sums, times the additive part's constant (fp16)
+  // lanes cover the 128 dwords); the rows' inverse scales, times the quants' operand scale, follow
   if (l < 8) extra[32 * 4 + r * 8 + l] = 0u;
-  if (l == 0) ((float*)extra)[64 * 4 + r] = inv * (F32A ? (FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f) : additive_constant<FMT>());
+  if (l == 0) ((float*)extra)[64 * 4 + r] = inv * (FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f);
+}
+
+// fp16 activations: the two A operands of a row tile's additive MFMAs, mean_hi and mean_lo apart
+// (`extra`: the row tile's additive words in the image).  Lanes (row, g' >= 2) have no blocks.
+__device__ __forceinline__ void mean_operands(const uint8_t* extra, uint32_t lane, uint32_t g, half8* hi, half8* lo) {
+  const u32x4_t w = *(const u32x4_t*)(extra + (lane & 31) * 16);
+  const bool has = g < 2;
+  *hi = as_half8(has ? w.x & 0xFFFFu : 0u, has ? w.y & 0xFFFFu : 0u, has ? w.z & 0xFFFFu : 0u, has ? w.w & 0xFFFFu : 0u);
+  *lo = as_half8(has ? w.x >> 16 : 0u, has ? w.y >> 16 : 0u, has ? w.z >> 16 : 0u, has ? w.w >> 16 : 0u);
 }
 
 // grid.x = row tiles * slices; 512 threads: half-wave r (0..15) converts row r of the tile,
@@ -275,21 +281,23 @@ __device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t*
 #pragma unroll
     for (int r = 0; r < R; r++) {
       const uint8_t* const ir = ib + lane * 16 + r * rstride + 8 * HL * 64 * 16;
-      const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, *(const u32x4_t*)ir), bm,
-                                                               floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-      // f32 activations: the rows' inverse slice scales (times 2^20 or 2^24: the operand scale of the
-      // quants); fp16 activations: the inverse scales of the rows' block sums times kAdd
-      const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
       if constexpr (F32A) {
+        const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, *(const u32x4_t*)ir), bm,
+                                                                 floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        // the rows' inverse slice scales (times 2^20 or 2^24: the operand scale of the quants)
+        const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
         acc[r][0] = __fmaf_rn(__fmaf_rn(kAdd, d[0], P[r][0]), inv.x, acc[r][0]);
         acc[r][1] = __fmaf_rn(__fmaf_rn(kAdd, d[1], P[r][1]), inv.y, acc[r][1]);
         acc[r][2] = __fmaf_rn(__fmaf_rn(kAdd, d[2], P[r][2]), inv.z, acc[r][2]);
         acc[r][3] = __fmaf_rn(__fmaf_rn(kAdd, d[3], P[r][3]), inv.w, acc[r][3]);
       } else {
-        acc[r][0] += __fmaf_rn(inv.x, d[0], P[r][0]);
-        acc[r][1] += __fmaf_rn(inv.y, d[1], P[r][1]);
-        acc[r][2] += __fmaf_rn(inv.z, d[2], P[r][2]);
-        acc[r][3] += __fmaf_rn(inv.w, d[3], P[r][3]);
+        // the means' hi and lo apart, lo's products times 2^-11 (see convert_task)
+        half8 ah, al;
+        mean_operands(ir - lane * 16, lane, g, &ah, &al);
+        const floatx4 dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bm, floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        const floatx4 dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bm, floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[r][i] += __fmaf_rn(kAdd / 2048.0f, dl[i], __fmaf_rn(kAdd, dh[i], P[r][i]));
       }
     }
   }
@@ -687,23 +695,28 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
 #pragma unroll
   for (int r = 0; r < R; r++) {
     const uint8_t* const ir = ib + lane * 16 + r * rstride + 8 * HL * 64 * 16;
-    const half8 am = __builtin_bit_cast(half8, *(const u32x4_t*)ir);
-    // f32 activations: the rows' inverse slice scales (times 2^20 or 2^24); fp16 activations: the
-    // inverse scales of the rows' block sums times kAdd
-    const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
+    if constexpr (F32A) {
+      const half8 am = __builtin_bit_cast(half8, *(const u32x4_t*)ir);
+      // the rows' inverse slice scales (times 2^20 or 2^24)
+      const float4 inv = *(const float4*)(ir - lane * 16 + 64 * 16 + g * 16);
 #pragma unroll
-    for (int u = 0; u < kSide; u++) {
-      const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm[u], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
-      if constexpr (F32A) {
+      for (int u = 0; u < kSide; u++) {
+        const floatx4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm[u], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
         acc[u][r][0] = __fmaf_rn(__fmaf_rn(kAdd, d[0], P[u][r][0]), inv.x, acc[u][r][0]);
         acc[u][r][1] = __fmaf_rn(__fmaf_rn(kAdd, d[1], P[u][r][1]), inv.y, acc[u][r][1]);
         acc[u][r][2] = __fmaf_rn(__fmaf_rn(kAdd, d[2], P[u][r][2]), inv.z, acc[u][r][2]);
         acc[u][r][3] = __fmaf_rn(__fmaf_rn(kAdd, d[3], P[u][r][3]), inv.w, acc[u][r][3]);
-      } else {
-        acc[u][r][0] += __fmaf_rn(inv.x, d[0], P[u][r][0]);
-        acc[u][r][1] += __fmaf_rn(inv.y, d[1], P[u][r][1]);
-        acc[u][r][2] += __fmaf_rn(inv.z, d[2], P[u][r][2]);
-        acc[u][r][3] += __fmaf_rn(inv.w, d[3], P[u][r][3]);
+      }
+    } else {
+      // the means' hi and lo apart, lo's products times 2^-11 (see convert_task)
+      half8 ah, al;
+      mean_operands(ir - lane * 16, lane, g, &ah, &al);
+#pragma unroll
+      for (int u = 0; u < kSide; u++) {
+        const floatx4 dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bm[u], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+        const floatx4 dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bm[u], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[u][r][i] += __fmaf_rn(kAdd / 2048.0f, dl[i], __fmaf_rn(kAdd, dh[i], P[u][r][i]));
       }
     }
   }

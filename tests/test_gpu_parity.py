@@ -808,6 +808,37 @@ def test_the_error_scales_with_the_activations(ctx, orc, fmt, f16, m, route):
     wt.free()
 
 
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m,route", [(16, "tile_mfma"), (40, "tile_mfma"), (70, "tile_mfma"), (40, "auto")])
+def test_fp16_block_sums_at_both_ends_of_the_range(ctx, orc, fmt, m, route):
+    """The 16x16x32 kernels carry a block's mean activation as an fp16 pair (the mean cut to fp16,
+    and the rest times 2^11).  Rows that put the pair at its limits: every element at 60000 (block
+    sums of 1.9e6, means near the largest half), alternating +-65504, every element the smallest
+    subnormal half (the mean IS the smallest half), a single smallest half per block (the mean, 2^-29,
+    lives in the low part alone), and ordinary rows between them."""
+    k, n = 1024, 96
+    w = synth.normal(1401, k * n, 0.02).reshape(k, n) + np.float32(0.01)  # (minima and byte bias well away from zero)
+    x = synth.normal(1402 + m, m * k, 1.0).reshape(m, k)
+    tiny = np.float32(2.0 ** -24)
+    x[0, :] = 60000.0
+    x[1, 0::2], x[1, 1::2] = 65504.0, -65504.0
+    x[2, :] = tiny
+    x[3, :] = 0.0
+    x[3, 5::32] = tiny
+    x[4, :] = 0.0
+    x[4, 0::32], x[4, 1::32] = 65504.0, tiny
+    x = x.astype(np.float16).astype(np.float32)
+    deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n)
+    wt = ctx.weight(fmt, w)
+    got = run_matmul(ctx, fmt, x, wt, ROUTES[route], f16=True)
+    assert_close_rowwise(got, orc.matmul_f64(x, deq), x)
+    # the additive part alone must come out: rows 2 and 3 against what the sums times the minima give
+    want = orc.matmul_f64(x, deq)
+    for r in (2, 3):
+        assert np.abs(got[r] - want[r]).max() <= 2e-3 * np.abs(want[r]).max(), r
+    wt.free()
+
+
 def weight_scaled_bar(got, want, x, factor, abs_bar=ABS):
     """The matmul bar for weights scaled by `factor`: outputs and errors scale with it, so the
     absolute part does too (and with each row's activation magnitude)."""
