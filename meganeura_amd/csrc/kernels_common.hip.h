@@ -78,6 +78,17 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+// src/shaders/swiglu_concat.wgsl:20-32: silu(gate) * up with sig = 1 / (1 + exp(-gate)).
+// The hardware's exp2 and reciprocal (1 ulp each) instead of the library's expf and an IEEE
+// division: six instructions instead of about thirty.  Every workgroup of a fused launch
+// evaluates this for all of K, so it is on the path of every column: 14336 x 4096 at one row
+// 10.9 -> 9.9 us.  exp(-gate) overflowing to infinity gives sig = 0 as in the plain formula.
+__device__ __forceinline__ float swiglu_act(float gate, float up) {
+  const float e = __builtin_amdgcn_exp2f(gate * -1.4426950408889634f);
+  const float sig = __builtin_amdgcn_rcpf(1.0f + e);
+  return gate * sig * up;
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for
 // every outstanding global load of the wave (its fences cover global memory),
 // which would stall a kernel that keeps weight loads in flight across the barrier.

@@ -393,8 +393,8 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     const uint32_t nwv = nwaves;
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
-      float tot = 0.0f;
-      for (uint32_t wv = 0; wv < nwv; wv++) tot += nrm[wv * MROWS + r];
+      // (one LDS read and a reduction over 16 lanes, not a read per wave one after the other)
+      const float tot = group_sum<16>((lane & 15u) < nwv ? nrm[(lane & 15u) * MROWS + r] : 0.0f);
       const float rstd = 1.0f / sqrtf(tot / (float)w.k + pro.eps);
 #pragma unroll
       for (int tt = 0; tt < TASKS; tt++)

@@ -44,12 +44,6 @@ __device__ __forceinline__ float sum_over_blocks(float v) {
   return v;
 }
 
-// src/shaders/swiglu_concat.wgsl:20-32: silu(gate) * up with sig = 1 / (1 + exp(-gate))
-__device__ __forceinline__ float swiglu_act(float gate, float up) {
-  const float sig = 1.0f / (1.0f + expf(-gate));
-  return gate * sig * up;
-}
-
 // ---- one activation row: integer digits on the int8 matrix instruction ----
 // With a single activation row the four A rows of v_mfma_i32_4x4x4_16B_i8 hold the base-128
 // digits of the activations instead of fp16 halves: x, scaled per 32-element block by a power of

@@ -302,16 +302,11 @@ __global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, c
   if (i < len) out[i] = a[i] + b[i];
 }
 
-// src/shaders/swiglu_concat.wgsl:20-32: silu(gate) * up with sig = 1 / (1 + exp(-gate))
-__device__ __forceinline__ float swiglu_value(float gate, float up) {
-  const float sig = 1.0f / (1.0f + expf(-gate));
-  return gate * sig * up;
-}
 
 __global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gate, const float* __restrict__ up,
                                                      float* __restrict__ out, size_t len) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < len) out[i] = swiglu_value(gate[i], up[i]);
+  if (i < len) out[i] = swiglu_act(gate[i], up[i]);
 }
 
 __global__ __launch_bounds__(256) void swiglu_concat_kernel(const float* __restrict__ in, float* __restrict__ out,
@@ -320,7 +315,7 @@ __global__ __launch_bounds__(256) void swiglu_concat_kernel(const float* __restr
   if (i >= len) return;
   const size_t row = i / half_n, col = i % half_n;
   const float* p = in + row * 2 * half_n;
-  out[i] = swiglu_value(p[col], p[half_n + col]);
+  out[i] = swiglu_act(p[col], p[half_n + col]);
 }
 
 // src/shaders/rms_norm.wgsl:1-57: one workgroup of 256 per row, strided sum of
