@@ -74,19 +74,27 @@ HEADLINE = "c5_q4_m1_4096x14336"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
 # same counters read for a 256 MiB device copy (one summary per workload under profiles/).
 MEASURED_TRAFFIC_BYTES = {
-    "c5_q4_m1_4096x14336": 37.01e6,
-    "c5_q8_m1_4096x14336": 63.59e6,
-    "c5_q4_m4_14336x4096": 39.6e6,
-    "c5_q4_m16_4096x14336": 47.4e6,
-    "c4_q4_prefill_up_512x1024x3072": 19.1e6,
+    "c5_q4_m1_4096x14336": 37.02e6,
+    "c5_q4_m1_14336x4096": 37.42e6,
+    "c5_q8_m1_4096x14336": 63.63e6,
+    "c5_q8_m1_14336x4096": 64.02e6,
+    "c5_q4_m4_4096x14336": 37.79e6,
+    "c5_q4_m4_14336x4096": 39.59e6,
+    "c5_q8_m4_4096x14336": 64.57e6,
+    "c5_q8_m4_14336x4096": 66.34e6,
+    "c5_q4_m16_4096x14336": 49.53e6,
+    "c5_q4_m16_14336x4096": 54.93e6,
+    "c5_q8_m16_4096x14336": 75.16e6,
+    "c5_q8_m16_14336x4096": 80.86e6,
     "c3_q4_lm_head_576x49152": 18.03e6,
-    "c1_q8_up_576x1536": 1.17e6,
-    "c2_q4_gate_up_576x3072": 1.32e6,
-    "c2_q4_down_1536x576_add": 0.72e6,
-    "c4_q4_prefill_down_512x3072x1024": 31.7e6,
-    "c5_q4_m1_14336x4096": 37.4e6,
-    "c5_q4_m4_4096x14336": 37.8e6,
-    "c5_q8_m16_4096x14336": 73.1e6,
+    "c1_q8_up_576x1536": 1.18e6,
+    "c2_q4_gate_up_576x3072": 1.34e6,
+    "c2_q4_down_1536x576_add": 0.73e6,
+    "c2_q4_q_576x576": 0.40e6,
+    "c4_q4_prefill_up_512x1024x3072": 19.08e6,
+    "c4_q4_prefill_down_512x3072x1024": 33.35e6,
+    "c4_f32a_q4_prefill_up_512x1024x3072": 27.31e6,
+    "c4_f32a_q4_prefill_down_512x3072x1024": 37.50e6,
 }
 
 
@@ -510,6 +518,9 @@ def main():
     ap.add_argument("--profile", action="store_true",
                     help="for rocprofv3 runs: only the timed cache-cold workload plus one 256 MiB device copy "
                          "(a known size to calibrate FETCH_SIZE / WRITE_SIZE against); no CPU leg, no warm leg")
+    ap.add_argument("--profile-chains", action="store_true",
+                    help="for rocprofv3 runs: only the decode layer through the Session (8 layers a step, as one chain "
+                         "launch a layer and as separate launches) and the FFN pair, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (column-parallel "
@@ -520,6 +531,13 @@ def main():
 
     from meganeura_amd import capi
     import oracle
+
+    if args.profile_chains:
+        ctx = capi.Context(0)
+        out = {"c5_q4_ffn_m1": ffn_chain_times(ctx), "c2_q4_decode_layer_session": decode_layer_times(200, 20)}
+        ctx.close()
+        print(json.dumps(out))
+        return
 
     ctx = capi.Context(0)
     sets = WeightSets(ctx)
