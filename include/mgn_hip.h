@@ -63,8 +63,9 @@ typedef enum mgn_route {
   MGN_ROUTE_GEMM_MFMA = 4, /* tiled dequant-GEMM on MFMA (32x32x16 tiles), larger M: the fast form, for weights whose
                               block minima stay below 2047 (Q8: scales below 15.99) and f32 activations below 65504 */
   MGN_ROUTE_TILE_MFMA = 5  /* tiled dequant-GEMM on MFMA (16x16x32 tiles, activations rescaled per row and 256-element
-                              K slice): any finite weight and activation magnitude, larger M; the automatic choice
-                              for weights outside the range of the form above */
+                              K slice): any finite weight, activations below 2^100 in magnitude (a slice that holds a
+                              larger one gives its row non-finite results), larger M; the automatic choice for weights
+                              outside the range of the form above */
 } mgn_route;
 
 typedef struct mgn_ctx mgn_ctx;
@@ -83,9 +84,12 @@ const char* mgn_last_error(const mgn_ctx* ctx);
 mgn_status mgn_sync(mgn_ctx* ctx);
 /* What the context may assume about f32 activations of matmuls with M >= 5.
  *   MGN_ACT_ANY (default): nothing.  Those matmuls run on the kernels that rescale every
- *     256-element slice of a row by a power of two before splitting it into fp16 pairs: every
- *     finite f32 is exact input whatever its magnitude, inf and NaN stay in their rows -- what the
- *     reference's f32 arithmetic on the scalar ALUs gives (src/shaders/matmul.wgsl:43-90).
+ *     256-element slice of a row by a power of two before splitting it into fp16 pairs (hi + lo:
+ *     22 significant bits relative to the slice's largest magnitude, products with the quants
+ *     exact on those): f32 of any magnitude below 2^100 is served with the same relative accuracy,
+ *     inf and NaN stay in their rows, and a slice holding a magnitude of 2^100 or more makes its
+ *     row's results non-finite (never a finite wrong number) -- in effect what the reference's f32
+ *     arithmetic on the scalar ALUs gives (src/shaders/matmul.wgsl:43-90) up to that magnitude.
  *   MGN_ACT_FP16_RANGE: the caller promises |x| < 65504 and accepts that values below 2^-4 are
  *     carried with an absolute step of 2^-25 instead of a relative one.  The matmuls may then run
  *     on the 32x32 tiled kernel, which splits without rescaling and is faster on some shapes

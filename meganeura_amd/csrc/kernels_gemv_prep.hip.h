@@ -82,12 +82,14 @@ __device__ __forceinline__ void make_digits(const float (&x)[8], const int (&ord
 }
 
 // Power of two that brings a block's largest magnitude below 2^12 (1 if the block
-// is all zero, tiny or not finite).  *inv gets the reciprocal.
+// is all zero, tiny or not finite).  *inv gets the reciprocal.  A finite magnitude of 2^100 or
+// more is not rescaled either, and the truncating fp16 conversion would clamp it to 65504: its
+// *inv is a NaN, so that the block's sums come out non-finite instead of finite and wrong.
 __device__ __forceinline__ float block_scale(float amax, float* inv) {
   const uint32_t amax_bits = __builtin_bit_cast(uint32_t, amax);
   const int e = (int)(amax_bits >> 23) - 127;  // floor(log2(amax)) for normal values
   if (amax_bits == 0 || e >= 100 || e <= -100) {
-    *inv = 1.0f;
+    *inv = (e >= 100 && e < 128) ? __builtin_nanf("") : 1.0f;
     return 1.0f;
   }
   const int sh = 11 - e;  // amax * 2^sh in [2^11, 2^12)

@@ -16,9 +16,11 @@
 //     8g..8g+7 as (q + 128) * 2^-24 in bits 0-7).
 //   A operand: the activations, converted into an "image" in the instruction's own lane order.
 //     f32 activations are scaled per (row, 256-element K slice) by a power of two and split
-//     hi + lo into two fp16 operands that are multiplied into the same accumulator, so products
-//     are exact, any finite magnitude is representable and only f32 accumulation rounds; fp16
-//     activations are used as they are.
+//     hi + lo into two fp16 operands that are multiplied into the same accumulator: 22
+//     significant bits relative to the slice's largest magnitude (each half is cut, not rounded,
+//     to 11), products with the quants exact on those, f32 accumulation rounds; any magnitude
+//     below 2^100 is representable (beyond, the slice's inverse scale is a NaN and the row comes
+//     out non-finite).  fp16 activations are used as they are.
 //   Per block: D = sum n x on the matrix cores, then P += d * D on the vector ALU (4 FMAs per
 //     lane).  The format's additive part (m * sum(x) for Q4, -128 * scale * sum(x) for Q8's byte
 //     bias) is one more MFMA per slice of 8 blocks: its A operand holds the blocks' mean

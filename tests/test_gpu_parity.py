@@ -914,6 +914,26 @@ def test_a_slice_beyond_2_to_the_100_gives_a_non_finite_row(ctx, orc, fmt, m):
     wt.free()
 
 
+@pytest.mark.parametrize("fmt", [Q4, Q8])
+@pytest.mark.parametrize("m", [1, 2, 4])
+def test_a_block_beyond_2_to_the_100_gives_a_non_finite_row_on_the_gemv(ctx, orc, fmt, m):
+    """The same on the GEMV kernels, which rescale per 32-element block: a block that holds a finite
+    magnitude of 2^100 or more makes its row non-finite on the fp16 forms (M = 2..4, Q8) as on the
+    one-row Q4 kernel's integer digits; the other rows stay within the bar."""
+    k, n = 1024, 96
+    w = synth.normal(1411, k * n, 0.02).reshape(k, n)
+    x = synth.normal(1412 + m, m * k, 1.0).reshape(m, k)
+    x[m - 1, 77] = np.float32(-2e33)
+    wt = ctx.weight(fmt, w)
+    want = orc.matmul_f64(x, orc.dequantize(fmt, orc.quantize(fmt, w), k, n))
+    for route in ("gemv_mfma", "auto"):
+        got = run_matmul(ctx, fmt, x, wt, ROUTES[route])
+        assert not np.isfinite(got[m - 1]).any(), route
+        if m > 1:
+            assert_close_rowwise(got[:m - 1], want[:m - 1], x[:m - 1])
+    wt.free()
+
+
 @pytest.mark.parametrize("fmt,m,k,n", [(Q4, 16, 4096, 2048), (Q8, 9, 4096, 1024), (Q4, 4, 14336, 518), (Q8, 3, 12288, 64)])
 def test_a_reader_that_gives_up_is_reported_and_the_context_recovers(ctx, orc, fmt, m, k, n):
     """K cut into parts for different workgroups: the part that adds the others up polls the
