@@ -192,16 +192,19 @@ mgn_status mgn_matmul_q_f16a(mgn_ctx* ctx, const mgn_buf* a_f16, const mgn_weigh
 
 /* mgn_matmul_q for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
- * Shapes whose K is cut into parts for different workgroups keep their partial sums and arrival
- * counters in a workspace; mgn_matmul_q uses one the context allocated, this entry uses an
+ * Shapes whose K is cut into parts for different workgroups keep their partial sums in a
+ * workspace (with arrival counters, or as hand-over words that read "empty" until a part has
+ * stored its sum); mgn_matmul_q uses workspaces the context allocated, this entry uses an
  * array inside the library's own device image (MGN_STATIC_WORKSPACE_BYTES = 4 MiB of partial
- * sums plus 4096 counters, held on every device the library runs on until the process ends)
- * and calls no hipMalloc / hipFree or any other allocating routine.  Same plan, same kernels
- * and bit-identical results as mgn_matmul_q; MGN_EUNSUPPORTED, with the byte counts in
- * mgn_last_error, when the shape's partial sums do not fit the static array.  All contexts
- * of a device share the array: calls that overlap on one device (two contexts, two threads)
- * race; calls on one context are ordered by its stream.  The arrival counters are cleared by a
- * small fill kernel in front of every launch that uses them. */
+ * sums, plus 4096 counters, plus as many bytes of hand-over words again, held on every device the
+ * library runs on until the process ends) and calls no hipMalloc / hipFree or any other
+ * allocating routine.  Same plan, same kernels and bit-identical results as mgn_matmul_q;
+ * MGN_EUNSUPPORTED, with the byte counts in mgn_last_error, when the shape's partial sums or
+ * hand-over words do not fit the static array.  All contexts of a device share the array: calls
+ * that overlap on one device (two contexts, two threads) race; calls on one context are ordered by
+ * its stream.  The array keeps the last call's contents: the counters are cleared and the
+ * hand-over words a launch will use are set to the empty pattern by a small fill kernel in front
+ * of every launch that uses them. */
 #define MGN_STATIC_WORKSPACE_BYTES ((size_t)4 << 20)
 mgn_status mgn_matmul_q_static(mgn_ctx* ctx, const mgn_buf* a, const mgn_weight* w, const mgn_buf* d,
                                mgn_buf* c, uint32_t m);
