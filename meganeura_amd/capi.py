@@ -91,7 +91,7 @@ def load():
         "mgn_sync": (C.c_int, [vp]),
         "mgn_ctx_set_route": (C.c_int, [vp, C.c_int]),
         "mgn_ctx_set_spin_limit": (C.c_int, [vp, C.c_uint32]),
-        "mgn_engine_clock_mhz": (C.c_int, [vp, C.POINTER(C.c_float)]),
+        "mgn_engine_clock_mhz": (C.c_int, [vp, C.c_int, C.POINTER(C.c_float)]),
         "mgn_ctx_set_activation_range": (C.c_int, [vp, C.c_int]),
         "mgn_buf_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
         "mgn_buf_free": (None, [vp, vp]),
@@ -283,9 +283,9 @@ class Context:
         """Polls a wave makes for another workgroup's partial sums before it gives up (tests only)."""
         self.check(self.lib.mgn_ctx_set_spin_limit(self.h, polls))
 
-    def engine_clock_mhz(self):
+    def engine_clock_mhz(self, loaded=False):
         mhz = C.c_float()
-        self.check(self.lib.mgn_engine_clock_mhz(self.h, C.byref(mhz)))
+        self.check(self.lib.mgn_engine_clock_mhz(self.h, 1 if loaded else 0, C.byref(mhz)))
         return float(mhz.value)
 
     def sync(self):

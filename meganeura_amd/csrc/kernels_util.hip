@@ -539,8 +539,37 @@ __global__ void clock_probe_kernel(uint64_t* __restrict__ out) {
   const uint64_t t1 = __builtin_amdgcn_s_memtime();
   if (threadIdx.x == 0) out[0] = t1 - t0, out[1] = r1 - r0;
 }
-int launch_clock_probe(ihipStream_t* s, uint64_t* out2_dev) {
-  hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, s, out2_dev);
+// The same under load: every CU runs 16 waves of fp16 matrix instructions fed from LDS (the mix
+// of the several-row GEMV kernels) for about 20 us; one wave reads the counters.  A box that
+// lowers its clock under such a load shows it here and not in the idle probe.
+__global__ __launch_bounds__(1024) void clock_probe_loaded_kernel(uint64_t* __restrict__ out, float* __restrict__ sink) {
+  typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+  typedef float floatx4 __attribute__((ext_vector_type(4)));
+  __shared__ uint4 lds[1024];
+  lds[threadIdx.x] = make_uint4(threadIdx.x, 0x3C003C00u, 0x38003800u, threadIdx.x * 7u);
+  __syncthreads();
+  const uint64_t t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+  uint64_t r1 = r0;
+  floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (uint32_t i = 0; i < (1u << 16) && r1 - r0 < 2000; i++) {  // (bounded: ends whatever the counters do)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const uint4 v = lds[(threadIdx.x + 64 * j + i) & 1023];
+      const uint2 a = make_uint2(v.x & 0x03FF03FFu, v.y), b = make_uint2(v.z, v.w & 0x03FF03FFu);
+      acc = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4, a), __builtin_bit_cast(half4, b), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4, b), __builtin_bit_cast(half4, a), acc, 0, 0, 0);
+    }
+    r1 = __builtin_amdgcn_s_memrealtime();
+  }
+  const uint64_t t1 = __builtin_amdgcn_s_memtime();
+  if (acc[0] == 123.456f) sink[threadIdx.x] = acc[1] + acc[2] + acc[3];  // (keeps the arithmetic)
+  if (blockIdx.x == 0 && threadIdx.x == 0) out[0] = t1 - t0, out[1] = r1 - r0;
+}
+int launch_clock_probe(ihipStream_t* s, uint64_t* out2_dev, int num_cus_loaded) {
+  if (num_cus_loaded > 0)
+    hipLaunchKernelGGL(clock_probe_loaded_kernel, dim3((unsigned)num_cus_loaded), dim3(1024), 0, s, out2_dev, (float*)(out2_dev + 8));
+  else
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, s, out2_dev);
   MGN_HIP_LAUNCH_CHECK();
   return 0;
 }

@@ -105,7 +105,9 @@ int launch_quantize_nk(ihipStream_t* s, int fmt, const float* w_nk_dev, uint32_t
 int launch_transpose(ihipStream_t* s, const float* in, float* out, uint32_t rows, uint32_t cols);
 // measurement aid: one pass of plain reads over the weight's quants and scales
 // two words: shader-clock ticks and 100 MHz ticks over the same ~20 us
-int launch_clock_probe(ihipStream_t* s, uint64_t* out2_dev);
+// (num_cus_loaded > 0: that many workgroups of matrix-instruction work run meanwhile; out2_dev then
+// needs 64 + 4096 bytes)
+int launch_clock_probe(ihipStream_t* s, uint64_t* out2_dev, int num_cus_loaded);
 // pattern 0: contiguous shares per workgroup; 1: the decode kernel's lane -> address map
 int launch_read_probe(ihipStream_t* s, const WeightView& w, int num_cus, uint32_t* sink, int pattern);
 int launch_matmul_generic(ihipStream_t* s, const LaunchArgs& a);
