@@ -284,9 +284,15 @@ def config_table(ctx, sets, steps=200, repeats=5, preheat_ms=100.0):
         roof = wl.roofline(r["median"])
         table[name] = {"us": r["median"] * 1e3, "us_min": r["min"] * 1e3, "us_max": r["max"] * 1e3,
                        # read right behind the timed regions: one idle wave, and under a matrix-instruction load
-                       "engine_mhz": round(ctx.engine_clock_mhz()), "engine_mhz_loaded": round(ctx.engine_clock_mhz(True)),
+                       "engine_mhz": round(ctx.engine_clock_mhz()), **dict(zip(("engine_mhz_loaded", "load_cycles_per_round"), map(round, ctx.engine_probe()))),
                        "bound": roof["bound"], "achieved": roof["achieved"], "unit": roof["unit"], "frac": roof["frac"],
                        "algorithmic_bytes": wl.bytes}
+        if m == 1 and wl.bytes >= (8 << 20):
+            # a bandwidth-bound one-row call beside its own floor on this box: the faster of the two
+            # read-only passes over the same rotating copies, pre-heated and timed the same way
+            fl = wl.read_floor(steps, 20, repeats, preheat_ms)
+            table[name]["read_floor_us"] = fl["median"] * 1e3
+            table[name]["frac_of_read_floor"] = fl["median"] / r["median"]
         if m > 4 and not f16:
             # f32 activations at M >= 5: the figure above is the context's default (activations of any
             # magnitude, the rescaling kernels); beside it, the same call on a context that was promised
@@ -544,7 +550,8 @@ def main():
     sets = WeightSets(ctx)
     wl = Workload(ctx, args.workload, 512 << 20, sets)
     timing = wl.measure(args.steps, args.warmup, repeats, preheat_ms=20.0 if args.profile else 100.0)
-    engine_mhz, engine_mhz_loaded = round(ctx.engine_clock_mhz()), round(ctx.engine_clock_mhz(True))
+    engine_mhz = round(ctx.engine_clock_mhz())
+    engine_mhz_loaded, load_cycles_per_round = map(round, ctx.engine_probe())
     ms = timing["median"]
     want = wl.check()  # the timed kernel's result against the oracle, before anything is reported
 
@@ -589,6 +596,7 @@ def main():
         "us_per_call_max": timing["max"] * 1e3,
         "engine_mhz": engine_mhz,
         "engine_mhz_loaded": engine_mhz_loaded,
+        "load_cycles_per_round": load_cycles_per_round,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -30,8 +30,10 @@ mgn_status mgn_ctx_set_spin_limit(mgn_ctx* ctx, uint32_t polls);
  * against the constant 100 MHz counter over about 20 us); synchronises.  loaded = 0: one wave on an
  * otherwise idle device; loaded = 1: while every CU runs 16 waves of fp16 matrix instructions fed
  * from LDS, the mix of the several-row kernels.  Timings of instruction-bound kernels move with it
- * from box to box, bandwidth-bound ones do not. */
-mgn_status mgn_engine_clock_mhz(mgn_ctx* ctx, int loaded, float* mhz);
+ * from box to box, bandwidth-bound ones do not.  cycles_per_round (may be null; 0 when not loaded):
+ * shader cycles one wave of the load took per round of eight 4x4x4 fp16 matrix instructions and
+ * four 16-byte LDS reads, with four such waves on its SIMD. */
+mgn_status mgn_engine_clock_mhz(mgn_ctx* ctx, int loaded, float* mhz, float* cycles_per_round);
 
 /* `steps` matmuls (mgn_matmul_q, or mgn_matmul_q_f16a when a_is_f16 != 0) enqueued back to back,
  * call i on weights[i % count]: the step loop of a compiled host

@@ -91,7 +91,7 @@ def load():
         "mgn_sync": (C.c_int, [vp]),
         "mgn_ctx_set_route": (C.c_int, [vp, C.c_int]),
         "mgn_ctx_set_spin_limit": (C.c_int, [vp, C.c_uint32]),
-        "mgn_engine_clock_mhz": (C.c_int, [vp, C.c_int, C.POINTER(C.c_float)]),
+        "mgn_engine_clock_mhz": (C.c_int, [vp, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
         "mgn_ctx_set_activation_range": (C.c_int, [vp, C.c_int]),
         "mgn_buf_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
         "mgn_buf_free": (None, [vp, vp]),
@@ -285,8 +285,14 @@ class Context:
 
     def engine_clock_mhz(self, loaded=False):
         mhz = C.c_float()
-        self.check(self.lib.mgn_engine_clock_mhz(self.h, 1 if loaded else 0, C.byref(mhz)))
+        self.check(self.lib.mgn_engine_clock_mhz(self.h, 1 if loaded else 0, C.byref(mhz), None))
         return float(mhz.value)
+
+    def engine_probe(self):
+        """(MHz under the matrix-instruction load, shader cycles per round of that load)."""
+        mhz, cyc = C.c_float(), C.c_float()
+        self.check(self.lib.mgn_engine_clock_mhz(self.h, 1, C.byref(mhz), C.byref(cyc)))
+        return float(mhz.value), float(cyc.value)
 
     def sync(self):
         self.check(self.lib.mgn_sync(self.h))

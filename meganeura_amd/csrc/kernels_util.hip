@@ -551,7 +551,8 @@ __global__ __launch_bounds__(1024) void clock_probe_loaded_kernel(uint64_t* __re
   const uint64_t t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
   uint64_t r1 = r0;
   floatx4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (uint32_t i = 0; i < (1u << 16) && r1 - r0 < 2000; i++) {  // (bounded: ends whatever the counters do)
+  uint32_t i = 0;
+  for (; i < (1u << 16) && r1 - r0 < 2000; i++) {  // (bounded: ends whatever the counters do)
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const uint4 v = lds[(threadIdx.x + 64 * j + i) & 1023];
@@ -563,7 +564,7 @@ __global__ __launch_bounds__(1024) void clock_probe_loaded_kernel(uint64_t* __re
   }
   const uint64_t t1 = __builtin_amdgcn_s_memtime();
   if (acc[0] == 123.456f) sink[threadIdx.x] = acc[1] + acc[2] + acc[3];  // (keeps the arithmetic)
-  if (blockIdx.x == 0 && threadIdx.x == 0) out[0] = t1 - t0, out[1] = r1 - r0;
+  if (blockIdx.x == 0 && threadIdx.x == 0) out[0] = t1 - t0, out[1] = r1 - r0, out[2] = i;
 }
 int launch_clock_probe(ihipStream_t* s, uint64_t* out2_dev, int num_cus_loaded) {
   if (num_cus_loaded > 0)

@@ -923,15 +923,16 @@ mgn_status mgn_weight_read_loop(mgn_ctx* ctx, const mgn_weight* const* weights, 
   return MGN_OK;
 }
 
-mgn_status mgn_engine_clock_mhz(mgn_ctx* ctx, int loaded, float* mhz) {
+mgn_status mgn_engine_clock_mhz(mgn_ctx* ctx, int loaded, float* mhz, float* cycles_per_round) {
   if (!ctx || !mhz) return fail(ctx, MGN_EINVAL, "null argument");
   // (the first bytes of the split-K workspace hold nothing between launches)
   const int rc = mgn::launch_clock_probe(ctx->stream, (uint64_t*)ctx->scratch, loaded ? ctx->num_cus : 0);
   if (rc != 0) return hip_fail(ctx, "clock probe launch", (hipError_t)rc);
-  uint64_t host[2] = {0, 0};
+  uint64_t host[3] = {0, 0, 0};
   MGN_HIP(ctx, hipMemcpyAsync(host, ctx->scratch, sizeof(host), hipMemcpyDeviceToHost, ctx->stream));
   MGN_HIP(ctx, hipStreamSynchronize(ctx->stream));
   *mhz = host[1] ? 100.0f * (float)host[0] / (float)host[1] : 0.0f;
+  if (cycles_per_round) *cycles_per_round = loaded && host[2] ? (float)host[0] / (float)host[2] : 0.0f;
   return MGN_OK;
 }
 

@@ -171,7 +171,7 @@ pub mod bench {
     extern "C" {
         pub fn mgn_ctx_set_route(ctx: *mut mgn_ctx, route: mgn_route) -> mgn_status;
         pub fn mgn_ctx_set_spin_limit(ctx: *mut mgn_ctx, polls: u32) -> mgn_status;
-        pub fn mgn_engine_clock_mhz(ctx: *mut mgn_ctx, loaded: c_int, mhz: *mut f32) -> mgn_status;
+        pub fn mgn_engine_clock_mhz(ctx: *mut mgn_ctx, loaded: c_int, mhz: *mut f32, cycles_per_round: *mut f32) -> mgn_status;
         pub fn mgn_matmul_q_loop(ctx: *mut mgn_ctx, a: *const mgn_buf, a_is_f16: c_int, weights: *const *const mgn_weight, count: usize, d: *const mgn_buf, c: *mut mgn_buf, m: u32, steps: u32) -> mgn_status;
         pub fn mgn_weight_read_loop(ctx: *mut mgn_ctx, weights: *const *const mgn_weight, count: usize, steps: u32, pattern: c_int) -> mgn_status;
     }
