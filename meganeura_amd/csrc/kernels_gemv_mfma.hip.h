@@ -672,24 +672,24 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     // no K split (always the case with QPW > 1): lanes 0..3 hold the four finished columns of a quad
 #pragma unroll
     for (int q = 0; q < QPW; q++) {
-#pragma unroll
-      for (int r = 0; r < MROWS; r++) {
-        const float tot = sum_over_blocks(acc[q][r]);
-        const uint32_t n = (quad + q) * 4 + lane;
-        if (lane < 4 && wave_live && (uint32_t)r < m && n < w.n) {
-          const size_t o = (size_t)r * w.n + n;
-          const float* const dres = pick3(widx, bt.d[0], bt.d[1], bt.d[2]);
-          float* const c = pick3(widx, bt.c[0], bt.c[1], bt.c[2]);
-          c[o] = apply_epilogue(dres ? tot + dres[o] : tot, sp.epilogue);
-        }
+      uint32_t r;
+      bool writer;
+      const float tot = sum_rows_over_blocks<MROWS>(acc[q], lane, &r, &writer);
+      const uint32_t n = (quad + q) * 4 + (lane & 3u);
+      if (writer && wave_live && r < m && n < w.n) {
+        const size_t o = (size_t)r * w.n + n;
+        const float* const dres = pick3(widx, bt.d[0], bt.d[1], bt.d[2]);
+        float* const c = pick3(widx, bt.c[0], bt.c[1], bt.c[2]);
+        c[o] = apply_epilogue(dres ? tot + dres[o] : tot, sp.epilogue);
       }
     }
     return;
   }
-#pragma unroll
-  for (int r = 0; r < MROWS; r++) {
-    const float tot = sum_over_blocks(acc[0][r]);
-    if (lane < 4 && wave_live) red[((wn * ksc + ks) * MROWS + r) * 4 + lane] = tot;
+  {
+    uint32_t r;
+    bool writer;
+    const float tot = sum_rows_over_blocks<MROWS>(acc[0], lane, &r, &writer);
+    if (writer && wave_live && r < (uint32_t)MROWS) red[((wn * ksc + ks) * MROWS + r) * 4 + (lane & 3u)] = tot;
   }
   lds_barrier();
   // ---- combine the K splits, then the K parts, add the residual, store ----

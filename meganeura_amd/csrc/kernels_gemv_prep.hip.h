@@ -44,6 +44,56 @@ __device__ __forceinline__ float sum_over_blocks(float v) {
   return v;
 }
 
+// The same for MROWS accumulators at once, without a trip through LDS: the halves and rows of the
+// wave are folded with the row-swap instructions while the activation rows are handed out to them
+// (3 swaps and 3 adds for four rows, where four separate sums take 8 cross-row exchanges), then
+// two rotations inside a row.  Every lane ends with the total of column lane % 4 for ONE
+// activation row, *row: lanes 16 j .. 16 j + 15 hold row {0, 2, 1, 3}[j] of four (rows past MROWS
+// are zero sums), row j / 2 of two, row 0 of one.  *writer: one lane per (row, column).
+template <int MROWS>
+__device__ __forceinline__ float sum_rows_over_blocks(const float (&acc)[MROWS], uint32_t lane, uint32_t* row, bool* writer) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  // (the instructions swap two registers in place: one value given twice needs a register of its own)
+  auto twin = [](float a) {
+    float b = a;
+    asm volatile("" : "+v"(b));
+    return b;
+  };
+  auto fold32 = [](float a, float b) {  // lanes 0..31: a(lane) + a(lane + 32); lanes 32..63: b(lane - 32) + b(lane)
+    const u32x2 s = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), false, false);
+    uint32_t x = s.x, y = s.y;
+    asm volatile("" : "+v"(x), "+v"(y));  // (without it the sum came out as x + x)
+    return __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
+  };
+  auto fold16 = [](float a, float b) {  // even rows of 16: a(row) + a(row + 1); odd rows: b(row - 1) + b(row)
+    const u32x2 s = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b), false, false);
+    uint32_t x = s.x, y = s.y;
+    asm volatile("" : "+v"(x), "+v"(y));
+    return __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
+  };
+  const uint32_t j = lane >> 4;
+  float v;
+  if constexpr (MROWS >= 3) {
+    const float t01 = fold32(acc[0], acc[1]), t23 = fold32(acc[2], MROWS > 3 ? acc[MROWS > 3 ? 3 : 0] : 0.0f);
+    v = fold16(t01, t23);
+    *row = ((j & 1u) << 1) | (j >> 1);
+    *writer = (lane & 15u) < 4u;
+  } else if constexpr (MROWS == 2) {
+    const float t = fold32(acc[0], acc[1]);  // lanes 0..31: row 0, lanes 32..63: row 1
+    v = fold16(t, twin(t));
+    *row = j >> 1;
+    *writer = (lane & 31u) < 4u;
+  } else {
+    const float t = fold32(acc[0], twin(acc[0]));
+    v = fold16(t, twin(t));
+    *row = 0;
+    *writer = lane < 4u;
+  }
+  v += dpp_move<kRowRor4>(v);
+  v += dpp_move<kRowRor8>(v);
+  return v;
+}
+
 // ---- one activation row: integer digits on the int8 matrix instruction ----
 // With a single activation row the four A rows of v_mfma_i32_4x4x4_16B_i8 hold the base-128
 // digits of the activations instead of fp16 halves: x, scaled per 32-element block by a power of
