@@ -268,8 +268,11 @@ __global__ __launch_bounds__(1024) void chain_kernel_q4(const ChainStageDev* __r
             acc = __fmaf_rn(v, ci0.y, acc);
             cs++;
             if (cs == my_steps) {  // the quad is done: its 16 lanes per column meet, lanes 0..3 hold the four columns
-              const float sum = sum_over_blocks(acc);
-              if (lane < 4) red[((slot + cq * nslots) * ksc + ks) * 4 + lane] = sum;
+              const float one[1] = {acc};
+              uint32_t row;
+              bool writer;
+              const float sum = sum_rows_over_blocks<1>(one, lane, &row, &writer);
+              if (writer) red[((slot + cq * nslots) * ksc + ks) * 4 + lane] = sum;
               acc = 0.0f, cs = 0, cq++;
             }
           }

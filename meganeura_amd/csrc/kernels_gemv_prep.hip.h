@@ -35,16 +35,8 @@ __device__ __forceinline__ float half_hi(uint32_t p) { return (float)__builtin_b
 
 constexpr int kRowRor4 = 0x124, kRowRor8 = 0x128;  // rotate right within a row of 16 lanes
 
-// sum over the 16 lanes sharing lane%4 (every such lane ends with the total)
-__device__ __forceinline__ float sum_over_blocks(float v) {
-  v += dpp_move<kRowRor4>(v);
-  v += dpp_move<kRowRor8>(v);
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  return v;
-}
-
-// The same for MROWS accumulators at once, without a trip through LDS: the halves and rows of the
+// Sums over the 16 lanes of a wave that share lane % 4 (the 16 K blocks of a step, per column), for
+// MROWS accumulators at once, without a trip through LDS: the halves and rows of the
 // wave are folded with the row-swap instructions while the activation rows are handed out to them
 // (3 swaps and 3 adds for four rows, where four separate sums take 8 cross-row exchanges), then
 // two rotations inside a row.  Every lane ends with the total of column lane % 4 for ONE
