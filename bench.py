@@ -76,20 +76,20 @@ HEADLINE = "c5_q4_m1_4096x14336"
 MEASURED_TRAFFIC_BYTES = {
     "c5_q4_m1_4096x14336": 37.02e6,
     "c5_q4_m1_14336x4096": 37.42e6,
-    "c5_q8_m1_4096x14336": 63.63e6,
+    "c5_q8_m1_4096x14336": 63.60e6,
     "c5_q8_m1_14336x4096": 64.02e6,
-    "c5_q4_m4_4096x14336": 37.79e6,
-    "c5_q4_m4_14336x4096": 39.59e6,
-    "c5_q8_m4_4096x14336": 64.57e6,
-    "c5_q8_m4_14336x4096": 66.34e6,
+    "c5_q4_m4_4096x14336": 37.74e6,
+    "c5_q4_m4_14336x4096": 39.60e6,
+    "c5_q8_m4_4096x14336": 64.58e6,
+    "c5_q8_m4_14336x4096": 66.33e6,
     "c5_q4_m16_4096x14336": 49.53e6,
     "c5_q4_m16_14336x4096": 54.93e6,
     "c5_q8_m16_4096x14336": 75.16e6,
     "c5_q8_m16_14336x4096": 80.86e6,
     "c3_q4_lm_head_576x49152": 18.03e6,
-    "c1_q8_up_576x1536": 1.18e6,
-    "c2_q4_gate_up_576x3072": 1.34e6,
-    "c2_q4_down_1536x576_add": 0.73e6,
+    "c1_q8_up_576x1536": 1.17e6,
+    "c2_q4_gate_up_576x3072": 1.33e6,
+    "c2_q4_down_1536x576_add": 0.74e6,
     "c2_q4_q_576x576": 0.40e6,
     "c4_q4_prefill_up_512x1024x3072": 19.08e6,
     "c4_q4_prefill_down_512x3072x1024": 33.35e6,
