@@ -367,11 +367,13 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
         }
   }
   if constexpr (PRO == kProRmsNorm) {
-    // row sums of squares: per thread, per wave (DPP), then across the waves through LDS
-    float ss[MROWS];
+    // x * rstd * g is staged as x * g: the row's rstd is one factor for all of K, so it is applied
+    // to the finished sums instead (rms_rstd below) and nothing waits for the row's sum of squares
+    // before the staging.  The sums of squares go to LDS per wave; the barrier behind the staging
+    // publishes them.
 #pragma unroll
     for (int r = 0; r < MROWS; r++) {
-      ss[r] = 0.0f;
+      float ss = 0.0f;
 #pragma unroll
       for (int tt = 0; tt < TASKS; tt++) {
         const uint32_t kb = (tid + tt * nthreads) >> 2;
@@ -379,32 +381,29 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
 #pragma unroll
           for (int h = 0; h < 2; h++) {
             const float4 v = xraw[tt][r][h];
-            ss[r] = __fmaf_rn(v.x, v.x, ss[r]);
-            ss[r] = __fmaf_rn(v.y, v.y, ss[r]);
-            ss[r] = __fmaf_rn(v.z, v.z, ss[r]);
-            ss[r] = __fmaf_rn(v.w, v.w, ss[r]);
+            ss = __fmaf_rn(v.x, v.x, ss);
+            ss = __fmaf_rn(v.y, v.y, ss);
+            ss = __fmaf_rn(v.z, v.z, ss);
+            ss = __fmaf_rn(v.w, v.w, ss);
           }
         }
       }
-      ss[r] = group_sum<64>(ss[r]);
-      if (lane == 0) nrm[wave * MROWS + r] = ss[r];
-    }
-    lds_barrier();
-    const uint32_t nwv = nwaves;
-#pragma unroll
-    for (int r = 0; r < MROWS; r++) {
-      // (one LDS read and a reduction over 16 lanes, not a read per wave one after the other)
-      const float tot = group_sum<16>((lane & 15u) < nwv ? nrm[(lane & 15u) * MROWS + r] : 0.0f);
-      const float rstd = 1.0f / sqrtf(tot / (float)w.k + pro.eps);
+      ss = group_sum<64>(ss);
+      if (lane == 0) nrm[wave * MROWS + r] = ss;
 #pragma unroll
       for (int tt = 0; tt < TASKS; tt++)
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           const float4 v = xraw[tt][r][h], g4 = gw[tt][h];
-          xraw[tt][r][h] = make_float4(v.x * rstd * g4.x, v.y * rstd * g4.y, v.z * rstd * g4.z, v.w * rstd * g4.w);
+          xraw[tt][r][h] = make_float4(v.x * g4.x, v.y * g4.y, v.z * g4.z, v.w * g4.w);
         }
     }
   }
+  // kProRmsNorm: 1 / sqrt(mean(x^2) + eps) of row r, from the waves' sums (valid behind the staging barrier)
+  auto rms_rstd = [&](uint32_t r) {
+    const float tot = group_sum<16>((lane & 15u) < nwaves ? nrm[(lane & 15u) * MROWS + r] : 0.0f);
+    return 1.0f / sqrtf(tot / (float)w.k + pro.eps);
+  };
 
   // ---- activations -> LDS (once per workgroup) ----
 #pragma unroll
@@ -676,11 +675,13 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
       bool writer;
       const float tot = sum_rows_over_blocks<MROWS>(acc[q], lane, &r, &writer);
       const uint32_t n = (quad + q) * 4 + (lane & 3u);
+      float tot_r = tot;
+      if constexpr (PRO == kProRmsNorm) tot_r *= rms_rstd(min(r, (uint32_t)MROWS - 1));
       if (writer && wave_live && r < m && n < w.n) {
         const size_t o = (size_t)r * w.n + n;
         const float* const dres = pick3(widx, bt.d[0], bt.d[1], bt.d[2]);
         float* const c = pick3(widx, bt.c[0], bt.c[1], bt.c[2]);
-        c[o] = apply_epilogue(dres ? tot + dres[o] : tot, sp.epilogue);
+        c[o] = apply_epilogue(dres ? tot_r + dres[o] : tot_r, sp.epilogue);
       }
     }
     return;
@@ -693,6 +694,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   }
   lds_barrier();
   // ---- combine the K splits, then the K parts, add the residual, store ----
+  float rstd_row[MROWS];
+#pragma unroll
+  for (int r = 0; r < MROWS; r++) rstd_row[r] = PRO == kProRmsNorm ? rms_rstd(r) : 1.0f;
   for (uint32_t t = tid; t < wnc * MROWS * 4; t += nthreads) {
     const uint32_t col = t & 3, r = (t >> 2) % MROWS, ql = t / (4 * MROWS);
     // the quads of a workgroup may belong to different weights of the batch
@@ -703,6 +707,12 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
     if (r < m && n < wn_cols) {
       float v = 0.0f;
       for (uint32_t s = 0; s < ksc; s++) v += red[((ql * ksc + s) * MROWS + r) * 4 + col];
+      if constexpr (PRO == kProRmsNorm) {
+        float f = rstd_row[0];
+#pragma unroll
+        for (int rr = 1; rr < MROWS; rr++) f = r == (uint32_t)rr ? rstd_row[rr] : f;
+        v *= f;
+      }
       if constexpr (KSPLIT) {
         float* const slot0 = sp.handover + (size_t)r * wn_cols + n;  // part p's word: slot0 + p * MROWS * wn_cols
         const size_t pstride = (size_t)MROWS * wn_cols;
