@@ -179,13 +179,11 @@ __global__ __launch_bounds__(1024) void chain_kernel_q4(const ChainStageDev* __r
       }
     }
     if (rms) {
-      // src/shaders/rms_norm.wgsl:1-57: x * rsqrt(mean(x^2) + eps) * weight
+      // src/shaders/rms_norm.wgsl:1-57: x * rsqrt(mean(x^2) + eps) * weight.  The activations are
+      // staged as x * weight; the row's one factor is applied to the finished sums below, so the
+      // staging does not wait for the sum of squares (the barrier behind the staging publishes it)
       ss = group_sum<64>(ss);
       if (lane == 0) nrm[wave] = ss;
-      lds_barrier();
-      float tot = 0.0f;
-      for (uint32_t wv = 0; wv < 16; wv++) tot += nrm[wv];
-      const float rstd = 1.0f / sqrtf(tot / (float)k + st.eps);
 #pragma unroll
       for (int tt = 0; tt < kMaxTasks; tt++) {
         const uint32_t t = tid + tt * 1024, kb = t >> 2, ch = t & 3;
@@ -194,7 +192,7 @@ __global__ __launch_bounds__(1024) void chain_kernel_q4(const ChainStageDev* __r
           const float4 g0 = gp[0], g1 = gp[1];
           const float g[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
 #pragma unroll
-          for (int e = 0; e < 8; e++) x[tt][e] = x[tt][e] * rstd * g[e];
+          for (int e = 0; e < 8; e++) x[tt][e] = x[tt][e] * g[e];
         }
       }
     }
@@ -282,11 +280,13 @@ __global__ __launch_bounds__(1024) void chain_kernel_q4(const ChainStageDev* __r
     lds_barrier();
 
     // ---- the K splits meet (fixed order), residual, unary operations, store ----
+    const float rstd = rms ? 1.0f / sqrtf(group_sum<16>(nrm[lane & 15u]) / (float)k + st.eps) : 1.0f;
     for (uint32_t t = tid; t < quads_here * 4; t += 1024) {
       const uint32_t ql = t >> 2, col = t & 3, nidx = (quad0 + ql) * 4 + col;
       if (nidx < n) {
         float v = 0.0f;
         for (uint32_t sp = 0; sp < ksc; sp++) v += red[(ql * ksc + sp) * 4 + col];
+        v *= rstd;
         if (st.d) v += st.d_poll ? load1_polled(st.d + nidx, spin_limit, &gave_up) : st.d[nidx];
         v = apply_epilogue(v, st.epilogue);
         st.c[nidx] = v;
