@@ -315,6 +315,7 @@ struct TileTail {  // arguments first needed in the epilogue
   float* handover;
   uint32_t spin_limit;
   uint32_t* fault_flag;
+  uint32_t spread;  // resident kernel: every part adds up a share of the tiles (all workgroups of the launch resident)
 };
 
 constexpr int park_stride(int fmt) { return fmt == MGN_FMT_Q4 ? 8 * 16 + 16 : 8 * 32 + 16; }  // bytes per parked column
@@ -947,6 +948,83 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
     const __amdgpu_buffer_rsrc_t partials =
         __builtin_amdgcn_make_buffer_rsrc(tail.handover, 0, (parts - 1) * part_stride, 0x00020000);
     const uint32_t my_off = ((rg * colgroups + cg) * 8u + wave) * (kSlots * 1024u) + lane * 16u;
+    if (tail.spread) {
+      // Every part adds up a share.  With many parts the one workgroup that reads all the others'
+      // tiles takes them in at the rate of a single CU (14 parts: 208 KB, 1.5 us); here every part
+      // stores ALL its tiles (its own share included), and tile T = wave * kSlots + slot of the
+      // group belongs to part T % parts, whose wave T / parts polls the `parts` copies of that one
+      // tile, adds them in part order, stores the outputs and puts the pattern back.  Every part
+      // waits for every other, so the planner asks for this only when the whole grid is resident
+      // at once (at most one workgroup per CU).  The workspace holds `parts` sets of tiles.
+      const __amdgpu_buffer_rsrc_t all_parts = __builtin_amdgcn_make_buffer_rsrc(tail.handover, 0, parts * part_stride, 0x00020000);
+#pragma unroll
+      for (int p = 0; p < Q; p++)
+#pragma unroll
+        for (int u = 0; u < kSide; u++)
+#pragma unroll
+          for (int r = 0; r < R; r++) {
+            u32x4_t v = __builtin_bit_cast(u32x4_t, res[p][u][r]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = v[i] == kHandoverEmpty ? 0x7FC00000u : v[i];
+            __builtin_amdgcn_raw_buffer_store_b128(v, all_parts, part * part_stride + my_off + ((p * kSide + u) * R + r) * 1024u, 0,
+                                                   kDeviceScope);
+          }
+      bool gave_up = false;
+      // the tiles this wave adds up: part + parts * (wave, wave + 8, ..) while the group has that many
+      for (uint32_t tile = part + wave * parts; tile < 8u * kSlots; tile += 8u * parts) {
+        const uint32_t src_wave = tile / kSlots, slot = tile - src_wave * kSlots;
+        const uint32_t t_off = ((rg * colgroups + cg) * 8u + src_wave) * (kSlots * 1024u) + slot * 1024u + lane * 16u;
+        floatx4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+        constexpr uint32_t PG = 8;
+        const u32x4_t empty4 = {kHandoverEmpty, kHandoverEmpty, kHandoverEmpty, kHandoverEmpty};
+        for (uint32_t pp0 = 0; pp0 < parts; pp0 += PG) {
+          uint32_t v[PG][4];  // (scalars: vectors assigned inside a divergent polling loop have come out wrong)
+#pragma unroll
+          for (uint32_t j = 0; j < PG; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[j][i] = kHandoverEmpty;
+          for (uint32_t polls = 0;; polls++) {
+            if (polls >= tail.spin_limit) {  // (a limit of 0 looks at nothing: the give-up path, for tests)
+              gave_up = true;
+              break;
+            }
+            bool missing = false;
+#pragma unroll
+            for (uint32_t j = 0; j < PG; j++) {
+              const u32x4_t x4 = __builtin_amdgcn_raw_buffer_load_b128(all_parts, min(pp0 + j, parts - 1) * part_stride + t_off, 0, kDeviceScope);
+              v[j][0] = x4.x, v[j][1] = x4.y, v[j][2] = x4.z, v[j][3] = x4.w;
+              missing |= x4.x == kHandoverEmpty || x4.y == kHandoverEmpty || x4.z == kHandoverEmpty || x4.w == kHandoverEmpty;
+            }
+            if (!__builtin_amdgcn_ballot_w64(missing)) break;
+            __builtin_amdgcn_s_sleep(1);
+            asm volatile("" ::: "memory");  // the loads are issued anew on every round
+          }
+#pragma unroll
+          for (uint32_t j = 0; j < PG; j++) {
+            if (pp0 + j < parts) {  // uniform
+#pragma unroll
+              for (int i = 0; i < 4; i++) sum[i] += __builtin_bit_cast(float, v[j][i]);
+              __builtin_amdgcn_raw_buffer_store_b128(empty4, all_parts, (pp0 + j) * part_stride + t_off, 0, kDeviceScope);
+            }
+          }
+        }
+        // the tile's place in the output: slot = (pair * kSide + side) * R + row tile of wave src_wave
+        const uint32_t tp = slot / (kSide * R), tu = (slot / R) % kSide, tr = slot % R;
+        const uint32_t col = (((cg * 8 + src_wave) * Q + tp) * kSide + tu) * 16 + c;
+        if (col < n) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const uint32_t row = row0 + tr * 16 + 4 * g + i;
+            if (row < m) {
+              const size_t o = (size_t)row * n + col;
+              tail.c[o] = apply_epilogue(tail.dres ? sum[i] + tail.dres[o] : sum[i], tail.epilogue);
+            }
+          }
+        }
+      }
+      if (gave_up && lane == 0 && tail.fault_flag) *tail.fault_flag = 1u;
+      return;
+    }
     if (part + 1 < parts) {
 #pragma unroll
       for (int p = 0; p < Q; p++)
@@ -1042,6 +1120,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
 struct ResidentPlan {
   uint32_t r, q, nsl, parts, colgroups, rowgroups, nslices;
   bool park;  // quants through a wave-private LDS strip (if there is room) instead of row swaps
+  bool spread;  // the K parts' tiles are added up by all parts, a share each (see the kernel)
   size_t lds, partial_bytes;
   double cost;
 };
@@ -1080,14 +1159,22 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
       const uint32_t colgroups = (n_tiles + per_wg - 1) / per_wg;
       if (parts > 65535 || (uint64_t)colgroups * rowgroups > 0x7FFFFFF0ull) continue;
       // a workgroup's partial tile: 8 waves x (q kSide r) float4 per lane; the last part keeps its own
-      const uint64_t partial = parts > 1 ? (uint64_t)(parts - 1) * rowgroups * colgroups * (8u * q * kSide * r * 1024u) : 0;
-      if (partial > x.handover_bytes || partial >= (1ull << 32)) continue;
+      // Every part adds up a share of the tiles when all workgroups are resident at once (every part then
+      // waits for every other); the workspace then holds the last part's tiles too.  Measured against
+      // the one reader at M = 16 (us, reader / shares): 14336 x 4096, 14 parts, 15.1 / 12.8 (Q8 19.0 /
+      // 15.8); 11008 x 4096, 11 parts, 16.0 / 12.1; 8192 x 4096, 8 parts, 13.5 / 11.1; 4096 x 4096, 4
+      // parts, 11.4 / 10.8; 3072 x 4096 11.3 / 10.7; 2048 x 14336, 2 parts, 11.7 / 11.1; fp16 512 x
+      // 3072 x 1024 14.8 / 14.6.  With four parts or fewer on a nearly full chip it is level or loses
+      // (4096 x 11008, 172 workgroups: 12.1 / 12.2; 4096 x 14336, 224 workgroups: 12.5 / 13.0).
       const uint64_t wgs = (uint64_t)parts * colgroups * rowgroups;
+      const bool spread = parts >= 2 && wgs <= (uint64_t)x.num_cus && (parts >= 5 || 3 * wgs <= 2 * (uint64_t)x.num_cus);
+      const uint64_t partial = parts > 1 ? (uint64_t)(spread ? parts : parts - 1) * rowgroups * colgroups * (8u * q * kSide * r * 1024u) : 0;
+      if (partial > x.handover_bytes || partial >= (1ull << 32)) continue;
       const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q * r * nsl / 4.0) * (r == 2 ? 0.9 : 1.0) + (parts > 1 ? 1.0 : 0.0);
       if (best == 0 || cost < best) {
         best = cost;
         bp.r = r, bp.q = q, bp.nsl = nsl, bp.parts = parts, bp.colgroups = colgroups, bp.rowgroups = rowgroups;
-        bp.nslices = nslices, bp.partial_bytes = partial, bp.cost = cost;
+        bp.nslices = nslices, bp.partial_bytes = partial, bp.cost = cost, bp.spread = spread;
         bp.park = resident_lds_bytes(x.w.fmt, f32a, r, q, true) <= 160 * 1024;
         bp.lds = resident_lds_bytes(x.w.fmt, f32a, r, q, bp.park);
       }
@@ -1104,7 +1191,7 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
-  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, (float*)x.handover, x.spin_limit, x.fault_flag};
+  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, (float*)x.handover, x.spin_limit, x.fault_flag, p.spread ? 1u : 0u};
   // (column groups x row groups, K parts); with K parts the first is rounded up to a multiple of 8 (see the kernel)
   const uint64_t groups = (uint64_t)p.colgroups * p.rowgroups;
   const dim3 grid((unsigned)(p.parts > 1 ? (groups + 7) / 8 * 8 : groups), p.parts, 1);
@@ -1223,7 +1310,7 @@ int launch_cpt(ihipStream_t* s, const LaunchArgs& x, const TilePlan& p, uint4* i
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
-  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, nullptr, 0, nullptr};
+  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, nullptr, 0, nullptr, 0};
   hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups, p.rowgroups), dim3(64 * p.ksc * p.wnc), p.lds, s, image, x.w.meta, x.w.quants,
                      x.m, x.w.k, x.w.n, p.wnc, p.ksc, p.nph, p.parts, p.nslices, tail);
   MGN_HIP_LAUNCH_CHECK();

@@ -98,9 +98,14 @@ def check_tile(p, fmt, m, k, n, f16):
         assert p.full_steps == 1 or f16  # row groups of 32 are for fp16 activations
         assert p.k_parts == ceil_div(nslices, p.steps)
         # partial tiles in whole workgroup slots: 8 waves x (pairs x 2 tiles x row tiles) float4 per lane;
-        # the part that adds the others up keeps its own, and the parts meet without counters
+        # the parts meet without counters.  Either the last part adds the others up and keeps its own
+        # tiles, or -- when the whole grid is resident at once (256 CUs here) and the parts are five or
+        # more, or the workgroups fill at most two thirds of the chip -- every part adds up a share and
+        # the workspace holds all parts' tiles.
         slot = 8 * (p.waves_n // 16) * 2 * p.full_steps * 1024
-        partial = (p.k_parts - 1) * p.grid[2] * p.grid[1] * slot
+        wgs = p.k_parts * p.grid[1] * p.grid[2]
+        shares = p.k_parts >= 2 and wgs <= 256 and (p.k_parts >= 5 or 3 * wgs <= 2 * 256)
+        partial = (p.k_parts if shares else p.k_parts - 1) * p.grid[2] * p.grid[1] * slot
         assert p.workspace_bytes == partial <= WORKSPACE
     else:
         assert p.full_steps in (1, 2, 4) and p.k_splits in (1, 2, 4) and p.threads == 64 * p.k_splits * p.waves_n
