@@ -97,6 +97,16 @@ mgn_status mgn_sync(mgn_ctx* ctx);
  *     detected while it is staged and the next synchronising call returns MGN_ERANGE.
  * fp16 activations (mgn_matmul_q_f16a) and M <= 4 never depend on this. */
 typedef enum mgn_act_range { MGN_ACT_ANY = 0, MGN_ACT_FP16_RANGE = 1 } mgn_act_range;
+/* Whether other work runs on the device beside this context's launches (other contexts, other
+ * processes).  Two kinds of launch let all their workgroups wait for each other, which needs them
+ * resident on the device together: a chain (mgn_chain_*), and a matmul whose K parts are added up
+ * by all parts, a share each.  Two such kernels at once can take each other's compute units and
+ * both stall until their bounded waits give up (MGN_ETIMEOUT at the next synchronising call, no
+ * hang, results not to be used).  shared = 0 (default): the context has the device to itself while
+ * it computes, and both are used.  shared != 0: neither is; chains are refused with
+ * MGN_EUNSUPPORTED and K parts are added up by the part that is dispatched last, which waits only
+ * for workgroups dispatched before it.  No counterpart in the reference (one Session per device). */
+mgn_status mgn_ctx_set_shared_device(mgn_ctx* ctx, int shared);
 mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, mgn_act_range range);
 /* ---- plain device buffers: the reference allocates every plan buffer
  *      zero-filled (src/runtime.rs:1737-1755) and moves data with memcpy

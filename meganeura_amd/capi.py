@@ -20,7 +20,7 @@ ROUTE_AUTO, ROUTE_GENERIC, ROUTE_GEMV_VALU, ROUTE_GEMV_MFMA, ROUTE_GEMM_MFMA, RO
 # every symbol include/mgn_hip.h, include/mgn_bench.h and include/mgn_session.h declare
 BENCH_SYMBOLS = ["mgn_ctx_set_route", "mgn_ctx_set_spin_limit", "mgn_engine_clock_mhz", "mgn_matmul_q_loop", "mgn_weight_read_loop"]
 HIP_SYMBOLS = [
-    "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync", "mgn_ctx_set_activation_range",
+    "mgn_ctx_create", "mgn_ctx_destroy", "mgn_last_error", "mgn_sync", "mgn_ctx_set_activation_range", "mgn_ctx_set_shared_device",
     "mgn_buf_alloc", "mgn_buf_free", "mgn_buf_size", "mgn_buf_device_ptr", "mgn_buf_upload",
     "mgn_buf_download", "mgn_buf_copy", "mgn_packed_size", "mgn_quantize_ref", "mgn_dequantize_ref",
     "mgn_weight_create", "mgn_weight_create_nk", "mgn_quantize_ref_nk", "mgn_weight_create_packed", "mgn_weight_create_device", "mgn_weight_free",
@@ -93,6 +93,7 @@ def load():
         "mgn_ctx_set_spin_limit": (C.c_int, [vp, C.c_uint32]),
         "mgn_engine_clock_mhz": (C.c_int, [vp, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
         "mgn_ctx_set_activation_range": (C.c_int, [vp, C.c_int]),
+        "mgn_ctx_set_shared_device": (C.c_int, [vp, C.c_int]),
         "mgn_buf_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
         "mgn_buf_free": (None, [vp, vp]),
         "mgn_buf_size": (sz, [vp]),
@@ -275,6 +276,11 @@ class Context:
         """f32 activations of M >= 5: False (default, ACT_ANY) takes any value; True (ACT_FP16_RANGE)
         promises |x| < 65504 and lets the faster unscaled tiled kernel run."""
         self.check(self.lib.mgn_ctx_set_activation_range(self.h, ACT_FP16_RANGE if fp16_range else ACT_ANY))
+
+    def set_shared_device(self, shared):
+        """True: other work runs on the device beside this context; launches whose workgroups all
+        wait for each other (chains, K parts added up by shares) are not used."""
+        self.check(self.lib.mgn_ctx_set_shared_device(self.h, 1 if shared else 0))
 
     def set_route(self, route):
         self.check(self.lib.mgn_ctx_set_route(self.h, route))

@@ -314,6 +314,12 @@ mgn_status mgn_ctx_set_activation_range(mgn_ctx* ctx, mgn_act_range range) {
   return MGN_OK;
 }
 
+mgn_status mgn_ctx_set_shared_device(mgn_ctx* ctx, int shared) {
+  if (!ctx) return MGN_EINVAL;
+  ctx->shared_device = shared != 0;
+  return MGN_OK;
+}
+
 mgn_status mgn_ctx_set_spin_limit(mgn_ctx* ctx, uint32_t polls) {
   if (!ctx) return MGN_EINVAL;
   ctx->spin_limit = polls;
@@ -688,6 +694,7 @@ static mgn_status matmul_impl(mgn_ctx* ctx, const mgn_buf* a, bool a_is_f16, con
   if (c->ptr == a->ptr) return fail(ctx, MGN_EINVAL, "C must not alias A");
   mgn::LaunchArgs x{view_of(w), a->ptr, d ? (const float*)d->ptr : nullptr, (float*)c->ptr, m, a_is_f16, ctx->num_cus};
   x.device = ctx->device;
+  x.shared_device = ctx->shared_device;
   x.range_flag = ctx->range_flag_dev;
   x.fault_flag = ctx->range_flag_dev + 1;
   x.spin_limit = ctx->spin_limit;
@@ -943,6 +950,7 @@ mgn_status mgn_chain_create(mgn_ctx* ctx, const mgn_chain_stage* stages, size_t 
   *out = nullptr;
   if (count == 0 || count > 4096) return fail(ctx, MGN_EINVAL, "a chain holds 1 to 4096 stages");
   if (m != 1) return fail(ctx, MGN_EUNSUPPORTED, "chains serve one activation row (M = 1)");
+  if (ctx->shared_device) return fail(ctx, MGN_EUNSUPPORTED, "chains need the device to themselves (mgn_ctx_set_shared_device)");
   const int chain_cus = ctx->num_cus;
   std::vector<mgn::ChainStageDev> dev(count);
   std::vector<int> a_from(count, -1), d_from(count, -1);

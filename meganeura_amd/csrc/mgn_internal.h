@@ -53,6 +53,9 @@ struct LaunchArgs {
   bool a_is_f16;
   int num_cus;
   int device = 0;  // HIP device ordinal of the context
+  // other work may run on the device beside this launch: no plan whose workgroups all wait for
+  // each other (they would have to be resident together, and a second such kernel can take their CUs)
+  bool shared_device = false;
   // further weights served by the same launch (GEMV-MFMA route only): same K, format and
   // activations, each with its own output and optional residual
   struct More {
@@ -170,6 +173,7 @@ struct mgn_ctx {
   void* handover = nullptr;  // counter-free hand-over workspace (LaunchArgs::handover), kHandoverEmpty between launches
   size_t handover_bytes = 0;
   uint32_t spin_limit = 1u << 20;
+  bool shared_device = false;  // mgn_ctx_set_shared_device
   uint32_t* range_flag_host = nullptr;  // pinned, mapped, two words: [0] range, [1] hand-over gave up; written by kernels, read at sync points
   uint32_t* range_flag_dev = nullptr;   // the same words as the device sees them
   void* static_scratch = nullptr;       // this device's copy of the library's static workspace (mgn_matmul_q_static)

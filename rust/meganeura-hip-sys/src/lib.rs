@@ -123,6 +123,7 @@ extern "C" {
     pub fn mgn_last_error(ctx: *const mgn_ctx) -> *const c_char;
     pub fn mgn_sync(ctx: *mut mgn_ctx) -> mgn_status;
     pub fn mgn_ctx_set_activation_range(ctx: *mut mgn_ctx, range: mgn_act_range) -> mgn_status;
+    pub fn mgn_ctx_set_shared_device(ctx: *mut mgn_ctx, shared: c_int) -> mgn_status;
     pub fn mgn_buf_alloc(ctx: *mut mgn_ctx, bytes: usize, out: *mut *mut mgn_buf) -> mgn_status;
     pub fn mgn_buf_free(ctx: *mut mgn_ctx, buf: *mut mgn_buf);
     pub fn mgn_buf_size(buf: *const mgn_buf) -> usize;

@@ -29,6 +29,28 @@ def rms_norm(x, g, eps):
     return (x64 / np.sqrt((x64 ** 2).mean() + eps) * g).astype(np.float32)
 
 
+def test_a_context_on_a_shared_device_refuses_chains(ctx, orc):
+    """mgn_ctx_set_shared_device: a chain's workgroups all wait for each other, which needs the
+    device to themselves; on a shared device the chain is refused and the caller launches the
+    stages one by one."""
+    k, n = 576, 576
+    wt = ctx.weight(Q4, synth.normal(3001, k * n, 0.02).reshape(k, n))
+    a, c = ctx.upload(synth.normal(3002, k, 1.0)), ctx.buffer(n * 4)
+    ctx.set_shared_device(True)
+    try:
+        with pytest.raises(capi.MgnError) as e:
+            ctx.chain([dict(w=wt, a=a, c=c)])
+        assert e.value.status == capi.EUNSUPPORTED
+    finally:
+        ctx.set_shared_device(False)
+    ch = ctx.chain([dict(w=wt, a=a, c=c)])
+    ch.run()
+    ctx.sync()
+    ch.free()
+    for h in (a, c, wt):
+        h.free()
+
+
 def swiglu(gate_up, k):
     # src/shaders/swiglu_concat.wgsl:20-32
     g, u = gate_up[:, :k].astype(np.float64), gate_up[:, k:].astype(np.float64)

@@ -934,6 +934,30 @@ def test_a_block_beyond_2_to_the_100_gives_a_non_finite_row_on_the_gemv(ctx, orc
     wt.free()
 
 
+@pytest.mark.parametrize("fmt,m,k,n", [(Q4, 16, 14336, 1024), (Q8, 9, 8192, 512), (Q4, 16, 2048, 4096)])
+def test_k_parts_added_up_by_shares_or_by_the_last_part_agree(ctx, orc, fmt, m, k, n):
+    """Shapes whose K parts are added up by all parts, a share each (the whole grid resident at
+    once), against the same call on a context that shares its device, where the part dispatched
+    last adds the others up: both within the bar, each repeatable bit for bit, and the two orders
+    of summation within a few ulps of each other."""
+    w = synth.normal(1501 + k, k * n, 0.02).reshape(k, n)
+    x = synth.normal(1502 + m, m * k, 1.0).reshape(m, k)
+    wt = ctx.weight(fmt, w)
+    want = orc.matmul_f64(x, orc.dequantize(fmt, orc.quantize(fmt, w), k, n))
+    assert capi.matmul_plan(fmt, m, k, n).k_parts > 1
+    shares = [run_matmul(ctx, fmt, x, wt, ROUTES["auto"]) for _ in range(3)]
+    ctx.set_shared_device(True)
+    try:
+        last = [run_matmul(ctx, fmt, x, wt, ROUTES["auto"]) for _ in range(3)]
+    finally:
+        ctx.set_shared_device(False)
+    for got in (shares, last):
+        assert (bits(got[0]) == bits(got[1])).all() and (bits(got[0]) == bits(got[2])).all()
+        orc.assert_close(got[0], want, REL, ABS)
+    np.testing.assert_allclose(shares[0], last[0], rtol=2e-5, atol=2e-5)
+    wt.free()
+
+
 @pytest.mark.parametrize("fmt,m,k,n", [(Q4, 16, 4096, 2048), (Q8, 9, 4096, 1024), (Q4, 4, 14336, 518), (Q8, 3, 12288, 64)])
 def test_a_reader_that_gives_up_is_reported_and_the_context_recovers(ctx, orc, fmt, m, k, n):
     """K cut into parts for different workgroups: the part that adds the others up polls the
