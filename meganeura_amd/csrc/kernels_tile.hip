@@ -1166,8 +1166,13 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
       // parts, 11.4 / 10.8; 3072 x 4096 11.3 / 10.7; 2048 x 14336, 2 parts, 11.7 / 11.1; fp16 512 x
       // 3072 x 1024 14.8 / 14.6.  With four parts or fewer on a nearly full chip it is level or loses
       // (4096 x 11008, 172 workgroups: 12.1 / 12.2; 4096 x 14336, 224 workgroups: 12.5 / 13.0).
+      // Resident at once means per XCD: workgroups go to the eight XCDs in turn by their linear index, the
+      // groups are in grid x (a multiple of 8) and the parts in y, so an XCD gets ceil(groups / 8) groups
+      // with all their parts, one workgroup per CU, on an eighth of the CUs.
       const uint64_t wgs = (uint64_t)parts * colgroups * rowgroups;
-      const bool spread = !x.shared_device && parts >= 2 && wgs <= (uint64_t)x.num_cus && (parts >= 5 || 3 * wgs <= 2 * (uint64_t)x.num_cus);
+      const uint64_t per_xcd = ((uint64_t)colgroups * rowgroups + 7) / 8 * parts;
+      const bool spread = !x.shared_device && parts >= 2 && per_xcd <= (uint64_t)x.num_cus / 8 &&
+                          (parts >= 5 || 3 * wgs <= 2 * (uint64_t)x.num_cus);
       const uint64_t partial = parts > 1 ? (uint64_t)(spread ? parts : parts - 1) * rowgroups * colgroups * (8u * q * kSide * r * 1024u) : 0;
       if (partial > x.handover_bytes || partial >= (1ull << 32)) continue;
       const double cost = std::ceil((double)wgs / x.num_cus) * (1.5 + q * r * nsl / 4.0) * (r == 2 ? 0.9 : 1.0) + (parts > 1 ? 1.0 : 0.0);

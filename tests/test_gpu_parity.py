@@ -934,7 +934,20 @@ def test_a_block_beyond_2_to_the_100_gives_a_non_finite_row_on_the_gemv(ctx, orc
     wt.free()
 
 
-@pytest.mark.parametrize("fmt,m,k,n", [(Q4, 16, 14336, 1024), (Q8, 9, 8192, 512), (Q4, 16, 2048, 4096)])
+def test_shares_are_planned_only_when_every_xcd_holds_its_workgroups():
+    """Every part adds up a share only if all workgroups are resident at once, and that is decided
+    per XCD: 17 column groups of 14 parts are 238 workgroups on 256 CUs, but XCD 0 would get three
+    groups = 42 workgroups on its 32 CUs.  Such a launch keeps the single reader (its workspace
+    holds 13 parts' tiles, not 14); 16 groups of 14 parts fit and take the shares."""
+    slot = 8 * 2 * 1024  # a workgroup's tiles: 8 waves x one pair of 16-column tiles x 1 KiB
+    p = capi.matmul_plan(Q4, 16, 14336, 17 * 256)
+    assert (p.route, p.k_parts, p.grid[1], p.grid[2]) == (capi.ROUTE_TILE_MFMA, 14, 17, 1)
+    assert p.workspace_bytes == 13 * 17 * slot
+    p = capi.matmul_plan(Q4, 16, 14336, 16 * 256)
+    assert (p.k_parts, p.grid[1]) == (14, 16) and p.workspace_bytes == 14 * 16 * slot
+
+
+@pytest.mark.parametrize("fmt,m,k,n", [(Q4, 16, 14336, 1024), (Q8, 9, 8192, 512), (Q4, 16, 2048, 4096), (Q4, 16, 14336, 17 * 256)])
 def test_k_parts_added_up_by_shares_or_by_the_last_part_agree(ctx, orc, fmt, m, k, n):
     """Shapes whose K parts are added up by all parts, a share each (the whole grid resident at
     once), against the same call on a context that shares its device, where the part dispatched

@@ -103,8 +103,10 @@ def check_tile(p, fmt, m, k, n, f16):
         # more, or the workgroups fill at most two thirds of the chip -- every part adds up a share and
         # the workspace holds all parts' tiles.
         slot = 8 * (p.waves_n // 16) * 2 * p.full_steps * 1024
+        # (resident at once is a matter of every XCD: it gets every eighth group with all its parts, on 32 CUs)
         wgs = p.k_parts * p.grid[1] * p.grid[2]
-        shares = p.k_parts >= 2 and wgs <= 256 and (p.k_parts >= 5 or 3 * wgs <= 2 * 256)
+        per_xcd = ceil_div(p.grid[1] * p.grid[2], 8) * p.k_parts
+        shares = p.k_parts >= 2 and per_xcd <= 32 and (p.k_parts >= 5 or 3 * wgs <= 2 * 256)
         partial = (p.k_parts if shares else p.k_parts - 1) * p.grid[2] * p.grid[1] * slot
         assert p.workspace_bytes == partial <= WORKSPACE
     else:
