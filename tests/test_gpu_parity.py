@@ -551,6 +551,17 @@ def test_matmul_loop_is_the_same_calls_in_a_row(ctx, orc):
         w.free()
 
 
+def test_engine_clock_probes_return_plausible_figures(ctx):
+    """mgn_engine_clock_mhz (a measurement aid): the shader clock against the 100 MHz counter, from one
+    idle wave and under a matrix-instruction load on every CU, with the load's cycles per round; the
+    probes use the head of the split-K workspace and must leave the context usable."""
+    idle = ctx.engine_clock_mhz()
+    loaded, cycles = ctx.engine_probe()
+    assert 500.0 < idle < 4000.0 and 500.0 < loaded < 4000.0
+    assert 64.0 <= cycles < 5000.0  # at least the eight matrix instructions of a round, at 8 cycles each
+    ctx.sync()
+
+
 def test_weight_read_loop_leaves_results_alone(ctx, orc):
     """mgn_weight_read_loop (a timing aid: plain reads of the packed bytes) runs on weights of
     both formats, the smallest included, and a K-part matmul enqueued right behind it, whose
