@@ -315,7 +315,8 @@ mgn_status mgn_matmul_q_batch(mgn_ctx* ctx, const mgn_buf* a, mgn_prologue prolo
  * synchronising call if it ever gives up).  Every C_j is also written to the caller's buffer.
  * mgn_chain_create: MGN_EUNSUPPORTED when a stage is not served (m != 1, a Q8 weight, K beyond
  * 16384, two stages writing one buffer, a stage writing a buffer that the chain also reads as
- * written before the launch): run the dispatches one by one then.  It allocates (tables and
+ * written before the launch), or when the context shares its device (mgn_ctx_set_shared_device:
+ * a chain's workgroups wait for each other): run the dispatches one by one then.  It allocates (tables and
  * workspace) and synchronises; mgn_chain_run allocates nothing and is asynchronous on the
  * context's stream.  The weights and buffers must outlive the chain; free it before them.
  * A chain must not be recorded into a HIP graph that is replayed: consecutive runs alternate
