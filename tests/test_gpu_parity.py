@@ -945,6 +945,50 @@ def test_a_block_beyond_2_to_the_100_gives_a_non_finite_row_on_the_gemv(ctx, orc
     wt.free()
 
 
+@pytest.mark.parametrize("seed,shared", [(11, False), (12, False), (13, True)])
+def test_random_shapes_on_the_automatic_route(ctx, orc, seed, shared):
+    """A seeded random sweep of the kind that found the per-XCD residency limit: 120 shapes per
+    seed over both formats, M from 1 to 1000, K from 32 to 16000, N from 1 to 30000, f32 and fp16
+    activations of several magnitudes, weights of several magnitudes and offsets, with and without a
+    residual, on the automatic route; one seed on a context that shares its device (K parts added
+    up by the last part only).  Every result within the matmul bar, with its absolute part scaled
+    by the magnitudes at hand; no launch may end in a give-up.  (Q8 weights with fp16-subnormal
+    scales and f32 activations at M >= 5 are held to the documented 2.5e-4 instead of 1e-4.)"""
+    rng = np.random.default_rng(seed)
+    ctx.set_shared_device(shared)
+    try:
+        done = 0
+        while done < 120:
+            fmt = int(rng.integers(0, 2))
+            m = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 48, 64, 65, 100, 128, 200, 513, 1000]))
+            k = 32 * int(rng.choice([rng.integers(1, 12), rng.integers(12, 100), rng.integers(100, 500)]))
+            n = int(rng.choice([rng.integers(1, 40), rng.integers(40, 600), rng.integers(600, 5000), rng.integers(5000, 30000)]))
+            if m * k * n > 1.5e9 or k * n > 6.0e7:
+                continue
+            f16 = bool(rng.integers(0, 2))
+            resid = bool(rng.integers(0, 2))
+            scale = float(rng.choice([1.0, 1e-2, 1e-4, 300.0]))
+            wscale = float(rng.choice([0.03, 0.03, 1e-5, 30.0]))
+            woff = float(rng.choice([0.0, 0.0, 1.0, -3.0])) * wscale
+            w = (rng.standard_normal((k, n)) * wscale + woff).astype(np.float32)
+            x = (rng.standard_normal((m, k)) * scale).astype(np.float32)
+            xa = x.astype(np.float16).astype(np.float32) if f16 else x
+            d = (rng.standard_normal((m, n)) * scale).astype(np.float32) if resid else None
+            deq = orc.dequantize(fmt, orc.quantize(fmt, w), k, n).astype(np.float64)
+            want = xa.astype(np.float64) @ deq + (d.astype(np.float64) if resid else 0.0)
+            got = run_matmul(ctx, fmt, x, w, d=d, f16=f16).astype(np.float64)
+            xr = np.sqrt((xa.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
+            typ = xr * np.sqrt((deq ** 2).mean(axis=0, keepdims=True)) * np.sqrt(k) + 1e-30 + (np.abs(d) if resid else 0.0)
+            abs_bar = 2.5e-4 if (fmt == Q8 and wscale < 1e-3 and not f16 and m >= 5) else ABS
+            err = np.abs(got - want)
+            where = f"seed {seed} shape {done}: fmt {fmt} m {m} k {k} n {n} f16 {f16} resid {resid} scale {scale} wscale {wscale} woff {woff}"
+            assert np.isfinite(got).all(), where
+            assert (err <= REL * np.abs(want) + abs_bar * typ).all(), where + f" worst {(err / typ).max():.2e} of typical"
+            done += 1
+    finally:
+        ctx.set_shared_device(False)
+
+
 def test_shares_are_planned_only_when_every_xcd_holds_its_workgroups():
     """Every part adds up a share only if all workgroups are resident at once, and that is decided
     per XCD: 17 column groups of 14 parts are 238 workgroups on 256 CUs, but XCD 0 would get three
