@@ -528,6 +528,12 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(const void* __restrict__
     }
   }
   if (writer) {
+    if (row0 + 8 * ((NI - 1) >> 2) + 8 <= g.m && !g.dres && tail.epilogue == 0) {  // (uniform) whole rows, nothing to add or apply
+      float* const dst = g.c + (size_t)(row0 + 4 * gh) * w.n + n;
+#pragma unroll
+      for (int i = 0; i < NI; i++) dst[(size_t)(8 * (i >> 2) + (i & 3)) * w.n] = outv[i];
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NI; i++) {
       const uint32_t row = row0 + 8 * (i >> 2) + 4 * gh + (i & 3);

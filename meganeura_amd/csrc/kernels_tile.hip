@@ -549,6 +549,16 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
     }
   }
   if (writer) {
+    if (row0 + R * 16 <= m && !tail.dres && tail.epilogue == 0) {  // (uniform) whole rows, nothing to add or apply
+      float* dst = tail.c + (size_t)(row0 + 4 * g) * n + col;
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[(size_t)i * n] = acc[r][i];
+        dst += (size_t)16 * n;
+      }
+      return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++)
 #pragma unroll
@@ -1012,12 +1022,18 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
         const uint32_t tp = slot / (kSide * R), tu = (slot / R) % kSide, tr = slot % R;
         const uint32_t col = (((cg * 8 + src_wave) * Q + tp) * kSide + tu) * 16 + c;
         if (col < n) {
+          if (row0 + R * 16 <= m && !tail.dres && tail.epilogue == 0) {  // (uniform) whole rows, nothing to add or apply
+            float* const dst = tail.c + (size_t)(row0 + tr * 16 + 4 * g) * n + col;
 #pragma unroll
-          for (int i = 0; i < 4; i++) {
-            const uint32_t row = row0 + tr * 16 + 4 * g + i;
-            if (row < m) {
-              const size_t o = (size_t)row * n + col;
-              tail.c[o] = apply_epilogue(tail.dres ? sum[i] + tail.dres[o] : sum[i], tail.epilogue);
+            for (int i = 0; i < 4; i++) dst[(size_t)i * n] = sum[i];
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+              const uint32_t row = row0 + tr * 16 + 4 * g + i;
+              if (row < m) {
+                const size_t o = (size_t)row * n + col;
+                tail.c[o] = apply_epilogue(tail.dres ? sum[i] + tail.dres[o] : sum[i], tail.epilogue);
+              }
             }
           }
         }
@@ -1097,12 +1113,26 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
         for (int r = 0; r < R; r++) res[p][u][r] = sum[(p * kSide + u) * R + r] + res[p][u][r];
     if (gave_up && lane == 0 && tail.fault_flag) *tail.fault_flag = 1u;
   }
+  // The stores end every wave's life, with nothing left to hide them behind: a row group that lies
+  // inside M whole, with no residual and no unary operation, stores through one pointer per tile and
+  // a running row stride, without a test or a 64-bit product per element.
+  const bool whole_rows = row0 + R * 16 <= m && !tail.dres && tail.epilogue == 0;  // uniform
 #pragma unroll
   for (int p = 0; p < Q; p++)
 #pragma unroll
     for (int u = 0; u < kSide; u++) {
       const uint32_t col = ((pair0 + p) * kSide + u) * 16 + c;
       if (col < n) {
+        if (whole_rows) {
+          float* dst = tail.c + (size_t)(row0 + 4 * g) * n + col;
+#pragma unroll
+          for (int r = 0; r < R; r++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[(size_t)i * n] = res[p][u][r][i];
+            dst += (size_t)16 * n;
+          }
+          continue;
+        }
 #pragma unroll
         for (int r = 0; r < R; r++)
 #pragma unroll

@@ -946,7 +946,7 @@ def test_a_block_beyond_2_to_the_100_gives_a_non_finite_row_on_the_gemv(ctx, orc
 
 
 @pytest.mark.parametrize("seed,shared", [(11, False), (12, False), (13, True)])
-def test_random_shapes_on_the_automatic_route(ctx, orc, seed, shared):
+def test_random_shapes_magnitudes_and_hand_over_forms(ctx, orc, seed, shared):
     """A seeded random sweep of the kind that found the per-XCD residency limit: 120 shapes per
     seed over both formats, M from 1 to 1000, K from 32 to 16000, N from 1 to 30000, f32 and fp16
     activations of several magnitudes, weights of several magnitudes and offsets, with and without a
