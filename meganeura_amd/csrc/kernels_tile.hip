@@ -1116,7 +1116,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   // The stores end every wave's life, with nothing left to hide them behind: a row group that lies
   // inside M whole, with no residual and no unary operation, stores through one pointer per tile and
   // a running row stride, without a test or a 64-bit product per element.
-  const bool whole_rows = row0 + R * 16 <= m && !tail.dres && tail.epilogue == 0;  // uniform
+  const bool whole_rows = row0 + R * 16 <= m && tail.epilogue == 0;  // uniform
 #pragma unroll
   for (int p = 0; p < Q; p++)
 #pragma unroll
@@ -1124,7 +1124,21 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
       const uint32_t col = ((pair0 + p) * kSide + u) * 16 + c;
       if (col < n) {
         if (whole_rows) {
-          float* dst = tail.c + (size_t)(row0 + 4 * g) * n + col;
+          const size_t first = (size_t)(row0 + 4 * g) * n + col;
+          float* dst = tail.c + first;
+          if (tail.dres) {  // (uniform) the residual's loads first, all of a tile column's at once
+            const float* src = tail.dres + first;
+            float dv[R][4];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+              for (int i = 0; i < 4; i++) dv[r][i] = src[(size_t)(16 * r + i) * n];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+              for (int i = 0; i < 4; i++) dst[(size_t)(16 * r + i) * n] = res[p][u][r][i] + dv[r][i];
+            continue;
+          }
 #pragma unroll
           for (int r = 0; r < R; r++) {
 #pragma unroll
