@@ -24,8 +24,9 @@
 //   Per block: D = sum n x on the matrix cores, then P += d * D on the vector ALU (4 FMAs per
 //     lane).  The format's additive part (m * sum(x) for Q4, -128 * scale * sum(x) for Q8's byte
 //     bias) is one more MFMA per slice of 8 blocks: its A operand holds the blocks' mean
-//     activations (hi, lo), its B operand the blocks' m (or scale), exact fp16 values.  (fp16
-//     activations: two MFMAs, hi and lo apart, because lo is kept times 2^11; see convert_task.)
+//     activations (hi, lo), its B operand the blocks' m (or scale), exact fp16 values times a
+//     power of two chosen per weight (AddLift).  (fp16 activations: two MFMAs, hi and lo apart,
+//     because lo is kept times 2^11; see convert_task.)
 //     With f32 activations a slice's P is multiplied by the rows' inverse power-of-two scales
 //     before it is added to the accumulators.
 //
@@ -42,6 +43,7 @@
 // With too few tiles to fill the chip K is also cut into parts for different workgroups, whose
 // partial tiles the last one to finish adds in part order (deterministic).
 #include <algorithm>
+#include <cmath>
 #include <type_traits>
 
 #include "kernels_operand.hip.h"
@@ -53,6 +55,19 @@ namespace {
 // 32 for the means and, for Q8, -128 for the byte bias, over the quants' operand scale.
 template <int FMT>
 constexpr float additive_constant() { return FMT == MGN_FMT_Q4 ? 32.0f / 1048576.0f : -4096.0f / 16777216.0f; }
+
+// The additive MFMA's B operand holds the blocks' own constants (m, or the Q8 scale) as fp16, and
+// the matrix cores lose low bits of products whose operand is an fp16 subnormal (Q8 scales below
+// 2^-14: 2 * 10^-4 of a typical output, measured).  The constants are therefore multiplied by a
+// power of two first, the largest that keeps the weight's largest constant finite (exact, one
+// packed multiplication per dword), and the instruction's result by its inverse.
+struct AddLift {
+  uint32_t up2;  // 2^s twice, as fp16
+  float down;    // 2^-s
+  __device__ __forceinline__ uint32_t up(uint32_t pair) const {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, pair) * __builtin_bit_cast(half2_t, up2));
+  }
+};
 
 // max over aligned groups of 32 consecutive lanes (every lane ends with the group's maximum)
 __device__ __forceinline__ float group_max32(float v) {
@@ -211,7 +226,7 @@ __global__ __launch_bounds__(512) void image_kernel(const void* __restrict__ a, 
 // tiles rstride bytes apart), the column's 8 scale words in mw.
 template <int FMT, bool F32A, int R>
 __device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t* ib, uint32_t rstride, const uint32_t (&mw)[8],
-                                          uint32_t g, uint32_t lane, floatx4 (&acc)[R]) {
+                                          uint32_t g, uint32_t lane, AddLift lift, floatx4 (&acc)[R]) {
   constexpr uint32_t HL = F32A ? 2 : 1;
     // Software pipeline over the 8 blocks: LDS reads two blocks ahead, unpack and MFMAs one
     // block ahead of the scaling FMAs that consume the previous block's products.
@@ -276,10 +291,10 @@ __device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t*
       // (bit arithmetic, not a select between array elements: that would be turned into an
       // indexed load from a stack copy of the array)
       const uint32_t w = mw[j] ^ ((mw[j] ^ mw[4 + j]) & upper);
-      bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
+      bw[j] = lift.up(FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u));
     }
     const half8 bm = as_half8(bw[0], bw[1], bw[2], bw[3]);
-    constexpr float kAdd = additive_constant<FMT>();
+    const float kAdd = additive_constant<FMT>() * lift.down;
 #pragma unroll
     for (int r = 0; r < R; r++) {
       const uint8_t* const ir = ib + lane * 16 + r * rstride + 8 * HL * 64 * 16;
@@ -299,7 +314,7 @@ __device__ __forceinline__ void slice_mac(const uint8_t* park_rd, const uint8_t*
         const floatx4 dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bm, floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
         const floatx4 dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bm, floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[r][i] += __fmaf_rn(kAdd / 2048.0f, dl[i], __fmaf_rn(kAdd, dh[i], P[r][i]));
+        for (int i = 0; i < 4; i++) acc[r][i] += __fmaf_rn(kAdd * (1.0f / 2048.0f), dl[i], __fmaf_rn(kAdd, dh[i], P[r][i]));
       }
     }
   }
@@ -316,6 +331,7 @@ struct TileTail {  // arguments first needed in the epilogue
   uint32_t spin_limit;
   uint32_t* fault_flag;
   uint32_t spread;  // resident kernel: every part adds up a share of the tiles (all workgroups of the launch resident)
+  AddLift lift;     // (needed in the walk; rides along here)
 };
 
 constexpr int park_stride(int fmt) { return fmt == MGN_FMT_Q4 ? 8 * 16 + 16 : 8 * 32 + 16; }  // bytes per parked column
@@ -470,7 +486,7 @@ __global__ __launch_bounds__(512) void tile_mfma_kernel(const uint4* __restrict_
           const uint8_t* const ib = (const uint8_t*)(imgbuf + (p & 1) * buf_units + ks * UNITS);
           constexpr uint32_t kRowTile = 16;  // bytes per uint4 unit
           const uint32_t rstride = ksc * UNITS * kRowTile;  // bytes between the row tiles of a buffer
-          slice_mac<FMT, F32A, R>(park_rd, ib, rstride, mw, g, lane, acc);
+          slice_mac<FMT, F32A, R>(park_rd, ib, rstride, mw, g, lane, tail.lift, acc);
         }
         copy_store((ph + 1) & 1, (p + 1) & 1);  // that LDS buffer was last read before the previous barrier
         lds_barrier();
@@ -617,7 +633,7 @@ constexpr int kSide = 2;            // column tiles a wave multiplies side by si
 template <int FMT, bool F32A, int R, bool PARK>
 __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == MGN_FMT_Q4 ? 2 : 4], const uint8_t* park_rd,
                                                const uint32_t (&mw)[kSide][8], const uint8_t* ib, uint32_t rstride, uint32_t g,
-                                               uint32_t lane, floatx4 (&acc)[kSide][R]) {
+                                               uint32_t lane, AddLift lift, floatx4 (&acc)[kSide][R]) {
   constexpr uint32_t HL = F32A ? 2 : 1;
   const uint32_t slot_off[2] = {image_slot(lane & 15, g, 0) * 16, image_slot(lane & 15, g, 1) * 16};
   u32x4_t aop[3][R][HL];
@@ -693,7 +709,7 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
   }
   // additive part of the slice's 8 blocks (see slice_mac)
   const uint32_t upper = 0u - (g & 1u);  // all ones in the lanes that take blocks 4..7
-  constexpr float kAdd = additive_constant<FMT>();
+  const float kAdd = additive_constant<FMT>() * lift.down;
   half8 bm[kSide];
 #pragma unroll
   for (int u = 0; u < kSide; u++) {
@@ -701,7 +717,7 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const uint32_t w = mw[u][j] ^ ((mw[u][j] ^ mw[u][4 + j]) & upper);
-      bw[j] = FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u);
+      bw[j] = lift.up(FMT == MGN_FMT_Q4 ? __builtin_amdgcn_perm(w, w, 0x07060706u) : __builtin_amdgcn_perm(w, w, 0x05040504u));
     }
     bm[u] = as_half8(bw[0], bw[1], bw[2], bw[3]);
   }
@@ -729,7 +745,7 @@ __device__ __forceinline__ void slice_mac_side(const u32x4_t (&q)[kSide][FMT == 
         const floatx4 dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bm[u], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
         const floatx4 dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, bm[u], floatx4{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[u][r][i] += __fmaf_rn(kAdd / 2048.0f, dl[i], __fmaf_rn(kAdd, dh[i], P[u][r][i]));
+        for (int i = 0; i < 4; i++) acc[u][r][i] += __fmaf_rn(kAdd * (1.0f / 2048.0f), dl[i], __fmaf_rn(kAdd, dh[i], P[u][r][i]));
       }
     }
   }
@@ -922,7 +938,7 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
           for (int e = 0; e < 8; e++) mw[u][e] = kb0 + e < bpc ? mw[u][e] : 0u;
       }
       slice_mac_side<FMT, F32A, R, PARK>(wq[slot], wpark + c * kStride + g * (QB / 4), mw, (const uint8_t*)(img + ws * R * UNITS),
-                                         UNITS * 16, g, lane, res[wp]);
+                                         UNITS * 16, g, lane, tail.lift, res[wp]);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -1161,6 +1177,13 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
     }
 }
 
+// s = WeightView::additive_lift: 2^s as an fp16 pair and 2^-s
+AddLift add_lift(const WeightView& w) {
+  const uint32_t s = std::min<uint32_t>(w.additive_lift, 15u);
+  const uint32_t h = (15u + s) << 10;  // fp16 bits of 2^s
+  return AddLift{h | (h << 16), std::ldexp(1.0f, -(int)s)};
+}
+
 struct ResidentPlan {
   uint32_t r, q, nsl, parts, colgroups, rowgroups, nslices;
   bool park;  // quants through a wave-private LDS strip (if there is room) instead of row swaps
@@ -1240,7 +1263,7 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
-  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, (float*)x.handover, x.spin_limit, x.fault_flag, p.spread ? 1u : 0u};
+  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, (float*)x.handover, x.spin_limit, x.fault_flag, p.spread ? 1u : 0u, add_lift(x.w)};
   // (column groups x row groups, K parts); with K parts the first is rounded up to a multiple of 8 (see the kernel)
   const uint64_t groups = (uint64_t)p.colgroups * p.rowgroups;
   const dim3 grid((unsigned)(p.parts > 1 ? (groups + 7) / 8 * 8 : groups), p.parts, 1);
@@ -1359,7 +1382,7 @@ int launch_cpt(ihipStream_t* s, const LaunchArgs& x, const TilePlan& p, uint4* i
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
-  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, nullptr, 0, nullptr, 0};
+  const TileTail tail{x.d, x.c, (float*)x.scratch, x.counters, x.epilogue, nullptr, 0, nullptr, 0, add_lift(x.w)};
   hipLaunchKernelGGL(kern, dim3(p.parts, p.colgroups, p.rowgroups), dim3(64 * p.ksc * p.wnc), p.lds, s, image, x.w.meta, x.w.quants,
                      x.m, x.w.k, x.w.n, p.wnc, p.ksc, p.nph, p.parts, p.nslices, tail);
   MGN_HIP_LAUNCH_CHECK();

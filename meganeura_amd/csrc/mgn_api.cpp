@@ -74,7 +74,7 @@ size_t quant_elem(mgn_fmt fmt) { return fmt == MGN_FMT_Q4 ? 16 : 32; }
 bool valid_fmt(mgn_fmt fmt) { return fmt == MGN_FMT_Q4 || fmt == MGN_FMT_Q8; }
 
 mgn::WeightView view_of(const mgn_weight* w) {
-  return mgn::WeightView{w->meta, w->quants, (uint32_t)w->rows, (uint32_t)w->cols, (int)w->fmt, w->mfma_gemm_range_ok};
+  return mgn::WeightView{w->meta, w->quants, (uint32_t)w->rows, (uint32_t)w->cols, (int)w->fmt, w->mfma_gemm_range_ok, w->additive_lift};
 }
 
 // Device storage for a [rows, cols] weight, contents undefined.
@@ -177,6 +177,12 @@ mgn_status finish_weight_range(mgn_ctx* ctx, mgn_weight* w, const char* what) {
   std::memcpy(&smax, &host[0], 4);
   std::memcpy(&mmax, &host[1], 4);
   w->mfma_gemm_range_ok = w->fmt == MGN_FMT_Q4 ? (mmax < 2047.0f && std::isfinite(smax)) : smax < 15.99f;
+  // the constant the additive part multiplies by: every block's minimum (Q4) or scale (Q8)
+  const float amax = w->fmt == MGN_FMT_Q4 ? mmax : smax;
+  w->additive_lift = 0;
+  if (std::isfinite(amax)) {
+    while (w->additive_lift < 15 && std::ldexp(amax, (int)w->additive_lift + 1) < 32768.0f) w->additive_lift++;
+  }
   return MGN_OK;
 }
 

@@ -40,6 +40,10 @@ struct WeightView {
   // The tiled MFMA kernel feeds 32 * min (Q4) or 4096 * scale (Q8) to the matrix cores as
   // fp16: true when every block of this weight keeps that finite (|min| < 2047, scale < 15.99).
   bool mfma_gemm_range_ok = true;
+  // The 16x16 tiled kernels multiply every block's additive constant (Q4: min, Q8: scale) by 2^additive_lift
+  // on its way into the matrix cores, which lose low product bits on fp16 subnormals: the largest
+  // power of two up to 2^15 that keeps the weight's largest such constant below 32768.
+  uint32_t additive_lift = 0;
 };
 
 enum { kProNone = 0, kProRmsNorm = 1, kProSwiglu = 2 };
@@ -214,4 +218,5 @@ struct mgn_weight {
   void* quants = nullptr;  // into base, 256-byte aligned
   size_t meta_bytes = 0, quant_bytes = 0;
   bool mfma_gemm_range_ok = true;  // see WeightView
+  uint32_t additive_lift = 0;      // see WeightView
 };
