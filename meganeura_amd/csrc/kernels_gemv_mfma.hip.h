@@ -288,7 +288,11 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   // in the load queue (which drains at HBM speed) before it could prepare any activations.
   // load t = q * STEPS + s: K step s of the wave's quad q
   constexpr int TS = STEPS * QPW;
-  constexpr int kDepth = prefetch_depth<FMT>();
+  // One row with the shared tail step (short K, e.g. 576 x 49152: four one-step quads and the tail
+  // make five loads per wave): all five go out before the activations are prepared, which is little
+  // work at such a K, so none of them pays a second trip to memory behind the barrier (5.94 -> 5.54
+  // us; 640 x 32768 5.06 -> 4.74; with more rows the prologue is longer and the deeper queue loses).
+  constexpr int kDepth = (TAIL && MROWS == 1) ? 5 : prefetch_depth<FMT>();
   // TAIL: K is STEPS full steps plus 1, 2 or 4 leftover blocks per column.  Instead of a second,
   // nearly empty step for every quad, one more step takes the leftovers of all QPW quads at once:
   // the MFMA's 16 blocks are independent, so slot b serves quad b / T, K block 16 * STEPS + b % T.
