@@ -15,7 +15,8 @@ template <int FMT>
 constexpr float operand_scale() { return FMT == MGN_FMT_Q4 ? 1048576.0f : 16777216.0f; }  // 2^20, 2^24
 constexpr int kMaxTasks = 2;  // activation chunks a thread prepares at most, per row
 // weight blocks in flight per lane ahead of the one in use (measured: 3 for Q4's 20-byte
-// blocks, 2 for Q8's 34-byte blocks; one more or less costs 0.3-0.4 us on a 4096 x 14336 weight)
+// blocks, 2 for Q8's 34-byte blocks; the one-row Q4 kernel takes one more where a wave has the
+// loads for it, see gemv_mfma_kernel)
 template <int FMT>
 constexpr int prefetch_depth() { return FMT == MGN_FMT_Q8 ? 2 : 3; }
 
