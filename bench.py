@@ -76,25 +76,25 @@ HEADLINE = "c5_q4_m1_4096x14336"
 MEASURED_TRAFFIC_BYTES = {
     "c5_q4_m1_4096x14336": 37.02e6,
     "c5_q4_m1_14336x4096": 37.42e6,
-    "c5_q8_m1_4096x14336": 63.60e6,
+    "c5_q8_m1_4096x14336": 63.57e6,
     "c5_q8_m1_14336x4096": 64.02e6,
-    "c5_q4_m4_4096x14336": 37.74e6,
-    "c5_q4_m4_14336x4096": 39.60e6,
-    "c5_q8_m4_4096x14336": 64.58e6,
-    "c5_q8_m4_14336x4096": 66.33e6,
-    "c5_q4_m16_4096x14336": 50.12e6,
-    "c5_q4_m16_14336x4096": 56.58e6,
-    "c5_q8_m16_4096x14336": 75.52e6,
-    "c5_q8_m16_14336x4096": 82.43e6,
-    "c3_q4_lm_head_576x49152": 18.03e6,
+    "c5_q4_m4_4096x14336": 37.71e6,
+    "c5_q4_m4_14336x4096": 39.55e6,
+    "c5_q8_m4_4096x14336": 64.56e6,
+    "c5_q8_m4_14336x4096": 66.31e6,
+    "c5_q4_m16_4096x14336": 50.11e6,
+    "c5_q4_m16_14336x4096": 56.63e6,
+    "c5_q8_m16_4096x14336": 74.80e6,
+    "c5_q8_m16_14336x4096": 82.33e6,
+    "c3_q4_lm_head_576x49152": 18.02e6,
     "c1_q8_up_576x1536": 1.17e6,
     "c2_q4_gate_up_576x3072": 1.33e6,
     "c2_q4_down_1536x576_add": 0.74e6,
-    "c2_q4_q_576x576": 0.40e6,
+    "c2_q4_q_576x576": 0.39e6,
     "c4_q4_prefill_up_512x1024x3072": 18.99e6,
-    "c4_q4_prefill_down_512x3072x1024": 32.98e6,
-    "c4_f32a_q4_prefill_up_512x1024x3072": 27.28e6,
-    "c4_f32a_q4_prefill_down_512x3072x1024": 37.84e6,
+    "c4_q4_prefill_down_512x3072x1024": 32.99e6,
+    "c4_f32a_q4_prefill_up_512x1024x3072": 27.29e6,
+    "c4_f32a_q4_prefill_down_512x3072x1024": 37.60e6,
 }
 
 

@@ -292,13 +292,12 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(
   // make five loads per wave): all five go out before the activations are prepared, which is little
   // work at such a K, so none of them pays a second trip to memory behind the barrier (5.94 -> 5.54
   // us; 640 x 32768 5.06 -> 4.74; with more rows the prologue is longer and the deeper queue loses).
-  // One row of Q4 with five or more loads per wave: four ahead instead of three (4096 x 14336 7.63 ->
-  // 7.45 us on one box, 7.73 -> 7.6 on another; 4096 x 28672 13.39 -> 13.06; five or six ahead, Q8
-  // with three, or more than one row with four measured level or slower, and so did a depth that
-  // covers all of a wave's loads where there is no tail step: 2048 x 8192 3.85 -> 4.03 us).
+  // (One row of Q4 with four ahead instead of three gains 0.15 us on 4096 x 14336 on three boxes of
+  // five and loses 0.26 us there and 0.55 us on 14336 x 4096 on a fourth: three it stays, 7.68-7.73
+  // us on all five.)
   // Three or four rows of Q4: two ahead (the rows' operands and sums leave fewer registers for loads
   // in flight; 4096 x 14336 at M = 4 11.7 -> 11.35 us, 14336 x 4096 13.7 -> 13.45; one ahead is slower again).
-  constexpr int kDepth = (TAIL && MROWS == 1) ? 5 : (MROWS == 1 && FMT == MGN_FMT_Q4 && STEPS * QPW >= 5) ? 4 : (MROWS > 2 && FMT == MGN_FMT_Q4) ? 2 : prefetch_depth<FMT>();
+  constexpr int kDepth = (TAIL && MROWS == 1) ? 5 : (MROWS > 2 && FMT == MGN_FMT_Q4) ? 2 : prefetch_depth<FMT>();
   // TAIL: K is STEPS full steps plus 1, 2 or 4 leftover blocks per column.  Instead of a second,
   // nearly empty step for every quad, one more step takes the leftovers of all QPW quads at once:
   // the MFMA's 16 blocks are independent, so slot b serves quad b / T, K block 16 * STEPS + b % T.
