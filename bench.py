@@ -91,8 +91,8 @@ MEASURED_TRAFFIC_BYTES = {
     "c2_q4_gate_up_576x3072": 1.33e6,
     "c2_q4_down_1536x576_add": 0.74e6,
     "c2_q4_q_576x576": 0.39e6,
-    "c4_q4_prefill_up_512x1024x3072": 18.99e6,
-    "c4_q4_prefill_down_512x3072x1024": 32.99e6,
+    "c4_q4_prefill_up_512x1024x3072": 19.00e6,
+    "c4_q4_prefill_down_512x3072x1024": 32.97e6,
     "c4_f32a_q4_prefill_up_512x1024x3072": 27.29e6,
     "c4_f32a_q4_prefill_down_512x3072x1024": 37.60e6,
 }

@@ -759,7 +759,7 @@ constexpr int resident_slices(bool f32a, int r) { return f32a && r == 2 ? 2 : 4;
 // a tile fall into different LDS banks.
 __host__ __device__ constexpr uint32_t meta_stride(int fmt, uint32_t nsl) { return nsl * kSliceBlocks * (fmt == MGN_FMT_Q4 ? 4 : 2) + 16; }
 
-template <int FMT, bool F32A, int R, int Q, bool PARK>
+template <int FMT, bool F32A, int R, int Q, bool PARK, bool LATE = false>
 __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restrict__ a, const void* __restrict__ meta_arg,
                                                              const void* __restrict__ quants_arg, uint32_t m, uint32_t kdim,
                                                              uint32_t n, uint32_t parts, uint32_t nslices, uint32_t colgroups,
@@ -867,7 +867,12 @@ __global__ __launch_bounds__(512) void tile_resident_kernel(const void* __restri
   // front of them delays the conversion that all waves wait for (first request after the second
   // task, one slice ahead from there on: 15.0 -> 14.0 us at M = 16 on 4096 x 14336; two slices
   // ahead or any request before the conversion measured 0.3-2.3 us slower).
-  constexpr int kFirstFetchAfterTask = NT > 1 ? 1 : 0;
+  // LATE (row groups of 32 fp16 rows on a chip that the launch fills): not before the last task.
+  // The eight tasks of such a workgroup read 64 KB of activations, and with every CU doing the
+  // same the weights requested in between only stand in their way: fp16 512 x 1024 x 3072 11.23 ->
+  // 10.93 us, 512 x 3072 x 1024 14.22 -> 14.0.  (On half a chip the early request wins: M = 64 on
+  // 4096 x 4096, 128 workgroups, 10.2 against 10.45 us; and with f32 activations a later one loses.)
+  constexpr int kFirstFetchAfterTask = NT > 1 ? (LATE ? NT - 1 : 1) : 0;
 #pragma unroll
   for (int t = 0; t < NT; t++) {
     convert_task<FMT, F32A>(xin[t], xok[t], img + t * UNITS, cr, cl);
@@ -1257,9 +1262,9 @@ bool plan_resident(const LaunchArgs& x, ResidentPlan* out) {
   return true;
 }
 
-template <int FMT, bool F32A, int R, int Q, bool PARK>
+template <int FMT, bool F32A, int R, int Q, bool PARK, bool LATE = false>
 int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& p) {
-  auto kern = tile_resident_kernel<FMT, F32A, R, Q, PARK>;
+  auto kern = tile_resident_kernel<FMT, F32A, R, Q, PARK, LATE>;
   static std::atomic<uint64_t> big_lds_done{0};
   if (p.lds > 64 * 1024)
     if (int e = enable_big_lds(kern, x.device, big_lds_done)) return e;
@@ -1276,8 +1281,12 @@ int launch_resident_q(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& 
 template <int FMT, bool F32A>
 int launch_resident_fa(ihipStream_t* s, const LaunchArgs& x, const ResidentPlan& p) {
   if constexpr (!F32A) {
-    if (p.r == 2)
-      return p.park ? launch_resident_q<FMT, F32A, 2, 1, true>(s, x, p) : launch_resident_q<FMT, F32A, 2, 1, false>(s, x, p);
+    if (p.r == 2) {
+      // the first weight request waits for the conversion when the launch fills the chip (see the kernel)
+      const bool late = (uint64_t)p.parts * p.colgroups * p.rowgroups * 10 >= (uint64_t)x.num_cus * 7;
+      if (p.park) return late ? launch_resident_q<FMT, F32A, 2, 1, true, true>(s, x, p) : launch_resident_q<FMT, F32A, 2, 1, true>(s, x, p);
+      return late ? launch_resident_q<FMT, F32A, 2, 1, false, true>(s, x, p) : launch_resident_q<FMT, F32A, 2, 1, false>(s, x, p);
+    }
   }
   if (p.r != 1) return (int)hipErrorInvalidValue;
   if (p.q == 1)
